@@ -1,0 +1,168 @@
+/*
+ * C ABI of the MI355X (gfx950) tiled-kernel library: dense GEMM (fp16 / bf16 / fp8),
+ * block-scaled MX GEMM (MXFP4 / MXFP8), and fused flash-attention forward / backward.
+ *
+ * Conventions shared by every entry point
+ *   - all pointers are DEVICE pointers unless stated otherwise; the caller owns every buffer
+ *     (the library allocates nothing and keeps nothing between calls);
+ *   - strides are in ELEMENTS of the tensor's dtype (packed fp4: in bytes);
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); calls are
+ *     asynchronous on that stream and never synchronise;
+ *   - the return value is 0 on success, a positive hipError_t when a launch failed, or a
+ *     negative MI355_E* code when an argument was rejected before anything was launched.
+ *     Nothing is thrown across this boundary.
+ *
+ * The reference interfaces each entry point stands in for are cited per function as
+ * path:line relative to the openai/triton source tree.
+ */
+#ifndef MI355_KERNELS_H
+#define MI355_KERNELS_H
+
+#include <stdint.h>
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* element types (the reference's names: python/triton/language/core.py:324-381) */
+enum {
+  MI355_F16 = 0,    /* fp16                        */
+  MI355_BF16 = 1,   /* bf16                        */
+  MI355_F8E4M3 = 2, /* fp8e4nv  (OCP e4m3fn)       */
+  MI355_F8E5M2 = 3, /* fp8e5    (OCP e5m2)         */
+  MI355_F32 = 4     /* fp32 (output only)          */
+};
+
+/* MX element formats for mi355_mx_gemm */
+enum {
+  MI355_MXFP4 = 0, /* e2m1, two codes per byte, element 2i in the low nibble */
+  MI355_MXFP8 = 1  /* e4m3fn, one code per byte                              */
+};
+
+/* code formats for mi355_dequant */
+enum {
+  MI355_DEQ_E4M3 = 0, /* one e4m3fn code per byte                          */
+  MI355_DEQ_E5M2 = 1, /* one e5m2 code per byte                            */
+  MI355_DEQ_E2M1 = 2, /* two e2m1 codes per byte, low nibble first         */
+  MI355_DEQ_E8M0 = 3  /* one e8m0 scale per byte: 2^(b-127), 255 -> NaN    */
+};
+
+/* activation fused on the fp32 accumulator (python/tutorials/03-matrix-multiplication.py:304-307, 320-322) */
+enum { MI355_ACT_NONE = 0, MI355_ACT_LEAKY_RELU = 1 };
+
+/* argument-error codes (negative); positive return values are hipError_t */
+enum {
+  MI355_OK = 0,
+  MI355_EINVAL = -1,   /* null pointer, non-positive size, unknown enum           */
+  MI355_EDTYPE = -2,   /* dtype combination not supported                         */
+  MI355_ESHAPE = -3,   /* shape constraint of the kernel family violated          */
+  MI355_ESTRIDE = -4,  /* stride / alignment constraint violated                  */
+  MI355_EDEVICE = -5   /* no gfx950 device current                                */
+};
+
+/* mi355_query selectors */
+enum {
+  MI355_Q_ABI_VERSION = 0,
+  MI355_Q_CU_COUNT = 1,
+  MI355_Q_IS_GFX950 = 2,
+  MI355_Q_LDS_BYTES = 3,
+  MI355_Q_CLOCK_KHZ = 4
+};
+
+/*
+ * C[M,N] = act( (a_scale*b_scale) * A[M,K] @ B[K,N] ), fp32 accumulation, one rounding to out_dtype.
+ *
+ * Stands in for the launch of `matmul_kernel` by the host wrappers
+ *   python/tutorials/03-matrix-multiplication.py:241-316 (kernel), :330-348 (`matmul`)
+ *   python/tutorials/09-persistent-matmul.py:48-102 (kernel), :105-138 (`matmul`, fp8e4nv)
+ * i.e. what the generated launcher third_party/amd/backend/driver.py:326-377 does for them.
+ * Same arguments as the kernel: three pointers, M N K, six strides (any strides are accepted;
+ * the MFMA path needs a unit stride on one axis of each operand, anything else runs a
+ * slower strided kernel on the GPU), plus ACTIVATION.  in_dtype is the type of A and B
+ * (they must match, python/triton/language/semantic.py:1355).  a_scale / b_scale are
+ * optional device pointers to one fp32 each (NULL = 1.0): per-tensor dequantisation
+ * scales for fp8 inputs, applied to the fp32 accumulator before activation and cast.
+ */
+int mi355_gemm(const void* A, const void* B, void* C,
+               int M, int N, int K,
+               int64_t stride_am, int64_t stride_ak,
+               int64_t stride_bk, int64_t stride_bn,
+               int64_t stride_cm, int64_t stride_cn,
+               int in_dtype, int out_dtype,
+               const float* a_scale, const float* b_scale,
+               int activation, void* stream);
+
+/*
+ * Block-scaled (OCP MX v1.0) GEMM: C[m,n] = sum_kb 2^(sA[m,kb]-127) 2^(sB[n,kb]-127) sum_{k in kb} A^[m,k] B^[n,k]
+ * with 32-element blocks along K.  A is [M, K] and B is [N, K] (both K-contiguous):
+ *   MXFP4: A_bytes[M, K/2], B_bytes[N, K/2];   MXFP8: A_bytes[M, K], B_bytes[N, K];
+ *   scales: sA[M, K/32], sB[N, K/32] e8m0 bytes (2^(b-127)); C[M,N] in out_dtype (bf16/fp16/fp32).
+ * lda/ldb are row pitches in BYTES, lds_a/lds_b row pitches of the scale matrices in bytes, ldc in elements.
+ * No counterpart exists in the reference snapshot (no dot_scaled / e8m0 / e2m1 anywhere in it);
+ * the operation is defined by the OCP Microscaling Formats specification v1.0.
+ */
+int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const uint8_t* sB, void* C,
+                  int M, int N, int K, int fmt, int out_dtype,
+                  int64_t lda, int64_t ldb, int64_t lds_a, int64_t lds_b, int64_t ldc,
+                  void* stream);
+
+/*
+ * Flash-attention forward: O = softmax(Q K^T * sm_scale [+ causal mask]) V per (z, h); also writes
+ * Mlse[z,h,n] = base-2 log-sum-exp of (q.k * sm_scale * log2 e), fp32.
+ * Stands in for the launch of `_attn_fwd` by `_attention.forward`
+ *   python/tutorials/06-fused-attention.py:98-187 (kernel), :25-75 (inner loop), :441-475 (host).
+ * q,k,v,o are [Z,H,N_CTX,D] with the four element strides given per tensor (last stride must be 1);
+ * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {64, 128}.
+ */
+int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* Mlse,
+                   int Z, int H, int N_CTX, int D,
+                   const int64_t* stride_q, const int64_t* stride_k,
+                   const int64_t* stride_v, const int64_t* stride_o, /* HOST arrays of 4 */
+                   float sm_scale, int causal, int dtype, void* stream);
+
+/*
+ * delta[z,h,n] = sum_d o[z,h,n,d] * do[z,h,n,d] in fp32.
+ * Stands in for `_attn_bwd_preprocess` (python/tutorials/06-fused-attention.py:190-204, launch :495-502).
+ * o and do share `stride` (HOST array of 4, last = 1); delta is contiguous [Z,H,N_CTX].
+ */
+int mi355_attn_bwd_preprocess(const void* o, const void* d_o, float* delta,
+                              int Z, int H, int N_CTX, int D,
+                              const int64_t* stride, int dtype, void* stream);
+
+/*
+ * Flash-attention backward: dq, dk, dv from q, k, v, do, Mlse (from the forward) and delta.
+ * Stands in for the launch of `_attn_bwd` by `_attention.backward`
+ *   python/tutorials/06-fused-attention.py:308-435 (kernel), :208-305 (inner loops), :478-517 (host).
+ * All of q,k,v,do,dq,dk,dv share one stride set (HOST array of 4, last = 1), as in the reference (:481).
+ * k is the ORIGINAL key tensor: the pre-scaling `k * (sm_scale / ln 2)` the reference does on the
+ * host (:490-492) is folded into the kernel.  causal = 0 gives the full (non-causal) backward,
+ * which the reference kernel cannot produce.  N_CTX must be a multiple of 128 (:494).
+ */
+int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
+                   const float* Mlse, const float* delta,
+                   void* dq, void* dk, void* dv,
+                   int Z, int H, int N_CTX, int D,
+                   const int64_t* stride,
+                   float sm_scale, int causal, int dtype, void* stream);
+
+/*
+ * out[i] = decode(codes[i]) in fp32 for n code BYTES (MI355_DEQ_E2M1 writes 2n values), using the
+ * decode routines the strided kernels use.  The formats are those of the reference type table
+ * (python/triton/language/core.py:352-363) and of its up-cast emulation
+ * (python/triton/runtime/interpreter.py:130-191, python/test/unit/language/test_conversions.py:178-209);
+ * e2m1 / e8m0 follow OCP MX v1.0.
+ */
+int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* stream);
+
+/* Device facts needed by callers (analogue of get_device_properties,
+ * third_party/amd/backend/driver.c:125-141).  Returns -1 for an unknown selector. */
+int mi355_query(int what);
+
+/* Static string for a return code of the functions above (never NULL). */
+const char* mi355_strerror(int code);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_KERNELS_H */

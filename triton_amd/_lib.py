@@ -1,0 +1,77 @@
+"""ctypes binding of the C ABI in include/mi355_kernels.h (the only way into the HIP kernels).
+
+There is deliberately no fallback: if the shared library has not been built, importing the
+operators fails with an instruction to build it, and every non-zero status of a C call
+becomes a Python exception.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libmi355_kernels.so"
+
+# enums of include/mi355_kernels.h
+F16, BF16, F8E4M3, F8E5M2, F32 = 0, 1, 2, 3, 4
+MXFP4, MXFP8 = 0, 1
+ACT_NONE, ACT_LEAKY_RELU = 0, 1
+DEQ_E4M3, DEQ_E5M2, DEQ_E2M1, DEQ_E8M0 = 0, 1, 2, 3
+Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ = 0, 1, 2, 3, 4
+
+I64x4 = c_int64 * 4
+
+# name -> (restype, argtypes); kept in one table so tests can check it against the header
+SIGNATURES = {
+    "mi355_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                           c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                           c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "mi355_mx_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_int, c_int, c_int, c_int, c_int,
+                              c_int64, c_int64, c_int64, c_int64, c_int64, c_void_p]),
+    "mi355_attn_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_int, c_int, c_int, c_int,
+                               POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+                               c_float, c_int, c_int, c_void_p]),
+    "mi355_attn_bwd_preprocess": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                          POINTER(c_int64), c_int, c_void_p]),
+    "mi355_attn_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                               POINTER(c_int64), c_float, c_int, c_int, c_void_p]),
+    "mi355_dequant": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "mi355_query": (c_int, [c_int]),
+    "mi355_strerror": (c_char_p, [c_int]),
+}
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the kernel library once; raise if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise ImportError(
+                f"{LIB_PATH} is missing: build the HIP kernels first with "
+                "`python -m triton_amd.build` (needs hipcc); there is no CPU fallback")
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def strerror(code: int) -> str:
+    return load().mi355_strerror(code).decode()
+
+
+def check(code: int, what: str) -> None:
+    """Map a C status to the reference's exception convention
+    (third_party/amd/backend/driver.py:258-269: HIP failures are RuntimeError)."""
+    if code == 0:
+        return
+    if code > 0:
+        raise RuntimeError(f"Triton Error [HIP]:  Code: {code}, Messsage: {strerror(code)} ({what})")
+    raise ValueError(f"{what}: {strerror(code)} (code {code})")

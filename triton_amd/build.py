@@ -1,0 +1,78 @@
+"""Build the gfx950 kernel library (`csrc/*.hip` -> `csrc/libmi355_kernels.so`) with hipcc.
+
+Plain ahead-of-time compilation: the reference compiles its kernels at first launch through a
+JIT (python/triton/runtime/jit.py:642-648); here every kernel is a fixed HIP source, so the
+"compiler" is one hipcc invocation per file and a link.  Run as `python -m triton_amd.build`.
+"""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+
+CSRC = Path(__file__).resolve().parent / "csrc"
+LIB_NAME = "libmi355_kernels.so"
+ARCH = "gfx950"
+
+# -packed-fp32-ops off: packed fp32 VALU forms are not used by these kernels.
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument", "-Wno-ignored-attributes",
+]
+
+
+def hipcc_path() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found (set HIPCC or install ROCm)")
+
+
+def lib_path() -> Path:
+    return CSRC / LIB_NAME
+
+
+def _compile(hipcc: str, src: Path, obj: Path, verbose: bool) -> None:
+    cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    # hipcc's host pass prints a harmless note about the device-only target feature
+    err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{err}")
+    if verbose and err.strip():
+        print(err, flush=True)
+
+
+def build(verbose: bool = False, jobs: int | None = None) -> Path:
+    """Compile every csrc/*.hip and link the shared library; always recompiles."""
+    hipcc = hipcc_path()
+    objdir = CSRC / "_build"
+    objdir.mkdir(exist_ok=True)
+    srcs = sorted(CSRC.glob("*.hip"))
+    if not srcs:
+        raise RuntimeError(f"no HIP sources under {CSRC}")
+    objs = [objdir / (s.stem + ".o") for s in srcs]
+    jobs = jobs or min(8, len(srcs), os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(lambda so: _compile(hipcc, so[0], so[1], verbose), zip(srcs, objs)))
+    out = lib_path()
+    tmp = out.with_suffix(".so.tmp")
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"link failed:\n{res.stderr}")
+    os.replace(tmp, out)
+    return out
+
+
+if __name__ == "__main__":
+    p = build(verbose="-v" in sys.argv)
+    print(p)

@@ -1,0 +1,227 @@
+// extern "C" entry points declared in include/mi355_kernels.h: argument validation, kernel
+// family / tile selection, launch.  Plays the role of the generated launcher of the reference
+// (third_party/amd/backend/driver.py:326-377): pointers and scalars in, one asynchronous
+// launch on the caller's stream out, an integer status back.
+#include <hip/hip_runtime.h>
+#include <stdlib.h>
+#include <string.h>
+#include <mutex>
+#include "../../include/mi355_kernels.h"
+#include "launch.h"
+
+using namespace mi355;
+
+namespace {
+
+struct DeviceInfo {
+  int ok = 0, cus = 0, gfx950 = 0, lds = 0, clock_khz = 0;
+};
+
+const DeviceInfo& device_info() {
+  static DeviceInfo info;
+  static std::once_flag once;
+  std::call_once(once, [] {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
+    info.cus = prop.multiProcessorCount;
+    info.gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+    info.lds = (int)prop.sharedMemPerBlock;
+    info.clock_khz = prop.clockRate;
+    info.ok = 1;
+  });
+  return info;
+}
+
+int env_int(const char* name, int dflt) {
+  const char* s = getenv(name);
+  return s && *s ? atoi(s) : dflt;
+}
+
+bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+int elem_size(int dtype) {
+  switch (dtype) {
+    case MI355_F16: case MI355_BF16: return 2;
+    case MI355_F8E4M3: case MI355_F8E5M2: return 1;
+    case MI355_F32: return 4;
+    default: return 0;
+  }
+}
+
+bool copy_strides(const int64_t* src, int64_t* dst) {
+  if (!src) return false;
+  for (int i = 0; i < 4; i++) dst[i] = src[i];
+  return true;
+}
+
+}  // namespace
+
+extern "C" {
+
+int mi355_query(int what) {
+  const DeviceInfo& d = device_info();
+  switch (what) {
+    case MI355_Q_ABI_VERSION: return 1;
+    case MI355_Q_CU_COUNT: return d.cus;
+    case MI355_Q_IS_GFX950: return d.gfx950;
+    case MI355_Q_LDS_BYTES: return d.lds;
+    case MI355_Q_CLOCK_KHZ: return d.clock_khz;
+    default: return -1;
+  }
+}
+
+const char* mi355_strerror(int code) {
+  switch (code) {
+    case MI355_OK: return "ok";
+    case MI355_EINVAL: return "invalid argument (null pointer, non-positive size or unknown enum)";
+    case MI355_EDTYPE: return "unsupported dtype combination";
+    case MI355_ESHAPE: return "shape not supported by this kernel family";
+    case MI355_ESTRIDE: return "stride or alignment not supported by this kernel family";
+    case MI355_EDEVICE: return "current device is not a gfx950 GPU";
+    default: break;
+  }
+  if (code > 0) return hipGetErrorString((hipError_t)code);
+  return "unknown error";
+}
+
+int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
+               int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+               int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+               int activation, void* stream_) {
+  if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
+  if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
+  if (in_dtype < MI355_F16 || in_dtype > MI355_F8E5M2) return MI355_EDTYPE;
+  if (out_dtype < MI355_F16 || out_dtype > MI355_F32) return MI355_EDTYPE;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  hipStream_t stream = (hipStream_t)stream_;
+  const int es = elem_size(in_dtype);
+  const bool is8 = es == 1;
+  const int vec = 16 / es;  // elements per 16-byte chunk
+
+  const bool out_ok = out_dtype == MI355_F16 || out_dtype == MI355_BF16 || out_dtype == MI355_F32;
+  const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
+  const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
+  const bool b_nmajor = !is8 && sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
+  // byte offsets inside one operand must fit the 32-bit-safe pointer arithmetic of the tile copies
+  const bool fast = out_ok && a_ok && (b_kmajor || b_nmajor) && env_int("MI355_GEMM_FORCE_STRIDED", 0) == 0;
+
+  if (!fast) {
+    GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype};
+    return gemm_strided_launch(s, stream);
+  }
+
+  GemmArgs p{};
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C;
+  p.M = M; p.N = N; p.K = K;
+  p.lda = sam * es;
+  p.ldb = (b_kmajor ? sbn : sbk) * es;
+  p.ldc = scm; p.scn = scn;
+  p.a_scale = a_scale; p.b_scale = b_scale;
+  p.activation = activation; p.out_dtype = out_dtype;
+  p.group_m = env_int("MI355_GEMM_GROUP_M", 8);
+  p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
+
+  const int cus = device_info().cus > 0 ? device_info().cus : 256;
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
+  tile = env_int("MI355_GEMM_TILE", tile);
+  if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
+  return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
+}
+
+int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const uint8_t* sB, void* C,
+                  int M, int N, int K, int fmt, int out_dtype,
+                  int64_t lda, int64_t ldb, int64_t lds_a, int64_t lds_b, int64_t ldc, void* stream_) {
+  if (!A || !sA || !B || !sB || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
+  if (fmt != MI355_MXFP4 && fmt != MI355_MXFP8) return MI355_EINVAL;
+  if (out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  if (K % 32 != 0) return MI355_ESHAPE;  // whole scale blocks only
+  const int64_t row_bytes = fmt == MI355_MXFP4 ? K / 2 : K;
+  if (lda < row_bytes || ldb < row_bytes || lds_a < K / 32 || lds_b < K / 32 || ldc < N) return MI355_ESTRIDE;
+  if (lda % 16 || ldb % 16 || !aligned(A, 16) || !aligned(B, 16)) return MI355_ESTRIDE;
+  MxGemmArgs p{A, sA, B, sB, (char*)C, M, N, K, lda, ldb, lds_a, lds_b, ldc, out_dtype,
+               env_int("MI355_GEMM_GROUP_M", 8)};
+  const int cus = device_info().cus > 0 ? device_info().cus : 256;
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
+  tile = env_int("MI355_GEMM_TILE", tile);
+  return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
+}
+
+int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* stream_) {
+  if (!codes || !out || n < 0) return MI355_EINVAL;
+  if (fmt < MI355_DEQ_E4M3 || fmt > MI355_DEQ_E8M0) return MI355_EINVAL;
+  if (n == 0) return MI355_OK;
+  if (n > (int64_t)0x7FFFFFFF * 256) return MI355_ESHAPE;
+  return dequant_launch(codes, out, n, fmt, (hipStream_t)stream_);
+}
+
+static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype) {
+  if (Z <= 0 || H <= 0 || N_CTX <= 0) return MI355_EINVAL;
+  if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
+  if (D != 64 && D != 128) return MI355_ESHAPE;
+  if (N_CTX % 128 != 0) return MI355_ESHAPE;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  p.Z = Z; p.H = H; p.N = N_CTX; p.D = D;
+  return MI355_OK;
+}
+
+static bool attn_stride_ok(const int64_t* s, const void* ptr, int D) {
+  return s[3] == 1 && s[2] >= D && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && aligned(ptr, 16);
+}
+
+int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* Mlse,
+                   int Z, int H, int N_CTX, int D,
+                   const int64_t* sq, const int64_t* sk, const int64_t* sv, const int64_t* so,
+                   float sm_scale, int causal, int dtype, void* stream_) {
+  if (!q || !k || !v || !o || !Mlse) return MI355_EINVAL;
+  AttnArgs p{};
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  if (rc) return rc;
+  if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))
+    return MI355_EINVAL;
+  if (!attn_stride_ok(p.sq, q, D) || !attn_stride_ok(p.sk, k, D) || !attn_stride_ok(p.sv, v, D) ||
+      !attn_stride_ok(p.so, o, D))
+    return MI355_ESTRIDE;
+  p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
+  p.sm_scale = sm_scale; p.causal = causal != 0;
+  return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
+}
+
+int mi355_attn_bwd_preprocess(const void* o, const void* d_o, float* delta,
+                              int Z, int H, int N_CTX, int D, const int64_t* stride, int dtype, void* stream_) {
+  if (!o || !d_o || !delta) return MI355_EINVAL;
+  AttnArgs p{};
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  if (rc) return rc;
+  if (!copy_strides(stride, p.so)) return MI355_EINVAL;
+  if (!attn_stride_ok(p.so, o, D) || !aligned(d_o, 16)) return MI355_ESTRIDE;
+  p.o = (char*)o; p.d_o = (const char*)d_o; p.delta = delta;
+  // delta is written through the non-const alias below
+  p.lse = delta;
+  return attn_bwd_pre_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
+}
+
+int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
+                   const float* Mlse, const float* delta, void* dq, void* dk, void* dv,
+                   int Z, int H, int N_CTX, int D, const int64_t* stride,
+                   float sm_scale, int causal, int dtype, void* stream_) {
+  if (!q || !k || !v || !d_o || !Mlse || !delta || !dq || !dk || !dv) return MI355_EINVAL;
+  AttnArgs p{};
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  if (rc) return rc;
+  if (!copy_strides(stride, p.sq)) return MI355_EINVAL;
+  if (!attn_stride_ok(p.sq, q, D) || !aligned(k, 16) || !aligned(v, 16) || !aligned(d_o, 16) ||
+      !aligned(dq, 16) || !aligned(dk, 16) || !aligned(dv, 16))
+    return MI355_ESTRIDE;
+  p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.d_o = (const char*)d_o;
+  p.lse = const_cast<float*>(Mlse); p.delta = delta;
+  p.dq = (char*)dq; p.dk = (char*)dk; p.dv = (char*)dv;
+  p.sm_scale = sm_scale; p.causal = causal != 0;
+  return attn_bwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
+}
+
+}  // extern "C"

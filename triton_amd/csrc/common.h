@@ -1,0 +1,167 @@
+// Shared device-side helpers for the gfx950 kernels: vector types, MFMA wrappers,
+// LDS swizzles, direct global->LDS tile copies and fp32 -> 16-bit conversions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <utility>
+#include <type_traits>
+
+namespace mi355 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) _Float16 f16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(8))) short s16x8;
+typedef __attribute__((ext_vector_type(2))) int i32x2;
+typedef __attribute__((ext_vector_type(4))) int i32x4;
+typedef __attribute__((ext_vector_type(8))) int i32x8;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+
+#define LDS_PTR(T) T __attribute__((address_space(3)))*
+
+struct bf16_t { using vec8 = bf16x8; using vec4 = bf16x4; using scalar = __bf16; };
+struct f16_t  { using vec8 = f16x8;  using vec4 = f16x4;  using scalar = _Float16; };
+
+// D(32x32 fp32) += A(32x16) * B(16x32).  Lane l supplies A[l%32][8*(l/32) .. +8] and
+// B[8*(l/32) .. +8][l%32]; accumulator register r of lane l is D[(r/4)*8 + 4*(l/32) + r%4][l%32].
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+}
+
+// fp32 -> 16-bit, round to nearest even (the compiler emits v_cvt_pk_bf16_f32 / v_cvt_f16_f32).
+template <typename S> __device__ __forceinline__ S cvt16(float x) { return (S)x; }
+
+// Byte offset of 16-byte chunk `chunk` (0..7) of row `row` in an LDS tile whose rows are
+// 128 bytes: the chunk index is XORed with the low 3 row bits, so 8 consecutive rows reading
+// the same logical chunk touch 8 distinct 16-byte bank groups.
+__device__ __forceinline__ int swz128(int row, int chunk) {
+  return row * 128 + (((chunk ^ row) & 7) << 4);
+}
+
+// Builtins that need gfx950 target features are hidden from hipcc's host pass: a kernel
+// template that reaches one there silently loses its host-side launch stub.
+#if defined(__HIP_DEVICE_COMPILE__)
+#define MI355_DEVICE_PASS 1
+#else
+#define MI355_DEVICE_PASS 0
+#endif
+
+// 16 bytes per lane straight from global memory into LDS: lane i of the wave writes
+// lds_wave_base + 16 * i (the LDS address is wave-uniform, the global address per lane).
+__device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds_wave_base) {
+#if MI355_DEVICE_PASS
+  __builtin_amdgcn_global_load_lds(gsrc, lds_wave_base, 16, 0, 0);
+#endif
+}
+
+// Copy a [ROWS x 128 bytes] tile (rows `pitch` bytes apart in global memory) into a swizzled
+// LDS tile with direct global->LDS loads.  One wave instruction moves 64 x 16 B = 8 rows; the
+// LDS side of such a load is linear in the lane id, so the swizzle is applied to the SOURCE
+// chunk each lane fetches.  `gsrc[i]` are per-lane source pointers prepared by tile_src_ptrs.
+template <int ROWS, int NWAVES>
+struct TileCopy128 {
+  static constexpr int kIters = ROWS / 8 / NWAVES;
+  static_assert(ROWS % (8 * NWAVES) == 0, "tile rows must split evenly over the waves");
+
+  // Pointer (to the k = 0 tile) that lane `lane` of wave `wave` fetches in iteration i.
+  // row_limit clamps rows past the matrix edge onto the last valid row (their products are
+  // never stored).
+  __device__ static const char* src(const char* base, int64_t pitch, int row0, int row_limit,
+                                    int wave, int lane, int i) {
+    int r = (i * NWAVES + wave) * 8 + (lane >> 3);
+    int lc = (lane & 7) ^ (r & 7);
+    int gr = row0 + r;
+    gr = gr < row_limit ? gr : row_limit - 1;
+    return base + (int64_t)gr * pitch + lc * 16;
+  }
+};
+
+// Compile-time counted loop: f(std::integral_constant<int, 0>) ... f(<N-1>), so that loop indices
+// can be used as template arguments / instruction immediates.
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, Is...>) {
+  (f(std::integral_constant<int, Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// LDS fragment reads issued as inline assembly.  The compiler cannot tell that a transpose
+// read of one LDS stage does not alias an in-flight direct global->LDS load into the other
+// stage and would wait for all outstanding loads first; reads it does not see are not
+// delayed.  The price is that their completion has to be awaited by hand: lds_wait<N>()
+// blocks until at most N LDS operations are outstanding, and lds_use(x) pins a register
+// written by such a read so that no consumer is scheduled before the wait.
+// (Hidden from the host pass like the builtins above.)
+template <int OFF>
+__device__ __forceinline__ i32x4 lds_read_b128(unsigned addr) {
+  i32x4 v = {};
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ i32x2 lds_read_tr16_b64(unsigned addr) {
+  i32x2 v = {};
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ i32x2 lds_read_tr8_b64(unsigned addr) {
+  i32x2 v = {};
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int N>
+__device__ __forceinline__ void lds_wait() {
+#if MI355_DEVICE_PASS
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"i"(N));
+#endif
+}
+template <typename V>
+__device__ __forceinline__ void lds_use(V& v) {
+#if MI355_DEVICE_PASS
+  asm volatile("" : "+v"(v));
+#endif
+}
+__device__ __forceinline__ unsigned lds_addr(LDS_PTR(const void) p) { return (unsigned)(uintptr_t)p; }
+
+__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
+__device__ __forceinline__ void wait_all() { __builtin_amdgcn_s_waitcnt(0); }
+
+// Map a hardware workgroup id to a logical one so that ids that are consecutive in the
+// logical order run on the same XCD (hardware deals workgroups round-robin over 8 XCDs,
+// each with its own L2).
+__device__ __forceinline__ int xcd_remap(int pid, int total) {
+  constexpr int X = 8;
+  int per = (total + X - 1) / X;
+  int tall = total % X;
+  int xcd = pid % X, local = pid / X;
+  if (tall == 0 || xcd < tall) return xcd * per + local;
+  return tall * per + (xcd - tall) * (per - 1) + local;
+}
+
+// Grouped ("super-row") tile order of the reference GEMM: consecutive ids walk GROUP_M tiles
+// down before stepping one tile right (python/tutorials/03-matrix-multiplication.py:265-273).
+__device__ __forceinline__ void grouped_tile(int pid, int num_m, int num_n, int group_m, int& pm, int& pn) {
+  int in_group = group_m * num_n;
+  int gid = pid / in_group;
+  int first = gid * group_m;
+  int gsz = min(num_m - first, group_m);
+  pm = first + (pid % in_group) % gsz;
+  pn = (pid % in_group) / gsz;
+}
+
+}  // namespace mi355

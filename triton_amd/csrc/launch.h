@@ -1,0 +1,59 @@
+// Host-side argument blocks and launcher prototypes shared by the kernel files and the C ABI.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace mi355 {
+
+struct GemmArgs {
+  const char* A;  // [M,K], K-contiguous on the MFMA paths
+  const char* B;  // [K,N] (N- or K-contiguous)
+  char* C;        // [M,N]
+  int M, N, K;
+  int64_t lda;    // MFMA paths: row pitch of A in BYTES
+  int64_t ldb;    // MFMA paths: pitch in BYTES between consecutive k rows (row-major B) or n rows (K-major B)
+  int64_t ldc;    // elements between consecutive C rows
+  int64_t scn;    // elements between consecutive C columns
+  const float* a_scale;
+  const float* b_scale;
+  int activation;
+  int out_dtype;  // MI355_F16 / MI355_BF16 / MI355_F32 (fp8 kernels also MI355_F8E4M3)
+  int group_m;
+  int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
+};
+
+// generic strided kernel: strides in elements, any dtype the ABI knows
+struct GemmStridedArgs {
+  const void* A; const void* B; void* C;
+  int M, N, K;
+  int64_t sam, sak, sbk, sbn, scm, scn;
+  const float* a_scale; const float* b_scale;
+  int activation, in_dtype, out_dtype;
+};
+
+struct MxGemmArgs {
+  const uint8_t* A; const uint8_t* sA; const uint8_t* B; const uint8_t* sB; char* C;
+  int M, N, K;
+  int64_t lda, ldb, lds_a, lds_b, ldc;
+  int out_dtype, group_m;
+};
+
+struct AttnArgs {
+  const char* q; const char* k; const char* v; char* o; float* lse;
+  const char* d_o; const float* delta; char* dq; char* dk; char* dv;
+  int Z, H, N, D;
+  int64_t sq[4], sk[4], sv[4], so[4];  // element strides
+  float sm_scale;
+  int causal;
+};
+
+int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
+int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
+int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
+int mx_gemm_launch(const MxGemmArgs& p, int fmt, int tile, hipStream_t stream);
+int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int dequant_launch(const uint8_t* codes, float* out, int64_t n, int fmt, hipStream_t stream);
+
+}  // namespace mi355

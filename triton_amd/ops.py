@@ -1,0 +1,239 @@
+"""Host wrappers: drop-in `matmul(a, b)` / `attention(q, k, v, causal, sm_scale)` of the
+reference tutorials plus `mx_matmul`, on top of the C ABI.
+
+Mirrors, argument for argument,
+  python/tutorials/03-matrix-multiplication.py:330-348   matmul(a, b, activation="")
+  python/tutorials/06-fused-attention.py:438-520         _attention / attention
+  python/tutorials/09-persistent-matmul.py:105-138       matmul(a, b) with out dtype = in dtype
+Tensors may be torch tensors or any object exposing data_ptr(), dtype, shape, stride(i)
+and device (the duck typing of the reference launcher, third_party/amd/backend/driver.py:285-323).
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+_TORCH_TO_ABI = {
+    torch.float16: _lib.F16,
+    torch.bfloat16: _lib.BF16,
+    torch.float8_e4m3fn: _lib.F8E4M3,
+    torch.float8_e5m2: _lib.F8E5M2,
+    torch.float32: _lib.F32,
+}
+# names the reference uses for reinterpret()-ed tensors (python/triton/runtime/jit.py:406-429)
+_NAME_TO_ABI = {
+    "fp16": _lib.F16, "bf16": _lib.BF16, "fp8e4nv": _lib.F8E4M3, "fp8e5": _lib.F8E5M2, "fp32": _lib.F32,
+    "float16": _lib.F16, "bfloat16": _lib.BF16, "float8_e4m3fn": _lib.F8E4M3, "float8_e5m2": _lib.F8E5M2,
+}
+_ABI_TO_TORCH = {v: k for k, v in _TORCH_TO_ABI.items()}
+
+
+def _abi_dtype(t) -> int:
+    dt = t.dtype
+    if dt in _TORCH_TO_ABI:
+        return _TORCH_TO_ABI[dt]
+    name = getattr(dt, "name", None) or str(dt)
+    name = name.split(".")[-1]
+    if name in _NAME_TO_ABI:
+        return _NAME_TO_ABI[name]
+    raise TypeError(f"unsupported dtype {dt}")
+
+
+def _check_device(idx: int, t) -> None:
+    dev = getattr(t, "device", None)
+    if dev is None and hasattr(t, "base"):
+        dev = getattr(t.base, "device", None)
+    if dev is not None and getattr(dev, "type", "cuda") != "cuda":
+        raise ValueError(f"Pointer argument (at {idx}) cannot be accessed from Triton (cpu tensor?)")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _is_contiguous(t) -> bool:
+    if hasattr(t, "is_contiguous"):
+        return t.is_contiguous()
+    expect = 1
+    for d in range(len(t.shape) - 1, -1, -1):
+        if t.shape[d] != 1 and t.stride(d) != expect:
+            return False
+        expect *= t.shape[d]
+    return True
+
+
+def _scale_ptr(s, device):
+    """None, a python float or a 1-element fp32 device tensor -> (pointer or None, keep-alive)."""
+    if s is None:
+        return None, None
+    if not isinstance(s, torch.Tensor):
+        s = torch.tensor([float(s)], dtype=torch.float32, device=device)
+    assert s.dtype == torch.float32 and s.numel() == 1, "scales are one fp32 value per tensor"
+    _check_device(-1, s)
+    return s.data_ptr(), s
+
+
+def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None):
+    """C = act((a_scale*b_scale) * A @ B) with fp32 accumulation.
+
+    Same contract as the reference wrapper (03:330-348): A must be contiguous, B may have any
+    strides (the reference passes `b.T` for fp8, 03:378-382), the result is fp16 for fp16 / fp8
+    inputs.  Extensions, all keyword-only and defaulting to the reference behaviour: bf16
+    inputs give a bf16 result, `out_dtype` overrides the result type, `a_scale` / `b_scale`
+    are per-tensor fp32 dequantisation scales.
+    """
+    assert a.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert _is_contiguous(a), "Matrix A must be contiguous"
+    in_dt = _abi_dtype(a)
+    assert in_dt == _abi_dtype(b), "Incompatible dtypes"
+    _check_device(0, a)
+    _check_device(1, b)
+    M, K = a.shape
+    K, N = b.shape
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if in_dt == _lib.BF16 else torch.float16
+    if activation not in ("", "leaky_relu"):
+        raise KeyError(f"unknown ACTIVATION {activation!r}")
+    device = a.device if isinstance(a, torch.Tensor) else torch.device("cuda", torch.cuda.current_device())
+    c = torch.empty((M, N), device=device, dtype=out_dtype)
+    if M == 0 or N == 0:
+        return c
+    if K == 0:
+        return c.zero_()
+    pa, keep_a = _scale_ptr(a_scale, device)
+    pb, keep_b = _scale_ptr(b_scale, device)
+    rc = _lib.load().mi355_gemm(
+        a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+        a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+        in_dt, _TORCH_TO_ABI[out_dtype], pa, pb,
+        _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE, _stream())
+    _lib.check(rc, "mi355_gemm")
+    return c
+
+
+def matmul_like_input(a, b):
+    """`matmul(a, b)` of the persistent-matmul tutorial (09:105-138): result dtype = input dtype
+    (fp16 -> fp16, fp8e4nv -> fp8e4nv); A need not be contiguous there."""
+    assert a.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert a.dtype == b.dtype, "Incompatible dtypes"
+    in_dt = _abi_dtype(a)
+    _check_device(0, a)
+    _check_device(1, b)
+    M, K = a.shape
+    K, N = b.shape
+    c = torch.empty((M, N), device=a.device, dtype=a.dtype)
+    rc = _lib.load().mi355_gemm(
+        a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+        a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+        in_dt, in_dt, None, None, _lib.ACT_NONE, _stream())
+    _lib.check(rc, "mi355_gemm")
+    return c
+
+
+def mx_matmul(a_packed, a_scale, b_packed, b_scale, fmt="mxfp4", out_dtype=torch.bfloat16):
+    """Block-scaled matmul C[M,N] = A[M,K] . B[N,K]^T (OCP MX v1.0, 32-element blocks along K).
+
+    mxfp4: a_packed [M, K/2] / b_packed [N, K/2] uint8 (e2m1, element 2i in the low nibble);
+    mxfp8: [M, K] / [N, K] float8_e4m3fn or uint8 codes; scales [M, K/32] / [N, K/32] uint8
+    e8m0.  No counterpart in the reference snapshot.
+    """
+    f = {"mxfp4": _lib.MXFP4, "mxfp8": _lib.MXFP8}[fmt]
+    for i, t in enumerate((a_packed, a_scale, b_packed, b_scale)):
+        _check_device(i, t)
+        assert t.dim() == 2 and t.stride(1) == 1, "operands and scales must be row-major 2-D"
+        assert t.element_size() == 1, "packed operands and scales are byte tensors"
+    M, KB = a_packed.shape
+    N = b_packed.shape[0]
+    K = KB * 2 if f == _lib.MXFP4 else KB
+    assert b_packed.shape[1] == KB, "Incompatible dimensions"
+    assert K % 32 == 0, "K must be a multiple of the 32-element scale block"
+    assert tuple(a_scale.shape) == (M, K // 32) and tuple(b_scale.shape) == (N, K // 32), "scale shape must be [rows, K/32]"
+    c = torch.empty((M, N), device=a_packed.device, dtype=out_dtype)
+    rc = _lib.load().mi355_mx_gemm(
+        a_packed.data_ptr(), a_scale.data_ptr(), b_packed.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
+        M, N, K, f, _TORCH_TO_ABI[out_dtype],
+        a_packed.stride(0), b_packed.stride(0), a_scale.stride(0), b_scale.stride(0), c.stride(0), _stream())
+    _lib.check(rc, "mi355_mx_gemm")
+    return c
+
+
+def dequantize(codes: torch.Tensor, fmt: str) -> torch.Tensor:
+    """Decode narrow-format codes on the GPU with the kernels' own decode routines.
+    fmt: 'e4m3' | 'e5m2' | 'e8m0' (one value per byte) or 'e2m1' (two per byte, low nibble first)."""
+    f = {"e4m3": _lib.DEQ_E4M3, "e5m2": _lib.DEQ_E5M2, "e2m1": _lib.DEQ_E2M1, "e8m0": _lib.DEQ_E8M0}[fmt]
+    _check_device(0, codes)
+    assert codes.is_contiguous() and codes.element_size() == 1
+    n = codes.numel()
+    shape = list(codes.shape)
+    if f == _lib.DEQ_E2M1:
+        shape[-1] *= 2
+    out = torch.empty(shape, dtype=torch.float32, device=codes.device)
+    if n:
+        _lib.check(_lib.load().mi355_dequant(codes.data_ptr(), out.data_ptr(), n, f, _stream()), "mi355_dequant")
+    return out
+
+
+class _attention(torch.autograd.Function):
+    """Autograd function with the reference's forward/backward split (06:438-517)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, causal, sm_scale):
+        HEAD_DIM_Q, HEAD_DIM_K = q.shape[-1], k.shape[-1]
+        HEAD_DIM_V = v.shape[-1]
+        assert HEAD_DIM_Q == HEAD_DIM_K and HEAD_DIM_K == HEAD_DIM_V
+        assert HEAD_DIM_K in {16, 32, 64, 128, 256}
+        for i, t in enumerate((q, k, v)):
+            _check_device(i, t)
+        assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
+        dt = _abi_dtype(q)
+        o = torch.empty_like(q)
+        Z, H, N_CTX = q.shape[0], q.shape[1], q.shape[2]
+        M = torch.empty((Z, H, N_CTX), device=q.device, dtype=torch.float32)
+        I4 = _lib.I64x4
+        rc = _lib.load().mi355_attn_fwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr(),
+            Z, H, N_CTX, HEAD_DIM_K,
+            I4(*q.stride()), I4(*k.stride()), I4(*v.stride()), I4(*o.stride()),
+            float(sm_scale), int(bool(causal)), dt, _stream())
+        _lib.check(rc, "mi355_attn_fwd")
+        ctx.save_for_backward(q, k, v, o, M)
+        ctx.sm_scale = sm_scale
+        ctx.HEAD_DIM = HEAD_DIM_K
+        ctx.causal = causal
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, o, M = ctx.saved_tensors
+        assert do.is_contiguous()
+        assert q.stride() == k.stride() == v.stride() == o.stride() == do.stride()
+        dq = torch.empty_like(q)
+        dk = torch.empty_like(k)
+        dv = torch.empty_like(v)
+        BATCH, N_HEAD, N_CTX = q.shape[:3]
+        PRE_BLOCK = 128
+        assert N_CTX % PRE_BLOCK == 0
+        delta = torch.empty_like(M)
+        dt = _abi_dtype(q)
+        I4 = _lib.I64x4
+        lib = _lib.load()
+        rc = lib.mi355_attn_bwd_preprocess(
+            o.data_ptr(), do.data_ptr(), delta.data_ptr(), BATCH, N_HEAD, N_CTX, ctx.HEAD_DIM,
+            I4(*o.stride()), dt, _stream())
+        _lib.check(rc, "mi355_attn_bwd_preprocess")
+        rc = lib.mi355_attn_bwd(
+            q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), M.data_ptr(), delta.data_ptr(),
+            dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), BATCH, N_HEAD, N_CTX, ctx.HEAD_DIM,
+            I4(*q.stride()), float(ctx.sm_scale), int(bool(ctx.causal)), dt, _stream())
+        _lib.check(rc, "mi355_attn_bwd")
+        return dq, dk, dv, None, None
+
+
+attention = _attention.apply
+
+
+def default_sm_scale(head_dim: int) -> float:
+    return 1.0 / math.sqrt(head_dim)
