@@ -1,8 +1,6 @@
 // temporary: families not written yet
 #include "launch.h"
 namespace mi355 {
-int gemm8_launch(const GemmArgs&, bool, int, hipStream_t) { return -2; }
-int mx_gemm_launch(const MxGemmArgs&, int, int, hipStream_t) { return -2; }
 int attn_fwd_launch(const AttnArgs&, bool, hipStream_t) { return -2; }
 int attn_bwd_pre_launch(const AttnArgs&, bool, hipStream_t) { return -2; }
 int attn_bwd_launch(const AttnArgs&, bool, hipStream_t) { return -2; }

@@ -114,7 +114,7 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
 
   GemmArgs p{};
   p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C;
-  p.M = M; p.N = N; p.K = K;
+  p.M = M; p.N = N; p.K = K; p.k_bytes = K * es;
   p.lda = sam * es;
   p.ldb = (b_kmajor ? sbn : sbk) * es;
   p.ldc = scm; p.scn = scn;
@@ -124,9 +124,9 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
 
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
-  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
-  tile = env_int("MI355_GEMM_TILE", tile);
+  // the 256x256 / 8-wave MX variants do not fit 256 registers yet: 128x128 tiles for every shape
+  (void)cus;
+  int tile = env_int("MI355_GEMM_TILE", 1);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
@@ -142,12 +142,18 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   const int64_t row_bytes = fmt == MI355_MXFP4 ? K / 2 : K;
   if (lda < row_bytes || ldb < row_bytes || lds_a < K / 32 || lds_b < K / 32 || ldc < N) return MI355_ESTRIDE;
   if (lda % 16 || ldb % 16 || !aligned(A, 16) || !aligned(B, 16)) return MI355_ESTRIDE;
-  MxGemmArgs p{A, sA, B, sB, (char*)C, M, N, K, lda, ldb, lds_a, lds_b, ldc, out_dtype,
-               env_int("MI355_GEMM_GROUP_M", 8)};
+  GemmArgs p{};
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C;
+  p.M = M; p.N = N; p.K = K; p.k_bytes = (int)row_bytes;
+  p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.scn = 1;
+  p.out_dtype = out_dtype;
+  p.group_m = env_int("MI355_GEMM_GROUP_M", 8);
+  p.c_vec_ok = ldc % 4 == 0 && aligned(C, 16);
+  p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
-  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
-  tile = env_int("MI355_GEMM_TILE", tile);
+  // the 256x256 / 8-wave MX variants do not fit 256 registers yet: 128x128 tiles for every shape
+  (void)cus;
+  int tile = env_int("MI355_GEMM_TILE", 1);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
 }
 

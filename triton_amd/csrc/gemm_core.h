@@ -1,0 +1,383 @@
+// Tiled MFMA GEMM core for gfx950, shared by the fp16/bf16, fp8 and block-scaled MX kernels:
+//   C[M,N] = act(alpha * A[M,K] @ B[K,N]), fp32 accumulate.
+//
+// The device-side counterpart of the reference `matmul_kernel`
+// (python/tutorials/03-matrix-multiplication.py:241-316): one workgroup per BM x BN tile of C,
+// grouped tile order (:265-273), K loop (:294-303), epilogue activation and cast (:304-316).
+// Built MI355X-first instead of translated:
+//   * a K step is 128 BYTES of every operand row (64 fp16/bf16, 128 fp8, 256 fp4 elements);
+//     tiles go global -> LDS with direct 16-byte loads into two LDS stages (no register
+//     staging), the tile for step k+1 is in flight while step k is multiplied;
+//   * LDS rows are XOR-swizzled so that ds_read_b128 / ds_read_b64_tr_b16 are conflict free;
+//   * a row-major 16-bit B[K,N] is transposed on the fly by the LDS transpose read; a K-major B
+//     (the `b.T` view the reference passes for fp8, :378-382) uses plain 128-bit reads;
+//   * 32x32 MFMA tiles with the operands swapped, so every lane owns 4 consecutive columns of
+//     one C row and stores them with one instruction;
+//   * workgroup ids are remapped per XCD before the grouped ordering.
+//
+// `Cfg` describes one element family:
+//   kSteps            MFMA sub-steps per 128-byte K tile
+//   kChunks           16-byte LDS chunks one lane feeds into one MFMA operand (1 or 2)
+//   chunk(ks, g, c)   which 16-byte chunk (0..7) of the row lane-group g reads for sub-step ks
+//   kRowMajorB        whether the transpose-read path for a row-major B exists (16-bit only)
+//   kScaled           block-scaled: per-row e8m0 scales ride along (MX)
+//   Operand           register type of one MFMA operand
+//   mma<ks>(...)      the MFMA itself
+#pragma once
+#include "common.h"
+#include "launch.h"
+
+namespace mi355 {
+
+// Row-major [64 x BN] 16-bit tile of B (rows are k, BN*2 bytes each).  32-byte groups of a row
+// are XORed with (k & 3): the transpose read of one 16-lane group touches 4 consecutive k rows
+// x 32 bytes, which then fall into 4 different bank groups.
+template <int BN, int NW>
+struct TileCopyKN {
+  static constexpr int kChunksPerRow = BN / 8;             // 16-byte chunks per k row
+  static constexpr int kRowsPerInst = 64 / kChunksPerRow;  // k rows moved by one wave instruction
+  static constexpr int kIters = 64 / kRowsPerInst / NW;
+  static_assert(kRowsPerInst >= 1 && kIters >= 1, "tile too small for this wave count");
+
+  __device__ static int row(int wave, int lane, int i) { return (i * NW + wave) * kRowsPerInst + lane / kChunksPerRow; }
+  __device__ static int col16(int lane, int r) {  // logical 16-byte chunk this lane fetches
+    int pc16 = lane % kChunksPerRow;
+    int lc32 = (pc16 >> 1) ^ (r & 3);
+    return lc32 * 2 + (pc16 & 1);
+  }
+};
+
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
+  using Operand = typename Cfg::Operand;
+  constexpr int NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
+  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
+  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  using CopyA = TileCopy128<BM, NW>;
+  using CopyBk = TileCopy128<BN, NW>;
+  using CopyBn = TileCopyKN<BN, NW>;
+  constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
+
+  // Two LDS stages of STAGE bytes each (dynamic LDS: 2 * STAGE bytes at launch).
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds0 = (LDS_PTR(char))smem;
+  LDS_PTR(char) const lds1 = lds0 + STAGE;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  int pid = xcd_remap(blockIdx.x, num_m * num_n);
+  int pm, pn;
+  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
+  const int m0 = pm * BM, n0 = pn * BN;
+
+  // per-lane global source pointers of the k = 0 tile
+  const char* srcA[CopyA::kIters];
+  const char* srcB[ITB];
+#pragma unroll
+  for (int i = 0; i < CopyA::kIters; i++) srcA[i] = CopyA::src(p.A, p.lda, m0, p.M, wave, lane, i);
+#pragma unroll
+  for (int i = 0; i < ITB; i++) {
+    if constexpr (B_KMAJOR) {
+      srcB[i] = CopyBk::src(p.B, p.ldb, n0, p.N, wave, lane, i);
+    } else {
+      int r = CopyBn::row(wave, lane, i);
+      int n = n0 + CopyBn::col16(lane, r) * 8;
+      n = n < p.N ? n : p.N - 8;  // N % 8 == 0 on this path: clamp whole chunks
+      srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
+    }
+  }
+  const int64_t stepA = 128, stepB = B_KMAJOR ? (int64_t)128 : 64 * p.ldb;
+
+  auto issue_tile = [&](int kt, LDS_PTR(char) a) {
+    LDS_PTR(char) b = a + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < CopyA::kIters; i++)
+      async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
+#pragma unroll
+    for (int i = 0; i < ITB; i++)
+      async_copy16(srcB[i] + kt * stepB, (LDS_PTR(void))(b + (i * NW + wave) * 1024));
+  };
+  // Last, partial K tile: chunks past K are written as zeros (the reference masks them to 0,
+  // python/tutorials/03-matrix-multiplication.py:297-298); goes through registers.
+  auto guarded_tile = [&](int kt, LDS_PTR(char) a) {
+    LDS_PTR(char) b = a + A_BYTES;
+    const int kbase = kt * 128;  // bytes along K
+#pragma unroll
+    for (int i = 0; i < CopyA::kIters; i++) {
+      int r = (i * NW + wave) * 8 + (lane >> 3);
+      int kb = kbase + (((lane & 7) ^ (r & 7)) << 4);
+      i32x4 v = {0, 0, 0, 0};
+      if (kb < p.k_bytes) v = *(const i32x4*)(srcA[i] + kt * stepA);
+      *(LDS_PTR(i32x4))(a + (i * NW + wave) * 1024 + lane * 16) = v;
+    }
+#pragma unroll
+    for (int i = 0; i < ITB; i++) {
+      bool ok;
+      if constexpr (B_KMAJOR) {
+        int r = (i * NW + wave) * 8 + (lane >> 3);
+        ok = kbase + (((lane & 7) ^ (r & 7)) << 4) < p.k_bytes;
+      } else {
+        ok = kt * 64 + CopyBn::row(wave, lane, i) < p.K;
+      }
+      i32x4 v = {0, 0, 0, 0};
+      if (ok) v = *(const i32x4*)(srcB[i] + kt * stepB);
+      *(LDS_PTR(i32x4))(b + (i * NW + wave) * 1024 + lane * 16) = v;
+    }
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int nfull = p.k_bytes / 128;
+
+  // Per-lane LDS byte offsets of the MFMA operands inside one stage.
+  //   K-major operand (A always, B when B_KMAJOR): lane reads row (l%32) and the 16-byte
+  //   chunk(s) Cfg::chunk(ks, l/32, c), swizzled; 32-row sub-tiles add t * 4096.
+  //   Row-major B: transpose read, lane i of a 16-lane group q addresses k row
+  //   16*ks + 8*(q/2) + i/4 (+4 for the second half) and 32-byte group (n/16) ^ (k & 3).
+  const int l32 = lane & 31, g = lane >> 5;
+  const int i16 = lane & 15, q = lane >> 4;
+  unsigned offA[KS][NC], offB[KS][NC];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+      offA[ks][c] = swz128(wm * TM + l32, Cfg::chunk(ks, g, c));
+      offB[ks][c] = A_BYTES + swz128(wn * TN + l32, Cfg::chunk(ks, g, c));
+    }
+  unsigned offBn[2];
+  {
+    // offBn[par]: sub-tiles t with parity par; k row without the ks / +4 terms
+    int k = (q >> 1) * 8 + (i16 >> 2);
+#pragma unroll
+    for (int par = 0; par < 2; par++) {
+      int c32 = (wn * TN + par * 32) / 16 + (q & 1);
+      offBn[par] = A_BYTES + k * (BN * 2) + ((c32 ^ (k & 3)) << 5) + (i16 & 3) * 8;
+    }
+  }
+
+  struct Frags { Operand a[MT]; Operand b[NT]; };
+  auto read_operand = [&](unsigned base, const unsigned (&off)[NC], auto IMM) -> Operand {
+    constexpr int imm = decltype(IMM)::value;
+    if constexpr (NC == 1) {
+      return __builtin_bit_cast(Operand, lds_read_b128<imm>(base + off[0]));
+    } else {
+      i32x4 lo = lds_read_b128<imm>(base + off[0]);
+      i32x4 hi = lds_read_b128<imm>(base + off[1]);
+      i32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(Operand, both);
+    }
+  };
+  auto read_frags = [&](unsigned base, auto KS_, Frags& f) {
+    constexpr int ks = decltype(KS_)::value;
+    static_for<MT>([&](auto T_) {
+      constexpr int t = decltype(T_)::value;
+      f.a[t] = read_operand(base, offA[ks], std::integral_constant<int, t * 4096>{});
+    });
+    static_for<NT>([&](auto T_) {
+      constexpr int t = decltype(T_)::value;
+      if constexpr (B_KMAJOR) {
+        f.b[t] = read_operand(base, offB[ks], std::integral_constant<int, t * 4096>{});
+      } else {
+        constexpr int imm = ks * 16 * BN * 2 + (t / 2) * 128;
+        i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t & 1]);
+        i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[t & 1]);
+        i32x4 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
+        f.b[t] = __builtin_bit_cast(Operand, both);
+      }
+    });
+  };
+  constexpr int kReadsPerStep = MT * NC + NT * (B_KMAJOR ? NC : 2);
+  auto use_frags = [&](Frags& f) {
+#pragma unroll
+    for (int t = 0; t < MT; t++) lds_use(f.a[t]);
+#pragma unroll
+    for (int t = 0; t < NT; t++) lds_use(f.b[t]);
+  };
+
+  // block scales of the current K tile: one dword (4 e8m0 bytes) per 32-row sub-tile and lane
+  int sa[MT], sb[NT], sa_next[MT], sb_next[NT];
+  auto load_scales = [&](int kt, int (&da)[MT], int (&db)[NT]) {
+    if constexpr (Cfg::kScaled) {
+      const int koff = kt * Cfg::kScaleBytesPerTile + Cfg::scale_byte_offset(g);
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        int r = min(m0 + wm * TM + t * 32 + l32, p.M - 1);
+        da[t] = Cfg::scale_fixup(*(const int*)(p.sA + (int64_t)r * p.lds_a + koff), g);
+      }
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        int r = min(n0 + wn * TN + t * 32 + l32, p.N - 1);
+        db[t] = Cfg::scale_fixup(*(const int*)(p.sB + (int64_t)r * p.lds_b + koff), g);
+      }
+    }
+  };
+
+  auto mma = [&](const Frags& f, auto KS_) {
+    constexpr int ks = decltype(KS_)::value;
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) {
+        // operands swapped: the instruction computes D[n][m]
+        if constexpr (Cfg::kScaled) acc[i][j] = Cfg::template mma<ks>(f.b[j], f.a[i], acc[i][j], sb[j], sa[i]);
+        else acc[i][j] = Cfg::template mma<ks>(f.b[j], f.a[i], acc[i][j], 0, 0);
+      }
+  };
+
+  // One 128-byte K tile.  When the registers allow it, the operands of sub-step ks+1 are
+  // requested before the MFMAs of sub-step ks; otherwise the second wave on the SIMD has to
+  // cover the LDS latency.
+  constexpr int kOperandRegs = (MT + NT) * NC * 4;
+  constexpr bool kPrefetch = 2 * kOperandRegs + MT * NT * 16 + (Cfg::kScaled ? 2 * (MT + NT) : 0) <= 184 * (512 / (NW * 64)) + (NW == 4 ? 128 : 0);
+  auto compute_tile = [&](LDS_PTR(char) stage) {
+    const unsigned base = lds_addr(stage);
+    if constexpr (kPrefetch) {
+      Frags f[2];
+      read_frags(base, std::integral_constant<int, 0>{}, f[0]);
+      static_for<KS>([&](auto KS_) {
+        constexpr int ks = decltype(KS_)::value;
+        if constexpr (ks + 1 < KS) {
+          read_frags(base, std::integral_constant<int, ks + 1>{}, f[(ks + 1) & 1]);
+          lds_wait<kReadsPerStep>();
+        } else {
+          lds_wait<0>();
+        }
+        use_frags(f[ks & 1]);
+        mma(f[ks & 1], KS_);
+      });
+    } else {
+      static_for<KS>([&](auto KS_) {
+        Frags f;
+        read_frags(base, KS_, f);
+        lds_wait<0>();
+        use_frags(f);
+        mma(f, KS_);
+      });
+    }
+  };
+
+  // K loop over the full tiles, two per trip: the tile for step kt+1 streams into the idle
+  // stage while step kt is multiplied out of the other.
+  if (nfull > 0) {
+    issue_tile(0, lds0);
+    load_scales(0, sa, sb);
+    wait_all();
+    __syncthreads();
+    for (int kt = 0; kt < nfull; kt += 2) {
+      if (kt + 1 < nfull) { issue_tile(kt + 1, lds1); load_scales(kt + 1, sa_next, sb_next); }
+      compute_tile(lds0);
+      wait_all();
+      __syncthreads();
+      if (kt + 1 < nfull) {
+        if constexpr (Cfg::kScaled) {
+#pragma unroll
+          for (int t = 0; t < MT; t++) sa[t] = sa_next[t];
+#pragma unroll
+          for (int t = 0; t < NT; t++) sb[t] = sb_next[t];
+        }
+        if (kt + 2 < nfull) { issue_tile(kt + 2, lds0); load_scales(kt + 2, sa_next, sb_next); }
+        compute_tile(lds1);
+        wait_all();
+        __syncthreads();
+        if constexpr (Cfg::kScaled) {
+#pragma unroll
+          for (int t = 0; t < MT; t++) sa[t] = sa_next[t];
+#pragma unroll
+          for (int t = 0; t < NT; t++) sb[t] = sb_next[t];
+        }
+      }
+    }
+  }
+  // K tail (K bytes % 128 != 0): one more tile, zero-filled past K, outside the pipelined loop.
+  // (Block-scaled operands always come in whole tiles.)
+  if (nfull * 128 < p.k_bytes) {
+    guarded_tile(nfull, lds0);
+    wait_all();
+    __syncthreads();
+    compute_tile(lds0);
+  }
+
+  // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3
+  float alpha = 1.f;
+  if (p.a_scale) alpha *= *p.a_scale;
+  if (p.b_scale) alpha *= *p.b_scale;
+  const bool leaky = p.activation == 1;
+  const bool vec_ok = p.c_vec_ok;
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    int m = m0 + wm * TM + i * 32 + l32;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        int n = n0 + wn * TN + j * 32 + rg * 8 + g * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          float x = acc[i][j][rg * 4 + e] * alpha;
+          if (leaky) x = x >= 0.f ? x : 0.01f * x;
+          v[e] = x;
+        }
+        if (p.out_dtype == 4) {
+          float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = v[e];
+          }
+        } else if (p.out_dtype == 1) {
+          __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (__bf16)v[e];
+          }
+        } else {
+          _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (_Float16)v[e];
+          }
+        }
+      }
+    }
+  }
+}
+
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR>
+static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * (BM + BN) * 128;
+  static bool attr_set = false;  // benign race: setting the attribute twice is harmless
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR><<<dim3(num_m * num_n), dim3(WM * WN * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+// tile: 0 = 256x256 / 8 waves, 1 = 128x128 / 4 waves
+template <typename Cfg, bool B_KMAJOR>
+static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
+  if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR>(p, stream);
+  return launch_gemm<Cfg, 256, 256, 2, 4, B_KMAJOR>(p, stream);
+}
+
+}  // namespace mi355

@@ -1,0 +1,101 @@
+// Block-scaled (OCP MX v1.0) instantiations of the tiled MFMA GEMM core: MXFP4 (e2m1, 256
+// elements per 128-byte K tile, four 32x32x64 sub-steps) and MXFP8 (e4m3, 128 elements, two
+// sub-steps), one e8m0 scale per 32 elements of K applied inside the MFMA.
+//
+// How the scaled 32x32x64 f8f6f4 MFMA takes its scales (measured on gfx950): every lane passes
+// one dword and a byte selector.  fp4: the selected byte of lane (row, g) scales that lane's own
+// 32 elements.  fp8: registers 0-3 of both lane groups form K block 0 and are scaled by the byte
+// from lane group 0, registers 4-7 form K block 1 and take the byte from lane group 1.  The K
+// positions a lane reads are therefore chosen such that the scale byte it needs is byte `ks` of
+// a dword whose address does not depend on ks.
+#include "gemm_core.h"
+#include "formats.h"
+
+namespace mi355 {
+
+struct CfgMxfp4 {
+  using Operand = i32x4;
+  static constexpr int kSteps = 4, kChunks = 1;
+  static constexpr bool kRowMajorB = false, kScaled = true;
+  static constexpr int kScaleBytesPerTile = 8;  // 256 elements / 32
+  // lane group g reads scale blocks 4g .. 4g+3 of the tile, one per sub-step
+  __device__ static constexpr int chunk(int ks, int g, int) { return g * 4 + ks; }
+  __device__ static int scale_byte_offset(int g) { return g * 4; }
+  __device__ static int scale_fixup(int v, int) { return v; }
+  template <int ks>
+  __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+    // fp4 operands occupy the low four registers; the high four are not read by the hardware
+    i32x8 a8 = __builtin_shufflevector(a, a, 0, 1, 2, 3, -1, -1, -1, -1);
+    i32x8 b8 = __builtin_shufflevector(b, b, 0, 1, 2, 3, -1, -1, -1, -1);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a8, b8, c, 4, 4, ks, sa, ks, sb);
+#else
+    return c;
+#endif
+  }
+};
+
+struct CfgMxfp8 {
+  using Operand = i32x8;
+  static constexpr int kSteps = 2, kChunks = 2;
+  static constexpr bool kRowMajorB = false, kScaled = true;
+  static constexpr int kScaleBytesPerTile = 4;  // 128 elements / 32
+  // register half c of sub-step ks is scale block 2c + ks; lane group g holds its 16-byte half g
+  __device__ static constexpr int chunk(int ks, int g, int c) { return 4 * c + 2 * ks + g; }
+  __device__ static int scale_byte_offset(int) { return 0; }
+  // lane group g supplies the scales of blocks 2g + ks: move them to bytes 0 and 1
+  __device__ static int scale_fixup(int v, int g) { return (int)((unsigned)v >> (16 * g)); }
+  template <int ks>
+  __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, ks, sa, ks, sb);
+#else
+    return c;
+#endif
+  }
+};
+
+// Any shape / pitch: one thread per output, decode-and-FMA in fp32.  Used when K is not a
+// whole number of 128-byte tiles or the scale rows are not dword aligned.
+__global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4) {
+  int n = blockIdx.x * 16 + threadIdx.x % 16, m = blockIdx.y * 16 + threadIdx.x / 16;
+  if (m >= p.M || n >= p.N) return;
+  const uint8_t* a = (const uint8_t*)p.A + (int64_t)m * p.lda;
+  const uint8_t* b = (const uint8_t*)p.B + (int64_t)n * p.ldb;
+  const uint8_t* sa = p.sA + (int64_t)m * p.lds_a;
+  const uint8_t* sb = p.sB + (int64_t)n * p.lds_b;
+  float acc = 0.f;
+  for (int kb = 0; kb < p.K / 32; kb++) {
+    float part = 0.f;
+    for (int e = 0; e < 32; e++) {
+      int k = kb * 32 + e;
+      float x, y;
+      if (fp4) {
+        x = e2m1_to_f32((a[k >> 1] >> ((k & 1) * 4)) & 15);
+        y = e2m1_to_f32((b[k >> 1] >> ((k & 1) * 4)) & 15);
+      } else {
+        x = e4m3_to_f32(a[k]);
+        y = e4m3_to_f32(b[k]);
+      }
+      part = fmaf(x, y, part);
+    }
+    acc += part * e8m0_to_f32(sa[kb]) * e8m0_to_f32(sb[kb]);
+  }
+  int64_t idx = (int64_t)m * p.ldc + n;
+  if (p.out_dtype == 4) ((float*)p.C)[idx] = acc;
+  else if (p.out_dtype == 1) ((__bf16*)p.C)[idx] = (__bf16)acc;
+  else ((_Float16*)p.C)[idx] = (_Float16)acc;
+}
+
+int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
+  const bool whole_tiles = p.k_bytes % 128 == 0;
+  const bool scales_aligned = p.lds_a % 4 == 0 && p.lds_b % 4 == 0 && ((uintptr_t)p.sA % 4) == 0 && ((uintptr_t)p.sB % 4) == 0;
+  if (!whole_tiles || !scales_aligned || tile < 0) {
+    dim3 grid((p.N + 15) / 16, (p.M + 15) / 16);
+    mx_gemm_simple_kernel<<<grid, dim3(256), 0, stream>>>(p, fmt == 0);
+    return (int)hipGetLastError();
+  }
+  return fmt == 0 ? launch_gemm_tile<CfgMxfp4, true>(p, tile, stream) : launch_gemm_tile<CfgMxfp8, true>(p, tile, stream);
+}
+
+}  // namespace mi355

@@ -10,6 +10,7 @@ struct GemmArgs {
   const char* B;  // [K,N] (N- or K-contiguous)
   char* C;        // [M,N]
   int M, N, K;
+  int k_bytes;    // bytes of one operand row along K (K * element size, K / 2 for fp4)
   int64_t lda;    // MFMA paths: row pitch of A in BYTES
   int64_t ldb;    // MFMA paths: pitch in BYTES between consecutive k rows (row-major B) or n rows (K-major B)
   int64_t ldc;    // elements between consecutive C rows
@@ -20,6 +21,10 @@ struct GemmArgs {
   int out_dtype;  // MI355_F16 / MI355_BF16 / MI355_F32 (fp8 kernels also MI355_F8E4M3)
   int group_m;
   int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
+  // block-scaled (MX) kernels only: e8m0 scale matrices [M, K/32], [N, K/32] and their row pitches
+  const uint8_t* sA;
+  const uint8_t* sB;
+  int64_t lds_a, lds_b;
 };
 
 // generic strided kernel: strides in elements, any dtype the ABI knows
@@ -29,13 +34,6 @@ struct GemmStridedArgs {
   int64_t sam, sak, sbk, sbn, scm, scn;
   const float* a_scale; const float* b_scale;
   int activation, in_dtype, out_dtype;
-};
-
-struct MxGemmArgs {
-  const uint8_t* A; const uint8_t* sA; const uint8_t* B; const uint8_t* sB; char* C;
-  int M, N, K;
-  int64_t lda, ldb, lds_a, lds_b, ldc;
-  int out_dtype, group_m;
 };
 
 struct AttnArgs {
@@ -50,7 +48,7 @@ struct AttnArgs {
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
-int mx_gemm_launch(const MxGemmArgs& p, int fmt, int tile, hipStream_t stream);
+int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
