@@ -1,0 +1,307 @@
+// Fused flash-attention forward for gfx950 (fp16 / bf16, head_dim 64 or 128).
+//
+// Same algorithm as the reference `_attn_fwd` / `_attn_fwd_inner`
+// (python/tutorials/06-fused-attention.py:25-75, :98-187): a Q tile stays resident, K/V stream
+// past it in BLOCK_N = 64 steps, online softmax in fp32 in the exp2 domain with
+// qk_scale = sm_scale * 1.44269504 (:160-161), P rounded to the input type before the second
+// product (:66-70) while the normaliser sums the unrounded P (:57-58), causal blocks above the
+// diagonal are skipped and only the diagonal block is masked (:33-40, :49-53), and
+// M = m + log2(l), O = acc / l at the end (:183-187).
+//
+// MI355X-first layout of the work:
+//   * every wave owns QT*32 query rows and all of head_dim; the score tile is computed
+//     TRANSPOSED (S^T = K Q^T), so a lane holds 16 scores of ONE query row per 32x32 MFMA tile:
+//     row max / row sum are in-lane reductions plus one 32-lane swap, the rescale factor is a
+//     per-lane scalar, and the fp32 -> 16-bit P^T registers are already the B operand of the
+//     second MFMA (O^T = V^T P^T) - P never goes through LDS;
+//   * K and V tiles go global -> LDS by direct 16-byte loads into two stages; K rows are read
+//     back as MFMA A operands with ds_read_b128, V is transposed on the fly by
+//     ds_read_b64_tr_b16; both layouts are XOR-swizzled against bank conflicts;
+//   * heads are laid out over XCDs so that the query blocks sharing one K/V stay on one L2,
+//     and causal query blocks are issued longest-first.
+#include "common.h"
+#include "launch.h"
+
+namespace mi355 {
+
+template <typename V8> struct Elem;
+template <> struct Elem<bf16x8> { using type = __bf16; };
+template <> struct Elem<f16x8> { using type = _Float16; };
+
+template <typename V8, int D, int QT, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
+  using S = typename Elem<V8>::type;
+  constexpr int BM = NW * QT * 32, BN = 64;
+  constexpr int RB = D * 2;            // bytes per K/V row
+  constexpr int CPR = RB / 16;         // 16-byte chunks per row
+  constexpr int RPI = 1024 / RB;       // rows moved by one wave instruction
+  constexpr int TILE = BN * RB;        // bytes of one K or V tile
+  constexpr int INST = TILE / 1024 / NW;  // direct-load instructions per wave and tile
+  constexpr int KSQ = D / 16;          // MFMA k-steps of S^T = K Q^T
+  constexpr int DT = D / 32;           // 32-row tiles of O^T
+  static_assert(INST >= 1, "too many waves for this tile");
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][K tile | V tile]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
+
+  // block -> (head, query block): consecutive logical ids (same XCD) walk the query blocks of
+  // one head; causal blocks in descending order of work
+  const int nqb = (p.N + BM - 1) / BM;
+  int pid = xcd_remap(blockIdx.x, nqb * p.Z * p.H);
+  const int hz = pid / nqb;
+  int qb = pid % nqb;
+  if (p.causal) qb = nqb - 1 - qb;
+  const int z = hz / p.H, h = hz % p.H;
+  const int m0 = qb * BM;
+  const int row0 = m0 + wave * QT * 32;  // first query row of this wave
+
+  const char* qbase = p.q + ((int64_t)z * p.sq[0] + (int64_t)h * p.sq[1]) * 2;
+  const char* kbase = p.k + ((int64_t)z * p.sk[0] + (int64_t)h * p.sk[1]) * 2;
+  const char* vbase = p.v + ((int64_t)z * p.sv[0] + (int64_t)h * p.sv[1]) * 2;
+  char* obase = p.o + ((int64_t)z * p.so[0] + (int64_t)h * p.so[1]) * 2;
+  const int64_t qpitch = p.sq[2] * 2, kpitch = p.sk[2] * 2, vpitch = p.sv[2] * 2, opitch = p.so[2] * 2;
+
+  // ---- Q fragments (B operand of S^T): lane (row l32, half g) holds Q[row][16*ks + 8*g .. +8]
+  V8 qf[QT][KSQ];
+#pragma unroll
+  for (int b = 0; b < QT; b++) {
+    int r = min(row0 + b * 32 + l32, p.N - 1);
+    const char* src = qbase + (int64_t)r * qpitch + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) qf[b][ks] = *(const V8*)(src + ks * 32);
+  }
+
+  // ---- direct global -> LDS copies of the K and V tiles
+  const char* srcK[INST];
+  const char* srcV[INST];
+#pragma unroll
+  for (int i = 0; i < INST; i++) {
+    int r = (i * NW + wave) * RPI + lane / CPR;
+    int pc = lane % CPR;
+    int lcK = pc ^ (r & 7);
+    int lcV = ((((pc >> 1) ^ (r & 3))) << 1) | (pc & 1);
+    srcK[i] = kbase + (int64_t)r * kpitch + lcK * 16;
+    srcV[i] = vbase + (int64_t)r * vpitch + lcV * 16;
+  }
+  auto issue_kv = [&](int j, int stage) {
+    LDS_PTR(char) kd = lds + stage * (2 * TILE);
+    LDS_PTR(char) vd = kd + TILE;
+#pragma unroll
+    for (int i = 0; i < INST; i++) {
+      async_copy16(srcK[i] + (int64_t)j * BN * kpitch, (LDS_PTR(void))(kd + (i * NW + wave) * 1024));
+      async_copy16(srcV[i] + (int64_t)j * BN * vpitch, (LDS_PTR(void))(vd + (i * NW + wave) * 1024));
+    }
+  };
+
+  // ---- per-lane LDS offsets
+  // K operand: row l32 (+32a), chunk 2*ks+g swizzled with the low row bits
+  unsigned offK[4];
+#pragma unroll
+  for (int k4 = 0; k4 < 4; k4++) offK[k4] = l32 * RB + ((((k4 * 2 + g) ^ l32) & 7) << 4);
+  // V operand (transpose read): lane i16 of 16-lane group q4 addresses row 4*g + i16/4 and the
+  // 8-byte piece i16%4 of 32-byte group 2c + (q4&1), swizzled with the low row bits
+  unsigned offV[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    int row = 4 * g + (i16 >> 2);
+    int c32 = (par * 2 + (q4 & 1)) ^ (row & 3);
+    offV[par] = TILE + row * RB + c32 * 32 + (i16 & 3) * 8;
+  }
+
+  f32x16 oacc[DT][QT];
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int b = 0; b < QT; b++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[c][b][r] = 0.f;
+  float m_i[QT], l_i[QT];
+#pragma unroll
+  for (int b = 0; b < QT; b++) { m_i[b] = -INFINITY; l_i[b] = 0.f; }
+
+  const float qk_scale = p.sm_scale * 1.44269504f;
+
+  // number of K/V steps of this block / wave
+  const int kv_end_blk = p.causal ? min(p.N, m0 + BM) : p.N;
+  const int nsteps = (kv_end_blk + BN - 1) / BN;
+  const int wave_last = p.causal ? (row0 + QT * 32 - 1) / BN : nsteps - 1;  // last step with unmasked columns
+  const int wave_first_masked = p.causal ? row0 / BN : nsteps;              // first step that needs the mask
+
+  issue_kv(0, 0);
+  wait_all();
+  __syncthreads();
+
+  for (int j = 0; j < nsteps; j++) {
+    const int stage = j & 1;
+    if (j + 1 < nsteps) issue_kv(j + 1, stage ^ 1);
+    if (j <= wave_last && row0 < p.N) {
+      const unsigned base = lds_addr(lds + stage * (2 * TILE));
+      // ---- S^T = K Q^T : [2 kv tiles][QT q tiles]
+      f32x16 s[2][QT];
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int b = 0; b < QT; b++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) s[a][b][r] = 0.f;
+      {
+        i32x4 kf[2][2];
+        kf[0][0] = lds_read_b128<0>(base + offK[0]);
+        kf[0][1] = lds_read_b128<32 * RB>(base + offK[0]);
+        static_for<KSQ>([&](auto KS_) {
+          constexpr int ks = decltype(KS_)::value;
+          constexpr int cur = ks & 1, nxt = cur ^ 1;
+          if constexpr (ks + 1 < KSQ) {
+            constexpr int imm = ((ks + 1) >> 2) * 128;
+            kf[nxt][0] = lds_read_b128<imm>(base + offK[(ks + 1) & 3]);
+            kf[nxt][1] = lds_read_b128<imm + 32 * RB>(base + offK[(ks + 1) & 3]);
+            lds_wait<2>();
+          } else {
+            lds_wait<0>();
+          }
+          lds_use(kf[cur][0]);
+          lds_use(kf[cur][1]);
+#pragma unroll
+          for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int b = 0; b < QT; b++)
+              s[a][b] = mfma32(__builtin_bit_cast(V8, kf[cur][a]), qf[b][ks], s[a][b]);
+        });
+      }
+      // ---- online softmax, one query row per lane (pair of lanes l, l+32 shares a row)
+      V8 pf[QT][4];  // P^T as B operand of the second product, per 16-column k-step
+#pragma unroll
+      for (int b = 0; b < QT; b++) {
+        if (j >= wave_first_masked) {
+          const int qrow = row0 + b * 32 + l32;
+#pragma unroll
+          for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+              if (kv > qrow) s[a][b][r] = -INFINITY;
+            }
+        }
+        float mx = s[0][b][0];
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[a][b][r]);
+        mx = pair_max(mx);
+        const float m_new = fmaxf(m_i[b], mx * qk_scale);
+        const float alpha = fast_exp2(m_i[b] - m_new);
+        float rs = 0.f;
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            float pv = fast_exp2(fmaf(s[a][b][r], qk_scale, -m_new));
+            s[a][b][r] = pv;
+            rs += pv;
+          }
+        l_i[b] = l_i[b] * alpha + rs;
+        m_i[b] = m_new;
+#pragma unroll
+        for (int c = 0; c < DT; c++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) oacc[c][b][r] *= alpha;
+        // k-step t = 2a + u covers columns 16t .. 16t+15: registers 8u .. 8u+7 of tile a
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) pf[b][t][e] = (S)s[t >> 1][b][(t & 1) * 8 + e];
+      }
+      // ---- O^T += V^T P^T : [DT d tiles][QT q tiles], 4 k-steps of 16 columns
+      {
+        i32x2 vf[2][DT][2];
+        auto read_v = [&](auto T_, i32x2 (&dst)[DT][2]) {
+          constexpr int t = decltype(T_)::value;
+          static_for<DT>([&](auto C_) {
+            constexpr int c = decltype(C_)::value;
+            constexpr int imm = (c >> 1) * 128 + 16 * t * RB;
+            dst[c][0] = lds_read_tr16_b64<imm>(base + offV[c & 1]);
+            dst[c][1] = lds_read_tr16_b64<imm + 8 * RB>(base + offV[c & 1]);
+          });
+        };
+        read_v(std::integral_constant<int, 0>{}, vf[0]);
+        static_for<4>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          constexpr int cur = t & 1, nxt = cur ^ 1;
+          if constexpr (t + 1 < 4) {
+            read_v(std::integral_constant<int, t + 1>{}, vf[nxt]);
+            lds_wait<2 * DT>();
+          } else {
+            lds_wait<0>();
+          }
+#pragma unroll
+          for (int c = 0; c < DT; c++) {
+            lds_use(vf[cur][c][0]);
+            lds_use(vf[cur][c][1]);
+            i32x4 both = __builtin_shufflevector(vf[cur][c][0], vf[cur][c][1], 0, 1, 2, 3);
+#pragma unroll
+            for (int b = 0; b < QT; b++) oacc[c][b] = mfma32(__builtin_bit_cast(V8, both), pf[b][t], oacc[c][b]);
+          }
+        });
+      }
+    }
+    wait_all();
+    __syncthreads();
+  }
+
+  // ---- epilogue: O = acc / l, M = m + log2(l)
+#pragma unroll
+  for (int b = 0; b < QT; b++) {
+    float l = l_i[b];
+    l = pair_sum(l);
+    const int row = row0 + b * 32 + l32;
+    if (row >= p.N) continue;
+    const float inv = 1.f / l;
+    if (g == 0) p.lse[(int64_t)hz * p.N + row] = m_i[b] + log2f(l);
+    char* dst = obase + (int64_t)row * opitch;
+#pragma unroll
+    for (int c = 0; c < DT; c++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        int d = c * 32 + rg * 8 + g * 4;
+        typedef __attribute__((ext_vector_type(4))) S S4;
+        S4 v;
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = (S)(oacc[c][b][rg * 4 + e] * inv);
+        *(S4*)(dst + d * 2) = v;
+      }
+  }
+}
+
+template <typename V8, int D, int QT, int NW>
+static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
+  constexpr int BM = NW * QT * 32;
+  constexpr int smem = 2 * 2 * 64 * D * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<V8, D, QT, NW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  int nqb = (p.N + BM - 1) / BM;
+  attn_fwd_kernel<V8, D, QT, NW><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+template <typename V8>
+static int launch_fwd_d(const AttnArgs& p, int variant, hipStream_t stream) {
+  if (p.D == 128) {
+    return variant == 1 ? launch_fwd<V8, 128, 1, 4>(p, stream) : launch_fwd<V8, 128, 2, 4>(p, stream);
+  }
+  return variant == 1 ? launch_fwd<V8, 64, 1, 4>(p, stream) : launch_fwd<V8, 64, 2, 4>(p, stream);
+}
+
+int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
+  int variant = p.variant;
+  return bf16 ? launch_fwd_d<bf16x8>(p, variant, stream) : launch_fwd_d<f16x8>(p, variant, stream);
+}
+
+}  // namespace mi355

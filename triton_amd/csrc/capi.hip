@@ -194,6 +194,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     return MI355_ESTRIDE;
   p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
   p.sm_scale = sm_scale; p.causal = causal != 0;
+  p.variant = env_int("MI355_ATTN_FWD_VARIANT", 0);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 
@@ -221,7 +222,7 @@ int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
   if (rc) return rc;
   if (!copy_strides(stride, p.sq)) return MI355_EINVAL;
   if (!attn_stride_ok(p.sq, q, D) || !aligned(k, 16) || !aligned(v, 16) || !aligned(d_o, 16) ||
-      !aligned(dq, 16) || !aligned(dk, 16) || !aligned(dv, 16))
+      !aligned(dq, 16) || !aligned(dk, 16) || !aligned(dv, 16) || !aligned(Mlse, 16) || !aligned(delta, 16))
     return MI355_ESTRIDE;
   p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.d_o = (const char*)d_o;
   p.lse = const_cast<float*>(Mlse); p.delta = delta;

@@ -60,6 +60,32 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds
 #endif
 }
 
+// 2^x by the hardware transcendental unit (denormal results flush to zero, as the reference
+// allows on AMD: python/tutorials/06-fused-attention.py:452-454 `allow_flush_denorm`).
+__device__ __forceinline__ float fast_exp2(float x) {
+#if MI355_DEVICE_PASS
+  return __builtin_amdgcn_exp2f(x);
+#else
+  return x;
+#endif
+}
+
+// Exchange between the two lanes (l, l+32) that share a row of a 32x32 MFMA accumulator.
+// v_permlane32_swap exchanges the upper half of its first register with the lower half of its
+// second; fed with two copies of x it leaves (own, partner) in lanes < 32 and (partner, own)
+// in lanes >= 32.  Issued as inline assembly (with the two wait states the instruction needs
+// after a VALU write of its operands): the compiler builtin folds the two results into one.
+__device__ __forceinline__ void swap32(float x, float& r0, float& r1) {
+  float a = x, b = x;
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+#endif
+  r0 = a;
+  r1 = b;
+}
+__device__ __forceinline__ float pair_max(float x) { float a, b; swap32(x, a, b); return fmaxf(a, b); }
+__device__ __forceinline__ float pair_sum(float x) { float a, b; swap32(x, a, b); return a + b; }
+
 // Copy a [ROWS x 128 bytes] tile (rows `pitch` bytes apart in global memory) into a swizzled
 // LDS tile with direct global->LDS loads.  One wave instruction moves 64 x 16 B = 8 rows; the
 // LDS side of such a load is linear in the lane id, so the swizzle is applied to the SOURCE
@@ -127,7 +153,8 @@ __device__ __forceinline__ i32x2 lds_read_tr8_b64(unsigned addr) {
 template <int N>
 __device__ __forceinline__ void lds_wait() {
 #if MI355_DEVICE_PASS
-  asm volatile("s_waitcnt lgkmcnt(%0)" ::"i"(N));
+  // the counter has 4 bits; asking for "at most 15" where more are in flight only waits longer
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"i"(N > 15 ? 15 : N));
 #endif
 }
 template <typename V>

@@ -43,6 +43,7 @@ struct AttnArgs {
   int64_t sq[4], sk[4], sv[4], so[4];  // element strides
   float sm_scale;
   int causal;
+  int variant;  // tiling variant (tuning knob)
 };
 
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
