@@ -1,0 +1,86 @@
+"""GEMM oracle (numpy, CPU; test infrastructure): the reference tile program restated, and
+the closed form that pins it.
+
+`matmul_tiled` follows `matmul_kernel` (python/tutorials/03-matrix-multiplication.py:241-316)
+as executed by the interpreter's serial grid loop (python/triton/runtime/interpreter.py:1088-1092)
+with `tl.dot` = `np.matmul(a, b, dtype=float32) + acc` per K chunk (:542-549).
+Arrays are float32 holding values already representable in the input type; outputs are float32
+holding the rounded result (see formats.round_to).
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import formats
+
+
+def cdiv(a: int, b: int) -> int:
+    return (a + b - 1) // b
+
+
+def grouped_pid_to_tile(pid: int, M: int, N: int, BM: int, BN: int, GROUP_M: int):
+    """pid -> (pid_m, pid_n), grouped ordering (03:265-273)."""
+    num_pid_m, num_pid_n = cdiv(M, BM), cdiv(N, BN)
+    num_pid_in_group = GROUP_M * num_pid_n
+    group_id = pid // num_pid_in_group
+    first_pid_m = group_id * GROUP_M
+    group_size_m = min(num_pid_m - first_pid_m, GROUP_M)
+    pid_m = first_pid_m + ((pid % num_pid_in_group) % group_size_m)
+    pid_n = (pid % num_pid_in_group) // group_size_m
+    return pid_m, pid_n
+
+
+def leaky_relu(x: np.ndarray) -> np.ndarray:
+    """03:320-322 on the fp32 accumulator."""
+    return np.where(x >= 0, x, np.float32(0.01) * x).astype(np.float32)
+
+
+def matmul_tiled(a: np.ndarray, b: np.ndarray, BM: int = 64, BN: int = 64, BK: int = 32, GROUP_M: int = 8,
+                 activation: str = "", out_dtype: str = "fp16", alpha: float = 1.0) -> np.ndarray:
+    """C = A @ B tile by tile, exactly in the reference's program order.
+
+    Row/column offsets of edge tiles wrap with % M / % N (03:282-283) and the store is masked
+    (03:312-316); the K tail is zero-filled (03:297-298); one fp32 add of the chunk product per
+    K step (03:300); activation on the accumulator (03:306-307); cast on store (03:308).
+    `alpha` is the per-tensor scale product a_scale*b_scale of the fp8 extension (1.0 = reference).
+    """
+    M, K = a.shape
+    K2, N = b.shape
+    assert K == K2, "Incompatible dimensions"
+    a = np.asarray(a, dtype=np.float32)
+    b = np.asarray(b, dtype=np.float32)
+    c = np.zeros((M, N), dtype=np.float32)
+    n_prog = cdiv(M, BM) * cdiv(N, BN)
+    offs_k = np.arange(BK)
+    for pid in range(n_prog):  # GridExecutor: serial loop over the 1-D grid
+        pid_m, pid_n = grouped_pid_to_tile(pid, M, N, BM, BN, GROUP_M)
+        offs_am = (pid_m * BM + np.arange(BM)) % M
+        offs_bn = (pid_n * BN + np.arange(BN)) % N
+        acc = np.zeros((BM, BN), dtype=np.float32)
+        for k in range(cdiv(K, BK)):
+            ks = k * BK + offs_k
+            kmask = ks < K
+            ksafe = np.where(kmask, ks, 0)
+            at = np.where(kmask[None, :], a[offs_am[:, None], ksafe[None, :]], np.float32(0))
+            bt = np.where(kmask[:, None], b[ksafe[:, None], offs_bn[None, :]], np.float32(0))
+            acc = np.matmul(at, bt, dtype=np.float32) + acc
+        if alpha != 1.0:
+            acc = acc * np.float32(alpha)
+        if activation == "leaky_relu":
+            acc = leaky_relu(acc)
+        out = formats.round_to(acc, out_dtype)
+        offs_cm = pid_m * BM + np.arange(BM)
+        offs_cn = pid_n * BN + np.arange(BN)
+        mm, nn = offs_cm < M, offs_cn < N
+        c[np.ix_(offs_cm[mm], offs_cn[nn])] = out[np.ix_(mm, nn)]
+    return c
+
+
+def matmul_closed_form(a: np.ndarray, b: np.ndarray, activation: str = "", out_dtype: str = "fp32",
+                       alpha: float = 1.0) -> np.ndarray:
+    """fp64 matmul of the (exactly representable) inputs, then one rounding: the golden of the
+    reference's own tests (`torch.matmul(a.float(), b.float())`, hopper/test_gemm.py:138-140)."""
+    acc = (np.asarray(a, dtype=np.float64) @ np.asarray(b, dtype=np.float64)) * alpha
+    if activation == "leaky_relu":
+        acc = np.where(acc >= 0, acc, 0.01 * acc)
+    return formats.round_to(acc.astype(np.float32), out_dtype)

@@ -1,0 +1,94 @@
+"""CPU: the attention oracle (tile programs restated) pinned by the fp64 closed form and by
+invariants a dropped term / wrong sign / transposed operand would break."""
+import numpy as np
+import pytest
+
+from oracle import attention as A
+from oracle import formats
+
+
+def _inputs(seed, shape, dtype, std=0.5):
+    rng = np.random.default_rng(seed)
+    q, k, v = (formats.round_to(rng.normal(0, std, shape).astype(np.float32), dtype) for _ in range(3))
+    do = formats.round_to(rng.standard_normal(shape).astype(np.float32), dtype)
+    return q, k, v, do
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_forward_tiled_matches_closed_form(dtype, causal):
+    q, k, v, _ = _inputs(20, (1, 2, 256, 64), dtype)
+    o, M = A.attn_fwd_tiled(q, k, v, causal, 0.5, dtype)
+    ref = A.attn_closed_form(q, k, v, causal, 0.5)
+    tol = 1e-2 if dtype == "bf16" else 2e-3
+    assert np.max(np.abs(o - ref["o"])) < tol
+    assert np.max(np.abs(M - ref["M"])) < 1e-4   # M = logsumexp(qk * sm_scale) / ln 2
+
+
+def test_forward_matches_reference_test_op_configuration():
+    # 06:523-559: (Z,H,N,D) = (1,2,1024,64), normal(0, 0.5), sm_scale 0.5, causal, atol 1e-2
+    q, k, v, _ = _inputs(20, (1, 2, 1024, 64), "fp16")
+    o, M = A.attn_fwd_tiled(q, k, v, True, 0.5, "fp16")
+    ref = A.attn_closed_form(q, k, v, True, 0.5)
+    assert np.allclose(o, ref["o"], atol=1e-2, rtol=0)
+
+
+def test_forward_invariants():
+    q, k, v, _ = _inputs(5, (1, 1, 128, 32), "fp16")
+    o, M = A.attn_fwd_tiled(q, k, v, True, 0.3, "fp16", BLOCK_M=64, BLOCK_N=32)
+    # causal: the first query sees only the first key
+    assert np.allclose(o[0, 0, 0], v[0, 0, 0], atol=1e-3)
+    # rows of O are convex combinations of rows of V
+    assert np.all(o.max(axis=2) <= v.max(axis=2) + 1e-3) and np.all(o.min(axis=2) >= v.min(axis=2) - 1e-3)
+    # V = const * ones  =>  O = const (row sums of P are 1)
+    ones = np.full_like(v, 0.75)
+    o1, _ = A.attn_fwd_tiled(q, k, ones, False, 0.3, "fp16", BLOCK_M=64, BLOCK_N=32)
+    assert np.allclose(o1, 0.75, atol=2e-3)
+    # tile sizes do not change the result beyond rounding
+    o2, M2 = A.attn_fwd_tiled(q, k, v, True, 0.3, "fp16", BLOCK_M=32, BLOCK_N=16)
+    assert np.allclose(o, o2, atol=2e-3) and np.allclose(M, M2, atol=1e-4)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_backward_tiled_matches_closed_form(dtype, causal):
+    q, k, v, do = _inputs(21, (1, 2, 256, 64), dtype)
+    o, M = A.attn_fwd_tiled(q, k, v, causal, 0.5, dtype)
+    dq, dk, dv, delta = A.attn_bwd_tiled(q, k, v, o, do, M, 0.5, causal, dtype)
+    ref = A.attn_closed_form(q, k, v, causal, 0.5, do)
+    tol = 3e-2 if dtype == "bf16" else 1e-2   # reference tolerance: atol 1e-2 for fp16 (06:551-559)
+    for name, got in (("dq", dq), ("dk", dk), ("dv", dv)):
+        assert np.max(np.abs(got - ref[name])) < tol, name
+    assert np.max(np.abs(delta - ref["delta"])) < (2e-2 if dtype == "bf16" else 3e-3)
+
+
+def test_backward_closed_form_against_finite_differences():
+    # pins the closed form itself: d/dx of L = sum(O * dO) by central differences in fp64
+    rng = np.random.default_rng(7)
+    shape = (1, 1, 8, 4)
+    q, k, v, do = (rng.normal(0, 0.7, shape) for _ in range(4))
+    ref = A.attn_closed_form(q, k, v, True, 0.6, do)
+    eps = 1e-6
+    for name, x in (("dq", q), ("dk", k), ("dv", v)):
+        g = np.zeros(shape)
+        for idx in np.ndindex(*shape):
+            xp = x.copy(); xp[idx] += eps
+            xm = x.copy(); xm[idx] -= eps
+            args_p = {"dq": (xp, k, v), "dk": (q, xp, v), "dv": (q, k, xp)}[name]
+            args_m = {"dq": (xm, k, v), "dk": (q, xm, v), "dv": (q, k, xm)}[name]
+            lp = (A.attn_closed_form(*args_p, True, 0.6)["o"] * do).sum()
+            lm = (A.attn_closed_form(*args_m, True, 0.6)["o"] * do).sum()
+            g[idx] = (lp - lm) / (2 * eps)
+        assert np.allclose(g, ref[name], atol=1e-6), name
+
+
+def test_backward_invariants():
+    q, k, v, do = _inputs(9, (1, 1, 128, 32), "fp16")
+    o, M = A.attn_fwd_tiled(q, k, v, False, 0.4, "fp16", BLOCK_M=64, BLOCK_N=32)
+    dq, dk, dv, delta = A.attn_bwd_tiled(q, k, v, o, do, M, 0.4, False, "fp16")
+    # softmax is shift invariant: sum_n dS[m,n] = 0  =>  sum over keys of dK-contributions:
+    # dQ . q summed equals dK . k summed (both equal sum(dS * S) / 1)
+    assert abs((dq * q).sum() - (dk * k).sum()) < 5e-2
+    # non-causal: column sums of P^T dO: sum_n dv[n] = sum_m do[m] (rows of P sum to 1)
+    assert np.allclose(dv.sum(axis=2), do.sum(axis=2), atol=5e-2)
+    assert np.allclose(delta, (o * do).sum(-1), atol=1e-5)

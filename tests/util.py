@@ -1,0 +1,29 @@
+"""Shared helpers for the parity tests: torch <-> float32 numpy and seeded input builders."""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+TORCH_DT = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+def to_np(t: torch.Tensor) -> np.ndarray:
+    """Any float tensor -> float32 numpy holding the same values."""
+    return t.detach().float().cpu().numpy()
+
+
+def from_np(x: np.ndarray, dtype: str, device) -> torch.Tensor:
+    """float32 numpy holding values representable in dtype -> tensor of that dtype (exact)."""
+    return torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(TORCH_DT[dtype]).to(device)
+
+
+def randn_rounded(rng: np.random.Generator, shape, dtype: str, std: float = 1.0) -> np.ndarray:
+    from oracle import formats
+
+    return formats.round_to(rng.normal(0.0, std, size=shape).astype(np.float32), dtype)
+
+
+def bits_equal(a: np.ndarray, b: np.ndarray) -> bool:
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    b = np.ascontiguousarray(b, dtype=np.float32)
+    return a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))
