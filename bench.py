@@ -1,0 +1,195 @@
+"""Benchmark of the hot path on one MI355X.
+
+`python bench.py --gpus 1 --steps K --warmup W` times K back-to-back launches of the headline
+workload (bf16 GEMM 8192^3, BASELINE config 2) with inputs resident in HBM, and prints ONE JSON
+line: TFLOP/s (work = 2*M*N*K as in python/tutorials/03-matrix-multiplication.py:437), the MFMA
+roofline fraction of the GEMM kernel from per-launch device events, and the CPU oracle timed on
+the host cores.  The other workloads of the path (fp8 / MX GEMM, attention forward / backward)
+are timed briefly and reported under "extra".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# dense MFMA peaks of MI355X in TFLOP/s (published, without sparsity) and HBM3E bandwidth in GB/s
+PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4": 10100.0}
+HBM_GBPS = 8000.0
+
+# HBM bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc
+# (FETCH_SIZE, WRITE_SIZE), see profiles/; None until measured
+MEASURED_TRAFFIC_BYTES = None
+
+
+def time_launches(fn, steps, warmup):
+    """W untimed warm-up launches, then exactly K launches timed two ways: wall clock between two
+    device synchronisations, and K+1 device events on the launch stream (per-launch durations)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    t0 = time.perf_counter()
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    per = [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
+    return wall_ms, sum(per) / len(per), per
+
+
+def quick(fn, iters=10, warmup=2):
+    _, ev_ms, _ = time_launches(fn, iters, warmup)
+    return ev_ms
+
+
+def cpu_baseline_gemm(budget_s=20.0):
+    """The CPU oracle (a port of the reference's interpreter execution model: serial grid loop,
+    one fp32 np.matmul per K chunk, python/triton/runtime/interpreter.py:1088-1092, :542-549) on a
+    bounded sample of the GEMM workload: same tile program, size reduced until it fits the budget."""
+    import numpy as np
+
+    from oracle import gemm
+
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+    except Exception:
+        threads = os.cpu_count() or 1
+    rng = np.random.default_rng(0)
+    n = 1024
+    best = None
+    while True:
+        a = rng.standard_normal((n, n)).astype(np.float32)
+        b = rng.standard_normal((n, n)).astype(np.float32)
+        t0 = time.perf_counter()
+        gemm.matmul_tiled(a, b, 128, 256, 64, 8, out_dtype="fp32")
+        dt = time.perf_counter() - t0
+        best = (n, dt)
+        if dt * 8 > budget_s or n >= 8192:
+            break
+        n *= 2
+    n, dt = best
+    return {
+        "value": round(2.0 * n ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
+        "sample": f"oracle.gemm.matmul_tiled {n}^3 (tiles 128x256x64, GROUP_M 8, fp32 accumulate), one pass, {dt:.2f} s; "
+                  f"host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also launch plain device copies of the A matrix (a kernel of known traffic, for scaling PMC byte counters)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the path has no collectives); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    import triton_amd
+    from triton_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    lib = _lib.load()
+    dev = torch.device("cuda", 0)
+    torch.manual_seed(0)
+    n = args.size
+    a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+    c = torch.empty(n, n, device=dev, dtype=torch.bfloat16)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def step():
+        rc = lib.mi355_gemm(a.data_ptr(), b.data_ptr(), c.data_ptr(), n, n, n, n, 1, n, 1, n, 1,
+                            _lib.BF16, _lib.BF16, None, None, 0, stream)
+        assert rc == 0, rc
+
+    if args.copy_calibration:
+        for _ in range(5):
+            c.copy_(a)   # reads n*n*2 bytes, writes n*n*2 bytes
+        torch.cuda.synchronize()
+    wall_ms, ev_ms, per = time_launches(step, args.steps, args.warmup)
+    flops = 2.0 * n ** 3
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (ev_ms * 1e-3) / 1e12
+    out = {
+        "metric": "TFLOP/s & % MFMA peak: bf16/fp8 GEMM 8192^3; flash-attn fwd D=128 N=4096",
+        "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"bf16 GEMM M=N=K={n}, A row-major MxK, B row-major KxN, fp32 accumulate, bf16 out (BASELINE config 2)"},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK["bf16"], "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK["bf16"], 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel": "gemm_kernel<Cfg16<bf16>,256,256,2,4,row-major B>", "launch_ms_avg": round(ev_ms, 5),
+                     "launch_ms_min": round(min(per), 5), "algorithmic_flops": flops,
+                     "algorithmic_bytes": 3 * 2 * n * n},
+        "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
+                   "clock_khz": lib.mi355_query(_lib.Q_CLOCK_KHZ)},
+    }
+
+    if not args.no_extra:
+        extra = {}
+        # fp8 e4m3 GEMM, K-major B, per-tensor scales, bf16 out (config 4) and its decode shape
+        a8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
+        b8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
+        sc = torch.tensor([0.01], device=dev)
+        ms = quick(lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sc, b_scale=sc))
+        extra["fp8_e4m3_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK["fp8"], 4)}
+        a16 = torch.randn(16, n, device=dev).to(torch.float8_e4m3fn)
+        ms = quick(lambda: triton_amd.matmul(a16, b8.t(), out_dtype=torch.bfloat16), iters=20)
+        byts = n * n + 16 * n + 2 * 16 * n
+        extra["fp8_decode_m16"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1), "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
+        del a8, a16
+        # MX GEMMs (config 5)
+        for fmt, kb in (("mxfp4", n // 2), ("mxfp8", n)):
+            pa = torch.randint(0, 120, (n, kb), device=dev, dtype=torch.uint8)
+            pb = torch.randint(0, 120, (n, kb), device=dev, dtype=torch.uint8)
+            sa = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
+            sb = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
+            ms = quick(lambda: triton_amd.mx_matmul(pa, sa, pb, sb, fmt))
+            extra[f"{fmt}_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK[fmt], 4)}
+        del b8
+        # flash attention (config 3), flops by the reference formula (06:630-636)
+        Z, H, N, D = 4, 32, 4096, 128
+        q = torch.empty(Z, H, N, D, device=dev, dtype=torch.bfloat16).normal_(0, 0.5).requires_grad_()
+        k = torch.empty_like(q).normal_(0, 0.5).requires_grad_()
+        v = torch.empty_like(q).normal_(0, 0.5).requires_grad_()
+        sm = D ** -0.5
+        for causal in (True, False):
+            fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
+            ms = quick(lambda: triton_amd.attention(q, k, v, causal, sm))
+            tag = "causal" if causal else "noncausal"
+            extra[f"attn_fwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["bf16"], 4)}
+            o = triton_amd.attention(q, k, v, causal, sm)
+            do = torch.randn_like(o)
+            ms = quick(lambda: o.backward(do, retain_graph=True), iters=5)
+            extra[f"attn_bwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(2.5 * fl / ms / 1e9, 1), "frac_of_peak": round(2.5 * fl / ms / 1e9 / PEAK["bf16"], 4)}
+        out["extra"] = extra
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline_gemm()
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -124,9 +124,10 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
 
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
-  // the 256x256 / 8-wave MX variants do not fit 256 registers yet: 128x128 tiles for every shape
-  (void)cus;
-  int tile = env_int("MI355_GEMM_TILE", 1);
+  // 256x256 tiles once they fill three quarters of the CUs, 128x128 tiles (two workgroups per CU) below that
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
+  tile = env_int("MI355_GEMM_TILE", tile);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
@@ -194,7 +195,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     return MI355_ESTRIDE;
   p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
   p.sm_scale = sm_scale; p.causal = causal != 0;
-  p.variant = env_int("MI355_ATTN_FWD_VARIANT", 0);
+  p.variant = env_int("MI355_ATTN_FWD_VARIANT", 1);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 

@@ -38,10 +38,12 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 template <typename S> __device__ __forceinline__ S cvt16(float x) { return (S)x; }
 
 // Byte offset of 16-byte chunk `chunk` (0..7) of row `row` in an LDS tile whose rows are
-// 128 bytes: the chunk index is XORed with the low 3 row bits, so 8 consecutive rows reading
-// the same logical chunk touch 8 distinct 16-byte bank groups.
+// 128 bytes.  LDS has 64 four-byte banks, i.e. 256 bytes = two such rows per bank sweep, and a
+// ds_read_b128 is served 16 lanes at a time: 16 consecutive rows reading the same logical chunk
+// must land in 16 different 16-byte slots of the sweep.  The slot is (row & 1) * 8 + chunk, so
+// the chunk index is XORed with bits 1..3 of the row.
 __device__ __forceinline__ int swz128(int row, int chunk) {
-  return row * 128 + (((chunk ^ row) & 7) << 4);
+  return row * 128 + (((chunk ^ (row >> 1)) & 7) << 4);
 }
 
 // Builtins that need gfx950 target features are hidden from hipcc's host pass: a kernel
@@ -101,7 +103,7 @@ struct TileCopy128 {
   __device__ static const char* src(const char* base, int64_t pitch, int row0, int row_limit,
                                     int wave, int lane, int i) {
     int r = (i * NWAVES + wave) * 8 + (lane >> 3);
-    int lc = (lane & 7) ^ (r & 7);
+    int lc = (lane & 7) ^ ((r >> 1) & 7);
     int gr = row0 + r;
     gr = gr < row_limit ? gr : row_limit - 1;
     return base + (int64_t)gr * pitch + lc * 16;

@@ -29,9 +29,10 @@
 
 namespace mi355 {
 
-// Row-major [64 x BN] 16-bit tile of B (rows are k, BN*2 bytes each).  32-byte groups of a row
-// are XORed with (k & 3): the transpose read of one 16-lane group touches 4 consecutive k rows
-// x 32 bytes, which then fall into 4 different bank groups.
+// Row-major [64 x BN] 16-bit tile of B (rows are k, BN*2 bytes each, a multiple of the 256-byte
+// bank sweep).  A transpose read is served 32 lanes at a time: two 16-lane groups that address
+// the same 4 consecutive k rows and two neighbouring 32-byte groups of columns.  The 32-byte
+// group index is XORed with 2 * (k & 3), which spreads those 4 rows x 64 bytes over all banks.
 template <int BN, int NW>
 struct TileCopyKN {
   static constexpr int kChunksPerRow = BN / 8;             // 16-byte chunks per k row
@@ -42,7 +43,7 @@ struct TileCopyKN {
   __device__ static int row(int wave, int lane, int i) { return (i * NW + wave) * kRowsPerInst + lane / kChunksPerRow; }
   __device__ static int col16(int lane, int r) {  // logical 16-byte chunk this lane fetches
     int pc16 = lane % kChunksPerRow;
-    int lc32 = (pc16 >> 1) ^ (r & 3);
+    int lc32 = (pc16 >> 1) ^ ((r & 3) << 1);
     return lc32 * 2 + (pc16 & 1);
   }
 };
@@ -108,7 +109,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 #pragma unroll
     for (int i = 0; i < CopyA::kIters; i++) {
       int r = (i * NW + wave) * 8 + (lane >> 3);
-      int kb = kbase + (((lane & 7) ^ (r & 7)) << 4);
+      int kb = kbase + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
       i32x4 v = {0, 0, 0, 0};
       if (kb < p.k_bytes) v = *(const i32x4*)(srcA[i] + kt * stepA);
       *(LDS_PTR(i32x4))(a + (i * NW + wave) * 1024 + lane * 16) = v;
@@ -118,7 +119,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
       bool ok;
       if constexpr (B_KMAJOR) {
         int r = (i * NW + wave) * 8 + (lane >> 3);
-        ok = kbase + (((lane & 7) ^ (r & 7)) << 4) < p.k_bytes;
+        ok = kbase + (((lane & 7) ^ ((r >> 1) & 7)) << 4) < p.k_bytes;
       } else {
         ok = kt * 64 + CopyBn::row(wave, lane, i) < p.K;
       }
@@ -142,7 +143,7 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   //   K-major operand (A always, B when B_KMAJOR): lane reads row (l%32) and the 16-byte
   //   chunk(s) Cfg::chunk(ks, l/32, c), swizzled; 32-row sub-tiles add t * 4096.
   //   Row-major B: transpose read, lane i of a 16-lane group q addresses k row
-  //   16*ks + 8*(q/2) + i/4 (+4 for the second half) and 32-byte group (n/16) ^ (k & 3).
+  //   16*ks + 8*(q/2) + i/4 (+4 for the second half) and 32-byte group (n/16) ^ 2*(k & 3).
   const int l32 = lane & 31, g = lane >> 5;
   const int i16 = lane & 15, q = lane >> 4;
   unsigned offA[KS][NC], offB[KS][NC];
@@ -153,14 +154,14 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
       offA[ks][c] = swz128(wm * TM + l32, Cfg::chunk(ks, g, c));
       offB[ks][c] = A_BYTES + swz128(wn * TN + l32, Cfg::chunk(ks, g, c));
     }
-  unsigned offBn[2];
+  unsigned offBn[NT];
   {
-    // offBn[par]: sub-tiles t with parity par; k row without the ks / +4 terms
+    // k row without the ks / +4 terms; (k & 3) is the same for every ks and both halves
     int k = (q >> 1) * 8 + (i16 >> 2);
 #pragma unroll
-    for (int par = 0; par < 2; par++) {
-      int c32 = (wn * TN + par * 32) / 16 + (q & 1);
-      offBn[par] = A_BYTES + k * (BN * 2) + ((c32 ^ (k & 3)) << 5) + (i16 & 3) * 8;
+    for (int t = 0; t < NT; t++) {
+      int c32 = (wn * TN + t * 32) / 16 + (q & 1);
+      offBn[t] = A_BYTES + k * (BN * 2) + ((c32 ^ ((k & 3) << 1)) << 5) + (i16 & 3) * 8;
     }
   }
 
@@ -187,9 +188,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
       if constexpr (B_KMAJOR) {
         f.b[t] = read_operand(base, offB[ks], std::integral_constant<int, t * 4096>{});
       } else {
-        constexpr int imm = ks * 16 * BN * 2 + (t / 2) * 128;
-        i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t & 1]);
-        i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[t & 1]);
+        constexpr int imm = ks * 16 * BN * 2;
+        i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t]);
+        i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[t]);
         i32x4 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3);
         f.b[t] = __builtin_bit_cast(Operand, both);
       }
