@@ -152,9 +152,9 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.c_vec_ok = ldc % 4 == 0 && aligned(C, 16);
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
-  // the 256x256 / 8-wave MX variants do not fit 256 registers yet: 128x128 tiles for every shape
-  (void)cus;
-  int tile = env_int("MI355_GEMM_TILE", 1);
+  const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
+  tile = env_int("MI355_GEMM_TILE", tile);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
 }
 

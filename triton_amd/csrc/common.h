@@ -37,15 +37,6 @@ __device__ __forceinline__ f32x16 mfma32(f16x8 a, f16x8 b, f32x16 c) {
 // fp32 -> 16-bit, round to nearest even (the compiler emits v_cvt_pk_bf16_f32 / v_cvt_f16_f32).
 template <typename S> __device__ __forceinline__ S cvt16(float x) { return (S)x; }
 
-// Byte offset of 16-byte chunk `chunk` (0..7) of row `row` in an LDS tile whose rows are
-// 128 bytes.  LDS has 64 four-byte banks, i.e. 256 bytes = two such rows per bank sweep, and a
-// ds_read_b128 is served 16 lanes at a time: 16 consecutive rows reading the same logical chunk
-// must land in 16 different 16-byte slots of the sweep.  The slot is (row & 1) * 8 + chunk, so
-// the chunk index is XORed with bits 1..3 of the row.
-__device__ __forceinline__ int swz128(int row, int chunk) {
-  return row * 128 + (((chunk ^ (row >> 1)) & 7) << 4);
-}
-
 // Builtins that need gfx950 target features are hidden from hipcc's host pass: a kernel
 // template that reaches one there silently loses its host-side launch stub.
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -87,28 +78,6 @@ __device__ __forceinline__ void swap32(float x, float& r0, float& r1) {
 }
 __device__ __forceinline__ float pair_max(float x) { float a, b; swap32(x, a, b); return fmaxf(a, b); }
 __device__ __forceinline__ float pair_sum(float x) { float a, b; swap32(x, a, b); return a + b; }
-
-// Copy a [ROWS x 128 bytes] tile (rows `pitch` bytes apart in global memory) into a swizzled
-// LDS tile with direct global->LDS loads.  One wave instruction moves 64 x 16 B = 8 rows; the
-// LDS side of such a load is linear in the lane id, so the swizzle is applied to the SOURCE
-// chunk each lane fetches.  `gsrc[i]` are per-lane source pointers prepared by tile_src_ptrs.
-template <int ROWS, int NWAVES>
-struct TileCopy128 {
-  static constexpr int kIters = ROWS / 8 / NWAVES;
-  static_assert(ROWS % (8 * NWAVES) == 0, "tile rows must split evenly over the waves");
-
-  // Pointer (to the k = 0 tile) that lane `lane` of wave `wave` fetches in iteration i.
-  // row_limit clamps rows past the matrix edge onto the last valid row (their products are
-  // never stored).
-  __device__ static const char* src(const char* base, int64_t pitch, int row0, int row_limit,
-                                    int wave, int lane, int i) {
-    int r = (i * NWAVES + wave) * 8 + (lane >> 3);
-    int lc = (lane & 7) ^ ((r >> 1) & 7);
-    int gr = row0 + r;
-    gr = gr < row_limit ? gr : row_limit - 1;
-    return base + (int64_t)gr * pitch + lc * 16;
-  }
-};
 
 // Compile-time counted loop: f(std::integral_constant<int, 0>) ... f(<N-1>), so that loop indices
 // can be used as template arguments / instruction immediates.
@@ -167,8 +136,25 @@ __device__ __forceinline__ void lds_use(V& v) {
 }
 __device__ __forceinline__ unsigned lds_addr(LDS_PTR(const void) p) { return (unsigned)(uintptr_t)p; }
 
-__device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 __device__ __forceinline__ void wait_all() { __builtin_amdgcn_s_waitcnt(0); }
+
+// Wait until at most N vector-memory operations (loads, direct global->LDS copies) of this wave
+// are outstanding; they complete in issue order.  vmcnt is split over bits 3:0 and 15:14 of the
+// immediate, the other counters are left at "no wait".
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  static_assert(N >= 0 && N < 64, "vmcnt has 6 bits");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0F70);
+}
+
+// Workgroup barrier WITHOUT the full memory wait the compiler puts in front of its own barrier:
+// the K loops keep younger direct loads in flight across it.  The caller waits (wait_vmcnt /
+// lds_wait) for exactly what the other waves are about to read.
+__device__ __forceinline__ void block_barrier() {
+#if MI355_DEVICE_PASS
+  asm volatile("s_barrier" ::: "memory");
+#endif
+}
 
 // Map a hardware workgroup id to a logical one so that ids that are consecutive in the
 // logical order run on the same XCD (hardware deals workgroups round-robin over 8 XCDs,

@@ -1,5 +1,5 @@
-// fp16 / bf16 instantiation of the tiled MFMA GEMM core: 64 elements (128 bytes) per K tile,
-// four 32x32x16 MFMA sub-steps, row-major or K-major B.
+// fp16 / bf16 instantiation of the tiled MFMA GEMM core: 32 elements (64 bytes) per K step,
+// two 32x32x16 MFMA sub-steps, row-major or K-major B.
 #include "gemm_core.h"
 
 namespace mi355 {
@@ -7,7 +7,7 @@ namespace mi355 {
 template <typename V8>
 struct Cfg16 {
   using Operand = V8;
-  static constexpr int kSteps = 4, kChunks = 1;
+  static constexpr int kSteps = 2, kChunks = 1;
   static constexpr bool kRowMajorB = true, kScaled = false;
   // lane group g of sub-step ks reads k elements 16*ks + 8*g .. +8
   __device__ static constexpr int chunk(int ks, int g, int) { return ks * 2 + g; }

@@ -5,10 +5,14 @@
 // (python/tutorials/03-matrix-multiplication.py:241-316): one workgroup per BM x BN tile of C,
 // grouped tile order (:265-273), K loop (:294-303), epilogue activation and cast (:304-316).
 // Built MI355X-first instead of translated:
-//   * a K step is 128 BYTES of every operand row (64 fp16/bf16, 128 fp8, 256 fp4 elements);
-//     tiles go global -> LDS with direct 16-byte loads into two LDS stages (no register
-//     staging), the tile for step k+1 is in flight while step k is multiplied;
-//   * LDS rows are XOR-swizzled so that ds_read_b128 / ds_read_b64_tr_b16 are conflict free;
+//   * a K step is RBK = 64 BYTES of every operand row (32 fp16/bf16, 64 fp8, 128 fp4 elements);
+//     tiles go global -> LDS with direct 16-byte loads into a ring of NS LDS stages (no register
+//     staging).  Loads run NS-1 steps ahead of the MFMAs: an L2 round trip under load is longer
+//     than one step, so a two-stage ring stalls every step on its own prefetch;
+//   * one barrier per step, entered after waiting only for the loads of the step about to be
+//     multiplied (the younger ones stay in flight);
+//   * LDS rows are XOR-swizzled for the 64-bank LDS so that ds_read_b128 / ds_read_b64_tr_b16
+//     are conflict free;
 //   * a row-major 16-bit B[K,N] is transposed on the fly by the LDS transpose read; a K-major B
 //     (the `b.T` view the reference passes for fp8, :378-382) uses plain 128-bit reads;
 //   * 32x32 MFMA tiles with the operands swapped, so every lane owns 4 consecutive columns of
@@ -16,9 +20,9 @@
 //   * workgroup ids are remapped per XCD before the grouped ordering.
 //
 // `Cfg` describes one element family:
-//   kSteps            MFMA sub-steps per 128-byte K tile
+//   kSteps            MFMA sub-steps per 64-byte K step
 //   kChunks           16-byte LDS chunks one lane feeds into one MFMA operand (1 or 2)
-//   chunk(ks, g, c)   which 16-byte chunk (0..7) of the row lane-group g reads for sub-step ks
+//   chunk(ks, g, c)   which 16-byte chunk (0..3) of the row lane-group g reads for sub-step ks
 //   kRowMajorB        whether the transpose-read path for a row-major B exists (16-bit only)
 //   kScaled           block-scaled: per-row e8m0 scales ride along (MX)
 //   Operand           register type of one MFMA operand
@@ -29,17 +33,40 @@
 
 namespace mi355 {
 
-// Row-major [64 x BN] 16-bit tile of B (rows are k, BN*2 bytes each, a multiple of the 256-byte
-// bank sweep).  A transpose read is served 32 lanes at a time: two 16-lane groups that address
-// the same 4 consecutive k rows and two neighbouring 32-byte groups of columns.  The 32-byte
-// group index is XORed with 2 * (k & 3), which spreads those 4 rows x 64 bytes over all banks.
+constexpr int RBK = 64;          // bytes of one operand row per K step
+constexpr int CPR = RBK / 16;    // 16-byte chunks per row of a K-major LDS tile
+
+// K-major LDS tile: rows of RBK bytes, four rows per 256-byte bank sweep.  A ds_read_b128 is
+// served 16 lanes at a time; 16 consecutive rows reading the same logical chunk must hit 16
+// different 16-byte slots of the sweep.  The slot is (row & 3) * 4 + chunk, so the chunk index
+// is XORed with bits 2..3 of the row.
+__device__ __forceinline__ int kswz(int row) { return (row >> 2) & (CPR - 1); }
+__device__ __forceinline__ int kmajor_off(int row, int chunk) { return row * RBK + (((chunk ^ kswz(row))) << 4); }
+
+// Direct global -> LDS copy of a K-major [ROWS x RBK] tile.  One wave instruction moves
+// 64 x 16 B = 16 rows; the LDS side of such a load is linear in the lane id, so the swizzle is
+// applied to the SOURCE chunk each lane fetches.
+template <int ROWS, int NW>
+struct TileCopyK {
+  static constexpr int kRowsPerInst = 1024 / RBK;
+  static constexpr int kIters = ROWS / kRowsPerInst / NW;
+  static_assert(ROWS % (kRowsPerInst * NW) == 0 && kIters >= 1, "tile rows must split evenly over the waves");
+  __device__ static int row(int wave, int lane, int i) { return (i * NW + wave) * kRowsPerInst + lane / CPR; }
+  __device__ static int chunk(int lane, int r) { return (lane % CPR) ^ kswz(r); }  // logical chunk fetched
+};
+
+// Row-major [RBK/2 x BN] 16-bit tile of B (rows are k, BN*2 bytes each, a multiple of the
+// 256-byte bank sweep).  A transpose read is served 32 lanes at a time: two 16-lane groups that
+// address the same 4 consecutive k rows and two neighbouring 32-byte groups of columns.  The
+// 32-byte group index is XORed with 2 * (k & 3), which spreads those 4 rows x 64 bytes over all
+// banks.
 template <int BN, int NW>
 struct TileCopyKN {
+  static constexpr int kRows = RBK / 2;
   static constexpr int kChunksPerRow = BN / 8;             // 16-byte chunks per k row
   static constexpr int kRowsPerInst = 64 / kChunksPerRow;  // k rows moved by one wave instruction
-  static constexpr int kIters = 64 / kRowsPerInst / NW;
+  static constexpr int kIters = kRows / kRowsPerInst / NW;
   static_assert(kRowsPerInst >= 1 && kIters >= 1, "tile too small for this wave count");
-
   __device__ static int row(int wave, int lane, int i) { return (i * NW + wave) * kRowsPerInst + lane / kChunksPerRow; }
   __device__ static int col16(int lane, int r) {  // logical 16-byte chunk this lane fetches
     int pc16 = lane % kChunksPerRow;
@@ -48,22 +75,23 @@ struct TileCopyKN {
   }
 };
 
-template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR>
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   using Operand = typename Cfg::Operand;
   constexpr int NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
-  constexpr int A_BYTES = BM * 128, B_BYTES = BN * 128, STAGE = A_BYTES + B_BYTES;
+  constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK, STAGE = A_BYTES + B_BYTES;
   constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
   static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
-  using CopyA = TileCopy128<BM, NW>;
-  using CopyBk = TileCopy128<BN, NW>;
+  using CopyA = TileCopyK<BM, NW>;
+  using CopyBk = TileCopyK<BN, NW>;
   using CopyBn = TileCopyKN<BN, NW>;
+  constexpr int ITA = CopyA::kIters;
   constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
+  constexpr int KROWS = RBK / 2;  // k rows of a row-major 16-bit B tile
 
-  // Two LDS stages of STAGE bytes each (dynamic LDS: 2 * STAGE bytes at launch).
+  // ring of NS LDS stages (dynamic LDS: NS * STAGE bytes at launch)
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  LDS_PTR(char) const lds0 = (LDS_PTR(char))smem;
-  LDS_PTR(char) const lds1 = lds0 + STAGE;
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -74,15 +102,22 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
   const int m0 = pm * BM, n0 = pn * BN;
 
-  // per-lane global source pointers of the k = 0 tile
-  const char* srcA[CopyA::kIters];
+  // per-lane global source pointers of the k = 0 tile; rows past the matrix edge are clamped
+  // onto the last valid row (their products are never stored)
+  const char* srcA[ITA];
   const char* srcB[ITB];
 #pragma unroll
-  for (int i = 0; i < CopyA::kIters; i++) srcA[i] = CopyA::src(p.A, p.lda, m0, p.M, wave, lane, i);
+  for (int i = 0; i < ITA; i++) {
+    int r = CopyA::row(wave, lane, i);
+    int gr = min(m0 + r, p.M - 1);
+    srcA[i] = p.A + (int64_t)gr * p.lda + CopyA::chunk(lane, r) * 16;
+  }
 #pragma unroll
   for (int i = 0; i < ITB; i++) {
     if constexpr (B_KMAJOR) {
-      srcB[i] = CopyBk::src(p.B, p.ldb, n0, p.N, wave, lane, i);
+      int r = CopyBk::row(wave, lane, i);
+      int gr = min(n0 + r, p.N - 1);
+      srcB[i] = p.B + (int64_t)gr * p.ldb + CopyBk::chunk(lane, r) * 16;
     } else {
       int r = CopyBn::row(wave, lane, i);
       int n = n0 + CopyBn::col16(lane, r) * 8;
@@ -90,38 +125,35 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
       srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
     }
   }
-  const int64_t stepA = 128, stepB = B_KMAJOR ? (int64_t)128 : 64 * p.ldb;
+  const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
 
   auto issue_tile = [&](int kt, LDS_PTR(char) a) {
     LDS_PTR(char) b = a + A_BYTES;
 #pragma unroll
-    for (int i = 0; i < CopyA::kIters; i++)
-      async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
+    for (int i = 0; i < ITA; i++) async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
 #pragma unroll
-    for (int i = 0; i < ITB; i++)
-      async_copy16(srcB[i] + kt * stepB, (LDS_PTR(void))(b + (i * NW + wave) * 1024));
+    for (int i = 0; i < ITB; i++) async_copy16(srcB[i] + kt * stepB, (LDS_PTR(void))(b + (i * NW + wave) * 1024));
   };
   // Last, partial K tile: chunks past K are written as zeros (the reference masks them to 0,
   // python/tutorials/03-matrix-multiplication.py:297-298); goes through registers.
   auto guarded_tile = [&](int kt, LDS_PTR(char) a) {
     LDS_PTR(char) b = a + A_BYTES;
-    const int kbase = kt * 128;  // bytes along K
+    const int kbase = kt * RBK;  // bytes along K
 #pragma unroll
-    for (int i = 0; i < CopyA::kIters; i++) {
-      int r = (i * NW + wave) * 8 + (lane >> 3);
-      int kb = kbase + (((lane & 7) ^ ((r >> 1) & 7)) << 4);
+    for (int i = 0; i < ITA; i++) {
+      int r = CopyA::row(wave, lane, i);
       i32x4 v = {0, 0, 0, 0};
-      if (kb < p.k_bytes) v = *(const i32x4*)(srcA[i] + kt * stepA);
+      if (kbase + CopyA::chunk(lane, r) * 16 < p.k_bytes) v = *(const i32x4*)(srcA[i] + kt * stepA);
       *(LDS_PTR(i32x4))(a + (i * NW + wave) * 1024 + lane * 16) = v;
     }
 #pragma unroll
     for (int i = 0; i < ITB; i++) {
       bool ok;
       if constexpr (B_KMAJOR) {
-        int r = (i * NW + wave) * 8 + (lane >> 3);
-        ok = kbase + (((lane & 7) ^ ((r >> 1) & 7)) << 4) < p.k_bytes;
+        int r = CopyBk::row(wave, lane, i);
+        ok = kbase + CopyBk::chunk(lane, r) * 16 < p.k_bytes;
       } else {
-        ok = kt * 64 + CopyBn::row(wave, lane, i) < p.K;
+        ok = kt * KROWS + CopyBn::row(wave, lane, i) < p.K;
       }
       i32x4 v = {0, 0, 0, 0};
       if (ok) v = *(const i32x4*)(srcB[i] + kt * stepB);
@@ -137,11 +169,9 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-  const int nfull = p.k_bytes / 128;
-
   // Per-lane LDS byte offsets of the MFMA operands inside one stage.
   //   K-major operand (A always, B when B_KMAJOR): lane reads row (l%32) and the 16-byte
-  //   chunk(s) Cfg::chunk(ks, l/32, c), swizzled; 32-row sub-tiles add t * 4096.
+  //   chunk(s) Cfg::chunk(ks, l/32, c), swizzled; 32-row sub-tiles add t * 32 * RBK.
   //   Row-major B: transpose read, lane i of a 16-lane group q addresses k row
   //   16*ks + 8*(q/2) + i/4 (+4 for the second half) and 32-byte group (n/16) ^ 2*(k & 3).
   const int l32 = lane & 31, g = lane >> 5;
@@ -151,8 +181,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   for (int ks = 0; ks < KS; ks++)
 #pragma unroll
     for (int c = 0; c < NC; c++) {
-      offA[ks][c] = swz128(wm * TM + l32, Cfg::chunk(ks, g, c));
-      offB[ks][c] = A_BYTES + swz128(wn * TN + l32, Cfg::chunk(ks, g, c));
+      offA[ks][c] = kmajor_off(wm * TM + l32, Cfg::chunk(ks, g, c));
+      offB[ks][c] = A_BYTES + kmajor_off(wn * TN + l32, Cfg::chunk(ks, g, c));
     }
   unsigned offBn[NT];
   {
@@ -181,12 +211,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
     constexpr int ks = decltype(KS_)::value;
     static_for<MT>([&](auto T_) {
       constexpr int t = decltype(T_)::value;
-      f.a[t] = read_operand(base, offA[ks], std::integral_constant<int, t * 4096>{});
+      f.a[t] = read_operand(base, offA[ks], std::integral_constant<int, t * 32 * RBK>{});
     });
     static_for<NT>([&](auto T_) {
       constexpr int t = decltype(T_)::value;
       if constexpr (B_KMAJOR) {
-        f.b[t] = read_operand(base, offB[ks], std::integral_constant<int, t * 4096>{});
+        f.b[t] = read_operand(base, offB[ks], std::integral_constant<int, t * 32 * RBK>{});
       } else {
         constexpr int imm = ks * 16 * BN * 2;
         i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t]);
@@ -204,21 +234,29 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
     for (int t = 0; t < NT; t++) lds_use(f.b[t]);
   };
 
-  // block scales of the current K tile: one dword (4 e8m0 bytes) per 32-row sub-tile and lane
+  // block scales of the K step being multiplied and of the next one: one dword per 32-row
+  // sub-tile and lane, already shifted so that byte `ks` is the scale of sub-step ks
   int sa[MT], sb[NT], sa_next[MT], sb_next[NT];
   auto load_scales = [&](int kt, int (&da)[MT], int (&db)[NT]) {
     if constexpr (Cfg::kScaled) {
-      const int koff = kt * Cfg::kScaleBytesPerTile + Cfg::scale_byte_offset(g);
 #pragma unroll
       for (int t = 0; t < MT; t++) {
         int r = min(m0 + wm * TM + t * 32 + l32, p.M - 1);
-        da[t] = Cfg::scale_fixup(*(const int*)(p.sA + (int64_t)r * p.lds_a + koff), g);
+        da[t] = Cfg::load_scale(p.sA + (int64_t)r * p.lds_a, kt, g);
       }
 #pragma unroll
       for (int t = 0; t < NT; t++) {
         int r = min(n0 + wn * TN + t * 32 + l32, p.N - 1);
-        db[t] = Cfg::scale_fixup(*(const int*)(p.sB + (int64_t)r * p.lds_b + koff), g);
+        db[t] = Cfg::load_scale(p.sB + (int64_t)r * p.lds_b, kt, g);
       }
+    }
+  };
+  auto rotate_scales = [&]() {
+    if constexpr (Cfg::kScaled) {
+#pragma unroll
+      for (int t = 0; t < MT; t++) sa[t] = sa_next[t];
+#pragma unroll
+      for (int t = 0; t < NT; t++) sb[t] = sb_next[t];
     }
   };
 
@@ -234,11 +272,11 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
       }
   };
 
-  // One 128-byte K tile.  When the registers allow it, the operands of sub-step ks+1 are
-  // requested before the MFMAs of sub-step ks; otherwise the second wave on the SIMD has to
-  // cover the LDS latency.
+  // One K step.  When the registers allow it, the operands of sub-step ks+1 are requested
+  // before the MFMAs of sub-step ks; otherwise the second wave on the SIMD has to cover the LDS
+  // latency.
   constexpr int kOperandRegs = (MT + NT) * NC * 4;
-  constexpr bool kPrefetch = 2 * kOperandRegs + MT * NT * 16 + (Cfg::kScaled ? 2 * (MT + NT) : 0) <= 184 * (512 / (NW * 64)) + (NW == 4 ? 128 : 0);
+  constexpr bool kPrefetch = KS > 1 && 2 * kOperandRegs + MT * NT * 16 + (Cfg::kScaled ? 2 * (MT + NT) : 0) <= 184 * (512 / (NW * 64));
   auto compute_tile = [&](LDS_PTR(char) stage) {
     const unsigned base = lds_addr(stage);
     if constexpr (kPrefetch) {
@@ -266,45 +304,40 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
     }
   };
 
-  // K loop over the full tiles, two per trip: the tile for step kt+1 streams into the idle
-  // stage while step kt is multiplied out of the other.
-  if (nfull > 0) {
-    issue_tile(0, lds0);
-    load_scales(0, sa, sb);
-    wait_all();
-    __syncthreads();
-    for (int kt = 0; kt < nfull; kt += 2) {
-      if (kt + 1 < nfull) { issue_tile(kt + 1, lds1); load_scales(kt + 1, sa_next, sb_next); }
-      compute_tile(lds0);
-      wait_all();
-      __syncthreads();
-      if (kt + 1 < nfull) {
-        if constexpr (Cfg::kScaled) {
+  // ---- K loop: loads run NS-1 steps ahead.  Step kt:  wait for the loads of tile kt only,
+  //      barrier (every wave's part of tile kt is in LDS, and every wave has finished reading
+  //      tile kt-1), refill the stage tile kt-1 occupied with tile kt+NS-1, multiply tile kt.
+  const int nfull = p.k_bytes / RBK;
+  constexpr int kLoadsPerTile = ITA + ITB;
+  constexpr int kScaleLoads = Cfg::kScaled ? MT + NT : 0;
 #pragma unroll
-          for (int t = 0; t < MT; t++) sa[t] = sa_next[t];
-#pragma unroll
-          for (int t = 0; t < NT; t++) sb[t] = sb_next[t];
-        }
-        if (kt + 2 < nfull) { issue_tile(kt + 2, lds0); load_scales(kt + 2, sa_next, sb_next); }
-        compute_tile(lds1);
-        wait_all();
-        __syncthreads();
-        if constexpr (Cfg::kScaled) {
-#pragma unroll
-          for (int t = 0; t < MT; t++) sa[t] = sa_next[t];
-#pragma unroll
-          for (int t = 0; t < NT; t++) sb[t] = sb_next[t];
-        }
-      }
-    }
+  for (int s = 0; s < NS - 1; s++)
+    if (s < nfull) issue_tile(s, lds + s * STAGE);
+  if (nfull > 0) load_scales(0, sa, sb);
+  int stage = 0, fill = NS - 1;  // stage of tile kt, stage to refill
+  for (int kt = 0; kt < nfull; kt++) {
+    // Younger than the loads of tile kt are, in steady state, NS-2 whole steps (their tile
+    // loads and the scale loads each of them issued) plus the scale loads of the step that issued
+    // tile kt.  The prologue and the last steps issue fewer: they wait for everything.
+    constexpr int kYounger = (NS - 2) * (kLoadsPerTile + kScaleLoads) + kScaleLoads;
+    const bool steady = kt + NS - 2 < nfull && (!Cfg::kScaled || kt >= NS - 1);
+    if (steady) wait_vmcnt<kYounger>(); else wait_vmcnt<0>();
+    block_barrier();
+    if (kt + NS - 1 < nfull) issue_tile(kt + NS - 1, lds + fill * STAGE);
+    if (kt + 1 < nfull) load_scales(kt + 1, sa_next, sb_next);
+    compute_tile(lds + stage * STAGE);
+    rotate_scales();
+    stage = stage + 1 == NS ? 0 : stage + 1;
+    fill = fill + 1 == NS ? 0 : fill + 1;
   }
-  // K tail (K bytes % 128 != 0): one more tile, zero-filled past K, outside the pipelined loop.
+  // K tail (K bytes % RBK != 0): one more tile, zero-filled past K, outside the pipelined loop.
   // (Block-scaled operands always come in whole tiles.)
-  if (nfull * 128 < p.k_bytes) {
-    guarded_tile(nfull, lds0);
+  if (nfull * RBK < p.k_bytes) {
+    block_barrier();  // every wave is done with the ring
+    guarded_tile(nfull, lds);
     wait_all();
     __syncthreads();
-    compute_tile(lds0);
+    compute_tile(lds);
   }
 
   // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3
@@ -359,26 +392,28 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   }
 }
 
-template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR>
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
 static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * (BM + BN) * 128;
+  constexpr int smem = NS * (BM + BN) * RBK;
+  static_assert(smem <= 160 * 1024, "LDS ring does not fit");
   static bool attr_set = false;  // benign race: setting the attribute twice is harmless
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR, NS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
-  gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR><<<dim3(num_m * num_n), dim3(WM * WN * 64), smem, stream>>>(p);
+  gemm_kernel<Cfg, BM, BN, WM, WN, B_KMAJOR, NS><<<dim3(num_m * num_n), dim3(WM * WN * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
-// tile: 0 = 256x256 / 8 waves, 1 = 128x128 / 4 waves
+// tile: 0 = 256x256 / 8 waves / 4 stages (one workgroup per CU),
+//       1 = 128x128 / 4 waves / 4 stages (two workgroups per CU)
 template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
-  if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR>(p, stream);
-  return launch_gemm<Cfg, 256, 256, 2, 4, B_KMAJOR>(p, stream);
+  if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR, 4>(p, stream);
+  return launch_gemm<Cfg, 256, 256, 2, 4, B_KMAJOR, 4>(p, stream);
 }
 
 }  // namespace mi355

@@ -1,13 +1,13 @@
-// Block-scaled (OCP MX v1.0) instantiations of the tiled MFMA GEMM core: MXFP4 (e2m1, 256
-// elements per 128-byte K tile, four 32x32x64 sub-steps) and MXFP8 (e4m3, 128 elements, two
-// sub-steps), one e8m0 scale per 32 elements of K applied inside the MFMA.
+// Block-scaled (OCP MX v1.0) instantiations of the tiled MFMA GEMM core: MXFP4 (e2m1, 128
+// elements per 64-byte K step, two 32x32x64 sub-steps) and MXFP8 (e4m3, 64 elements, one
+// sub-step), one e8m0 scale per 32 elements of K applied inside the MFMA.
 //
 // How the scaled 32x32x64 f8f6f4 MFMA takes its scales (measured on gfx950): every lane passes
 // one dword and a byte selector.  fp4: the selected byte of lane (row, g) scales that lane's own
 // 32 elements.  fp8: registers 0-3 of both lane groups form K block 0 and are scaled by the byte
 // from lane group 0, registers 4-7 form K block 1 and take the byte from lane group 1.  The K
-// positions a lane reads are therefore chosen such that the scale byte it needs is byte `ks` of
-// a dword whose address does not depend on ks.
+// positions a lane reads are therefore chosen such that the scale byte it needs sits at a byte
+// position that does not depend on the lane.
 #include "gemm_core.h"
 #include "formats.h"
 
@@ -15,13 +15,14 @@ namespace mi355 {
 
 struct CfgMxfp4 {
   using Operand = i32x4;
-  static constexpr int kSteps = 4, kChunks = 1;
+  static constexpr int kSteps = 2, kChunks = 1;
   static constexpr bool kRowMajorB = false, kScaled = true;
-  static constexpr int kScaleBytesPerTile = 8;  // 256 elements / 32
-  // lane group g reads scale blocks 4g .. 4g+3 of the tile, one per sub-step
-  __device__ static constexpr int chunk(int ks, int g, int) { return g * 4 + ks; }
-  __device__ static int scale_byte_offset(int g) { return g * 4; }
-  __device__ static int scale_fixup(int v, int) { return v; }
+  // lane group g reads scale blocks 2g, 2g+1 of the step (16 bytes = 32 elements each), one per sub-step
+  __device__ static constexpr int chunk(int ks, int g, int) { return g * 2 + ks; }
+  // the step has 4 scale bytes per row; move bytes 2g, 2g+1 to positions 0, 1 (selector = ks)
+  __device__ static int load_scale(const uint8_t* row, int kt, int g) {
+    return (int)(*(const uint32_t*)(row + kt * 4) >> (16 * g));
+  }
   template <int ks>
   __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
 #if MI355_DEVICE_PASS
@@ -37,18 +38,18 @@ struct CfgMxfp4 {
 
 struct CfgMxfp8 {
   using Operand = i32x8;
-  static constexpr int kSteps = 2, kChunks = 2;
+  static constexpr int kSteps = 1, kChunks = 2;
   static constexpr bool kRowMajorB = false, kScaled = true;
-  static constexpr int kScaleBytesPerTile = 4;  // 128 elements / 32
-  // register half c of sub-step ks is scale block 2c + ks; lane group g holds its 16-byte half g
-  __device__ static constexpr int chunk(int ks, int g, int c) { return 4 * c + 2 * ks + g; }
-  __device__ static int scale_byte_offset(int) { return 0; }
-  // lane group g supplies the scales of blocks 2g + ks: move them to bytes 0 and 1
-  __device__ static int scale_fixup(int v, int g) { return (int)((unsigned)v >> (16 * g)); }
+  // register half c is scale block c of the step; lane group g holds its 16-byte half g
+  __device__ static constexpr int chunk(int, int g, int c) { return 2 * c + g; }
+  // the step has 2 scale bytes per row; lane group g supplies the scale of block g in byte 0
+  __device__ static int load_scale(const uint8_t* row, int kt, int g) {
+    return (int)(*(const uint16_t*)(row + kt * 2)) >> (8 * g);
+  }
   template <int ks>
   __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
 #if MI355_DEVICE_PASS
-    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, ks, sa, ks, sb);
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, sa, 0, sb);
 #else
     return c;
 #endif
@@ -56,7 +57,7 @@ struct CfgMxfp8 {
 };
 
 // Any shape / pitch: one thread per output, decode-and-FMA in fp32.  Used when K is not a
-// whole number of 128-byte tiles or the scale rows are not dword aligned.
+// whole number of 64-byte steps or the scale rows are not dword aligned.
 __global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4) {
   int n = blockIdx.x * 16 + threadIdx.x % 16, m = blockIdx.y * 16 + threadIdx.x / 16;
   if (m >= p.M || n >= p.N) return;
@@ -88,7 +89,7 @@ __global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4
 }
 
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
-  const bool whole_tiles = p.k_bytes % 128 == 0;
+  const bool whole_tiles = p.k_bytes % RBK == 0;
   const bool scales_aligned = p.lds_a % 4 == 0 && p.lds_b % 4 == 0 && ((uintptr_t)p.sA % 4) == 0 && ((uintptr_t)p.sB % 4) == 0;
   if (!whole_tiles || !scales_aligned || tile < 0) {
     dim3 grid((p.N + 15) / 16, (p.M + 15) / 16);
