@@ -53,6 +53,13 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds
 #endif
 }
 
+// 4 bytes per lane, same addressing: lane i writes lds_wave_base + 4 * i.
+__device__ __forceinline__ void async_copy4(const void* gsrc, LDS_PTR(void) lds_wave_base) {
+#if MI355_DEVICE_PASS
+  __builtin_amdgcn_global_load_lds(gsrc, lds_wave_base, 4, 0, 0);
+#endif
+}
+
 // 2^x by the hardware transcendental unit (denormal results flush to zero, as the reference
 // allows on AMD: python/tutorials/06-fused-attention.py:452-454 `allow_flush_denorm`).
 __device__ __forceinline__ float fast_exp2(float x) {
@@ -102,6 +109,14 @@ __device__ __forceinline__ i32x4 lds_read_b128(unsigned addr) {
   i32x4 v = {};
 #if MI355_DEVICE_PASS
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ int lds_read_b32(unsigned addr) {
+  int v = 0;
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
 #endif
   return v;
 }

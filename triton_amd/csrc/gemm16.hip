@@ -9,6 +9,7 @@ struct Cfg16 {
   using Operand = V8;
   static constexpr int kSteps = 2, kChunks = 1;
   static constexpr bool kRowMajorB = true, kScaled = false;
+  static constexpr int kStepsPerScaleDword = 1;
   // lane group g of sub-step ks reads k elements 16*ks + 8*g .. +8
   __device__ static constexpr int chunk(int ks, int g, int) { return ks * 2 + g; }
   template <int ks>

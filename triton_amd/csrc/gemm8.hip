@@ -11,6 +11,7 @@ struct Cfg8 {
   using Operand = i32x8;
   static constexpr int kSteps = 1, kChunks = 2;
   static constexpr bool kRowMajorB = false, kScaled = false;
+  static constexpr int kStepsPerScaleDword = 1;
   // A lane feeds 32 bytes per sub-step as two 16-byte halves; any assignment of K positions
   // works as long as both operands use the same one.
   __device__ static constexpr int chunk(int, int g, int c) { return c * 2 + g; }

@@ -75,6 +75,63 @@ struct TileCopyKN {
   }
 };
 
+// Epilogue shared by the GEMM kernels: alpha, activation, cast, store.  With the operands
+// swapped (D[n][m]) lane l owns C row `mrow0 + 32 i + l%32` and, per register group rg of tile
+// (i, j), the four consecutive columns `ncol0 + 32 j + 8 rg + 4 (l/32) ..`.
+template <int MT, int NT>
+__device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l32, int g) {
+  // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3
+  float alpha = 1.f;
+  if (p.a_scale) alpha *= *p.a_scale;
+  if (p.b_scale) alpha *= *p.b_scale;
+  const bool leaky = p.activation == 1;
+  const bool vec_ok = p.c_vec_ok;
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    int m = mrow0 + i * 32 + l32;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int j = 0; j < NT; j++) {
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        int n = ncol0 + j * 32 + rg * 8 + g * 4;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          float x = acc[i][j][rg * 4 + e] * alpha;
+          if (leaky) x = x >= 0.f ? x : 0.01f * x;
+          v[e] = x;
+        }
+        if (p.out_dtype == 4) {
+          float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = v[e];
+          }
+        } else if (p.out_dtype == 1) {
+          __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (__bf16)v[e];
+          }
+        } else {
+          _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+          if (vec_ok && n + 3 < p.N) {
+            *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+          } else {
+#pragma unroll
+            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (_Float16)v[e];
+          }
+        }
+      }
+    }
+  }
+}
+
 template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   using Operand = typename Cfg::Operand;
@@ -340,56 +397,244 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
     compute_tile(lds);
   }
 
-  // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3
-  float alpha = 1.f;
-  if (p.a_scale) alpha *= *p.a_scale;
-  if (p.b_scale) alpha *= *p.b_scale;
-  const bool leaky = p.activation == 1;
-  const bool vec_ok = p.c_vec_ok;
+  gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Ping-pong variant for the 8-wave tiles.  With one barrier per K step all eight waves stall,
+// issue loads and wait for their first LDS reads at the same time, and the MFMA pipes idle
+// meanwhile.  Here the two waves that share a SIMD (wave w and wave w+4) run half a step apart:
+// every K step of a wave is a MEMORY phase (issue its share of the direct loads for the tile
+// NS-1 steps ahead, read ALL operands of the current tile from LDS into registers) and a
+// COMPUTE phase (nothing but MFMAs), separated by workgroup barriers.  Waves 4-7 execute one
+// extra barrier before their loop and waves 0-3 one after, so at every barrier one wave of each
+// SIMD arrives from MFMAs and the other from memory work.
+//
+// Hazards:  a stage is refilled (tile kt+NS-1 into the stage of tile kt-1) in MEM(kt); waves 0-3
+// do that in phase 2kt, after the barrier that ended waves 4-7's MEM(kt-1), the last reader of
+// tile kt-1.  Tile kt is first read in phase 2kt; every wave waits for its own share of tile kt
+// before the barrier that ends phase 2kt-1 (waves 0-3 at the end of COMPUTE(kt-1), waves 4-7 at
+// the end of MEM(kt-1)), leaving its NS-2 younger shares in flight.
+//
+// Block scales (MX) travel with the tile: every wave copies 64 rows x 4 scale bytes per step
+// with a 4-byte direct load (waves 0-3 the A rows, waves 4-7 the B rows).
+// ---------------------------------------------------------------------------------------------
+template <typename Cfg, int BM, int BN, bool B_KMAJOR, int NS>
+__global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
+  using Operand = typename Cfg::Operand;
+  constexpr int WM = 2, WN = 4, NW = 8, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
+  constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK;
+  constexpr int SC_BYTES = Cfg::kScaled ? (BM + BN) * 4 : 0;
+  constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+  constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
+  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  static_assert(!Cfg::kScaled || (BM == 256 && BN == 256), "scale copies assume 64 rows per wave");
+  using CopyA = TileCopyK<BM, NW>;
+  using CopyBk = TileCopyK<BN, NW>;
+  using CopyBn = TileCopyKN<BN, NW>;
+  constexpr int ITA = CopyA::kIters;
+  constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
+  constexpr int KROWS = RBK / 2;
+  constexpr int kShare = ITA + ITB + (Cfg::kScaled ? 1 : 0);  // direct loads per wave and tile
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+  // the half of the waves that runs one phase behind (kept in a scalar register: the barriers
+  // below must be skipped by a real branch)
+  const bool late = __builtin_amdgcn_readfirstlane(tid) >= 256;
+
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  int pid = xcd_remap(blockIdx.x, num_m * num_n);
+  int pm, pn;
+  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
+  const int m0 = pm * BM, n0 = pn * BN;
+
+  const char* srcA[ITA];
+  const char* srcB[ITB];
 #pragma unroll
-  for (int i = 0; i < MT; i++) {
-    int m = m0 + wm * TM + i * 32 + l32;
-    if (m >= p.M) continue;
+  for (int i = 0; i < ITA; i++) {
+    int r = CopyA::row(wave, lane, i);
+    int gr = min(m0 + r, p.M - 1);
+    srcA[i] = p.A + (int64_t)gr * p.lda + CopyA::chunk(lane, r) * 16;
+  }
 #pragma unroll
-    for (int j = 0; j < NT; j++) {
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        int n = n0 + wn * TN + j * 32 + rg * 8 + g * 4;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          float x = acc[i][j][rg * 4 + e] * alpha;
-          if (leaky) x = x >= 0.f ? x : 0.01f * x;
-          v[e] = x;
-        }
-        if (p.out_dtype == 4) {
-          float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = v[e];
-          }
-        } else if (p.out_dtype == 1) {
-          __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (__bf16)v[e];
-          }
-        } else {
-          _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (_Float16)v[e];
-          }
-        }
-      }
+  for (int i = 0; i < ITB; i++) {
+    if constexpr (B_KMAJOR) {
+      int r = CopyBk::row(wave, lane, i);
+      int gr = min(n0 + r, p.N - 1);
+      srcB[i] = p.B + (int64_t)gr * p.ldb + CopyBk::chunk(lane, r) * 16;
+    } else {
+      int r = CopyBn::row(wave, lane, i);
+      int n = n0 + CopyBn::col16(lane, r) * 8;
+      n = n < p.N ? n : p.N - 8;
+      srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
     }
   }
+  const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
+  // scale rows this lane copies: waves 0-3 rows 64*wave + lane of A, waves 4-7 of B
+  const uint8_t* srcS = nullptr;
+  if constexpr (Cfg::kScaled) {
+    if (!late) srcS = p.sA + (int64_t)min(m0 + wave * 64 + lane, p.M - 1) * p.lds_a;
+    else srcS = p.sB + (int64_t)min(n0 + (wave - 4) * 64 + lane, p.N - 1) * p.lds_b;
+  }
+
+  auto issue_share = [&](int kt, LDS_PTR(char) a) {
+    LDS_PTR(char) b = a + A_BYTES;
+#pragma unroll
+    for (int i = 0; i < ITA; i++) async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
+#pragma unroll
+    for (int i = 0; i < ITB; i++) async_copy16(srcB[i] + kt * stepB, (LDS_PTR(void))(b + (i * NW + wave) * 1024));
+    if constexpr (Cfg::kScaled) async_copy4(srcS + Cfg::scale_dword_offset(kt), (LDS_PTR(void))(a + A_BYTES + B_BYTES + wave * 256));
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int l32 = lane & 31, g = lane >> 5;
+  const int i16 = lane & 15, q = lane >> 4;
+  unsigned offA[KS][NC], offB[KS][NC];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+      offA[ks][c] = kmajor_off(wm * TM + l32, Cfg::chunk(ks, g, c));
+      offB[ks][c] = A_BYTES + kmajor_off(wn * TN + l32, Cfg::chunk(ks, g, c));
+    }
+  unsigned offBn[NT];
+  {
+    int k = (q >> 1) * 8 + (i16 >> 2);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      int c32 = (wn * TN + t * 32) / 16 + (q & 1);
+      offBn[t] = A_BYTES + k * (BN * 2) + ((c32 ^ ((k & 3) << 1)) << 5) + (i16 & 3) * 8;
+    }
+  }
+  const unsigned offSA = A_BYTES + B_BYTES + (wm * TM + l32) * 4;
+  const unsigned offSB = A_BYTES + B_BYTES + BM * 4 + (wn * TN + l32) * 4;
+
+  Operand fa[KS][MT], fb[KS][NT];
+  int sa[MT], sb[NT];
+  auto read_tile = [&](unsigned base, int kt) {
+    static_for<KS>([&](auto KS_) {
+      constexpr int ks = decltype(KS_)::value;
+      static_for<MT>([&](auto T_) {
+        constexpr int t = decltype(T_)::value;
+        if constexpr (NC == 1) {
+          fa[ks][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offA[ks][0]));
+        } else {
+          i32x4 lo = lds_read_b128<t * 32 * RBK>(base + offA[ks][0]);
+          i32x4 hi = lds_read_b128<t * 32 * RBK>(base + offA[ks][1]);
+          fa[ks][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      });
+      static_for<NT>([&](auto T_) {
+        constexpr int t = decltype(T_)::value;
+        if constexpr (!B_KMAJOR) {
+          constexpr int imm = ks * 16 * BN * 2;
+          i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t]);
+          i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[t]);
+          fb[ks][t] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+        } else if constexpr (NC == 1) {
+          fb[ks][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offB[ks][0]));
+        } else {
+          i32x4 lo = lds_read_b128<t * 32 * RBK>(base + offB[ks][0]);
+          i32x4 hi = lds_read_b128<t * 32 * RBK>(base + offB[ks][1]);
+          fb[ks][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        }
+      });
+    });
+    if constexpr (Cfg::kScaled) {
+      static_for<MT>([&](auto T_) { constexpr int t = decltype(T_)::value; sa[t] = lds_read_b32<t * 128>(base + offSA); });
+      static_for<NT>([&](auto T_) { constexpr int t = decltype(T_)::value; sb[t] = lds_read_b32<t * 128>(base + offSB); });
+    }
+    lds_wait<0>();
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+#pragma unroll
+      for (int t = 0; t < MT; t++) lds_use(fa[ks][t]);
+#pragma unroll
+      for (int t = 0; t < NT; t++) lds_use(fb[ks][t]);
+    }
+    if constexpr (Cfg::kScaled) {
+#pragma unroll
+      for (int t = 0; t < MT; t++) { lds_use(sa[t]); sa[t] = Cfg::scale_fixup(sa[t], kt, g); }
+#pragma unroll
+      for (int t = 0; t < NT; t++) { lds_use(sb[t]); sb[t] = Cfg::scale_fixup(sb[t], kt, g); }
+    }
+  };
+  auto multiply_tile = [&]() {
+    static_for<KS>([&](auto KS_) {
+      constexpr int ks = decltype(KS_)::value;
+#pragma unroll
+      for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int j = 0; j < NT; j++) {
+          if constexpr (Cfg::kScaled) acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], sb[j], sa[i]);
+          else acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], 0, 0);
+        }
+    });
+  };
+  auto phase_barrier = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    block_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // wait for this wave's share of tile `next`, given that shares up to tile `issued_upto` are out
+  auto wait_share = [&](int next_plus, int nfull) {
+    // called with next_plus = j + NS - 1 where j is the current step: in steady state NS-2
+    // younger shares stay in flight, near the end of K everything is awaited
+    if (next_plus < nfull) wait_vmcnt<(NS - 2) * kShare>(); else wait_vmcnt<0>();
+  };
+
+  const int nfull = p.k_bytes / RBK;
+#pragma unroll
+  for (int s = 0; s < NS - 1; s++)
+    if (s < nfull) issue_share(s, lds + s * STAGE);
+  if (NS - 1 <= nfull) wait_vmcnt<(NS - 2) * kShare>(); else wait_vmcnt<0>();
+  phase_barrier();            // tile 0 is in LDS
+  if (late) phase_barrier();  // waves 4-7 start one phase later
+
+  int stage = 0, fill = NS - 1;
+  for (int kt = 0; kt < nfull; kt++) {
+    // ---- memory phase
+    if (kt + NS - 1 < nfull) issue_share(kt + NS - 1, lds + fill * STAGE);
+    read_tile(lds_addr(lds + stage * STAGE), kt);
+    if (late) wait_share(kt + NS - 1, nfull);
+    phase_barrier();
+    // ---- compute phase
+    multiply_tile();
+    if (!late) wait_share(kt + NS - 1, nfull);
+    phase_barrier();
+    stage = stage + 1 == NS ? 0 : stage + 1;
+    fill = fill + 1 == NS ? 0 : fill + 1;
+  }
+  if (!late) phase_barrier();  // waves 0-3 catch up: every wave has executed the same number of barriers
+
+  gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+}
+
+template <typename Cfg, int BM, int BN, bool B_KMAJOR, int NS>
+static int launch_gemm_pp(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = NS * ((BM + BN) * RBK + (Cfg::kScaled ? (BM + BN) * 4 : 0));
+  static_assert(smem <= 160 * 1024, "LDS ring does not fit");
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_pp_kernel<Cfg, BM, BN, B_KMAJOR, NS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  gemm_pp_kernel<Cfg, BM, BN, B_KMAJOR, NS><<<dim3(num_m * num_n), dim3(512), smem, stream>>>(p);
+  return (int)hipGetLastError();
 }
 
 template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
@@ -408,11 +653,13 @@ static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-// tile: 0 = 256x256 / 8 waves / 4 stages (one workgroup per CU),
-//       1 = 128x128 / 4 waves / 4 stages (two workgroups per CU)
+// tile: 0 = 256x256 / 8 waves / 4 stages, ping-pong phases (whole K steps only, else tile 2),
+//       1 = 128x128 / 4 waves / 4 stages (two workgroups per CU),
+//       2 = 256x256 / 8 waves / 4 stages, one barrier per step
 template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
   if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR, 4>(p, stream);
+  if (tile == 0 && p.k_bytes % (RBK * Cfg::kStepsPerScaleDword) == 0) return launch_gemm_pp<Cfg, 256, 256, B_KMAJOR, 4>(p, stream);
   return launch_gemm<Cfg, 256, 256, 2, 4, B_KMAJOR, 4>(p, stream);
 }
 

@@ -16,6 +16,7 @@ namespace mi355 {
 struct CfgMxfp4 {
   using Operand = i32x4;
   static constexpr int kSteps = 2, kChunks = 1;
+  static constexpr int kStepsPerScaleDword = 1;  // 4 scale bytes per row and K step
   static constexpr bool kRowMajorB = false, kScaled = true;
   // lane group g reads scale blocks 2g, 2g+1 of the step (16 bytes = 32 elements each), one per sub-step
   __device__ static constexpr int chunk(int ks, int g, int) { return g * 2 + ks; }
@@ -23,6 +24,8 @@ struct CfgMxfp4 {
   __device__ static int load_scale(const uint8_t* row, int kt, int g) {
     return (int)(*(const uint32_t*)(row + kt * 4) >> (16 * g));
   }
+  __device__ static int scale_dword_offset(int kt) { return kt * 4; }          // dword copied to LDS for step kt
+  __device__ static int scale_fixup(int v, int, int g) { return (int)((unsigned)v >> (16 * g)); }
   template <int ks>
   __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
 #if MI355_DEVICE_PASS
@@ -39,6 +42,7 @@ struct CfgMxfp4 {
 struct CfgMxfp8 {
   using Operand = i32x8;
   static constexpr int kSteps = 1, kChunks = 2;
+  static constexpr int kStepsPerScaleDword = 2;  // 2 scale bytes per row and K step
   static constexpr bool kRowMajorB = false, kScaled = true;
   // register half c is scale block c of the step; lane group g holds its 16-byte half g
   __device__ static constexpr int chunk(int, int g, int c) { return 2 * c + g; }
@@ -46,6 +50,9 @@ struct CfgMxfp8 {
   __device__ static int load_scale(const uint8_t* row, int kt, int g) {
     return (int)(*(const uint16_t*)(row + kt * 2)) >> (8 * g);
   }
+  // the dword holding the scales of steps kt and kt^1; bytes 2*(kt&1) + g
+  __device__ static int scale_dword_offset(int kt) { return (kt >> 1) * 4; }
+  __device__ static int scale_fixup(int v, int kt, int g) { return (int)((unsigned)v >> (16 * (kt & 1) + 8 * g)); }
   template <int ks>
   __device__ static f32x16 mma(Operand a, Operand b, f32x16 c, int sa, int sb) {
 #if MI355_DEVICE_PASS
