@@ -24,6 +24,15 @@ HIPCC_FLAGS = [
     "-Wno-unused-command-line-argument", "-Wno-ignored-attributes",
 ]
 
+# Per-file additions.  The attention kernels rescale their MFMA accumulators with VALU code every
+# key/value block, so the accumulators must live in architectural VGPRs: left to itself the
+# register allocator parks them in AGPRs and spends more VALU issue slots on
+# v_accvgpr_read/write pairs than on the softmax.
+EXTRA_FLAGS = {
+    "attn_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "attn_bwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
 
 def hipcc_path() -> str:
     for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
@@ -37,7 +46,7 @@ def lib_path() -> Path:
 
 
 def _compile(hipcc: str, src: Path, obj: Path, verbose: bool) -> None:
-    cmd = [hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)]
+    cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(src.name, []), "-c", str(src), "-o", str(obj)]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, capture_output=True, text=True)

@@ -22,8 +22,8 @@
 //                 the B operands of dV^T = dO^T p and dK^T = Q^T ds; K and V fragments stay in
 //                 registers, Q / dO tiles stream through LDS.
 // Every streamed tile is read both row-wise (ds_read_b128) and transposed
-// (ds_read_b64_tr_b16); one XOR swizzle serves both access patterns.
-#include "common.h"
+// (ds_read_b64_tr_b16); one XOR swizzle (attn_tiles.h) serves both access patterns.
+#include "attn_tiles.h"
 #include "launch.h"
 
 namespace mi355 {
@@ -56,47 +56,6 @@ __global__ __launch_bounds__(256) void attn_bwd_pre_kernel(AttnArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// shared LDS tile helpers: [rows][D*2 bytes], 16-byte chunk index XORed with
-//   f(row) = ((row & 3) << 1) | ((row >> 2) & 1)
-// 8 consecutive rows reading one logical chunk hit 8 distinct 16-byte bank groups (row-wise
-// reads), 4 consecutive rows reading one logical 32-byte group hit 4 distinct 32-byte groups
-// (transpose reads).
-// ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ int fsw(int row) { return ((row & 3) << 1) | ((row >> 2) & 1); }
-
-template <int D, int ROWS, int NW>
-struct BwdTile {
-  static constexpr int RB = D * 2, CPR = RB / 16, RPI = 1024 / RB;
-  static constexpr int BYTES = ROWS * RB;
-  static constexpr int INST = BYTES / 1024 / NW;
-  static_assert(INST >= 1, "tile too small for this wave count");
-  // source pointer of lane `lane`, wave `wave`, instruction i for the tile starting at row 0
-  __device__ static const char* src(const char* base, int64_t pitch, int wave, int lane, int i) {
-    int r = (i * NW + wave) * RPI + lane / CPR;
-    int lc = (lane % CPR) ^ fsw(r);
-    return base + (int64_t)r * pitch + lc * 16;
-  }
-};
-
-// per-lane offsets: row-wise operand read of row l32 (+32*tile), chunk 2*ks + g
-template <int RB>
-__device__ __forceinline__ void row_offsets(unsigned (&off)[4], int l32, int g) {
-#pragma unroll
-  for (int k4 = 0; k4 < 4; k4++) off[k4] = l32 * RB + ((((k4 * 2 + g) ^ fsw(l32)) & 7) << 4);
-}
-// per-lane offsets: transpose read; rows R0 + 4g + i16/4, 32 columns of sub-tile c (parity par)
-template <int RB>
-__device__ __forceinline__ void tr_offsets(unsigned (&off)[2], int i16, int q4) {
-  const int g = q4 >> 1, sub = q4 & 1;
-  const int row = 4 * g + (i16 >> 2);
-#pragma unroll
-  for (int par = 0; par < 2; par++) {
-    int l16 = par * 4 + 2 * sub + ((i16 & 3) >> 1);
-    off[par] = row * RB + (((l16 ^ fsw(row)) & 7) << 4) + (i16 & 1) * 8;
-  }
-}
-
-// ---------------------------------------------------------------------------------------------
 // dQ: one wave owns QT*32 query rows; K / V tiles of 64 rows stream through LDS.
 // ---------------------------------------------------------------------------------------------
 template <typename V8, int D, int QT, int NW>
@@ -104,7 +63,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
   using S = typename ElemB<V8>::type;
   typedef __attribute__((ext_vector_type(4))) S S4;
   constexpr int BM = NW * QT * 32, BN = 64, RB = D * 2, KSQ = D / 16, DT = D / 32;
-  using Tile = BwdTile<D, BN, NW>;
+  using Tile = AttnTile<RB, BN, NW>;
   constexpr int TILE = Tile::BYTES;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -161,9 +120,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     }
   };
 
-  unsigned offR[4], offT[2];
-  row_offsets<RB>(offR, l32, g);
-  tr_offsets<RB>(offT, i16, q4);
+  const RowRead<RB> rr(l32, g);
+  const TrRead<RB> tt(i16, q4);
 
   f32x16 dq[DT][QT];
 #pragma unroll
@@ -199,15 +157,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; r++) { s[b][r] = 0.f; dp[b][r] = 0.f; }
         i32x4 kf[2], vf[2];
-        kf[0] = a == 0 ? lds_read_b128<0>(kb + offR[0]) : lds_read_b128<32 * RB>(kb + offR[0]);
-        vf[0] = a == 0 ? lds_read_b128<0>(vb + offR[0]) : lds_read_b128<32 * RB>(vb + offR[0]);
+        kf[0] = a == 0 ? lds_read_b128<0>(rr.template addr<0>(kb)) : lds_read_b128<32 * RB>(rr.template addr<0>(kb));
+        vf[0] = a == 0 ? lds_read_b128<0>(rr.template addr<0>(vb)) : lds_read_b128<32 * RB>(rr.template addr<0>(vb));
         static_for<KSQ>([&](auto KS_) {
           constexpr int ks = decltype(KS_)::value;
           constexpr int cur = ks & 1, nxt = cur ^ 1;
           if constexpr (ks + 1 < KSQ) {
-            constexpr int imm = ((ks + 1) >> 2) * 128;
-            kf[nxt] = a == 0 ? lds_read_b128<imm>(kb + offR[(ks + 1) & 3]) : lds_read_b128<imm + 32 * RB>(kb + offR[(ks + 1) & 3]);
-            vf[nxt] = a == 0 ? lds_read_b128<imm>(vb + offR[(ks + 1) & 3]) : lds_read_b128<imm + 32 * RB>(vb + offR[(ks + 1) & 3]);
+            kf[nxt] = a == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(kb)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(kb));
+            vf[nxt] = a == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(vb)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(vb));
             lds_wait<2>();
           } else {
             lds_wait<0>();
@@ -243,9 +200,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
           constexpr int t = decltype(T_)::value;
           static_for<DT>([&](auto C_) {
             constexpr int c = decltype(C_)::value;
-            constexpr int imm = (c >> 1) * 128 + 16 * t * RB;
-            dst[c][0] = lds_read_tr16_b64<imm>(kb + offT[c & 1]);
-            dst[c][1] = lds_read_tr16_b64<imm + 8 * RB>(kb + offT[c & 1]);
+            dst[c][0] = lds_read_tr16_b64<16 * t * RB>(tt.template addr<c, 0>(kb));
+            dst[c][1] = lds_read_tr16_b64<(16 * t + 8) * RB>(tt.template addr<c, 1>(kb));
           });
         };
         read_t(std::integral_constant<int, 0>{}, tf[0]);
@@ -299,7 +255,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   using S = typename ElemB<V8>::type;
   typedef __attribute__((ext_vector_type(4))) S S4;
   constexpr int BN = NW * 32, BM = 64, MT = BM / 32, RB = D * 2, KSQ = D / 16, DT = D / 32;
-  using Tile = BwdTile<D, BM, NW>;
+  using Tile = AttnTile<RB, BM, NW>;
   constexpr int TILE = Tile::BYTES;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -352,9 +308,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     }
   };
 
-  unsigned offR[4], offT[2];
-  row_offsets<RB>(offR, l32, g);
-  tr_offsets<RB>(offT, i16, q4);
+  const RowRead<RB> rr(l32, g);
+  const TrRead<RB> tt(i16, q4);
 
   f32x16 dk[DT], dv[DT];
 #pragma unroll
@@ -397,15 +352,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
         for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
         {
           i32x4 qf[2], df[2];
-          qf[0] = mt == 0 ? lds_read_b128<0>(qb + offR[0]) : lds_read_b128<32 * RB>(qb + offR[0]);
-          df[0] = mt == 0 ? lds_read_b128<0>(db + offR[0]) : lds_read_b128<32 * RB>(db + offR[0]);
+          qf[0] = mt == 0 ? lds_read_b128<0>(rr.template addr<0>(qb)) : lds_read_b128<32 * RB>(rr.template addr<0>(qb));
+          df[0] = mt == 0 ? lds_read_b128<0>(rr.template addr<0>(db)) : lds_read_b128<32 * RB>(rr.template addr<0>(db));
           static_for<KSQ>([&](auto KS_) {
             constexpr int ks = decltype(KS_)::value;
             constexpr int cur = ks & 1, nxt = cur ^ 1;
             if constexpr (ks + 1 < KSQ) {
-              constexpr int imm = ((ks + 1) >> 2) * 128;
-              qf[nxt] = mt == 0 ? lds_read_b128<imm>(qb + offR[(ks + 1) & 3]) : lds_read_b128<imm + 32 * RB>(qb + offR[(ks + 1) & 3]);
-              df[nxt] = mt == 0 ? lds_read_b128<imm>(db + offR[(ks + 1) & 3]) : lds_read_b128<imm + 32 * RB>(db + offR[(ks + 1) & 3]);
+              qf[nxt] = mt == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(qb)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(qb));
+              df[nxt] = mt == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(db)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(db));
               lds_wait<2>();
             } else {
               lds_wait<0>();
@@ -435,17 +389,17 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
             constexpr int t = decltype(T_)::value;
             static_for<DT>([&](auto C_) {
               constexpr int c = decltype(C_)::value;
-              constexpr int imm0 = (c >> 1) * 128 + 16 * t * RB;
+              constexpr int imm0 = 16 * t * RB;
               if (mt == 0) {
-                dq_[c][0] = lds_read_tr16_b64<imm0>(qb + offT[c & 1]);
-                dq_[c][1] = lds_read_tr16_b64<imm0 + 8 * RB>(qb + offT[c & 1]);
-                dd_[c][0] = lds_read_tr16_b64<imm0>(db + offT[c & 1]);
-                dd_[c][1] = lds_read_tr16_b64<imm0 + 8 * RB>(db + offT[c & 1]);
+                dq_[c][0] = lds_read_tr16_b64<imm0>(tt.template addr<c, 0>(qb));
+                dq_[c][1] = lds_read_tr16_b64<imm0 + 8 * RB>(tt.template addr<c, 1>(qb));
+                dd_[c][0] = lds_read_tr16_b64<imm0>(tt.template addr<c, 0>(db));
+                dd_[c][1] = lds_read_tr16_b64<imm0 + 8 * RB>(tt.template addr<c, 1>(db));
               } else {
-                dq_[c][0] = lds_read_tr16_b64<imm0 + 32 * RB>(qb + offT[c & 1]);
-                dq_[c][1] = lds_read_tr16_b64<imm0 + 40 * RB>(qb + offT[c & 1]);
-                dd_[c][0] = lds_read_tr16_b64<imm0 + 32 * RB>(db + offT[c & 1]);
-                dd_[c][1] = lds_read_tr16_b64<imm0 + 40 * RB>(db + offT[c & 1]);
+                dq_[c][0] = lds_read_tr16_b64<imm0 + 32 * RB>(tt.template addr<c, 0>(qb));
+                dq_[c][1] = lds_read_tr16_b64<imm0 + 40 * RB>(tt.template addr<c, 1>(qb));
+                dd_[c][0] = lds_read_tr16_b64<imm0 + 32 * RB>(tt.template addr<c, 0>(db));
+                dd_[c][1] = lds_read_tr16_b64<imm0 + 40 * RB>(tt.template addr<c, 1>(db));
               }
             });
           };

@@ -16,10 +16,10 @@
 //     second MFMA (O^T = V^T P^T) - P never goes through LDS;
 //   * K and V tiles go global -> LDS by direct 16-byte loads into two stages; K rows are read
 //     back as MFMA A operands with ds_read_b128, V is transposed on the fly by
-//     ds_read_b64_tr_b16; both layouts are XOR-swizzled against bank conflicts;
+//     ds_read_b64_tr_b16; one XOR swizzle (attn_tiles.h) keeps both conflict free;
 //   * heads are laid out over XCDs so that the query blocks sharing one K/V stay on one L2,
 //     and causal query blocks are issued longest-first.
-#include "common.h"
+#include "attn_tiles.h"
 #include "launch.h"
 
 namespace mi355 {
@@ -33,13 +33,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   using S = typename Elem<V8>::type;
   constexpr int BM = NW * QT * 32, BN = 64;
   constexpr int RB = D * 2;            // bytes per K/V row
-  constexpr int CPR = RB / 16;         // 16-byte chunks per row
-  constexpr int RPI = 1024 / RB;       // rows moved by one wave instruction
-  constexpr int TILE = BN * RB;        // bytes of one K or V tile
-  constexpr int INST = TILE / 1024 / NW;  // direct-load instructions per wave and tile
+  using Tile = AttnTile<RB, BN, NW>;
+  constexpr int TILE = Tile::BYTES;    // bytes of one K or V tile
+  constexpr int INST = Tile::INST;     // direct-load instructions per wave and tile
   constexpr int KSQ = D / 16;          // MFMA k-steps of S^T = K Q^T
   constexpr int DT = D / 32;           // 32-row tiles of O^T
-  static_assert(INST >= 1, "too many waves for this tile");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][K tile | V tile]
@@ -79,12 +77,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   const char* srcV[INST];
 #pragma unroll
   for (int i = 0; i < INST; i++) {
-    int r = (i * NW + wave) * RPI + lane / CPR;
-    int pc = lane % CPR;
-    int lcK = pc ^ (r & 7);
-    int lcV = ((((pc >> 1) ^ (r & 3))) << 1) | (pc & 1);
-    srcK[i] = kbase + (int64_t)r * kpitch + lcK * 16;
-    srcV[i] = vbase + (int64_t)r * vpitch + lcV * 16;
+    srcK[i] = Tile::src(kbase, kpitch, wave, lane, i);
+    srcV[i] = Tile::src(vbase, vpitch, wave, lane, i);
   }
   auto issue_kv = [&](int j, int stage) {
     LDS_PTR(char) kd = lds + stage * (2 * TILE);
@@ -96,20 +90,9 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     }
   };
 
-  // ---- per-lane LDS offsets
-  // K operand: row l32 (+32a), chunk 2*ks+g swizzled with the low row bits
-  unsigned offK[4];
-#pragma unroll
-  for (int k4 = 0; k4 < 4; k4++) offK[k4] = l32 * RB + ((((k4 * 2 + g) ^ l32) & 7) << 4);
-  // V operand (transpose read): lane i16 of 16-lane group q4 addresses row 4*g + i16/4 and the
-  // 8-byte piece i16%4 of 32-byte group 2c + (q4&1), swizzled with the low row bits
-  unsigned offV[2];
-#pragma unroll
-  for (int par = 0; par < 2; par++) {
-    int row = 4 * g + (i16 >> 2);
-    int c32 = (par * 2 + (q4 & 1)) ^ (row & 3);
-    offV[par] = TILE + row * RB + c32 * 32 + (i16 & 3) * 8;
-  }
+  // ---- per-lane LDS addressing (row-wise K operand, transposed V operand)
+  const RowRead<RB> rk(l32, g);
+  const TrRead<RB> tv(i16, q4);
 
   f32x16 oacc[DT][QT];
 #pragma unroll
@@ -149,15 +132,15 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           for (int r = 0; r < 16; r++) s[a][b][r] = 0.f;
       {
         i32x4 kf[2][2];
-        kf[0][0] = lds_read_b128<0>(base + offK[0]);
-        kf[0][1] = lds_read_b128<32 * RB>(base + offK[0]);
+        kf[0][0] = lds_read_b128<0>(rk.template addr<0>(base));
+        kf[0][1] = lds_read_b128<32 * RB>(rk.template addr<0>(base));
         static_for<KSQ>([&](auto KS_) {
           constexpr int ks = decltype(KS_)::value;
           constexpr int cur = ks & 1, nxt = cur ^ 1;
           if constexpr (ks + 1 < KSQ) {
-            constexpr int imm = ((ks + 1) >> 2) * 128;
-            kf[nxt][0] = lds_read_b128<imm>(base + offK[(ks + 1) & 3]);
-            kf[nxt][1] = lds_read_b128<imm + 32 * RB>(base + offK[(ks + 1) & 3]);
+            const unsigned ka = rk.template addr<ks + 1>(base);
+            kf[nxt][0] = lds_read_b128<0>(ka);
+            kf[nxt][1] = lds_read_b128<32 * RB>(ka);
             lds_wait<2>();
           } else {
             lds_wait<0>();
@@ -221,9 +204,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           constexpr int t = decltype(T_)::value;
           static_for<DT>([&](auto C_) {
             constexpr int c = decltype(C_)::value;
-            constexpr int imm = (c >> 1) * 128 + 16 * t * RB;
-            dst[c][0] = lds_read_tr16_b64<imm>(base + offV[c & 1]);
-            dst[c][1] = lds_read_tr16_b64<imm + 8 * RB>(base + offV[c & 1]);
+            dst[c][0] = lds_read_tr16_b64<16 * t * RB>(tv.template addr<c, 0>(base + TILE));
+            dst[c][1] = lds_read_tr16_b64<(16 * t + 8) * RB>(tv.template addr<c, 1>(base + TILE));
           });
         };
         read_v(std::integral_constant<int, 0>{}, vf[0]);
