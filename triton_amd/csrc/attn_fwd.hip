@@ -90,9 +90,18 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     }
   };
 
-  // ---- per-lane LDS addressing (row-wise K operand, transposed V operand)
+  // ---- per-lane LDS addresses (row-wise K operand, transposed V operand), one register per
+  // k-step / column block; stage and sub-tile offsets go into the instructions' immediates
   const RowRead<RB> rk(l32, g);
   const TrRead<RB> tv(i16, q4);
+  const unsigned lds0 = lds_addr(lds);
+  unsigned ka[KSQ], va[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KSQ; ks++) ka[ks] = lds0 + rk.rowb + (rk.xk ^ (ks * 32));
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++) va[c][h2] = lds0 + (tv.tl ^ ((c << 6) | (h2 << 5)));
 
   f32x16 oacc[DT][QT];
 #pragma unroll
@@ -106,6 +115,10 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   for (int b = 0; b < QT; b++) { m_i[b] = -INFINITY; l_i[b] = 0.f; }
 
   const float qk_scale = p.sm_scale * 1.44269504f;
+  // The running maximum only has to bound the scores loosely: it is raised (and the
+  // accumulators rescaled) when some row of the wave outgrows it by more than 2^RESCALE_LOG2,
+  // so P stays below 2^RESCALE_LOG2 and the result O = acc / l, M = m + log2(l) is unchanged.
+  constexpr float RESCALE_LOG2 = 8.f;
 
   // number of K/V steps of this block / wave
   const int kv_end_blk = p.causal ? min(p.N, m0 + BM) : p.N;
@@ -117,11 +130,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   wait_all();
   __syncthreads();
 
-  for (int j = 0; j < nsteps; j++) {
-    const int stage = j & 1;
+  auto step = [&](const int j, auto STAGE_) {
+    constexpr int stage = decltype(STAGE_)::value;
+    constexpr int KOFF = stage * 2 * TILE, VOFF = KOFF + TILE;
     if (j + 1 < nsteps) issue_kv(j + 1, stage ^ 1);
     if (j <= wave_last && row0 < p.N) {
-      const unsigned base = lds_addr(lds + stage * (2 * TILE));
       // ---- S^T = K Q^T : [2 kv tiles][QT q tiles]
       f32x16 s[2][QT];
 #pragma unroll
@@ -132,15 +145,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           for (int r = 0; r < 16; r++) s[a][b][r] = 0.f;
       {
         i32x4 kf[2][2];
-        kf[0][0] = lds_read_b128<0>(rk.template addr<0>(base));
-        kf[0][1] = lds_read_b128<32 * RB>(rk.template addr<0>(base));
+        kf[0][0] = lds_read_b128<KOFF>(ka[0]);
+        kf[0][1] = lds_read_b128<KOFF + 32 * RB>(ka[0]);
         static_for<KSQ>([&](auto KS_) {
           constexpr int ks = decltype(KS_)::value;
           constexpr int cur = ks & 1, nxt = cur ^ 1;
           if constexpr (ks + 1 < KSQ) {
-            const unsigned ka = rk.template addr<ks + 1>(base);
-            kf[nxt][0] = lds_read_b128<0>(ka);
-            kf[nxt][1] = lds_read_b128<32 * RB>(ka);
+            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + 1]);
+            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + 1]);
             lds_wait<2>();
           } else {
             lds_wait<0>();
@@ -175,22 +187,26 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[a][b][r]);
         mx = pair_max(mx);
         const float m_new = fmaxf(m_i[b], mx * qk_scale);
-        const float alpha = fast_exp2(m_i[b] - m_new);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_i[b] + RESCALE_LOG2) != 0) {
+          const float alpha = fast_exp2(m_i[b] - m_new);
+          l_i[b] *= alpha;
+          m_i[b] = m_new;
+#pragma unroll
+          for (int c = 0; c < DT; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[c][b][r] *= alpha;
+        }
+        const float m_cur = m_i[b];
         float rs = 0.f;
 #pragma unroll
         for (int a = 0; a < 2; a++)
 #pragma unroll
           for (int r = 0; r < 16; r++) {
-            float pv = fast_exp2(fmaf(s[a][b][r], qk_scale, -m_new));
+            float pv = fast_exp2(fmaf(s[a][b][r], qk_scale, -m_cur));
             s[a][b][r] = pv;
             rs += pv;
           }
-        l_i[b] = l_i[b] * alpha + rs;
-        m_i[b] = m_new;
-#pragma unroll
-        for (int c = 0; c < DT; c++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) oacc[c][b][r] *= alpha;
+        l_i[b] += rs;
         // k-step t = 2a + u covers columns 16t .. 16t+15: registers 8u .. 8u+7 of tile a
 #pragma unroll
         for (int t = 0; t < 4; t++)
@@ -204,8 +220,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           constexpr int t = decltype(T_)::value;
           static_for<DT>([&](auto C_) {
             constexpr int c = decltype(C_)::value;
-            dst[c][0] = lds_read_tr16_b64<16 * t * RB>(tv.template addr<c, 0>(base + TILE));
-            dst[c][1] = lds_read_tr16_b64<(16 * t + 8) * RB>(tv.template addr<c, 1>(base + TILE));
+            dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0]);
+            dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1]);
           });
         };
         read_v(std::integral_constant<int, 0>{}, vf[0]);
@@ -231,6 +247,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     }
     wait_all();
     __syncthreads();
+  };
+
+  for (int j = 0; j < nsteps; j += 2) {
+    step(j, std::integral_constant<int, 0>{});
+    if (j + 1 < nsteps) step(j + 1, std::integral_constant<int, 1>{});
   }
 
   // ---- epilogue: O = acc / l, M = m + log2(l)
