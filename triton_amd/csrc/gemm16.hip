@@ -10,6 +10,9 @@ struct Cfg16 {
   static constexpr int kSteps = 2, kChunks = 1;
   static constexpr bool kRowMajorB = true, kScaled = false;
   static constexpr int kStepsPerScaleDword = 1;
+  // no block scales: placeholders so that generic code naming them compiles
+  __device__ static int scale_dword_offset(int) { return 0; }
+  __device__ static int scale_fixup(int v, int, int) { return v; }
   // lane group g of sub-step ks reads k elements 16*ks + 8*g .. +8
   __device__ static constexpr int chunk(int ks, int g, int) { return ks * 2 + g; }
   template <int ks>

@@ -12,6 +12,9 @@ struct Cfg8 {
   static constexpr int kSteps = 1, kChunks = 2;
   static constexpr bool kRowMajorB = false, kScaled = false;
   static constexpr int kStepsPerScaleDword = 1;
+  // no block scales: placeholders so that generic code naming them compiles
+  __device__ static int scale_dword_offset(int) { return 0; }
+  __device__ static int scale_fixup(int v, int, int) { return v; }
   // A lane feeds 32 bytes per sub-step as two 16-byte halves; any assignment of K positions
   // works as long as both operands use the same one.
   __device__ static constexpr int chunk(int, int g, int c) { return c * 2 + g; }

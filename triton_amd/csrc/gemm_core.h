@@ -621,6 +621,277 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
   gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
 }
 
+// ---------------------------------------------------------------------------------------------
+// Four-wave variant of the 256x256 tile: one wave per SIMD, each owning a 128x128 quarter of C
+// (256 accumulator registers).  Per K step a wave reads (4 + 4) x 32 operand rows from LDS for
+// 32 MFMAs - two thirds of the LDS traffic per flop of the 128x64 wave tiles above - and, with
+// no second wave on the SIMD to hide latencies, everything is software pipelined inside the wave:
+//   * direct loads run NS tiles ahead (tile kt+NS goes into the stage tile kt just vacated);
+//   * ALL operands of tile kt+1 are read from LDS into a second register set while the MFMAs of
+//     tile kt issue; the reads and the direct loads of a step are spread over the first MFMAs of
+//     the step, one or two per MFMA, in program order (scheduling barriers keep them there);
+//   * one barrier per step, at its top: by then every wave holds tile kt in registers (so its
+//     stage may be overwritten) and has seen its own share of tile kt+1 arrive.
+// ---------------------------------------------------------------------------------------------
+template <typename Cfg, int WN, bool B_KMAJOR, int NS>
+__global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
+  using Operand = typename Cfg::Operand;
+  constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
+  static_assert(WN == 2 || WN == 4, "four or eight waves");
+  constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK;
+  constexpr int SC_BYTES = Cfg::kScaled ? (BM + BN) * 4 : 0;
+  constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+  constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
+  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  using CopyA = TileCopyK<BM, NW>;
+  using CopyBk = TileCopyK<BN, NW>;
+  using CopyBn = TileCopyKN<BN, NW>;
+  constexpr int ITA = CopyA::kIters;
+  constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
+  constexpr int KROWS = RBK / 2;
+  constexpr int NSC = Cfg::kScaled ? 8 / NW : 0;  // scale copies per wave and tile (64 rows of 4 bytes each)
+  constexpr int kShare = ITA + ITB + NSC;         // direct loads per wave and tile
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  int pid = xcd_remap(blockIdx.x, num_m * num_n);
+  int pm, pn;
+  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
+  const int m0 = pm * BM, n0 = pn * BN;
+
+  const char* srcA[ITA];
+  const char* srcB[ITB];
+#pragma unroll
+  for (int i = 0; i < ITA; i++) {
+    int r = CopyA::row(wave, lane, i);
+    int gr = min(m0 + r, p.M - 1);
+    srcA[i] = p.A + (int64_t)gr * p.lda + CopyA::chunk(lane, r) * 16;
+  }
+#pragma unroll
+  for (int i = 0; i < ITB; i++) {
+    if constexpr (B_KMAJOR) {
+      int r = CopyBk::row(wave, lane, i);
+      int gr = min(n0 + r, p.N - 1);
+      srcB[i] = p.B + (int64_t)gr * p.ldb + CopyBk::chunk(lane, r) * 16;
+    } else {
+      int r = CopyBn::row(wave, lane, i);
+      int n = n0 + CopyBn::col16(lane, r) * 8;
+      n = n < p.N ? n : p.N - 8;
+      srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
+    }
+  }
+  const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
+  const uint8_t* srcSA = nullptr;
+  const uint8_t* srcSB = nullptr;
+  if constexpr (Cfg::kScaled) {
+    // four waves: every wave copies 64 A rows and 64 B rows; eight waves: waves 0-3 the A rows,
+    // waves 4-7 the B rows (the LDS side is A scales then B scales, 256 bytes per wave either way)
+    const int w4 = wave & 3;
+    srcSA = p.sA + (int64_t)min(m0 + w4 * 64 + lane, p.M - 1) * p.lds_a;
+    srcSB = p.sB + (int64_t)min(n0 + w4 * 64 + lane, p.N - 1) * p.lds_b;
+    if (NW == 8 && wave >= 4) srcSA = srcSB;
+  }
+
+  // direct load number `i` of this wave's share of tile kt
+  auto issue_one = [&](auto I_, int kt, LDS_PTR(char) a) {
+    constexpr int i = decltype(I_)::value;
+    if constexpr (i < ITA) {
+      async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
+    } else if constexpr (i < ITA + ITB) {
+      constexpr int ib = i - ITA;
+      async_copy16(srcB[ib] + kt * stepB, (LDS_PTR(void))(a + A_BYTES + (ib * NW + wave) * 1024));
+    } else if constexpr (i == ITA + ITB) {
+      async_copy4(srcSA + Cfg::scale_dword_offset(kt), (LDS_PTR(void))(a + A_BYTES + B_BYTES + wave * 256));
+    } else {
+      async_copy4(srcSB + Cfg::scale_dword_offset(kt), (LDS_PTR(void))(a + A_BYTES + B_BYTES + BM * 4 + wave * 256));
+    }
+  };
+
+  f32x16 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+  const int l32 = lane & 31, g = lane >> 5;
+  const int i16 = lane & 15, q = lane >> 4;
+  unsigned offA[KS][NC], offB[KS][NC];
+#pragma unroll
+  for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+    for (int c = 0; c < NC; c++) {
+      offA[ks][c] = kmajor_off(wm * TM + l32, Cfg::chunk(ks, g, c));
+      offB[ks][c] = A_BYTES + kmajor_off(wn * TN + l32, Cfg::chunk(ks, g, c));
+    }
+  unsigned offBn[NT];
+  {
+    int k = (q >> 1) * 8 + (i16 >> 2);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      int c32 = (wn * TN + t * 32) / 16 + (q & 1);
+      offBn[t] = A_BYTES + k * (BN * 2) + ((c32 ^ ((k & 3) << 1)) << 5) + (i16 & 3) * 8;
+    }
+  }
+  const unsigned offSA = A_BYTES + B_BYTES + (wm * TM + l32) * 4;
+  const unsigned offSB = A_BYTES + B_BYTES + BM * 4 + (wn * TN + l32) * 4;
+
+  // operand registers of the two MFMA sub-steps; sub-step ks of the next tile is read while the
+  // MFMAs of the other sub-step issue
+  static_assert(KS == 2, "the pipeline alternates between two sub-steps");
+  Operand fa[KS][MT], fb[KS][NT];
+  int sa[MT], sb[NT], sa_in[MT], sb_in[NT];
+
+  // LDS read number `r` of sub-step ks: A operands, B operands, then (with ks == 0) the scale dwords
+  constexpr int kOperandReads = MT + NT;
+  auto read_one = [&](auto R_, auto KS_, unsigned base) {
+    constexpr int r = decltype(R_)::value, ks = decltype(KS_)::value;
+    if constexpr (r < MT) {
+      constexpr int t = r;
+      if constexpr (NC == 1) {
+        fa[ks][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offA[ks][0]));
+      } else {
+        i32x4 lo = lds_read_b128<t * 32 * RBK>(base + offA[ks][0]);
+        i32x4 hi = lds_read_b128<t * 32 * RBK>(base + offA[ks][1]);
+        fa[ks][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    } else if constexpr (r < kOperandReads) {
+      constexpr int u = r - MT;
+      if constexpr (!B_KMAJOR) {
+        constexpr int imm = ks * 16 * BN * 2;
+        i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[u]);
+        i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[u]);
+        fb[ks][u] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+      } else if constexpr (NC == 1) {
+        fb[ks][u] = __builtin_bit_cast(Operand, lds_read_b128<u * 32 * RBK>(base + offB[ks][0]));
+      } else {
+        i32x4 lo = lds_read_b128<u * 32 * RBK>(base + offB[ks][0]);
+        i32x4 hi = lds_read_b128<u * 32 * RBK>(base + offB[ks][1]);
+        fb[ks][u] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+      }
+    } else {
+      constexpr int t = r - kOperandReads;
+      if constexpr (t < MT) sa_in[t] = lds_read_b32<t * 128>(base + offSA);
+      else sb_in[t - MT] = lds_read_b32<(t - MT) * 128>(base + offSB);
+    }
+  };
+  // after the reads of a sub-step have been waited for: tie the registers to the wait; with the
+  // first sub-step of a tile come its scales
+  auto settle = [&](auto KS_, int kt) {
+    constexpr int ks = decltype(KS_)::value;
+    lds_wait<0>();
+#pragma unroll
+    for (int t = 0; t < MT; t++) lds_use(fa[ks][t]);
+#pragma unroll
+    for (int t = 0; t < NT; t++) lds_use(fb[ks][t]);
+    if constexpr (Cfg::kScaled && ks == 0) {
+#pragma unroll
+      for (int t = 0; t < MT; t++) { lds_use(sa_in[t]); sa[t] = Cfg::scale_fixup(sa_in[t], kt, g); }
+#pragma unroll
+      for (int t = 0; t < NT; t++) { lds_use(sb_in[t]); sb[t] = Cfg::scale_fixup(sb_in[t], kt, g); }
+    }
+  };
+
+  constexpr int kMfmas = MT * NT;  // per sub-step
+  constexpr int kReads0 = kOperandReads + (Cfg::kScaled ? MT + NT : 0);  // reads of a tile's sub-step 0
+  const int nfull = p.k_bytes / RBK;
+
+  // MFMAs of (tile kt, sub-step KS_) with the memory instructions of the half step in between:
+  // first the `nreads` LDS reads, two per MFMA (they are needed at the top of the next half),
+  // then the `nloads` direct loads, one per MFMA
+  auto half = [&](auto KS_, auto NREADS_, auto NLOADS_, auto&& memop) {
+    constexpr int ks = decltype(KS_)::value, nreads = decltype(NREADS_)::value, nloads = decltype(NLOADS_)::value;
+    constexpr int rslots = (nreads + 1) / 2;
+    constexpr int lper = nloads == 0 ? 1 : (nloads + (kMfmas - rslots) - 1) / (kMfmas - rslots);
+    static_for<kMfmas>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      if constexpr (Cfg::kScaled) acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], sb[j], sa[i]);
+      else acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], 0, 0);
+      if constexpr (n < rslots) {
+        static_for<2>([&](auto O_) {
+          constexpr int op = 2 * n + decltype(O_)::value;
+          if constexpr (op < nreads) memop(std::integral_constant<int, op>{});
+        });
+      } else {
+        static_for<lper>([&](auto O_) {
+          constexpr int op = (n - rslots) * lper + decltype(O_)::value;
+          if constexpr (op < nloads) memop(std::integral_constant<int, nreads + op>{});
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+
+  // prologue: NS tiles in flight (past the end of K the last tile again, which keeps the number
+  // of outstanding loads - and with it the partial waits - uniform), sub-step 0 of tile 0 requested
+#pragma unroll
+  for (int s = 0; s < NS; s++) static_for<kShare>([&](auto I_) { issue_one(I_, min(s, nfull - 1), lds + s * STAGE); });
+  wait_vmcnt<(NS - 1) * kShare>();
+  __builtin_amdgcn_sched_barrier(0);
+  block_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  static_for<kReads0>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, lds_addr(lds)); });
+
+  int stage = 0;
+  for (int kt = 0; kt < nfull; kt++) {
+    const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+    // ---- first half: multiply sub-step 0, fetch sub-step 1 of the same tile
+    settle(std::integral_constant<int, 0>{}, kt);
+    {
+      const unsigned base = lds_addr(lds + stage * STAGE);
+      half(std::integral_constant<int, 0>{}, std::integral_constant<int, kOperandReads>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
+        read_one(OP_, std::integral_constant<int, 1>{}, base);
+      });
+    }
+    // ---- second half: every wave holds the whole of tile kt in registers and has seen its own
+    //      share of tile kt+1 arrive (NS-2 younger shares stay in flight); after the barrier the
+    //      stage of tile kt is refilled with tile kt+NS and sub-step 0 of tile kt+1 is fetched
+    settle(std::integral_constant<int, 1>{}, kt);
+    wait_vmcnt<(NS - 2) * kShare>();
+    __builtin_amdgcn_sched_barrier(0);
+    block_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    {
+      const unsigned base = lds_addr(lds + next_stage * STAGE);
+      LDS_PTR(char) const fill = lds + stage * STAGE;
+      const int kfill = min(kt + NS, nfull - 1);
+      half(std::integral_constant<int, 1>{}, std::integral_constant<int, kReads0>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
+        constexpr int op = decltype(OP_)::value;
+        if constexpr (op < kReads0) read_one(OP_, std::integral_constant<int, 0>{}, base);
+        else issue_one(std::integral_constant<int, op - kReads0>{}, kfill, fill);
+      });
+    }
+    stage = next_stage;
+  }
+  // nothing may still be writing this workgroup's LDS when it retires
+  wait_all();
+
+  gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+}
+
+template <typename Cfg, int WN, bool B_KMAJOR, int NS>
+static int launch_gemm_w4(const GemmArgs& p, hipStream_t stream) {
+  constexpr int BM = 256, BN = 256;
+  constexpr int smem = NS * ((BM + BN) * RBK + (Cfg::kScaled ? (BM + BN) * 4 : 0));
+  static_assert(smem <= 160 * 1024, "LDS ring does not fit");
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS><<<dim3(num_m * num_n), dim3(2 * WN * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 template <typename Cfg, int BM, int BN, bool B_KMAJOR, int NS>
 static int launch_gemm_pp(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = NS * ((BM + BN) * RBK + (Cfg::kScaled ? (BM + BN) * 4 : 0));
@@ -655,9 +926,17 @@ static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
 
 // tile: 0 = 256x256 / 8 waves / 4 stages, ping-pong phases (whole K steps only, else tile 2),
 //       1 = 128x128 / 4 waves / 4 stages (two workgroups per CU),
-//       2 = 256x256 / 8 waves / 4 stages, one barrier per step
+//       2 = 256x256 / 8 waves / 4 stages, one barrier per step,
+//       3 = 256x256 / 4 waves / 4 stages, software pipelined (whole K steps only, else tile 2),
+//       4 = the same pipeline with 8 waves
 template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
+  if constexpr (Cfg::kSteps == 2) {
+    const bool whole = p.k_bytes >= RBK && p.k_bytes % (RBK * Cfg::kStepsPerScaleDword) == 0;
+    if (tile == 3 && whole) return launch_gemm_w4<Cfg, 2, B_KMAJOR, 4>(p, stream);
+    if (tile == 4 && whole) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4>(p, stream);
+  }
+  if (tile >= 3) tile = 2;
   if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR, 4>(p, stream);
   if (tile == 0 && p.k_bytes % (RBK * Cfg::kStepsPerScaleDword) == 0) return launch_gemm_pp<Cfg, 256, 256, B_KMAJOR, 4>(p, stream);
   return launch_gemm<Cfg, 256, 256, 2, 4, B_KMAJOR, 4>(p, stream);
