@@ -126,8 +126,8 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   // 256x256 tiles once they fill three quarters of the CUs, 128x128 tiles (two workgroups per CU) below that
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  // large problems: fp8 runs the ping-pong kernel, 16-bit types the software-pipelined one
-  int tile = (tiles256 * 4 >= 3L * cus) ? (is8 ? 0 : 4) : 1;
+  // large problems run the software-pipelined 8-wave kernel
+  int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);

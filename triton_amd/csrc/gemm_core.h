@@ -742,55 +742,66 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   const unsigned offSA = A_BYTES + B_BYTES + (wm * TM + l32) * 4;
   const unsigned offSB = A_BYTES + B_BYTES + BM * 4 + (wn * TN + l32) * 4;
 
-  // operand registers of the two MFMA sub-steps; sub-step ks of the next tile is read while the
-  // MFMAs of the other sub-step issue
-  static_assert(KS == 2, "the pipeline alternates between two sub-steps");
-  Operand fa[KS][MT], fb[KS][NT];
+  // A K step is multiplied in two halves, and the operands of the next half are read from LDS
+  // while the MFMAs of the current one issue.  With two MFMA sub-steps per K step (16-bit, fp4)
+  // a half is a sub-step: all A and B operands of that sub-step.  With one sub-step (fp8) a half
+  // is the upper or lower half of the wave's A rows against all of its B columns; the B
+  // operands then live for the whole step and alternate between two register sets by tile parity.
+  constexpr bool KSPLIT = KS == 2;
+  static_assert(KS == 1 || KS == 2, "one or two MFMA sub-steps per K step");
+  constexpr int AH = KSPLIT ? MT : MT / 2;  // A operands per half
+  Operand fa[KSPLIT ? 2 : 1][MT], fb[2][NT];
   int sa[MT], sb[NT], sa_in[MT], sb_in[NT];
 
-  // LDS read number `r` of sub-step ks: A operands, B operands, then (with ks == 0) the scale dwords
-  constexpr int kOperandReads = MT + NT;
-  auto read_one = [&](auto R_, auto KS_, unsigned base) {
-    constexpr int r = decltype(R_)::value, ks = decltype(KS_)::value;
-    if constexpr (r < MT) {
-      constexpr int t = r;
+  // LDS reads of half H of a tile with parity P: A operands, then (K-split: always, M-split: with
+  // the first half) the B operands, then with the first half the scale dwords
+  auto n_reads = [](int H) constexpr { return AH + ((KSPLIT || H == 0) ? NT : 0) + ((Cfg::kScaled && H == 0) ? MT + NT : 0); };
+  auto read_one = [&](auto R_, auto H_, auto P_, unsigned base) {
+    constexpr int r = decltype(R_)::value, H = decltype(H_)::value, P = decltype(P_)::value;
+    constexpr int ks = KSPLIT ? H : 0, aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P;
+    constexpr int nb = (KSPLIT || H == 0) ? NT : 0;
+    if constexpr (r < AH) {
+      constexpr int t = (KSPLIT ? 0 : H * AH) + r;
       if constexpr (NC == 1) {
-        fa[ks][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offA[ks][0]));
+        fa[aset][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offA[ks][0]));
       } else {
         i32x4 lo = lds_read_b128<t * 32 * RBK>(base + offA[ks][0]);
         i32x4 hi = lds_read_b128<t * 32 * RBK>(base + offA[ks][1]);
-        fa[ks][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        fa[aset][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
-    } else if constexpr (r < kOperandReads) {
-      constexpr int u = r - MT;
+    } else if constexpr (r < AH + nb) {
+      constexpr int u = r - AH;
       if constexpr (!B_KMAJOR) {
         constexpr int imm = ks * 16 * BN * 2;
         i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[u]);
         i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[u]);
-        fb[ks][u] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+        fb[bset][u] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo, hi, 0, 1, 2, 3));
       } else if constexpr (NC == 1) {
-        fb[ks][u] = __builtin_bit_cast(Operand, lds_read_b128<u * 32 * RBK>(base + offB[ks][0]));
+        fb[bset][u] = __builtin_bit_cast(Operand, lds_read_b128<u * 32 * RBK>(base + offB[ks][0]));
       } else {
         i32x4 lo = lds_read_b128<u * 32 * RBK>(base + offB[ks][0]);
         i32x4 hi = lds_read_b128<u * 32 * RBK>(base + offB[ks][1]);
-        fb[ks][u] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        fb[bset][u] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     } else {
-      constexpr int t = r - kOperandReads;
+      constexpr int t = r - AH - nb;
       if constexpr (t < MT) sa_in[t] = lds_read_b32<t * 128>(base + offSA);
       else sb_in[t - MT] = lds_read_b32<(t - MT) * 128>(base + offSB);
     }
   };
-  // after the reads of a sub-step have been waited for: tie the registers to the wait; with the
-  // first sub-step of a tile come its scales
-  auto settle = [&](auto KS_, int kt) {
-    constexpr int ks = decltype(KS_)::value;
+  // after the reads of a half have been waited for: tie the registers to the wait; with the
+  // first half of a tile come its scales
+  auto settle = [&](auto H_, auto P_, int kt) {
+    constexpr int H = decltype(H_)::value, P = decltype(P_)::value;
+    constexpr int aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P, alo = KSPLIT ? 0 : H * AH;
     lds_wait<0>();
 #pragma unroll
-    for (int t = 0; t < MT; t++) lds_use(fa[ks][t]);
+    for (int t = 0; t < AH; t++) lds_use(fa[aset][alo + t]);
+    if constexpr (KSPLIT || H == 0) {
 #pragma unroll
-    for (int t = 0; t < NT; t++) lds_use(fb[ks][t]);
-    if constexpr (Cfg::kScaled && ks == 0) {
+      for (int t = 0; t < NT; t++) lds_use(fb[bset][t]);
+    }
+    if constexpr (Cfg::kScaled && H == 0) {
 #pragma unroll
       for (int t = 0; t < MT; t++) { lds_use(sa_in[t]); sa[t] = Cfg::scale_fixup(sa_in[t], kt, g); }
 #pragma unroll
@@ -798,24 +809,27 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     }
   };
 
-  constexpr int kMfmas = MT * NT;  // per sub-step
-  constexpr int kReads0 = kOperandReads + (Cfg::kScaled ? MT + NT : 0);  // reads of a tile's sub-step 0
+  constexpr int kMfmas = AH * NT;  // per half
   const int nfull = p.k_bytes / RBK;
 
-  // MFMAs of (tile kt, sub-step KS_) with the memory instructions of the half step in between:
-  // first the `nreads` LDS reads, two per MFMA (they are needed at the top of the next half),
-  // then the `nloads` direct loads, one per MFMA
-  auto half = [&](auto KS_, auto NREADS_, auto NLOADS_, auto&& memop) {
-    constexpr int ks = decltype(KS_)::value, nreads = decltype(NREADS_)::value, nloads = decltype(NLOADS_)::value;
-    constexpr int rslots = (nreads + 1) / 2;
+  // MFMAs of half H with the memory instructions of the half in between: the `nreads` LDS reads
+  // over the first MFMAs (they are needed at the top of the next half), then the `nloads`
+  // direct loads over the rest
+  auto half = [&](auto H_, auto P_, auto NREADS_, auto NLOADS_, auto&& memop) {
+    constexpr int H = decltype(H_)::value, P = decltype(P_)::value;
+    constexpr int nreads = decltype(NREADS_)::value, nloads = decltype(NLOADS_)::value;
+    constexpr int ks = KSPLIT ? H : 0, aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P, alo = KSPLIT ? 0 : H * AH;
+    constexpr int half_slots = (kMfmas + 1) / 2;
+    constexpr int rper = (nreads + half_slots - 1) / half_slots;
+    constexpr int rslots = (nreads + rper - 1) / rper;
     constexpr int lper = nloads == 0 ? 1 : (nloads + (kMfmas - rslots) - 1) / (kMfmas - rslots);
     static_for<kMfmas>([&](auto N_) {
-      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
-      if constexpr (Cfg::kScaled) acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], sb[j], sa[i]);
-      else acc[i][j] = Cfg::template mma<ks>(fb[ks][j], fa[ks][i], acc[i][j], 0, 0);
+      constexpr int n = decltype(N_)::value, i = alo + n / NT, j = n % NT;
+      if constexpr (Cfg::kScaled) acc[i][j] = Cfg::template mma<ks>(fb[bset][j], fa[aset][i], acc[i][j], sb[j], sa[i]);
+      else acc[i][j] = Cfg::template mma<ks>(fb[bset][j], fa[aset][i], acc[i][j], 0, 0);
       if constexpr (n < rslots) {
-        static_for<2>([&](auto O_) {
-          constexpr int op = 2 * n + decltype(O_)::value;
+        static_for<rper>([&](auto O_) {
+          constexpr int op = rper * n + decltype(O_)::value;
           if constexpr (op < nreads) memop(std::integral_constant<int, op>{});
         });
       } else {
@@ -829,30 +843,35 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   };
 
   // prologue: NS tiles in flight (past the end of K the last tile again, which keeps the number
-  // of outstanding loads - and with it the partial waits - uniform), sub-step 0 of tile 0 requested
+  // of outstanding loads - and with it the partial waits - uniform), first half of tile 0 requested
 #pragma unroll
   for (int s = 0; s < NS; s++) static_for<kShare>([&](auto I_) { issue_one(I_, min(s, nfull - 1), lds + s * STAGE); });
   wait_vmcnt<(NS - 1) * kShare>();
   __builtin_amdgcn_sched_barrier(0);
   block_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  static_for<kReads0>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, lds_addr(lds)); });
+  static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(lds)); });
 
   int stage = 0;
-  for (int kt = 0; kt < nfull; kt++) {
+  // one K step of a tile with parity P
+  auto step = [&](int kt, auto P_) {
+    constexpr int P = decltype(P_)::value;
+    using H0 = std::integral_constant<int, 0>;
+    using H1 = std::integral_constant<int, 1>;
+    using PN = std::integral_constant<int, P ^ 1>;
     const int next_stage = stage + 1 == NS ? 0 : stage + 1;
-    // ---- first half: multiply sub-step 0, fetch sub-step 1 of the same tile
-    settle(std::integral_constant<int, 0>{}, kt);
+    // ---- first half: multiply it, fetch the second half of the same tile
+    settle(H0{}, P_, kt);
     {
       const unsigned base = lds_addr(lds + stage * STAGE);
-      half(std::integral_constant<int, 0>{}, std::integral_constant<int, kOperandReads>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
-        read_one(OP_, std::integral_constant<int, 1>{}, base);
+      half(H0{}, P_, std::integral_constant<int, n_reads(1)>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
+        read_one(OP_, H1{}, P_, base);
       });
     }
     // ---- second half: every wave holds the whole of tile kt in registers and has seen its own
     //      share of tile kt+1 arrive (NS-2 younger shares stay in flight); after the barrier the
-    //      stage of tile kt is refilled with tile kt+NS and sub-step 0 of tile kt+1 is fetched
-    settle(std::integral_constant<int, 1>{}, kt);
+    //      stage of tile kt is refilled with tile kt+NS and the first half of tile kt+1 is fetched
+    settle(H1{}, P_, kt);
     wait_vmcnt<(NS - 2) * kShare>();
     __builtin_amdgcn_sched_barrier(0);
     block_barrier();
@@ -861,13 +880,22 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       const unsigned base = lds_addr(lds + next_stage * STAGE);
       LDS_PTR(char) const fill = lds + stage * STAGE;
       const int kfill = min(kt + NS, nfull - 1);
-      half(std::integral_constant<int, 1>{}, std::integral_constant<int, kReads0>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
+      constexpr int nr = n_reads(0);
+      half(H1{}, P_, std::integral_constant<int, nr>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
         constexpr int op = decltype(OP_)::value;
-        if constexpr (op < kReads0) read_one(OP_, std::integral_constant<int, 0>{}, base);
-        else issue_one(std::integral_constant<int, op - kReads0>{}, kfill, fill);
+        if constexpr (op < nr) read_one(OP_, H0{}, PN{}, base);
+        else issue_one(std::integral_constant<int, op - nr>{}, kfill, fill);
       });
     }
     stage = next_stage;
+  };
+  if constexpr (KSPLIT) {
+    for (int kt = 0; kt < nfull; kt++) step(kt, std::integral_constant<int, 0>{});
+  } else {
+    for (int kt = 0; kt < nfull; kt += 2) {
+      step(kt, std::integral_constant<int, 0>{});
+      if (kt + 1 < nfull) step(kt + 1, std::integral_constant<int, 1>{});
+    }
   }
   // nothing may still be writing this workgroup's LDS when it retires
   wait_all();
@@ -931,10 +959,12 @@ static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
 //       4 = the same pipeline with 8 waves
 template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
-  if constexpr (Cfg::kSteps == 2) {
+  {
     const bool whole = p.k_bytes >= RBK && p.k_bytes % (RBK * Cfg::kStepsPerScaleDword) == 0;
-    if (tile == 3 && whole) return launch_gemm_w4<Cfg, 2, B_KMAJOR, 4>(p, stream);
-    if (tile == 4 && whole) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4>(p, stream);
+    if constexpr (Cfg::kSteps == 2) {  // the four-wave form of the one-sub-step types runs out of registers
+      if (tile == 3 && whole) return launch_gemm_w4<Cfg, 2, B_KMAJOR, 4>(p, stream);
+    }
+    if (tile >= 3 && whole) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4>(p, stream);
   }
   if (tile >= 3) tile = 2;
   if (tile == 1) return launch_gemm<Cfg, 128, 128, 2, 2, B_KMAJOR, 4>(p, stream);
