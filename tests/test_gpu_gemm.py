@@ -94,6 +94,31 @@ def test_exact_integers_on_mfma_path_bitwise_vs_tiled_oracle(gpu):
             assert bits_equal(got, ref)
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+def test_every_kernel_variant_is_bit_exact_on_integers(gpu, monkeypatch, tile):
+    # MI355_GEMM_TILE forces one MFMA kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves)
+    # for shapes the size heuristic would give to another; K = 520 has a partial last K step, which
+    # the ping-pong and pipelined kernels hand to the one-barrier kernel
+    monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
+    rng = np.random.default_rng(11 + tile)
+    for (M, N, K) in [(512, 768, 512), (300, 264, 520), (256, 256, 64)]:
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ref = gemm.matmul_closed_form(a, b, out_dtype="fp32")
+        for dtype in ("fp16", "bf16"):
+            got = to_np(triton_amd.matmul(from_np(a, dtype, gpu), from_np(b, dtype, gpu), out_dtype=torch.float32))
+            assert bits_equal(got, ref), (tile, dtype, M, N, K, "row-major B")
+            bt = from_np(np.ascontiguousarray(b.T), dtype, gpu).t()  # K-major B
+            got = to_np(triton_amd.matmul(from_np(a, dtype, gpu), bt, out_dtype=torch.float32))
+            assert bits_equal(got, ref), (tile, dtype, M, N, K, "K-major B")
+        # fp8: small integers are exact e4m3 / e5m2 values
+        for fmt, tdt in (("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)):
+            ca, cb = formats.encode_fp8(a, fmt), formats.encode_fp8(np.ascontiguousarray(b.T), fmt)
+            got = to_np(triton_amd.matmul(torch.from_numpy(ca).to(gpu).view(tdt), torch.from_numpy(cb).to(gpu).view(tdt).t(),
+                                          out_dtype=torch.float32))
+            assert bits_equal(got, ref), (tile, fmt, M, N, K)
+
+
 def test_single_nonzero_locates_every_tile(gpu):
     M, N, K = 520, 776, 136   # edge tiles for both tile sizes, K tail
     for (i, k, j) in [(0, 0, 0), (519, 135, 775), (255, 63, 256), (256, 64, 255), (300, 128, 511), (512, 7, 768)]:

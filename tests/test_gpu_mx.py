@@ -105,3 +105,25 @@ def test_full_size_8192_sampled_rows(gpu, fmt):
     ref = mx.mx_matmul(a[rows], sa[rows], b, sb, fmt, out_dtype="bf16")
     got = to_np(c[rows])
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max() / 64)
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
+def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile):
+    # MI355_GEMM_TILE forces one kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves) for
+    # shapes the size heuristic would give to another; K = 1536 covers three 16-byte scale groups per
+    # row in the pipelined kernels, K = 1056 (not a multiple of 512) their fall-back.
+    monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
+    rng = np.random.default_rng(tile)
+    for (M, N, K) in [(512, 256, 1536), (300, 520, 1056)]:
+        if fmt == "mxfp4":
+            a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
+        else:
+            # e4m3 codes of small multiples of 1/2 (exact products, exact sums)
+            vals = np.array([0x00, 0x30, 0x38, 0x3C, 0x40, 0xB0, 0xB8, 0xC0], dtype=np.uint8)  # 0, .5, 1, 1.5, 2, -.5, -1, -2
+            a = vals[rng.integers(0, len(vals), size=(M, K))]
+            b = vals[rng.integers(0, len(vals), size=(N, K))]
+            sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+            sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
+        assert bits_equal(_run(gpu, a, sa, b, sb, fmt, torch.float32), ref32), (fmt, tile, M, N, K)

@@ -154,7 +154,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  int tile = (tiles256 * 4 >= 3L * cus) ? 0 : 1;
+  int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
 }

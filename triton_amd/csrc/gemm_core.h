@@ -622,7 +622,7 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Four-wave variant of the 256x256 tile: one wave per SIMD, each owning a 128x128 quarter of C
+// Software-pipelined variant of the 256x256 tile, four or eight waves.  With four: one wave per SIMD, each owning a 128x128 quarter of C
 // (256 accumulator registers).  Per K step a wave reads (4 + 4) x 32 operand rows from LDS for
 // 32 MFMAs - two thirds of the LDS traffic per flop of the 128x64 wave tiles above - and, with
 // no second wave on the SIMD to hide latencies, everything is software pipelined inside the wave:
@@ -639,8 +639,10 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   static_assert(WN == 2 || WN == 4, "four or eight waves");
   constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK;
-  constexpr int SC_BYTES = Cfg::kScaled ? (BM + BN) * 4 : 0;
-  constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
+  constexpr int STAGE = A_BYTES + B_BYTES;
+  // block scales: 16 bytes per row (SPG K steps) at a time into a two-slot ring behind the tiles
+  constexpr int SPG = 4 * Cfg::kStepsPerScaleDword;
+  constexpr int SC_SLOT = (BM + BN) * 16;
   constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
   static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
   using CopyA = TileCopyK<BM, NW>;
@@ -649,8 +651,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   constexpr int ITA = CopyA::kIters;
   constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
   constexpr int KROWS = RBK / 2;
-  constexpr int NSC = Cfg::kScaled ? 8 / NW : 0;  // scale copies per wave and tile (64 rows of 4 bytes each)
-  constexpr int kShare = ITA + ITB + NSC;         // direct loads per wave and tile
+  constexpr int kShare = ITA + ITB;               // direct loads per wave and tile
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
@@ -702,13 +703,21 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     constexpr int i = decltype(I_)::value;
     if constexpr (i < ITA) {
       async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
-    } else if constexpr (i < ITA + ITB) {
+    } else {
       constexpr int ib = i - ITA;
       async_copy16(srcB[ib] + kt * stepB, (LDS_PTR(void))(a + A_BYTES + (ib * NW + wave) * 1024));
-    } else if constexpr (i == ITA + ITB) {
-      async_copy4(srcSA + Cfg::scale_dword_offset(kt), (LDS_PTR(void))(a + A_BYTES + B_BYTES + wave * 256));
-    } else {
-      async_copy4(srcSB + Cfg::scale_dword_offset(kt), (LDS_PTR(void))(a + A_BYTES + B_BYTES + BM * 4 + wave * 256));
+    }
+  };
+  // scale group sg (the 16 scale bytes per row of K steps sg*SPG ..) into ring slot sg % 2: one
+  // direct load moves 64 rows; past the last group the last one is fetched again
+  LDS_PTR(char) const sc_ring = lds + NS * STAGE;
+  const int ngroups = p.k_bytes / (RBK * SPG);
+  auto issue_scales = [&](int sg) {
+    if constexpr (Cfg::kScaled) {
+      LDS_PTR(char) dst = sc_ring + (sg & 1) * SC_SLOT + wave * 1024;
+      const int off = min(sg, ngroups - 1) * 16;
+      async_copy16(srcSA + off, (LDS_PTR(void))dst);
+      if constexpr (NW == 4) async_copy16(srcSB + off, (LDS_PTR(void))(dst + BM * 16));
     }
   };
 
@@ -739,8 +748,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       offBn[t] = A_BYTES + k * (BN * 2) + ((c32 ^ ((k & 3) << 1)) << 5) + (i16 & 3) * 8;
     }
   }
-  const unsigned offSA = A_BYTES + B_BYTES + (wm * TM + l32) * 4;
-  const unsigned offSB = A_BYTES + B_BYTES + BM * 4 + (wn * TN + l32) * 4;
+  const unsigned offSA = (wm * TM + l32) * 16;
+  const unsigned offSB = BM * 16 + (wn * TN + l32) * 16;
 
   // A K step is multiplied in two halves, and the operands of the next half are read from LDS
   // while the MFMAs of the current one issue.  With two MFMA sub-steps per K step (16-bit, fp4)
@@ -756,7 +765,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // LDS reads of half H of a tile with parity P: A operands, then (K-split: always, M-split: with
   // the first half) the B operands, then with the first half the scale dwords
   auto n_reads = [](int H) constexpr { return AH + ((KSPLIT || H == 0) ? NT : 0) + ((Cfg::kScaled && H == 0) ? MT + NT : 0); };
-  auto read_one = [&](auto R_, auto H_, auto P_, unsigned base) {
+  auto read_one = [&](auto R_, auto H_, auto P_, unsigned base, unsigned scbase) {
     constexpr int r = decltype(R_)::value, H = decltype(H_)::value, P = decltype(P_)::value;
     constexpr int ks = KSPLIT ? H : 0, aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P;
     constexpr int nb = (KSPLIT || H == 0) ? NT : 0;
@@ -785,8 +794,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       }
     } else {
       constexpr int t = r - AH - nb;
-      if constexpr (t < MT) sa_in[t] = lds_read_b32<t * 128>(base + offSA);
-      else sb_in[t - MT] = lds_read_b32<(t - MT) * 128>(base + offSB);
+      if constexpr (t < MT) sa_in[t] = lds_read_b32<t * 512>(scbase + offSA);
+      else sb_in[t - MT] = lds_read_b32<(t - MT) * 512>(scbase + offSB);
     }
   };
   // after the reads of a half have been waited for: tie the registers to the wait; with the
@@ -844,13 +853,14 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
 
   // prologue: NS tiles in flight (past the end of K the last tile again, which keeps the number
   // of outstanding loads - and with it the partial waits - uniform), first half of tile 0 requested
+  issue_scales(0);
 #pragma unroll
   for (int s = 0; s < NS; s++) static_for<kShare>([&](auto I_) { issue_one(I_, min(s, nfull - 1), lds + s * STAGE); });
   wait_vmcnt<(NS - 1) * kShare>();
   __builtin_amdgcn_sched_barrier(0);
   block_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(lds)); });
+  static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(lds), lds_addr(sc_ring)); });
 
   int stage = 0;
   // one K step of a tile with parity P
@@ -865,7 +875,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     {
       const unsigned base = lds_addr(lds + stage * STAGE);
       half(H0{}, P_, std::integral_constant<int, n_reads(1)>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
-        read_one(OP_, H1{}, P_, base);
+        read_one(OP_, H1{}, P_, base, 0u);
       });
     }
     // ---- second half: every wave holds the whole of tile kt in registers and has seen its own
@@ -876,14 +886,22 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     __builtin_amdgcn_sched_barrier(0);
     block_barrier();
     __builtin_amdgcn_sched_barrier(0);
+    // the first step of a scale group fetches the next group: its slot was last read two steps
+    // ago, and the loads are older than the NS-2 shares the partial waits leave in flight by the
+    // time the group is first read (SPG - 1 >= NS - 1 steps from now)
+    if constexpr (Cfg::kScaled) {
+      if (kt % SPG == 0) issue_scales(kt / SPG + 1);
+    }
     {
+      const int ktn = kt + 1;
+      const unsigned scbase = lds_addr(sc_ring) + ((ktn / SPG) & 1) * SC_SLOT + Cfg::scale_dword_offset(ktn % SPG);
       const unsigned base = lds_addr(lds + next_stage * STAGE);
       LDS_PTR(char) const fill = lds + stage * STAGE;
       const int kfill = min(kt + NS, nfull - 1);
       constexpr int nr = n_reads(0);
       half(H1{}, P_, std::integral_constant<int, nr>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
         constexpr int op = decltype(OP_)::value;
-        if constexpr (op < nr) read_one(OP_, H0{}, PN{}, base);
+        if constexpr (op < nr) read_one(OP_, H0{}, PN{}, base, scbase);
         else issue_one(std::integral_constant<int, op - nr>{}, kfill, fill);
       });
     }
@@ -906,7 +924,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
 template <typename Cfg, int WN, bool B_KMAJOR, int NS>
 static int launch_gemm_w4(const GemmArgs& p, hipStream_t stream) {
   constexpr int BM = 256, BN = 256;
-  constexpr int smem = NS * ((BM + BN) * RBK + (Cfg::kScaled ? (BM + BN) * 4 : 0));
+  constexpr int smem = NS * (BM + BN) * RBK + (Cfg::kScaled ? 2 * (BM + BN) * 16 : 0);
   static_assert(smem <= 160 * 1024, "LDS ring does not fit");
   static bool attr_set = false;
   if (!attr_set) {
@@ -960,7 +978,12 @@ static int launch_gemm(const GemmArgs& p, hipStream_t stream) {
 template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
   {
-    const bool whole = p.k_bytes >= RBK && p.k_bytes % (RBK * Cfg::kStepsPerScaleDword) == 0;
+    // whole K steps; block scales are fetched 16 bytes per row at a time
+    bool whole = p.k_bytes >= RBK && p.k_bytes % RBK == 0;
+    if constexpr (Cfg::kScaled) {
+      whole = p.k_bytes % (RBK * 4 * Cfg::kStepsPerScaleDword) == 0 && p.lds_a % 16 == 0 && p.lds_b % 16 == 0 &&
+              ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0;
+    }
     if constexpr (Cfg::kSteps == 2) {  // the four-wave form of the one-sub-step types runs out of registers
       if (tile == 3 && whole) return launch_gemm_w4<Cfg, 2, B_KMAJOR, 4>(p, stream);
     }
