@@ -259,7 +259,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   constexpr int TILE = Tile::BYTES;
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][Q tile | dO tile]
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][Q tile | dO tile | M rows | delta rows]
+  constexpr int STAGE = 2 * Tile::BYTES + 2 * BM * 4;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
@@ -298,14 +299,19 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     srcQ[i] = Tile::src(qbase, pitch, wave, lane, i);
     srcD[i] = Tile::src(dobase, pitch, wave, lane, i);
   }
+  // the M and delta values of the tile's query rows ride along (4 bytes per lane: wave 0 copies
+  // the 64 M values, wave 1 the 64 deltas), so the loop issues no register loads that would have to
+  // wait behind the tile copies
+  const float* src_stat = (wave == 0 ? lse : delta) + lane;
   auto issue_qd = [&](int mstart, int stage) {
-    LDS_PTR(char) qd = lds + stage * (2 * TILE);
+    LDS_PTR(char) qd = lds + stage * STAGE;
     LDS_PTR(char) dd = qd + TILE;
 #pragma unroll
     for (int i = 0; i < Tile::INST; i++) {
       async_copy16(srcQ[i] + (int64_t)mstart * pitch, (LDS_PTR(void))(qd + (i * NW + wave) * 1024));
       async_copy16(srcD[i] + (int64_t)mstart * pitch, (LDS_PTR(void))(dd + (i * NW + wave) * 1024));
     }
+    if (wave < 2) async_copy4(src_stat + mstart, (LDS_PTR(void))(qd + 2 * TILE + wave * (BM * 4)));
   };
 
   const RowRead<RB> rr(l32, g);
@@ -332,8 +338,9 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     const int ms = m_begin + j * BM;
     if (j + 1 < nsteps) issue_qd(ms + BM, stage ^ 1);
     if (nrow0 < p.N) {
-      const unsigned qb = lds_addr(lds + stage * (2 * TILE));
+      const unsigned qb = lds_addr(lds + stage * STAGE);
       const unsigned db = qb + TILE;
+      const unsigned sb = qb + 2 * TILE + g * 16;
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) {
         const int mrow0 = ms + mt * 32;
@@ -341,12 +348,17 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
         if (p.causal && mrow0 + 31 < nrow0) continue;
         const bool masked = p.causal && mrow0 < nrow0 + 31;
         // M and delta of the 16 query rows this lane's registers stand for
-        f32x4 mv[4], dl[4];
-#pragma unroll
-        for (int rg = 0; rg < 4; rg++) {
-          mv[rg] = *(const f32x4*)(lse + mrow0 + rg * 8 + g * 4);
-          dl[rg] = *(const f32x4*)(delta + mrow0 + rg * 8 + g * 4);
-        }
+        i32x4 mvi[4], dli[4];
+        static_for<4>([&](auto RG_) {
+          constexpr int rg = decltype(RG_)::value;
+          if (mt == 0) {
+            mvi[rg] = lds_read_b128<rg * 32>(sb);
+            dli[rg] = lds_read_b128<BM * 4 + rg * 32>(sb);
+          } else {
+            mvi[rg] = lds_read_b128<128 + rg * 32>(sb);
+            dli[rg] = lds_read_b128<BM * 4 + 128 + rg * 32>(sb);
+          }
+        });
         f32x16 s, dp;
 #pragma unroll
         for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
@@ -366,9 +378,19 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
             }
             lds_use(qf[cur]);
             lds_use(df[cur]);
+            if constexpr (ks + 1 == KSQ) {
+#pragma unroll
+              for (int rg = 0; rg < 4; rg++) { lds_use(mvi[rg]); lds_use(dli[rg]); }
+            }
             s = mfma32(__builtin_bit_cast(V8, qf[cur]), kf[ks], s);    // S[m][n]
             dp = mfma32(__builtin_bit_cast(V8, df[cur]), vf[ks], dp);  // dP[m][n]
           });
+        }
+        f32x4 mv[4], dl[4];
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          mv[rg] = __builtin_bit_cast(f32x4, mvi[rg]);
+          dl[rg] = __builtin_bit_cast(f32x4, dli[rg]);
         }
         V8 pf[2], dsf[2];
 #pragma unroll
@@ -453,7 +475,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
 template <typename V8, int D>
 static int launch_bwd_d(const AttnArgs& p, hipStream_t stream) {
   {
-    constexpr int QT = 2, NW = 4, BM = NW * QT * 32;
+    constexpr int QT = 1, NW = 4, BM = NW * QT * 32;
     constexpr int smem = 2 * 2 * 64 * D * 2;
     static bool attr_set = false;
     if (!attr_set) {
@@ -469,7 +491,7 @@ static int launch_bwd_d(const AttnArgs& p, hipStream_t stream) {
   }
   {
     constexpr int NW = 4, BN = NW * 32;
-    constexpr int smem = 2 * 2 * 64 * D * 2;
+    constexpr int smem = 2 * (2 * 64 * D * 2 + 2 * 64 * 4);
     static bool attr_set = false;
     if (!attr_set) {
       hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<V8, D, NW>,
