@@ -1,0 +1,312 @@
+// Flash-attention backward for gfx950, dK/dV pass (see attn_bwd.hip for the algorithm, the
+// reference lines it follows and the operand plan).  A file of its own because it is compiled
+// with the accumulators in AGPRs - dK and dV are touched by MFMAs only - while the kernels in
+// attn_bwd.hip want theirs in architectural VGPRs.
+#include "attn_tiles.h"
+#include "launch.h"
+
+namespace mi355 {
+
+template <typename V8> struct ElemB;
+template <> struct ElemB<bf16x8> { using type = __bf16; };
+template <> struct ElemB<f16x8> { using type = _Float16; };
+
+// ---------------------------------------------------------------------------------------------
+// dK/dV: one wave owns 32 key rows (K / V fragments and both accumulators in registers: one wave
+// per SIMD); Q / dO tiles of 64 rows stream through a ring of four LDS stages, each carrying the
+// M and delta values of its rows.
+//
+// With a single wave per SIMD nothing hides a latency for free, so the loop is software
+// pipelined over the 32-row query tiles t = 0, 1, ...:
+//     A(t):  S = Q K^T and dP = dO V^T          (2 * D/16 MFMAs, row-wise LDS operands)
+//     X(t):  p = exp2(S*s2 - M), ds = p (dP - delta), rounded to the input type   (VALU)
+//     C(t):  dV^T += dO^T p,  dK^T += Q^T ds    (2 * D/16 MFMAs, transposed LDS operands)
+// run as  ... [A(t+1) with X(t) and the transposed reads of t in between] [C(t) with the row-wise
+// reads of t+2 and the M/delta reads of t+1 in between] ...  so every MFMA group covers the other
+// pipes' work of its neighbours.  Tiles that lie entirely above the causal diagonal of a wave are
+// multiplied like the diagonal one: the mask turns p and ds into exact zeros.
+// One barrier per stage (two tiles), placed where every wave has finished reading the stage
+// before and has seen its own share of the next one arrive; the stage before is refilled there,
+// three stages ahead.
+// ---------------------------------------------------------------------------------------------
+template <typename V8, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
+  using S = typename ElemB<V8>::type;
+  typedef __attribute__((ext_vector_type(4))) S S4;
+  constexpr int BN = NW * 32, BM = 64, RB = D * 2, KSQ = D / 16, DT = D / 32, NS = 4;
+  using Tile = AttnTile<RB, BM, NW>;
+  constexpr int TILE = Tile::BYTES;
+  constexpr int STAGE = 2 * TILE + 2 * BM * 4;  // Q tile | dO tile | M rows | delta rows
+  constexpr int kShare = 2 * Tile::INST + 1;    // direct loads per wave and stage
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
+
+  const int nkb = (p.N + BN - 1) / BN;
+  int pid = xcd_remap(blockIdx.x, nkb * p.Z * p.H);
+  const int hz = pid / nkb;
+  const int kbk = pid % nkb;  // causal: low key blocks have the most work, ascending order = longest first
+  const int z = hz / p.H, h = hz % p.H;
+  const int n0 = kbk * BN, nrow0 = n0 + wave * 32;
+
+  const int64_t head_off = ((int64_t)z * p.sq[0] + (int64_t)h * p.sq[1]) * 2;
+  const int64_t pitch = p.sq[2] * 2;
+  const char* qbase = p.q + head_off;
+  const char* dobase = p.d_o + head_off;
+  const float* lse = p.lse + (int64_t)hz * p.N;
+  const float* delta = p.delta + (int64_t)hz * p.N;
+
+  // K / V fragments of this wave's key rows: lane (row l32, half g) holds X[row][16*ks + 8*g .. +8]
+  V8 kf[KSQ], vf[KSQ];
+  {
+    int r = min(nrow0 + l32, p.N - 1);
+    const char* sk = p.k + head_off + (int64_t)r * pitch + g * 16;
+    const char* sv = p.v + head_off + (int64_t)r * pitch + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) {
+      kf[ks] = *(const V8*)(sk + ks * 32);
+      vf[ks] = *(const V8*)(sv + ks * 32);
+    }
+  }
+
+  // query rows m >= n0 (causal) or all of them, in stages of BM rows
+  const int m_begin = p.causal ? (n0 / BM) * BM : 0;
+  const int nsteps = (p.N - m_begin + BM - 1) / BM;
+  const int ncol = nrow0 + l32;  // this lane's key row
+
+  const char* srcQ[Tile::INST];
+  const char* srcD[Tile::INST];
+#pragma unroll
+  for (int i = 0; i < Tile::INST; i++) {
+    srcQ[i] = Tile::src(qbase, pitch, wave, lane, i) + (int64_t)m_begin * pitch;
+    srcD[i] = Tile::src(dobase, pitch, wave, lane, i) + (int64_t)m_begin * pitch;
+  }
+  // even waves copy the stage's 64 M values, odd waves its 64 deltas (4 bytes per lane; the
+  // duplicates keep the number of loads per wave uniform for the partial waits)
+  const float* src_stat = ((wave & 1) == 0 ? lse : delta) + m_begin + lane;
+  // stage-step js (clamped to the last one) into ring slot js % NS
+  auto issue_stage = [&](int js) {
+    LDS_PTR(char) qd = lds + (js % NS) * STAGE;
+    LDS_PTR(char) dd = qd + TILE;
+    const int jc = min(js, nsteps - 1);
+#pragma unroll
+    for (int i = 0; i < Tile::INST; i++) {
+      async_copy16(srcQ[i] + (int64_t)jc * BM * pitch, (LDS_PTR(void))(qd + (i * NW + wave) * 1024));
+      async_copy16(srcD[i] + (int64_t)jc * BM * pitch, (LDS_PTR(void))(dd + (i * NW + wave) * 1024));
+    }
+    async_copy4(src_stat + jc * BM, (LDS_PTR(void))(qd + 2 * TILE + (wave & 1) * (BM * 4)));
+  };
+
+  // per-lane LDS offsets inside a stage: row-wise operand per k-step, transposed operand per
+  // (column block, half); stage, tile and sub-row offsets are added as scalars / immediates
+  const RowRead<RB> rr(l32, g);
+  const TrRead<RB> tt(i16, q4);
+  unsigned ra[KSQ], ta[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KSQ; ks++) ra[ks] = rr.rowb + (rr.xk ^ (ks * 32));
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++) ta[c][h2] = tt.tl ^ ((c << 6) | (h2 << 5));
+  const unsigned lds0 = lds_addr(lds);
+
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dk[c][r] = 0.f; dv[c][r] = 0.f; }
+  f32x16 sacc[2], dpacc[2];   // S and dP of the tile being multiplied / the tile being exponentiated
+  i32x4 rq[KSQ], rd[KSQ];     // row-wise Q / dO operands of the next A
+  i32x2 tq[2][DT][2], td[2][DT][2];  // transposed Q / dO operands of the next C
+  i32x4 mvi[4], dli[4];       // M and delta of the 16 query rows this lane's S registers stand for
+  V8 pf[2], dsf[2];           // p and ds as B operands of C, per 16-row k-step
+
+  const float qk_scale = p.sm_scale * 1.4426950408889634f;
+
+  // ---- pieces of the pipeline; MT = which 32-row half of the stage the tile is
+  auto read_rows = [&](auto I_, auto MT_, unsigned sbase) {  // read number I of 2*KSQ
+    constexpr int i = decltype(I_)::value, mt = decltype(MT_)::value, ks = i >> 1;
+    if constexpr ((i & 1) == 0) rq[ks] = lds_read_b128<mt * 32 * RB>(sbase + ra[ks]);
+    else rd[ks] = lds_read_b128<TILE + mt * 32 * RB>(sbase + ra[ks]);
+  };
+  auto read_stats = [&](auto I_, auto MT_, unsigned sbase) {  // read number I of 8
+    constexpr int i = decltype(I_)::value, mt = decltype(MT_)::value, rg = i >> 1;
+    if constexpr ((i & 1) == 0) mvi[rg] = lds_read_b128<2 * TILE + mt * 128 + rg * 32>(sbase + g * 16);
+    else dli[rg] = lds_read_b128<2 * TILE + BM * 4 + mt * 128 + rg * 32>(sbase + g * 16);
+  };
+  auto read_tr = [&](auto I_, auto MT_, unsigned sbase) {  // read number I of 8*DT
+    constexpr int i = decltype(I_)::value, mt = decltype(MT_)::value;
+    constexpr int which = i & 1, h2 = (i >> 1) & 1, c = (i >> 2) % DT, t = i / (4 * DT);
+    constexpr int imm = (mt * 32 + 16 * t + 8 * h2) * RB;
+    if constexpr (which == 0) tq[t][c][h2] = lds_read_tr16_b64<imm>(sbase + ta[c][h2]);
+    else td[t][c][h2] = lds_read_tr16_b64<TILE + imm>(sbase + ta[c][h2]);
+  };
+  auto settle_rows = [&]() {
+    lds_wait<0>();
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) { lds_use(rq[ks]); lds_use(rd[ks]); }
+  };
+  auto settle_stats = [&]() {
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) { lds_use(mvi[rg]); lds_use(dli[rg]); }
+  };
+  auto settle_tr = [&]() {
+    lds_wait<0>();
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int c = 0; c < DT; c++)
+#pragma unroll
+        for (int h2 = 0; h2 < 2; h2++) { lds_use(tq[t][c][h2]); lds_use(td[t][c][h2]); }
+  };
+  // X: elements r0 .. r0+n-1 of the tile whose S / dP sit in set PAR; mrow0 = its first query row
+  auto softmax_part = [&](auto PAR_, auto R0_, auto N_, int mrow0, bool masked) {
+    constexpr int par = decltype(PAR_)::value, r0 = decltype(R0_)::value, n = decltype(N_)::value;
+#pragma unroll
+    for (int r = r0; r < r0 + n; r++) {
+      const float mval = __builtin_bit_cast(f32x4, mvi[r >> 2])[r & 3];
+      const float dval = __builtin_bit_cast(f32x4, dli[r >> 2])[r & 3];
+      float pv = fast_exp2(fmaf(sacc[par][r], qk_scale, -mval));
+      if (masked) {
+        int m = mrow0 + (r >> 2) * 8 + g * 4 + (r & 3);
+        if (m < ncol) pv = 0.f;
+      }
+      float dsv = pv * (dpacc[par][r] - dval);
+      pf[r >> 3][r & 7] = (S)pv;
+      dsf[r >> 3][r & 7] = (S)dsv;
+    }
+  };
+  // A(next tile) into set PAR with X(previous tile, set PAR^1) and its transposed reads in between
+  auto phase_a = [&](auto PAR_, auto MTX_, bool do_x, int mrow0_x, unsigned sbase_x) {
+    constexpr int par = decltype(PAR_)::value;
+    constexpr int EPK = 16 / KSQ;             // X elements per k-step
+    constexpr int TRK = 2 * (8 * DT) / KSQ;   // transposed reads per k-step, all within the first half
+    const bool masked = p.causal && mrow0_x < nrow0 + 31;
+    settle_rows();
+    settle_stats();
+    static_for<KSQ>([&](auto KS_) {
+      constexpr int ks = decltype(KS_)::value;
+      if constexpr (ks == 0) {
+        f32x16 zero;
+#pragma unroll
+        for (int r = 0; r < 16; r++) zero[r] = 0.f;
+        sacc[par] = mfma32(__builtin_bit_cast(V8, rq[0]), kf[0], zero);
+        dpacc[par] = mfma32(__builtin_bit_cast(V8, rd[0]), vf[0], zero);
+      } else {
+        sacc[par] = mfma32(__builtin_bit_cast(V8, rq[ks]), kf[ks], sacc[par]);
+        dpacc[par] = mfma32(__builtin_bit_cast(V8, rd[ks]), vf[ks], dpacc[par]);
+      }
+      if (do_x) {
+        static_for<TRK>([&](auto O_) {
+          constexpr int i = ks * TRK + decltype(O_)::value;
+          if constexpr (i < 8 * DT) read_tr(std::integral_constant<int, i>{}, MTX_, sbase_x);
+        });
+        softmax_part(std::integral_constant<int, par ^ 1>{}, std::integral_constant<int, ks * EPK>{},
+                     std::integral_constant<int, EPK>{}, mrow0_x, masked);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  // C(tile) with the row-wise reads of the tile after next (stage sbase_r, half MTR) and the
+  // M / delta reads of the next tile (stage sbase_s, half MTS) in between
+  auto phase_c = [&](auto MTR_, unsigned sbase_r, auto MTS_, unsigned sbase_s) {
+    constexpr int NM = 2 * DT;               // MFMA pairs
+    constexpr int NRD = 2 * KSQ + 8;         // reads to place
+    constexpr int PER = (2 * NRD + NM - 1) / NM;  // all within the first half of the MFMAs
+    settle_tr();
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, t = n / DT, c = n % DT;
+      i32x4 qt = __builtin_shufflevector(tq[t][c][0], tq[t][c][1], 0, 1, 2, 3);
+      i32x4 dt = __builtin_shufflevector(td[t][c][0], td[t][c][1], 0, 1, 2, 3);
+      dv[c] = mfma32(__builtin_bit_cast(V8, dt), pf[t], dv[c]);
+      dk[c] = mfma32(__builtin_bit_cast(V8, qt), dsf[t], dk[c]);
+      static_for<PER>([&](auto O_) {
+        constexpr int i = n * PER + decltype(O_)::value;
+        if constexpr (i < 2 * KSQ) read_rows(std::integral_constant<int, i>{}, MTR_, sbase_r);
+        else if constexpr (i < NRD) read_stats(std::integral_constant<int, i - 2 * KSQ>{}, MTS_, sbase_s);
+      });
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  using I0 = std::integral_constant<int, 0>;
+  using I1 = std::integral_constant<int, 1>;
+
+  // ---- prologue: three stages in flight; A(0) alone; operands of A(1) and M/delta of tile 0
+#pragma unroll
+  for (int js = 0; js < NS - 1; js++) issue_stage(js);
+  wait_vmcnt<(NS - 2) * kShare>();
+  __builtin_amdgcn_sched_barrier(0);
+  block_barrier();
+  __builtin_amdgcn_sched_barrier(0);
+  static_for<2 * KSQ>([&](auto I_) { read_rows(I_, I0{}, lds0); });
+  static_for<8>([&](auto I_) { read_stats(I_, I0{}, lds0); });
+  phase_a(I0{}, I0{}, false, 0, 0u);
+  static_for<2 * KSQ>([&](auto I_) { read_rows(I_, I1{}, lds0); });
+
+  for (int j = 0; j < nsteps; j++) {
+    const unsigned sb_cur = lds0 + (j % NS) * STAGE;
+    const unsigned sb_nxt = lds0 + ((j + 1) % NS) * STAGE;
+    const int ms = m_begin + j * BM;
+    // A(2j+1) | X(2j), transposed reads of tile 2j
+    phase_a(I1{}, I0{}, true, ms, sb_cur);
+    // every wave is done with stage j-1 and has seen its share of stage j+1 arrive
+    wait_vmcnt<kShare>();
+    __builtin_amdgcn_sched_barrier(0);
+    block_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    issue_stage(j + NS - 1);
+    // C(2j) | row-wise reads of tile 2j+2 (next stage), M/delta of tile 2j+1
+    phase_c(I0{}, sb_nxt, I1{}, sb_cur);
+    // A(2j+2) | X(2j+1), transposed reads of tile 2j+1
+    phase_a(I0{}, I1{}, true, ms + 32, sb_cur);
+    // C(2j+1) | row-wise reads of tile 2j+3, M/delta of tile 2j+2
+    phase_c(I1{}, sb_nxt, I0{}, sb_nxt);
+  }
+  // nothing may still be writing this workgroup's LDS when it retires
+  wait_all();
+
+  if (ncol < p.N) {
+    char* dkd = p.dk + head_off + (int64_t)ncol * pitch;
+    char* dvd = p.dv + head_off + (int64_t)ncol * pitch;
+#pragma unroll
+    for (int c = 0; c < DT; c++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        int d = c * 32 + rg * 8 + g * 4;
+        S4 a, b;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          a[e] = (S)(dk[c][rg * 4 + e] * p.sm_scale);
+          b[e] = (S)dv[c][rg * 4 + e];
+        }
+        *(S4*)(dkd + d * 2) = a;
+        *(S4*)(dvd + d * 2) = b;
+      }
+  }
+}
+
+template <typename V8, int D>
+static int launch_dkdv(const AttnArgs& p, hipStream_t stream) {
+  constexpr int NW = 4, BN = NW * 32;
+  constexpr int smem = 4 * (2 * 64 * D * 2 + 2 * 64 * 4);
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<V8, D, NW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  int nkb = (p.N + BN - 1) / BN;
+  attn_bwd_dkdv_kernel<V8, D, NW><<<dim3(nkb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+int attn_bwd_dkdv_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
+  if (bf16) return p.D == 128 ? launch_dkdv<bf16x8, 128>(p, stream) : launch_dkdv<bf16x8, 64>(p, stream);
+  return p.D == 128 ? launch_dkdv<f16x8, 128>(p, stream) : launch_dkdv<f16x8, 64>(p, stream);
+}
+
+}  // namespace mi355
