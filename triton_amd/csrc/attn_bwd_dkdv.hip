@@ -42,7 +42,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: branches on it are uniform
   const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
 
   const int nkb = (p.N + BN - 1) / BN;
@@ -163,14 +164,15 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
         for (int h2 = 0; h2 < 2; h2++) { lds_use(tq[t][c][h2]); lds_use(td[t][c][h2]); }
   };
   // X: elements r0 .. r0+n-1 of the tile whose S / dP sit in set PAR; mrow0 = its first query row
-  auto softmax_part = [&](auto PAR_, auto R0_, auto N_, int mrow0, bool masked) {
+  auto softmax_part = [&](auto PAR_, auto R0_, auto N_, int mrow0, auto MASKED_) {
     constexpr int par = decltype(PAR_)::value, r0 = decltype(R0_)::value, n = decltype(N_)::value;
+    constexpr bool masked = decltype(MASKED_)::value;
 #pragma unroll
     for (int r = r0; r < r0 + n; r++) {
       const float mval = __builtin_bit_cast(f32x4, mvi[r >> 2])[r & 3];
       const float dval = __builtin_bit_cast(f32x4, dli[r >> 2])[r & 3];
       float pv = fast_exp2(fmaf(sacc[par][r], qk_scale, -mval));
-      if (masked) {
+      if constexpr (masked) {
         int m = mrow0 + (r >> 2) * 8 + g * 4 + (r & 3);
         if (m < ncol) pv = 0.f;
       }
@@ -180,11 +182,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     }
   };
   // A(next tile) into set PAR with X(previous tile, set PAR^1) and its transposed reads in between
-  auto phase_a = [&](auto PAR_, auto MTX_, bool do_x, int mrow0_x, unsigned sbase_x) {
+  auto phase_a_impl = [&](auto PAR_, auto MTX_, auto DOX_, auto MASKED_, int mrow0_x, unsigned sbase_x) {
     constexpr int par = decltype(PAR_)::value;
+    constexpr bool do_x = decltype(DOX_)::value;
     constexpr int EPK = 16 / KSQ;             // X elements per k-step
     constexpr int TRK = 2 * (8 * DT) / KSQ;   // transposed reads per k-step, all within the first half
-    const bool masked = p.causal && mrow0_x < nrow0 + 31;
     settle_rows();
     settle_stats();
     static_for<KSQ>([&](auto KS_) {
@@ -199,17 +201,18 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
         sacc[par] = mfma32(__builtin_bit_cast(V8, rq[ks]), kf[ks], sacc[par]);
         dpacc[par] = mfma32(__builtin_bit_cast(V8, rd[ks]), vf[ks], dpacc[par]);
       }
-      if (do_x) {
+      if constexpr (do_x) {
         static_for<TRK>([&](auto O_) {
           constexpr int i = ks * TRK + decltype(O_)::value;
           if constexpr (i < 8 * DT) read_tr(std::integral_constant<int, i>{}, MTX_, sbase_x);
         });
         softmax_part(std::integral_constant<int, par ^ 1>{}, std::integral_constant<int, ks * EPK>{},
-                     std::integral_constant<int, EPK>{}, mrow0_x, masked);
+                     std::integral_constant<int, EPK>{}, mrow0_x, MASKED_);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
   };
+
   // C(tile) with the row-wise reads of the tile after next (stage sbase_r, half MTR) and the
   // M / delta reads of the next tile (stage sbase_s, half MTS) in between
   auto phase_c = [&](auto MTR_, unsigned sbase_r, auto MTS_, unsigned sbase_s) {
@@ -243,15 +246,16 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   __builtin_amdgcn_sched_barrier(0);
   static_for<2 * KSQ>([&](auto I_) { read_rows(I_, I0{}, lds0); });
   static_for<8>([&](auto I_) { read_stats(I_, I0{}, lds0); });
-  phase_a(I0{}, I0{}, false, 0, 0u);
+  phase_a_impl(I0{}, I0{}, std::false_type{}, std::false_type{}, 0, 0u);
   static_for<2 * KSQ>([&](auto I_) { read_rows(I_, I1{}, lds0); });
 
-  for (int j = 0; j < nsteps; j++) {
+  // one stage (two tiles) of the pipeline
+  auto stage_step = [&](int j, auto MASKED_) {
     const unsigned sb_cur = lds0 + (j % NS) * STAGE;
     const unsigned sb_nxt = lds0 + ((j + 1) % NS) * STAGE;
     const int ms = m_begin + j * BM;
     // A(2j+1) | X(2j), transposed reads of tile 2j
-    phase_a(I1{}, I0{}, true, ms, sb_cur);
+    phase_a_impl(I1{}, I0{}, std::true_type{}, MASKED_, ms, sb_cur);
     // every wave is done with stage j-1 and has seen its share of stage j+1 arrive
     wait_vmcnt<kShare>();
     __builtin_amdgcn_sched_barrier(0);
@@ -261,10 +265,15 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     // C(2j) | row-wise reads of tile 2j+2 (next stage), M/delta of tile 2j+1
     phase_c(I0{}, sb_nxt, I1{}, sb_cur);
     // A(2j+2) | X(2j+1), transposed reads of tile 2j+1
-    phase_a(I0{}, I1{}, true, ms + 32, sb_cur);
+    phase_a_impl(I0{}, I1{}, std::true_type{}, MASKED_, ms + 32, sb_cur);
     // C(2j+1) | row-wise reads of tile 2j+3, M/delta of tile 2j+2
     phase_c(I1{}, sb_nxt, I0{}, sb_nxt);
-  }
+  };
+  // causal: the workgroup's 128 key rows meet the diagonal in its first two stages (query rows
+  // n0 .. n0+127); only those pay for the mask
+  const int nmasked = p.causal ? min(2, nsteps) : 0;
+  for (int j = 0; j < nmasked; j++) stage_step(j, std::true_type{});
+  for (int j = nmasked; j < nsteps; j++) stage_step(j, std::false_type{});
   // nothing may still be writing this workgroup's LDS when it retires
   wait_all();
 
