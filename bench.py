@@ -23,9 +23,10 @@ if ROOT not in sys.path:
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4": 10100.0}
 HBM_GBPS = 8000.0
 
-# HBM bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc
-# (FETCH_SIZE, WRITE_SIZE), see profiles/; None until measured
-MEASURED_TRAFFIC_BYTES = None
+# HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc:
+# FETCH_SIZE 790628 KiB x 2.000 + WRITE_SIZE 196184 KiB x 1.000, the factors being what the same
+# counters read for a plain copy of known size (profiles/gemm_bf16_8192.md)
+MEASURED_TRAFFIC_BYTES = int((790628 * 2.000 + 196184 * 1.000) * 1024)
 
 
 def time_launches(fn, steps, warmup):
@@ -138,7 +139,7 @@ def main():
         "config": {"workload": f"bf16 GEMM M=N=K={n}, A row-major MxK, B row-major KxN, fp32 accumulate, bf16 out (BASELINE config 2)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK["bf16"], 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gemm_kernel<Cfg16<bf16>,256,256,2,4,row-major B>", "launch_ms_avg": round(ev_ms, 5),
+                     "kernel": "gemm_w4_kernel<Cfg16<bf16>, 8 waves, row-major B, 4 stages> (256x256 tile, software pipelined)", "launch_ms_avg": round(ev_ms, 5),
                      "launch_ms_min": round(min(per), 5), "algorithmic_flops": flops,
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
