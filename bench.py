@@ -155,7 +155,14 @@ def main():
         ms = quick(lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sc, b_scale=sc))
         extra["fp8_e4m3_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK["fp8"], 4)}
         a16 = torch.randn(16, n, device=dev).to(torch.float8_e4m3fn)
-        ms = quick(lambda: triton_amd.matmul(a16, b8.t(), out_dtype=torch.bfloat16), iters=20)
+        c16 = torch.empty(16, n, device=dev, dtype=torch.bfloat16)
+
+        def decode():  # straight through the C ABI: at ~20 us per launch the Python wrapper would dominate
+            rc = lib.mi355_gemm(a16.data_ptr(), b8.data_ptr(), c16.data_ptr(), 16, n, n, n, 1, 1, n, n, 1,
+                                _lib.F8E4M3, _lib.BF16, None, None, 0, stream)
+            assert rc == 0, rc
+
+        ms = quick(decode, iters=50, warmup=5)
         byts = n * n + 16 * n + 2 * 16 * n
         extra["fp8_decode_m16"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1), "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
         del a8, a16
@@ -181,7 +188,8 @@ def main():
             extra[f"attn_fwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["bf16"], 4)}
             o = triton_amd.attention(q, k, v, causal, sm)
             do = torch.randn_like(o)
-            ms = quick(lambda: o.backward(do, retain_graph=True), iters=5)
+            # gradients returned, not accumulated into .grad (that would add three elementwise kernels)
+            ms = quick(lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True), iters=5)
             extra[f"attn_bwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(2.5 * fl / ms / 1e9, 1), "frac_of_peak": round(2.5 * fl / ms / 1e9 / PEAK["bf16"], 4)}
         out["extra"] = extra
 

@@ -129,6 +129,7 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   // large problems run the software-pipelined 8-wave kernel
   int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
+  if (is8 && gemm8_skinny_ok(p) && env_int("MI355_GEMM_SKINNY", 1)) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }

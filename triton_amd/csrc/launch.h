@@ -48,6 +48,8 @@ struct AttnArgs {
 
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
+bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
+int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
