@@ -147,7 +147,13 @@ def main():
     }
 
     if not args.no_extra:
+        from triton_amd import testing
+
         extra = {}
+        # the reference's own timing protocol (cache flushed before every call, per-call events)
+        med, p20, p80 = testing.do_bench(step, warmup=25, rep=100, quantiles=[0.5, 0.2, 0.8])
+        extra["bf16_gemm_do_bench"] = {"ms_median": round(med, 4), "ms_p20": round(p20, 4), "ms_p80": round(p80, 4),
+                                       "tflops_median": round(testing.matmul_tflops(n, n, n, med), 1)}
         # fp8 e4m3 GEMM, K-major B, per-tensor scales, bf16 out (config 4) and its decode shape
         a8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
         b8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
