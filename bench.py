@@ -172,6 +172,13 @@ def main():
         byts = n * n + 16 * n + 2 * 16 * n
         extra["fp8_decode_m16"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1), "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
         del a8, a16
+        # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch
+        ga = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        gb = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        ms = quick(lambda: triton_amd.group_gemm_fn(ga, gb))
+        gfl = 16 * 2.0 * 2048 ** 3
+        extra["grouped_gemm_16x2048"] = {"ms": round(ms, 4), "tflops": round(gfl / ms / 1e9, 1), "frac_of_peak": round(gfl / ms / 1e9 / PEAK["fp16"], 4)}
+        del ga, gb
         # MX GEMMs (config 5)
         for fmt, kb in (("mxfp4", n // 2), ("mxfp8", n)):
             pa = torch.randint(0, 120, (n, kb), device=dev, dtype=torch.uint8)

@@ -94,6 +94,25 @@ int mi355_gemm(const void* A, const void* B, void* C,
                int activation, void* stream);
 
 /*
+ * Grouped GEMM: C_g[M_g,N_g] = A_g[M_g,K_g] @ B_g[K_g,N_g] for g = 0 .. group_size-1 in ONE launch.
+ *
+ * Stands in for the launch of `grouped_matmul_kernel` by `group_gemm_fn`
+ *   python/tutorials/08-grouped-gemm.py:64-140 (kernel), :143-187 (host wrapper)
+ * with the kernel's own arguments: device arrays of matrix addresses (uint64), a device int32 array
+ * `d_sizes[group_size][3]` = <M, N, K> and a device int32 array `d_lds[group_size][3]` =
+ * <lda, ldb, ldc> in elements; all matrices row major (unit column stride), A, B and C of type
+ * `dtype` (MI355_F16 as in the reference, or MI355_BF16), fp32 accumulation.
+ * `num_programs` workgroups walk the tiles of all problems (the reference's NUM_SM); 0 picks two
+ * per compute unit.  Any sizes are accepted (partial tiles are handled; the reference assumes
+ * full tiles); problems whose lda, ldb, N or K are not multiples of 8 elements, or whose A / B
+ * are not 16-byte aligned, run a slower loop inside the same kernel.  Nothing about the device
+ * arrays can be checked on the host: they must hold `group_size` valid entries.
+ */
+int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,
+                       const int32_t* d_sizes, const int32_t* d_lds, int group_size,
+                       int dtype, int num_programs, void* stream);
+
+/*
  * Block-scaled (OCP MX v1.0) GEMM: C[m,n] = sum_kb 2^(sA[m,kb]-127) 2^(sB[n,kb]-127) sum_{k in kb} A^[m,k] B^[n,k]
  * with 32-element blocks along K.  A is [M, K] and B is [N, K] (both K-contiguous):
  *   MXFP4: A_bytes[M, K/2], B_bytes[N, K/2];   MXFP8: A_bytes[M, K], B_bytes[N, K];

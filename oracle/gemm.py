@@ -84,3 +84,45 @@ def matmul_closed_form(a: np.ndarray, b: np.ndarray, activation: str = "", out_d
     if activation == "leaky_relu":
         acc = np.where(acc >= 0, acc, 0.01 * acc)
     return formats.round_to(acc.astype(np.float32), out_dtype)
+
+
+def grouped_tile_walk(sizes, BM: int, BN: int, num_programs: int):
+    """The tile schedule of `grouped_matmul_kernel` (python/tutorials/08-grouped-gemm.py:86-134):
+    tiles are numbered problem after problem, row major inside a problem; program b visits
+    tiles b, b + num_programs, ...  Returns, per program, the list of (problem, tile_m, tile_n)."""
+    walks = []
+    for b in range(num_programs):
+        tile_idx, last_problem_end, visited = b, 0, []
+        for g, (gm, gn, _gk) in enumerate(sizes):
+            num_n_tiles = cdiv(gn, BN)
+            num_tiles = cdiv(gm, BM) * num_n_tiles
+            while last_problem_end <= tile_idx < last_problem_end + num_tiles:
+                t = tile_idx - last_problem_end
+                visited.append((g, t // num_n_tiles, t % num_n_tiles))
+                tile_idx += num_programs
+            last_problem_end += num_tiles
+        walks.append(visited)
+    return walks
+
+
+def grouped_matmul(group_a, group_b, BM: int = 128, BN: int = 128, BK: int = 32, num_programs: int = 84,
+                   out_dtype: str = "fp16"):
+    """`group_gemm_fn` (08:143-187) executed program by program in the order of `grouped_tile_walk`:
+    every tile accumulates `np.matmul(a, b, dtype=float32)` per K chunk (interpreter.py:542-549)
+    and is rounded once to the output type.  Partial tiles are clipped (the reference assumes full
+    tiles, 08:118 and :130)."""
+    sizes = [(a.shape[0], b.shape[1], a.shape[1]) for a, b in zip(group_a, group_b)]
+    outs = [np.zeros((m, n), dtype=np.float32) for (m, n, _k) in sizes]
+    done = [np.zeros((cdiv(m, BM), cdiv(n, BN)), dtype=np.int32) for (m, n, _k) in sizes]
+    for visited in grouped_tile_walk(sizes, BM, BN, num_programs):
+        for g, tm, tn in visited:
+            a = np.asarray(group_a[g], dtype=np.float32)
+            b = np.asarray(group_b[g], dtype=np.float32)
+            m0, n0, K = tm * BM, tn * BN, a.shape[1]
+            acc = np.zeros((min(BM, a.shape[0] - m0), min(BN, b.shape[1] - n0)), dtype=np.float32)
+            for k0 in range(0, K, BK):
+                acc = np.matmul(a[m0:m0 + BM, k0:k0 + BK], b[k0:k0 + BK, n0:n0 + BN], dtype=np.float32) + acc
+            outs[g][m0:m0 + BM, n0:n0 + BN] = formats.round_to(acc, out_dtype)
+            done[g][tm, tn] += 1
+    assert all((d == 1).all() for d in done), "every tile exactly once"
+    return outs

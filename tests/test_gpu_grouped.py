@@ -1,0 +1,59 @@
+"""GPU parity: grouped GEMM through the C ABI (`group_gemm_fn`) against the CPU oracle.
+The reference's own check is `torch.allclose(ref, out, atol=1e-2, rtol=0)` on rand() inputs of
+sizes 1024, 512, 256, 128 (python/tutorials/08-grouped-gemm.py:190-214)."""
+import numpy as np
+import pytest
+import torch
+
+import triton_amd
+from oracle import formats, gemm
+from util import bits_equal, from_np, to_np
+
+pytestmark = pytest.mark.gpu
+
+
+def _run(gpu, ga, gb, dtype, **kw):
+    ta = [from_np(a, dtype, gpu) for a in ga]
+    tb = [from_np(b, dtype, gpu) for b in gb]
+    return [to_np(c) for c in triton_amd.group_gemm_fn(ta, tb, **kw)]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_reference_example_sizes(gpu, dtype):
+    # 08:190-205: square problems 1024, 512, 256, 128 of uniform [0, 1) values
+    rng = np.random.default_rng(0)
+    ga = [formats.round_to(rng.random((d, d)).astype(np.float32), dtype) for d in (1024, 512, 256, 128)]
+    gb = [formats.round_to(rng.random((d, d)).astype(np.float32), dtype) for d in (1024, 512, 256, 128)]
+    outs = _run(gpu, ga, gb, dtype)
+    for a, b, c in zip(ga, gb, outs):
+        ref = gemm.matmul_closed_form(a, b, out_dtype=dtype)
+        # results reach 2^8: one unit in the last place is 0.25 (fp16) / 2 (bf16), so the reference's
+        # absolute 1e-2 only holds where both sides round the same way; the bar here is rtol 1e-2
+        assert np.allclose(c, ref, rtol=1e-2, atol=1e-2)
+        assert np.mean(c == ref) > 0.98
+
+
+@pytest.mark.parametrize("nprog", [0, 1, 7, 100])
+def test_ragged_problems_are_bit_exact_on_integers(gpu, nprog):
+    # partial tiles, a single row, K tails (K % 32 != 0), and problems without 16-byte rows
+    rng = np.random.default_rng(nprog)
+    shapes = [(256, 128, 64), (130, 72, 40), (1, 304, 8), (128, 128, 128), (100, 70, 50), (37, 19, 7), (300, 264, 520)]
+    ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]
+    gb = [rng.integers(-2, 3, size=(k, n)).astype(np.float32) for m, n, k in shapes]
+    ref = gemm.grouped_matmul(ga, gb, num_programs=max(nprog, 1), out_dtype="fp32")
+    for dtype in ("fp16", "bf16"):
+        outs = _run(gpu, ga, gb, dtype, num_programs=nprog)
+        for c, r in zip(outs, ref):
+            assert bits_equal(c, r)   # integer results below 2^11 are exact in fp16 and bf16
+
+
+def test_strided_rows_and_empty_group(gpu):
+    rng = np.random.default_rng(9)
+    big_a = torch.from_numpy(rng.integers(-2, 3, size=(96, 200)).astype(np.float32)).to(gpu).half()
+    big_b = torch.from_numpy(rng.integers(-2, 3, size=(64, 400)).astype(np.float32)).to(gpu).half()
+    a, b = big_a[:, :64], big_b[:, 8:136]          # lda = 200, ldb = 400 elements
+    (c,) = triton_amd.group_gemm_fn([a], [b])
+    assert torch.equal(c.float(), a.float() @ b.float())
+    assert triton_amd.group_gemm_fn([], []) == []
+    with pytest.raises(AssertionError):
+        triton_amd.group_gemm_fn([a], [b, b])

@@ -134,6 +134,21 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 
+int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,
+                       const int32_t* d_sizes, const int32_t* d_lds, int group_size,
+                       int dtype, int num_programs, void* stream_) {
+  if (!d_a_ptrs || !d_b_ptrs || !d_c_ptrs || !d_sizes || !d_lds || group_size < 0 || num_programs < 0) return MI355_EINVAL;
+  if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  if (group_size == 0) return MI355_OK;
+  GroupedArgs ga{};
+  ga.a_ptrs = (const uint64_t*)d_a_ptrs; ga.b_ptrs = (const uint64_t*)d_b_ptrs; ga.c_ptrs = (const uint64_t*)d_c_ptrs;
+  ga.sizes = d_sizes; ga.lds = d_lds; ga.group_size = group_size; ga.out_dtype = dtype;
+  const int cus = device_info().cus > 0 ? device_info().cus : 256;
+  const int nprog = num_programs > 0 ? num_programs : 2 * cus;
+  return gemm16_grouped_launch(ga, dtype == MI355_BF16, nprog, (hipStream_t)stream_);
+}
+
 int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const uint8_t* sB, void* C,
                   int M, int N, int K, int fmt, int out_dtype,
                   int64_t lda, int64_t ldb, int64_t lds_a, int64_t lds_b, int64_t ldc, void* stream_) {

@@ -132,8 +132,11 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmA
   }
 }
 
+// One BM x BN tile of C (tile row pm, tile column pn) with a ring of NS LDS stages at `lds`
+// (NS * (BM + BN) * RBK bytes).  Shared by the one-tile-per-workgroup kernel below and by the
+// grouped kernel, whose workgroups walk the tiles of several problems.
 template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
-__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, const int pn, LDS_PTR(char) const lds) {
   using Operand = typename Cfg::Operand;
   constexpr int NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK, STAGE = A_BYTES + B_BYTES;
@@ -146,17 +149,8 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
   constexpr int KROWS = RBK / 2;  // k rows of a row-major 16-bit B tile
 
-  // ring of NS LDS stages (dynamic LDS: NS * STAGE bytes at launch)
-  extern __shared__ __attribute__((aligned(1024))) char smem[];
-  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
-
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-
-  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
-  int pid = xcd_remap(blockIdx.x, num_m * num_n);
-  int pm, pn;
-  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
   const int m0 = pm * BM, n0 = pn * BN;
 
   // per-lane global source pointers of the k = 0 tile; rows past the matrix edge are clamped
@@ -398,6 +392,91 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   }
 
   gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+}
+
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
+  // ring of NS LDS stages (dynamic LDS: NS * STAGE bytes at launch)
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  int pid = xcd_remap(blockIdx.x, num_m * num_n);
+  int pm, pn;
+  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
+  gemm_tile_body<Cfg, BM, BN, WM, WN, B_KMAJOR, NS>(p, pm, pn, (LDS_PTR(char))smem);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Grouped GEMM: a fixed number of workgroups walks the tiles of `group_size` independent
+// problems C_g = A_g @ B_g, whose pointers, sizes and leading dimensions live in device arrays -
+// the contract of the reference's `grouped_matmul_kernel`
+// (python/tutorials/08-grouped-gemm.py:64-140): tiles are numbered problem after problem, row
+// major inside a problem, and program b takes tiles b, b + nprog, b + 2 nprog, ...
+// Here b is first remapped so that the programs of one XCD take neighbouring tiles (shared A
+// panels stay in one L2), a tile is the 128x128 MFMA tile above with its edge handling (the
+// reference assumes full tiles), and a problem whose leading dimensions or N, K are not multiples
+// of 8 elements - no 16-byte rows - is computed by a plain dot-product loop instead.
+// ---------------------------------------------------------------------------------------------
+template <typename Cfg, typename T>
+__global__ __launch_bounds__(256, 1) void gemm_grouped_kernel(GroupedArgs ga) {
+  constexpr int BM = 128, BN = 128, NS = 4;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+  const int nprog = gridDim.x;
+  int tile_idx = xcd_remap(blockIdx.x, nprog);
+  int last_problem_end = 0;
+  for (int gi = 0; gi < ga.group_size; gi++) {
+    const int gm = ga.sizes[gi * 3], gn = ga.sizes[gi * 3 + 1], gk = ga.sizes[gi * 3 + 2];
+    const int num_m = (gm + BM - 1) / BM, num_n = (gn + BN - 1) / BN;
+    const int num_tiles = num_m * num_n;
+    if (tile_idx >= last_problem_end && tile_idx < last_problem_end + num_tiles) {
+      const int lda = ga.lds[gi * 3], ldb = ga.lds[gi * 3 + 1], ldc = ga.lds[gi * 3 + 2];
+      GemmArgs p{};
+      p.A = (const char*)ga.a_ptrs[gi]; p.B = (const char*)ga.b_ptrs[gi]; p.C = (char*)ga.c_ptrs[gi];
+      p.M = gm; p.N = gn; p.K = gk; p.k_bytes = gk * 2;
+      p.lda = (int64_t)lda * 2; p.ldb = (int64_t)ldb * 2; p.ldc = ldc; p.scn = 1;
+      p.out_dtype = ga.out_dtype; p.group_m = 1;
+      p.c_vec_ok = (ldc % 4 == 0) && (((uintptr_t)p.C) % 16 == 0);
+      const bool rows16 = ((lda | ldb | gn | gk) % 8 == 0) && ((((uintptr_t)p.A) | ((uintptr_t)p.B)) % 16 == 0);
+      while (tile_idx >= last_problem_end && tile_idx < last_problem_end + num_tiles) {
+        const int t = tile_idx - last_problem_end;
+        const int pm = t / num_n, pn = t % num_n;
+        if (rows16) {
+          gemm_tile_body<Cfg, BM, BN, 2, 2, false, NS>(p, pm, pn, lds);
+          // the next tile refills the ring: every wave must be done reading it
+          wait_all();
+          __syncthreads();
+        } else {
+          const T* A = (const T*)p.A;
+          const T* B = (const T*)p.B;
+          T* C = (T*)p.C;
+          for (int e = threadIdx.x; e < BM * BN; e += 256) {
+            const int m = pm * BM + e / BN, n = pn * BN + e % BN;
+            if (m < gm && n < gn) {
+              float acc = 0.f;
+              for (int k = 0; k < gk; k++) acc = fmaf((float)A[(int64_t)m * lda + k], (float)B[(int64_t)k * ldb + n], acc);
+              C[(int64_t)m * ldc + n] = (T)acc;
+            }
+          }
+        }
+        tile_idx += nprog;
+      }
+    }
+    last_problem_end += num_tiles;
+  }
+}
+
+template <typename Cfg, typename T>
+static int launch_gemm_grouped(const GroupedArgs& ga, int nprog, hipStream_t stream) {
+  constexpr int smem = 4 * (128 + 128) * RBK;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_grouped_kernel<Cfg, T>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  gemm_grouped_kernel<Cfg, T><<<dim3(nprog), dim3(256), smem, stream>>>(ga);
+  return (int)hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -46,6 +46,18 @@ struct AttnArgs {
   int variant;  // tiling variant (tuning knob)
 };
 
+// Device-side tables of a grouped GEMM (layout of python/tutorials/08-grouped-gemm.py:66-77).
+struct GroupedArgs {
+  const uint64_t* a_ptrs;  // [group_size] device addresses
+  const uint64_t* b_ptrs;
+  const uint64_t* c_ptrs;
+  const int* sizes;        // [group_size][3] = M, N, K
+  const int* lds;          // [group_size][3] = lda, ldb, ldc in elements
+  int group_size;
+  int out_dtype;           // element type of A, B and C: 0 = fp16, 1 = bf16
+};
+
+int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
 bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256

@@ -133,6 +133,48 @@ def matmul_like_input(a, b):
     return c
 
 
+def group_gemm_fn(group_A, group_B, *, num_programs: int = 0):
+    """The reference's `group_gemm_fn(group_A, group_B)` (python/tutorials/08-grouped-gemm.py:143-187):
+    `[A_i @ B_i for i]` in one launch.  Builds the same five device tables (matrix addresses,
+    <M, N, K>, <lda, ldb, ldc>) and hands them to the grouped kernel; outputs have A's dtype.
+    fp16 as in the reference, or bf16.  `num_programs` is the reference's NUM_SM (0 = two per CU)."""
+    assert len(group_A) == len(group_B)
+    group_size = len(group_A)
+    if group_size == 0:
+        return []
+    device = group_A[0].device
+    dt = _abi_dtype(group_A[0])
+    assert dt in (_lib.F16, _lib.BF16), "grouped GEMM takes fp16 or bf16 matrices"
+    A_addrs, B_addrs, C_addrs, g_sizes, g_lds, group_C = [], [], [], [], [], []
+    for i in range(group_size):
+        A, B = group_A[i], group_B[i]
+        _check_device(2 * i, A)
+        _check_device(2 * i + 1, B)
+        assert A.shape[1] == B.shape[0]
+        assert A.dtype == B.dtype == group_A[0].dtype, "all matrices of a group share one dtype"
+        assert A.stride(1) == 1 and B.stride(1) == 1, "matrices must be row major"
+        M, K = A.shape
+        K, N = B.shape
+        C = torch.empty((M, N), device=device, dtype=A.dtype)
+        group_C.append(C)
+        A_addrs.append(A.data_ptr())
+        B_addrs.append(B.data_ptr())
+        C_addrs.append(C.data_ptr())
+        g_sizes += [M, N, K]
+        g_lds += [A.stride(0), B.stride(0), C.stride(0)]
+    # device tables, as in the reference (08:166-170)
+    d_a_ptrs = torch.tensor(A_addrs, device=device, dtype=torch.int64)
+    d_b_ptrs = torch.tensor(B_addrs, device=device, dtype=torch.int64)
+    d_c_ptrs = torch.tensor(C_addrs, device=device, dtype=torch.int64)
+    d_g_sizes = torch.tensor(g_sizes, dtype=torch.int32, device=device)
+    d_g_lds = torch.tensor(g_lds, dtype=torch.int32, device=device)
+    rc = _lib.load().mi355_grouped_gemm(d_a_ptrs.data_ptr(), d_b_ptrs.data_ptr(), d_c_ptrs.data_ptr(),
+                                        d_g_sizes.data_ptr(), d_g_lds.data_ptr(), group_size, dt,
+                                        int(num_programs), _stream())
+    _lib.check(rc, "mi355_grouped_gemm")
+    return group_C
+
+
 def mx_matmul(a_packed, a_scale, b_packed, b_scale, fmt="mxfp4", out_dtype=torch.bfloat16):
     """Block-scaled matmul C[M,N] = A[M,K] . B[N,K]^T (OCP MX v1.0, 32-element blocks along K).
 
