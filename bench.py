@@ -217,6 +217,14 @@ def main():
             # gradients returned, not accumulated into .grad (that would add three elementwise kernels)
             ms = quick(lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True), iters=5)
             extra[f"attn_bwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(2.5 * fl / ms / 1e9, 1), "frac_of_peak": round(2.5 * fl / ms / 1e9 / PEAK["bf16"], 4)}
+        # fp8 forward (06:609-614): e5m2 inputs, V transposed in memory
+        q8, k8 = q.detach().to(torch.float8_e5m2), k.detach().to(torch.float8_e5m2)
+        v8 = v.detach().permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2).to(torch.float8_e5m2)
+        for causal in (True, False):
+            fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
+            ms = quick(lambda: triton_amd.attention(q8, k8, v8, causal, sm))
+            tag = "causal" if causal else "noncausal"
+            extra[f"attn_fwd_fp8_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["fp8"], 4)}
         out["extra"] = extra
 
     if not args.no_cpu:

@@ -5,8 +5,9 @@ Tiled functions follow python/tutorials/06-fused-attention.py: `_attn_fwd` / `_a
 (:25-75, :98-187), `_attn_bwd_preprocess` (:190-204), `_attn_bwd_dkdv` (:208-257),
 `_attn_bwd_dq` (:261-305) and the driver `_attn_bwd` (:308-435), executed one program at a time
 like the interpreter's grid loop (python/triton/runtime/interpreter.py:1088-1092).  Inputs are
-float32 arrays [Z, H, N, D] holding values representable in `dtype` ('fp16' | 'bf16'); rounding
-points use formats.round_to(.., dtype).
+float32 arrays [Z, H, N, D] holding values representable in `dtype` ('fp16' | 'bf16', and for the
+forward also 'e5m2' | 'e4m3': the fp8 path of 06:66-67, :609-614); rounding points use
+formats.round_to(.., dtype).
 """
 from __future__ import annotations
 

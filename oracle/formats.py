@@ -131,6 +131,9 @@ def round_to(x: np.ndarray, dtype: str) -> np.ndarray:
         return round_bf16(x)
     if dtype == "fp32":
         return np.asarray(x, dtype=np.float32)
+    if dtype in FP8_FORMATS:
+        # `x.to(tl.float8e5)` / `.to(tl.float8e4nv)`: RTNE, saturating (see encode_fp8)
+        return fp8_table(dtype)[encode_fp8(np.asarray(x, dtype=np.float32), dtype)].astype(np.float32)
     raise ValueError(dtype)
 
 

@@ -203,6 +203,22 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
                    float sm_scale, int causal, int dtype, void* stream_) {
   if (!q || !k || !v || !o || !Mlse) return MI355_EINVAL;
   AttnArgs p{};
+  if (dtype == MI355_F8E5M2 || dtype == MI355_F8E4M3) {
+    // fp8 forward: q, k, o with D contiguous, v with N_CTX contiguous (transposed in memory)
+    int rc8 = attn_common(p, Z, H, N_CTX, D, MI355_F16);
+    if (rc8) return rc8;
+    if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))
+      return MI355_EINVAL;
+    auto rows16 = [&](const int64_t* s, const void* ptr) {
+      return s[3] == 1 && s[2] >= D && s[0] % 16 == 0 && s[1] % 16 == 0 && s[2] % 16 == 0 && aligned(ptr, 16);
+    };
+    if (!rows16(p.sq, q) || !rows16(p.sk, k) || !rows16(p.so, o)) return MI355_ESTRIDE;
+    if (!(p.sv[2] == 1 && p.sv[3] >= N_CTX && p.sv[0] % 16 == 0 && p.sv[1] % 16 == 0 && p.sv[3] % 16 == 0 && aligned(v, 16)))
+      return MI355_ESTRIDE;
+    p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
+    p.sm_scale = sm_scale; p.causal = causal != 0;
+    return attn_fwd8_launch(p, dtype == MI355_F8E5M2, (hipStream_t)stream_);
+  }
   int rc = attn_common(p, Z, H, N_CTX, D, dtype);
   if (rc) return rc;
   if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))

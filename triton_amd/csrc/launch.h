@@ -65,6 +65,7 @@ int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int attn_fwd8_launch(const AttnArgs& p, bool e5m2, hipStream_t stream);  // fp8 inputs, V with N contiguous
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int dequant_launch(const uint8_t* codes, float* out, int64_t n, int fmt, hipStream_t stream);

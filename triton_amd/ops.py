@@ -231,6 +231,10 @@ class _attention(torch.autograd.Function):
             _check_device(i, t)
         assert q.dtype == k.dtype == v.dtype, "q, k, v must share a dtype"
         dt = _abi_dtype(q)
+        if dt in (_lib.F8E4M3, _lib.F8E5M2):
+            # the reference passes V transposed in memory for fp8 (06:609-614) and has no fp8 backward
+            assert v.stride(2) == 1, "fp8 attention takes v transposed in memory: v.permute(0,1,3,2).contiguous().permute(0,1,3,2)"
+            assert not (q.requires_grad or k.requires_grad or v.requires_grad), "fp8 attention is forward only"
         o = torch.empty_like(q)
         Z, H, N_CTX = q.shape[0], q.shape[1], q.shape[2]
         M = torch.empty((Z, H, N_CTX), device=q.device, dtype=torch.float32)
