@@ -104,8 +104,9 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
   const bool b_nmajor = !is8 && sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
-  // byte offsets inside one operand must fit the 32-bit-safe pointer arithmetic of the tile copies
-  const bool fast = out_ok && a_ok && (b_kmajor || b_nmajor) && env_int("MI355_GEMM_FORCE_STRIDED", 0) == 0;
+  // the tile copies address 256 rows of an operand with 32-bit byte offsets from a 64-bit tile base
+  const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
+  const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && env_int("MI355_GEMM_FORCE_STRIDED", 0) == 0;
 
   if (!fast) {
     GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype};
@@ -160,6 +161,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   const int64_t row_bytes = fmt == MI355_MXFP4 ? K / 2 : K;
   if (lda < row_bytes || ldb < row_bytes || lds_a < K / 32 || lds_b < K / 32 || ldc < N) return MI355_ESTRIDE;
   if (lda % 16 || ldb % 16 || !aligned(A, 16) || !aligned(B, 16)) return MI355_ESTRIDE;
+  if (lda >= (1 << 23) || ldb >= (1 << 23)) return MI355_ESTRIDE;  // 32-bit offsets inside a 256-row tile
   GemmArgs p{};
   p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C;
   p.M = M; p.N = N; p.K = K; p.k_bytes = (int)row_bytes;

@@ -53,6 +53,18 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds
 #endif
 }
 
+// The same copy with the global address split into a wave-uniform 64-bit base (scalar registers)
+// and a 32-bit per-lane byte offset: the address add happens in the memory pipeline instead of
+// costing a 64-bit vector add per load.  `lds_wave_base` must be wave-uniform.  The load is
+// invisible to the compiler's wait-count bookkeeping: callers wait with wait_vmcnt<>.
+__device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned lane_off, unsigned lds_wave_base) {
+#if MI355_DEVICE_PASS
+  // one idle issue slot between the M0 write and the LDS-DMA instruction that reads it
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+               :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base) : "memory");
+#endif
+}
+
 // 4 bytes per lane, same addressing: lane i writes lds_wave_base + 4 * i.
 __device__ __forceinline__ void async_copy4(const void* gsrc, LDS_PTR(void) lds_wave_base) {
 #if MI355_DEVICE_PASS

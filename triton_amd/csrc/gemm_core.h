@@ -735,7 +735,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS destinations of the direct loads are scalar math
   const int wm = wave / WN, wn = wave % WN;
 
   const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
@@ -744,25 +745,29 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
   const int m0 = pm * BM, n0 = pn * BN;
 
-  const char* srcA[ITA];
-  const char* srcB[ITB];
+  // Sources of the direct loads: a scalar tile base that advances with kt plus a 32-bit per-lane
+  // offset that never changes (the host keeps 256 rows of either operand within 2^31 bytes), so a
+  // load costs no vector arithmetic.
+  const char* const baseA = p.A + (int64_t)m0 * p.lda;
+  const char* const baseB = B_KMAJOR ? p.B + (int64_t)n0 * p.ldb : p.B + (int64_t)n0 * 2;
+  unsigned offGA[ITA], offGB[ITB];
 #pragma unroll
   for (int i = 0; i < ITA; i++) {
     int r = CopyA::row(wave, lane, i);
-    int gr = min(m0 + r, p.M - 1);
-    srcA[i] = p.A + (int64_t)gr * p.lda + CopyA::chunk(lane, r) * 16;
+    int gr = min(m0 + r, p.M - 1) - m0;
+    offGA[i] = (unsigned)gr * (unsigned)p.lda + CopyA::chunk(lane, r) * 16;
   }
 #pragma unroll
   for (int i = 0; i < ITB; i++) {
     if constexpr (B_KMAJOR) {
       int r = CopyBk::row(wave, lane, i);
-      int gr = min(n0 + r, p.N - 1);
-      srcB[i] = p.B + (int64_t)gr * p.ldb + CopyBk::chunk(lane, r) * 16;
+      int gr = min(n0 + r, p.N - 1) - n0;
+      offGB[i] = (unsigned)gr * (unsigned)p.ldb + CopyBk::chunk(lane, r) * 16;
     } else {
       int r = CopyBn::row(wave, lane, i);
       int n = n0 + CopyBn::col16(lane, r) * 8;
-      n = n < p.N ? n : p.N - 8;
-      srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
+      n = (n < p.N ? n : p.N - 8) - n0;
+      offGB[i] = (unsigned)r * (unsigned)p.ldb + (unsigned)n * 2;
     }
   }
   const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
@@ -781,10 +786,10 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   auto issue_one = [&](auto I_, int kt, LDS_PTR(char) a) {
     constexpr int i = decltype(I_)::value;
     if constexpr (i < ITA) {
-      async_copy16(srcA[i] + kt * stepA, (LDS_PTR(void))(a + (i * NW + wave) * 1024));
+      async_copy16_sbase(baseA + kt * stepA, offGA[i], lds_addr(a) + (i * NW + wave) * 1024);
     } else {
       constexpr int ib = i - ITA;
-      async_copy16(srcB[ib] + kt * stepB, (LDS_PTR(void))(a + A_BYTES + (ib * NW + wave) * 1024));
+      async_copy16_sbase(baseB + kt * stepB, offGB[ib], lds_addr(a) + A_BYTES + (ib * NW + wave) * 1024);
     }
   };
   // scale group sg (the 16 scale bytes per row of K steps sg*SPG ..) into ring slot sg % 2: one
@@ -844,32 +849,51 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // LDS reads of half H of a tile with parity P: A operands, then (K-split: always, M-split: with
   // the first half) the B operands, then with the first half the scale dwords
   auto n_reads = [](int H) constexpr { return AH + ((KSPLIT || H == 0) ? NT : 0) + ((Cfg::kScaled && H == 0) ? MT + NT : 0); };
-  auto read_one = [&](auto R_, auto H_, auto P_, unsigned base, unsigned scbase) {
+  // Operand addresses carry the stage as an instruction immediate: the 16-bit offset field reaches
+  // two stages, so there are two copies of the per-lane offsets (stages 0-1 and 2-3) and the K loop
+  // is unrolled over the ring.
+  static_assert(NS == 4 && 2 * STAGE + 3 * 32 * RBK + 16 * BN * 2 + 4 * BN * 2 < 65536 + STAGE, "stage immediates");
+  const unsigned lds0 = lds_addr(lds);
+  unsigned adrA[2][KS][NC], adrB[2][KS][NC], adrBn[2][NT];
+#pragma unroll
+  for (int hi = 0; hi < 2; hi++) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++)
+#pragma unroll
+      for (int c = 0; c < NC; c++) {
+        adrA[hi][ks][c] = lds0 + hi * 2 * STAGE + offA[ks][c];
+        adrB[hi][ks][c] = lds0 + hi * 2 * STAGE + offB[ks][c];
+      }
+#pragma unroll
+    for (int t = 0; t < NT; t++) adrBn[hi][t] = lds0 + hi * 2 * STAGE + offBn[t];
+  }
+  auto read_one = [&](auto R_, auto H_, auto P_, auto STG_, unsigned scbase) {
     constexpr int r = decltype(R_)::value, H = decltype(H_)::value, P = decltype(P_)::value;
+    constexpr int hi = decltype(STG_)::value >> 1, SO = (decltype(STG_)::value & 1) * STAGE;
     constexpr int ks = KSPLIT ? H : 0, aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P;
     constexpr int nb = (KSPLIT || H == 0) ? NT : 0;
     if constexpr (r < AH) {
       constexpr int t = (KSPLIT ? 0 : H * AH) + r;
       if constexpr (NC == 1) {
-        fa[aset][t] = __builtin_bit_cast(Operand, lds_read_b128<t * 32 * RBK>(base + offA[ks][0]));
+        fa[aset][t] = __builtin_bit_cast(Operand, lds_read_b128<SO + t * 32 * RBK>(adrA[hi][ks][0]));
       } else {
-        i32x4 lo = lds_read_b128<t * 32 * RBK>(base + offA[ks][0]);
-        i32x4 hi = lds_read_b128<t * 32 * RBK>(base + offA[ks][1]);
-        fa[aset][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        i32x4 lo4 = lds_read_b128<SO + t * 32 * RBK>(adrA[hi][ks][0]);
+        i32x4 hi4 = lds_read_b128<SO + t * 32 * RBK>(adrA[hi][ks][1]);
+        fa[aset][t] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     } else if constexpr (r < AH + nb) {
       constexpr int u = r - AH;
       if constexpr (!B_KMAJOR) {
-        constexpr int imm = ks * 16 * BN * 2;
-        i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[u]);
-        i32x2 hi = lds_read_tr16_b64<imm + 4 * BN * 2>(base + offBn[u]);
-        fb[bset][u] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo, hi, 0, 1, 2, 3));
+        constexpr int imm = SO + ks * 16 * BN * 2;
+        i32x2 lo2 = lds_read_tr16_b64<imm>(adrBn[hi][u]);
+        i32x2 hi2 = lds_read_tr16_b64<imm + 4 * BN * 2>(adrBn[hi][u]);
+        fb[bset][u] = __builtin_bit_cast(Operand, (i32x4)__builtin_shufflevector(lo2, hi2, 0, 1, 2, 3));
       } else if constexpr (NC == 1) {
-        fb[bset][u] = __builtin_bit_cast(Operand, lds_read_b128<u * 32 * RBK>(base + offB[ks][0]));
+        fb[bset][u] = __builtin_bit_cast(Operand, lds_read_b128<SO + u * 32 * RBK>(adrB[hi][ks][0]));
       } else {
-        i32x4 lo = lds_read_b128<u * 32 * RBK>(base + offB[ks][0]);
-        i32x4 hi = lds_read_b128<u * 32 * RBK>(base + offB[ks][1]);
-        fb[bset][u] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+        i32x4 lo4 = lds_read_b128<SO + u * 32 * RBK>(adrB[hi][ks][0]);
+        i32x4 hi4 = lds_read_b128<SO + u * 32 * RBK>(adrB[hi][ks][1]);
+        fb[bset][u] = __builtin_bit_cast(Operand, (i32x8)__builtin_shufflevector(lo4, hi4, 0, 1, 2, 3, 4, 5, 6, 7));
       }
     } else {
       constexpr int t = r - AH - nb;
@@ -939,28 +963,25 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   __builtin_amdgcn_sched_barrier(0);
   block_barrier();
   __builtin_amdgcn_sched_barrier(0);
-  static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(lds), lds_addr(sc_ring)); });
+  static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(sc_ring)); });
 
-  int stage = 0;
-  // one K step of a tile with parity P
-  auto step = [&](int kt, auto P_) {
-    constexpr int P = decltype(P_)::value;
+  // one K step of the tile in ring stage STG (its parity, for the one-sub-step types, is STG % 2)
+  auto step = [&](int kt, auto STG_) {
+    constexpr int stage = decltype(STG_)::value, P = stage & 1;
     using H0 = std::integral_constant<int, 0>;
     using H1 = std::integral_constant<int, 1>;
+    using P_ = std::integral_constant<int, P>;
     using PN = std::integral_constant<int, P ^ 1>;
-    const int next_stage = stage + 1 == NS ? 0 : stage + 1;
+    using SN = std::integral_constant<int, (stage + 1) % NS>;
     // ---- first half: multiply it, fetch the second half of the same tile
-    settle(H0{}, P_, kt);
-    {
-      const unsigned base = lds_addr(lds + stage * STAGE);
-      half(H0{}, P_, std::integral_constant<int, n_reads(1)>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
-        read_one(OP_, H1{}, P_, base, 0u);
-      });
-    }
+    settle(H0{}, P_{}, kt);
+    half(H0{}, P_{}, std::integral_constant<int, n_reads(1)>{}, std::integral_constant<int, 0>{}, [&](auto OP_) {
+      read_one(OP_, H1{}, P_{}, STG_, 0u);
+    });
     // ---- second half: every wave holds the whole of tile kt in registers and has seen its own
     //      share of tile kt+1 arrive (NS-2 younger shares stay in flight); after the barrier the
     //      stage of tile kt is refilled with tile kt+NS and the first half of tile kt+1 is fetched
-    settle(H1{}, P_, kt);
+    settle(H1{}, P_{}, kt);
     wait_vmcnt<(NS - 2) * kShare>();
     __builtin_amdgcn_sched_barrier(0);
     block_barrier();
@@ -974,25 +995,21 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     {
       const int ktn = kt + 1;
       const unsigned scbase = lds_addr(sc_ring) + ((ktn / SPG) & 1) * SC_SLOT + Cfg::scale_dword_offset(ktn % SPG);
-      const unsigned base = lds_addr(lds + next_stage * STAGE);
       LDS_PTR(char) const fill = lds + stage * STAGE;
       const int kfill = min(kt + NS, nfull - 1);
       constexpr int nr = n_reads(0);
-      half(H1{}, P_, std::integral_constant<int, nr>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
+      half(H1{}, P_{}, std::integral_constant<int, nr>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
         constexpr int op = decltype(OP_)::value;
-        if constexpr (op < nr) read_one(OP_, H0{}, PN{}, base, scbase);
+        if constexpr (op < nr) read_one(OP_, H0{}, PN{}, SN{}, scbase);
         else issue_one(std::integral_constant<int, op - nr>{}, kfill, fill);
       });
     }
-    stage = next_stage;
   };
-  if constexpr (KSPLIT) {
-    for (int kt = 0; kt < nfull; kt++) step(kt, std::integral_constant<int, 0>{});
-  } else {
-    for (int kt = 0; kt < nfull; kt += 2) {
-      step(kt, std::integral_constant<int, 0>{});
-      if (kt + 1 < nfull) step(kt + 1, std::integral_constant<int, 1>{});
-    }
+  for (int kt = 0; kt < nfull; kt += NS) {
+    step(kt, std::integral_constant<int, 0>{});
+    if (kt + 1 < nfull) step(kt + 1, std::integral_constant<int, 1>{});
+    if (kt + 2 < nfull) step(kt + 2, std::integral_constant<int, 2>{});
+    if (kt + 3 < nfull) step(kt + 3, std::integral_constant<int, 3>{});
   }
   // nothing may still be writing this workgroup's LDS when it retires
   wait_all();

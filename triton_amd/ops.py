@@ -133,6 +133,13 @@ def matmul_like_input(a, b):
     return c
 
 
+def matmul_persistent(a, b):
+    """`matmul_persistent(a, b)` of the same tutorial (09:190-224): there, NUM_SMS programs walk the
+    tiles; here the schedule is the library's own (one workgroup per 256x256 tile fills the 256 CUs
+    in whole rounds at these sizes) and the result is the same `a @ b` in the input dtype."""
+    return matmul_like_input(a, b)
+
+
 def group_gemm_fn(group_A, group_B, *, num_programs: int = 0):
     """The reference's `group_gemm_fn(group_A, group_B)` (python/tutorials/08-grouped-gemm.py:143-187):
     `[A_i @ B_i for i]` in one launch.  Builds the same five device tables (matrix addresses,
