@@ -42,7 +42,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][K tile | V tile]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
 
   // block -> (head, query block): consecutive logical ids (same XCD) walk the query blocks of
@@ -72,21 +73,24 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     for (int ks = 0; ks < KSQ; ks++) qf[b][ks] = *(const V8*)(src + ks * 32);
   }
 
-  // ---- direct global -> LDS copies of the K and V tiles
-  const char* srcK[INST];
-  const char* srcV[INST];
+  // ---- direct global -> LDS copies of the K and V tiles: a scalar tile base that advances with
+  // the step plus a 32-bit per-lane offset (64 rows of K or V span less than 2^31 bytes, which the
+  // host checks), so a load costs no vector arithmetic
+  unsigned offK[INST], offV[INST];
 #pragma unroll
   for (int i = 0; i < INST; i++) {
-    srcK[i] = Tile::src(kbase, kpitch, wave, lane, i);
-    srcV[i] = Tile::src(vbase, vpitch, wave, lane, i);
+    offK[i] = (unsigned)Tile::off(kpitch, wave, lane, i);
+    offV[i] = (unsigned)Tile::off(vpitch, wave, lane, i);
   }
+  const unsigned lds_base = lds_addr(lds);
   auto issue_kv = [&](int j, int stage) {
-    LDS_PTR(char) kd = lds + stage * (2 * TILE);
-    LDS_PTR(char) vd = kd + TILE;
+    const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
+    const char* ksrc = kbase + (int64_t)j * BN * kpitch;
+    const char* vsrc = vbase + (int64_t)j * BN * vpitch;
 #pragma unroll
     for (int i = 0; i < INST; i++) {
-      async_copy16(srcK[i] + (int64_t)j * BN * kpitch, (LDS_PTR(void))(kd + (i * NW + wave) * 1024));
-      async_copy16(srcV[i] + (int64_t)j * BN * vpitch, (LDS_PTR(void))(vd + (i * NW + wave) * 1024));
+      async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
+      async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
     }
   };
 
@@ -297,8 +301,10 @@ static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
 template <typename V8>
 static int launch_fwd_d(const AttnArgs& p, int variant, hipStream_t stream) {
   if (p.D == 128) {
+    if (variant == 2) return launch_fwd<V8, 128, 1, 8>(p, stream);
     return variant == 1 ? launch_fwd<V8, 128, 1, 4>(p, stream) : launch_fwd<V8, 128, 2, 4>(p, stream);
   }
+  if (variant == 2) return launch_fwd<V8, 64, 1, 8>(p, stream);
   return variant == 1 ? launch_fwd<V8, 64, 1, 4>(p, stream) : launch_fwd<V8, 64, 2, 4>(p, stream);
 }
 

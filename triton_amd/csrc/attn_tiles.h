@@ -43,10 +43,14 @@ struct AttnTile {
   static constexpr int BYTES = ROWS * RB;
   static constexpr int INST = BYTES / 1024 / NW;
   static_assert(INST >= 1, "tile too small for this wave count");
-  __device__ static const char* src(const char* base, int64_t pitch, int wave, int lane, int i) {
+  // byte offset of the lane's source chunk from the tile's first row
+  __device__ static int64_t off(int64_t pitch, int wave, int lane, int i) {
     int r = (i * NW + wave) * RPI + lane / CPR;
     int lc = (lane % CPR) ^ tile_swz<RB>(r);
-    return base + (int64_t)r * pitch + lc * 16;
+    return (int64_t)r * pitch + lc * 16;
+  }
+  __device__ static const char* src(const char* base, int64_t pitch, int wave, int lane, int i) {
+    return base + off(pitch, wave, lane, i);
   }
 };
 

@@ -196,7 +196,8 @@ static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype) {
 }
 
 static bool attn_stride_ok(const int64_t* s, const void* ptr, int D) {
-  return s[3] == 1 && s[2] >= D && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && aligned(ptr, 16);
+  // rows at most 2^24 elements apart: the kernels address 64 rows of a tile with 32-bit byte offsets
+  return s[3] == 1 && s[2] >= D && s[2] < (1 << 24) && s[0] % 8 == 0 && s[1] % 8 == 0 && s[2] % 8 == 0 && aligned(ptr, 16);
 }
 
 int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* Mlse,
@@ -230,7 +231,9 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     return MI355_ESTRIDE;
   p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
   p.sm_scale = sm_scale; p.causal = causal != 0;
-  p.variant = env_int("MI355_ATTN_FWD_VARIANT", 1);
+  // eight waves (256 query rows) per K/V stream halve the L2 -> LDS traffic; under the causal mask
+  // the uneven row ranges of eight waves cost as much as that saves, so four waves stay
+  p.variant = env_int("MI355_ATTN_FWD_VARIANT", causal ? 1 : 2);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 
