@@ -55,19 +55,22 @@ def test_forward_backward_against_oracle(gpu, dtype, causal, shape):
     assert np.allclose(o, ro, atol=tol, rtol=1e-2)
 
 
+@pytest.mark.parametrize("n_ctx", [512, 384])
 @pytest.mark.parametrize("causal", [True, False])
-def test_forward_variants_and_lse(gpu, causal, monkeypatch):
+def test_forward_variants_and_lse(gpu, causal, n_ctx, monkeypatch):
     # M = m + log2(l) (06:183-185) is what the backward consumes: check it directly through the C ABI
     from triton_amd import _lib
-    (q, k, v, _), (tq, tk, tv, _) = _inputs(3, (2, 2, 512, 128), "bf16", gpu)
+    (q, k, v, _), (tq, tk, tv, _) = _inputs(3, (2, 2, n_ctx, 128), "bf16", gpu)
     cf = A.attn_closed_form(q, k, v, causal, 0.125)
-    for variant in ("0", "1"):
+    # 0: 64 query rows per wave, 1: four waves of 32 rows, 2: eight waves of 32 rows (n_ctx = 384 leaves
+    # half of its second 256-row block empty)
+    for variant in ("0", "1", "2"):
         monkeypatch.setenv("MI355_ATTN_FWD_VARIANT", variant)
         o = torch.empty_like(tq)
-        M = torch.empty(2, 2, 512, dtype=torch.float32, device=gpu)
+        M = torch.empty(2, 2, n_ctx, dtype=torch.float32, device=gpu)
         I4 = _lib.I64x4
         rc = _lib.load().mi355_attn_fwd(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(), M.data_ptr(),
-                                        2, 2, 512, 128, I4(*tq.stride()), I4(*tk.stride()), I4(*tv.stride()), I4(*o.stride()),
+                                        2, 2, n_ctx, 128, I4(*tq.stride()), I4(*tk.stride()), I4(*tv.stride()), I4(*o.stride()),
                                         0.125, int(causal), _lib.BF16, torch.cuda.current_stream().cuda_stream)
         assert rc == 0
         assert np.allclose(to_np(M), cf["M"], atol=2e-3, rtol=0)

@@ -69,7 +69,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][K tile | V tile]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
 
   const int nqb = (p.N + BM - 1) / BM;
@@ -103,20 +104,19 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     d_row[b] = p.delta[(int64_t)hz * p.N + r];
   }
 
-  const char* srcK[Tile::INST];
-  const char* srcV[Tile::INST];
+  // direct loads: scalar tile base + 32-bit lane offset (the host bounds the row pitch)
+  unsigned offKV[Tile::INST];
 #pragma unroll
-  for (int i = 0; i < Tile::INST; i++) {
-    srcK[i] = Tile::src(kbase, pitch, wave, lane, i);
-    srcV[i] = Tile::src(vbase, pitch, wave, lane, i);
-  }
+  for (int i = 0; i < Tile::INST; i++) offKV[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+  const unsigned lds_base = lds_addr(lds);
   auto issue_kv = [&](int j, int stage) {
-    LDS_PTR(char) kd = lds + stage * (2 * TILE);
-    LDS_PTR(char) vd = kd + TILE;
+    const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
+    const char* ksrc = kbase + (int64_t)j * BN * pitch;
+    const char* vsrc = vbase + (int64_t)j * BN * pitch;
 #pragma unroll
     for (int i = 0; i < Tile::INST; i++) {
-      async_copy16(srcK[i] + (int64_t)j * BN * pitch, (LDS_PTR(void))(kd + (i * NW + wave) * 1024));
-      async_copy16(srcV[i] + (int64_t)j * BN * pitch, (LDS_PTR(void))(vd + (i * NW + wave) * 1024));
+      async_copy16_sbase(ksrc, offKV[i], kd + (i * NW + wave) * 1024);
+      async_copy16_sbase(vsrc, offKV[i], vd + (i * NW + wave) * 1024);
     }
   };
 

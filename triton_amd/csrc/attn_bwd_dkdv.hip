@@ -78,25 +78,27 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   const int nsteps = (p.N - m_begin + BM - 1) / BM;
   const int ncol = nrow0 + l32;  // this lane's key row
 
-  const char* srcQ[Tile::INST];
-  const char* srcD[Tile::INST];
+  // direct loads: scalar tile base + 32-bit lane offset (the host bounds the row pitch)
+  unsigned offQD[Tile::INST];
 #pragma unroll
-  for (int i = 0; i < Tile::INST; i++) {
-    srcQ[i] = Tile::src(qbase, pitch, wave, lane, i) + (int64_t)m_begin * pitch;
-    srcD[i] = Tile::src(dobase, pitch, wave, lane, i) + (int64_t)m_begin * pitch;
-  }
+  for (int i = 0; i < Tile::INST; i++) offQD[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+  const char* const qsrc0 = qbase + (int64_t)m_begin * pitch;
+  const char* const dsrc0 = dobase + (int64_t)m_begin * pitch;
+  const unsigned lds_base = lds_addr(lds);
   // even waves copy the stage's 64 M values, odd waves its 64 deltas (4 bytes per lane; the
   // duplicates keep the number of loads per wave uniform for the partial waits)
   const float* src_stat = ((wave & 1) == 0 ? lse : delta) + m_begin + lane;
   // stage-step js (clamped to the last one) into ring slot js % NS
   auto issue_stage = [&](int js) {
     LDS_PTR(char) qd = lds + (js % NS) * STAGE;
-    LDS_PTR(char) dd = qd + TILE;
+    const unsigned qda = lds_base + (js % NS) * STAGE, dda = qda + TILE;
     const int jc = min(js, nsteps - 1);
+    const char* qsrc = qsrc0 + (int64_t)jc * BM * pitch;
+    const char* dsrc = dsrc0 + (int64_t)jc * BM * pitch;
 #pragma unroll
     for (int i = 0; i < Tile::INST; i++) {
-      async_copy16(srcQ[i] + (int64_t)jc * BM * pitch, (LDS_PTR(void))(qd + (i * NW + wave) * 1024));
-      async_copy16(srcD[i] + (int64_t)jc * BM * pitch, (LDS_PTR(void))(dd + (i * NW + wave) * 1024));
+      async_copy16_sbase(qsrc, offQD[i], qda + (i * NW + wave) * 1024);
+      async_copy16_sbase(dsrc, offQD[i], dda + (i * NW + wave) * 1024);
     }
     async_copy4(src_stat + jc * BM, (LDS_PTR(void))(qd + 2 * TILE + (wave & 1) * (BM * 4)));
   };

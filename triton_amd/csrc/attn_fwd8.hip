@@ -97,27 +97,27 @@ __global__ __launch_bounds__(256, 2) void attn_fwd8_kernel(AttnArgs p) {
   auto vswz8 = [](int row) { return (row >> 2) & 3; };
 
   // direct loads: one wave instruction moves 1 KiB = 1024/D K rows or 16 V^T rows
-  const char* srcK[KINST];
-  const char* srcV[VINST];
+  // (scalar tile base + 32-bit lane offset: the host bounds the row pitches)
+  unsigned offK[KINST], offV[VINST];
 #pragma unroll
   for (int i = 0; i < KINST; i++) {
     const int r = (i * NW + wave) * (1024 / D) + lane / KCH;
-    srcK[i] = kbase + (int64_t)r * kpitch + (((lane % KCH) ^ kswz8(r)) << 4);
+    offK[i] = (unsigned)(r * kpitch) + (((lane % KCH) ^ kswz8(r)) << 4);
   }
 #pragma unroll
   for (int i = 0; i < VINST; i++) {
     const int r = (i * NW + wave) * 16 + lane / 4;   // d row
-    srcV[i] = vbase + (int64_t)r * vpitch + (((lane % 4) ^ vswz8(r)) << 4);
+    offV[i] = (unsigned)(r * vpitch) + (((lane % 4) ^ vswz8(r)) << 4);
   }
+  const unsigned lds_base = lds_addr(lds);
   auto issue_kv = [&](int j, int stage) {
-    LDS_PTR(char) kd = lds + stage * STAGE;
-    LDS_PTR(char) vd = kd + KTILE;
+    const unsigned kd = lds_base + stage * STAGE, vd = kd + KTILE;
+    const char* ksrc = kbase + (int64_t)j * BN * kpitch;
+    const char* vsrc = vbase + (int64_t)j * BN;
 #pragma unroll
-    for (int i = 0; i < KINST; i++)
-      async_copy16(srcK[i] + (int64_t)j * BN * kpitch, (LDS_PTR(void))(kd + (i * NW + wave) * 1024));
+    for (int i = 0; i < KINST; i++) async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
 #pragma unroll
-    for (int i = 0; i < VINST; i++)
-      async_copy16(srcV[i] + (int64_t)j * BN, (LDS_PTR(void))(vd + (i * NW + wave) * 1024));
+    for (int i = 0; i < VINST; i++) async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
   };
 
   // per-lane LDS offsets.  K operand of tile row l32 = 8a + 4b + e is key row 16b + 4a + e

@@ -213,10 +213,10 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))
       return MI355_EINVAL;
     auto rows16 = [&](const int64_t* s, const void* ptr) {
-      return s[3] == 1 && s[2] >= D && s[0] % 16 == 0 && s[1] % 16 == 0 && s[2] % 16 == 0 && aligned(ptr, 16);
+      return s[3] == 1 && s[2] >= D && s[2] < (1 << 24) && s[0] % 16 == 0 && s[1] % 16 == 0 && s[2] % 16 == 0 && aligned(ptr, 16);
     };
     if (!rows16(p.sq, q) || !rows16(p.sk, k) || !rows16(p.so, o)) return MI355_ESTRIDE;
-    if (!(p.sv[2] == 1 && p.sv[3] >= N_CTX && p.sv[0] % 16 == 0 && p.sv[1] % 16 == 0 && p.sv[3] % 16 == 0 && aligned(v, 16)))
+    if (!(p.sv[2] == 1 && p.sv[3] >= N_CTX && p.sv[3] < (1 << 24) && p.sv[0] % 16 == 0 && p.sv[1] % 16 == 0 && p.sv[3] % 16 == 0 && aligned(v, 16)))
       return MI355_ESTRIDE;
     p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
     p.sm_scale = sm_scale; p.causal = causal != 0;
