@@ -252,3 +252,42 @@ def test_decode_shape_m16(gpu):
     c = to_np(triton_amd.matmul(torch.from_numpy(ca).to(gpu).view(torch.float8_e4m3fn),
                                 torch.from_numpy(cb).to(gpu).view(torch.float8_e4m3fn).t(), out_dtype=torch.bfloat16))
     assert np.allclose(c, ref, rtol=3e-2, atol=3e-2)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(16, 256, 512), (64, 128, 1024), (33, 96, 64), (1, 32, 32), (7, 2048, 4096),
+                                   (256, 64, 512), (128, 32, 256), (1024, 16, 2048), (96, 40, 96)])
+def test_skinny_16bit_kernel_is_bit_exact_on_integers(gpu, monkeypatch, dtype, shape):
+    # at most 64 rows on one side (shapes of python/test/regression/test_performance.py:36-44): the
+    # streaming kernel (K split over the waves of a workgroup) for row-major and K-major B; M > 64
+    # with N <= 64 takes it with the operands swapped (a row-major B then needs N = 32 or 64; the
+    # other cases here fall through to the tile kernels).  Every partial sum is an exact integer,
+    # so the result does not depend on how K is split.
+    M, N, K = shape
+    rng = np.random.default_rng(M + 3 * N + 7 * K)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    ref = gemm.matmul_closed_form(a, b, out_dtype="fp32")
+    ta = from_np(a, dtype, gpu)
+    for tb in (from_np(b, dtype, gpu), from_np(np.ascontiguousarray(b.T), dtype, gpu).t()):
+        got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+        assert bits_equal(got, ref), (dtype, shape, tb.stride())
+        monkeypatch.setenv("MI355_GEMM_SKINNY", "0")      # the tile kernels on the same inputs
+        assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), ref)
+        monkeypatch.delenv("MI355_GEMM_SKINNY")
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_skinny_16bit_decode_shapes_against_closed_form(gpu, dtype):
+    # M = 16 and 64 against N = K = 4096, and the transposed 4096 x 64: random data, output in the
+    # input type, leaky-ReLU epilogue on one of them
+    rng = np.random.default_rng(21)
+    for (M, N, K), act in (((16, 4096, 4096), ""), ((64, 4096, 4096), "leaky_relu"), ((4096, 64, 4096), "")):
+        a = randn_rounded(rng, (M, K), dtype)
+        b = randn_rounded(rng, (K, N), dtype)
+        ref = gemm.matmul_closed_form(a, b, out_dtype=dtype, activation=act)
+        tb = from_np(b, dtype, gpu)
+        c = to_np(triton_amd.matmul(from_np(a, dtype, gpu), tb, activation=act))
+        assert np.allclose(c, ref, rtol=1e-2, atol=1e-2), (M, N, K, "row-major B")
+        c = to_np(triton_amd.matmul(from_np(a, dtype, gpu), tb.t().contiguous().t(), activation=act))
+        assert np.allclose(c, ref, rtol=1e-2, atol=1e-2), (M, N, K, "K-major B")

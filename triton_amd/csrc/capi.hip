@@ -130,6 +130,24 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   // large problems run the software-pipelined 8-wave kernel
   int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
+  if (!is8 && env_int("MI355_GEMM_SKINNY", 1)) {
+    // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
+    SkinnyArgs sk{};
+    sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
+    sk.activation = activation; sk.out_dtype = out_dtype;
+    bool use = false, y_kmajor = false, x_kmajor = true;
+    if (M <= 64) {
+      sk.X = (const char*)A; sk.Y = (const char*)B; sk.S = M; sk.L = N;
+      sk.x_pitch = p.lda; sk.y_pitch = p.ldb; sk.cs = scm; sk.cl = scn;
+      y_kmajor = b_kmajor; use = true;
+    } else if (N <= 64) {
+      sk.X = (const char*)B; sk.Y = (const char*)A; sk.S = N; sk.L = M;
+      sk.x_pitch = p.ldb; sk.y_pitch = p.lda; sk.cs = scn; sk.cl = scm;
+      y_kmajor = true; x_kmajor = b_kmajor; use = true;
+    }
+    if (use && gemm16_skinny_ok(sk, y_kmajor, x_kmajor))
+      return gemm16_skinny_launch(sk, in_dtype == MI355_BF16, y_kmajor, x_kmajor, stream);
+  }
   if (is8 && gemm8_skinny_ok(p) && env_int("MI355_GEMM_SKINNY", 1)) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);

@@ -65,6 +65,18 @@ __device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned l
 #endif
 }
 
+// 16 bytes per lane from (wave-uniform 64-bit base + 32-bit lane offset + immediate) into
+// registers, issued as inline assembly so that the compiler neither counts it nor waits for it:
+// for loops that keep many loads in flight and wait with wait_vmcnt<> by hand.  The result may be
+// used only after such a wait followed by lds_use() on the register.
+template <int OFF, typename V>
+__device__ __forceinline__ void load16_sbase(V& dst, const void* sbase, unsigned lane_off) {
+  static_assert(sizeof(V) == 16 && OFF >= 0 && OFF < 4096, "one 16-byte register group, 12-bit offset");
+#if MI355_DEVICE_PASS
+  asm volatile("global_load_dwordx4 %0, %1, %2 offset:%3" : "=v"(dst) : "v"(lane_off), "s"(sbase), "i"(OFF));
+#endif
+}
+
 // 4 bytes per lane, same addressing: lane i writes lds_wave_base + 4 * i.
 __device__ __forceinline__ void async_copy4(const void* gsrc, LDS_PTR(void) lds_wave_base) {
 #if MI355_DEVICE_PASS

@@ -1,0 +1,278 @@
+// Skinny fp16 / bf16 GEMM: one side of the product has at most 64 rows (decode-style M = 16..64,
+// or N <= 64), so the work is reading the other operand once from HBM
+// (shapes of python/test/regression/test_performance.py:36-44; kernel contract of
+// python/tutorials/03-matrix-multiplication.py:241-316).
+//
+// Written for out[s][l] = sum_k X[s][k] * Y[l][k]: X the small operand (S <= 64 rows), Y the
+// streamed one (L rows).  The host maps (A, B) or (B^T, A^T) onto (X, Y).
+//   * one workgroup per 32 rows of Y, its waves split K into contiguous ranges and meet in LDS at
+//     the end - no tile reuse to organise, what matters is bytes in flight: every wave keeps
+//     NS - 1 stages of 32 k (2 KiB of Y) outstanding;
+//   * Y with K contiguous: each lane streams its own row straight into MFMA operand registers;
+//   * Y with L contiguous (a row-major B): stages go global -> LDS by direct loads into a ring
+//     private to the wave (no barriers in the loop) and come back transposed (ds_read_b64_tr_b16);
+//   * X is re-read by every workgroup from L2, prefetched with the same depth through the same
+//     ring: read back row-wise when K is contiguous, transposed when S is (the row-major B of a
+//     product with N = 32 or 64).
+#include "common.h"
+#include "launch.h"
+
+namespace mi355 {
+
+template <typename V8, bool Y_LDS, int XM, int ST, int NW, int NS>
+__global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
+  constexpr int PD = NS - 1;          // stages in flight
+  constexpr int LPS = 2 + 2 * ST;     // vector-memory operations per stage: 2 of Y, 2 per 32 rows of X
+  // X: 0 = K contiguous, straight into registers (32-byte pieces of 32 rows per instruction: slower,
+  //        kept for comparison); 1 = S contiguous, through LDS with a transposed read;
+  //    2 = K contiguous, through LDS (64-byte pieces of 16 rows per instruction)
+  constexpr bool X_LDS = XM != 0;
+  static_assert(!(Y_LDS && XM == 1), "one operand at most is transposed through LDS");
+  constexpr int XROW = 64 * ST;       // bytes of one k row of an S-contiguous X tile: S = 32 ST
+  constexpr int YSLOT = Y_LDS ? 2048 : 0;        // [32 k][32 l] 16-bit
+  constexpr int XSLOT = X_LDS ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
+  constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
+  static_assert(PD * LPS < 64, "vmcnt has 6 bits");
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q = lane >> 4;
+  // neighbouring 32-column blocks (the two halves of a 128-byte line of an L-contiguous Y) on one XCD
+  const int l0 = xcd_remap(blockIdx.x, gridDim.x) * 32;
+
+  const int nstages = p.K / 32;
+  const int per = (nstages + NW - 1) / NW;
+  const int j_lo = wave * per, j_hi = min(nstages, j_lo + per);
+
+  f32x16 acc[ST];
+#pragma unroll
+  for (int t = 0; t < ST; t++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
+
+  // Every load is a wave-uniform base (advancing with the stage) plus a fixed 32-bit lane offset.
+  // lane (row l32, half g) feeds k = 16 ks + 8 g .. + 8 of MFMA sub-step ks
+  unsigned xoff[ST];
+#pragma unroll
+  for (int t = 0; t < ST; t++) xoff[t] = (unsigned)min(32 * t + l32, p.S - 1) * (unsigned)p.x_pitch + g * 16;
+  // S-contiguous X (x_pitch between k rows): direct load i of a stage moves k rows (16 / ST) i .. of XROW bytes
+  const unsigned xdma = (unsigned)(lane / (4 * ST)) * (unsigned)p.x_pitch + (lane % (4 * ST)) * 16;
+  // K-contiguous X through LDS: direct load i moves rows 16 i .. 16 i + 15, 64 bytes of k each; the
+  // 16-byte chunk c of row r sits at position c ^ ((r >> 2) & 3) so that row-wise reads spread over the banks
+  unsigned xdma2[2 * ST];
+#pragma unroll
+  for (int i = 0; i < 2 * ST; i++) {
+    const int r = 16 * i + (lane >> 2);
+    xdma2[i] = (unsigned)min(r, p.S - 1) * (unsigned)p.x_pitch + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+  }
+  // K-contiguous Y: the lane's own row
+  const char* const ybase = Y_LDS ? p.Y + (int64_t)l0 * 2 : p.Y + (int64_t)l0 * p.y_pitch;
+  // L-contiguous Y: direct load i of a stage moves k rows 16 i .. 16 i + 15, 64 bytes (32 l) each
+  const unsigned yoff = Y_LDS ? (unsigned)(lane >> 2) * (unsigned)p.y_pitch + (lane & 3) * 16
+                              : (unsigned)l32 * (unsigned)p.y_pitch + g * 16;
+  const unsigned ring = lds_addr(lds) + wave * (NS * SLOT);
+  // transposed read: 16 lanes fetch 4 k rows x 16 l and receive 4 k values of one l each;
+  // lane -> k row 8 g + i16 / 4 (+ 4 for the second read), l = 16 (q & 1) + i16
+  const unsigned tl = ring + (8 * (q >> 1) + (i16 >> 2)) * (XM == 1 ? XROW : 64) + (q & 1) * 32 + (i16 & 3) * 8;
+  // row-wise read of the K-contiguous X tile: row s = 32 t + l32, chunk (2 ks + g) ^ ((s >> 2) & 3)
+  unsigned xrd[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) xrd[ks] = ring + YSLOT + l32 * 64 + (((2 * ks + g) ^ ((l32 >> 2) & 3)) << 4);
+
+  V8 xr[NS][2][ST], yr[NS][2];
+  auto issue = [&](int j, auto SLOT_) {
+    constexpr int sl = decltype(SLOT_)::value;
+    if constexpr (Y_LDS) {
+      const char* src = ybase + (int64_t)j * 32 * p.y_pitch;
+      async_copy16_sbase(src, yoff, ring + sl * SLOT);
+      async_copy16_sbase(src + 16 * p.y_pitch, yoff, ring + sl * SLOT + 1024);
+    } else {
+      const char* src = ybase + (int64_t)j * 64;
+      load16_sbase<0>(yr[sl][0], src, yoff);
+      load16_sbase<32>(yr[sl][1], src, yoff);
+    }
+    if constexpr (XM == 1) {
+      const char* xsrc = p.X + (int64_t)j * 32 * p.x_pitch;
+#pragma unroll
+      for (int i = 0; i < 2 * ST; i++)
+        async_copy16_sbase(xsrc + (int64_t)i * (16 / ST) * p.x_pitch, xdma, ring + sl * SLOT + i * 1024);
+    } else if constexpr (XM == 2) {
+      const char* xsrc = p.X + (int64_t)j * 64;
+#pragma unroll
+      for (int i = 0; i < 2 * ST; i++) async_copy16_sbase(xsrc, xdma2[i], ring + sl * SLOT + YSLOT + i * 1024);
+    } else {
+      const char* xsrc = p.X + (int64_t)j * 64;
+#pragma unroll
+      for (int t = 0; t < ST; t++) {
+        load16_sbase<0>(xr[sl][0][t], xsrc, xoff[t]);
+        load16_sbase<32>(xr[sl][1][t], xsrc, xoff[t]);
+      }
+    }
+  };
+  auto compute = [&](auto SLOT_) {
+    constexpr int sl = decltype(SLOT_)::value;
+    V8 yf[2];
+    if constexpr (Y_LDS) {
+      i32x2 lo[2], hi[2];
+      lo[0] = lds_read_tr16_b64<sl * SLOT>(tl);
+      hi[0] = lds_read_tr16_b64<sl * SLOT + 4 * 64>(tl);
+      lo[1] = lds_read_tr16_b64<sl * SLOT + 16 * 64>(tl);
+      hi[1] = lds_read_tr16_b64<sl * SLOT + 20 * 64>(tl);
+      lds_wait<0>();
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++) {
+        lds_use(lo[ks]);
+        lds_use(hi[ks]);
+        yf[ks] = __builtin_bit_cast(V8, (i32x4)__builtin_shufflevector(lo[ks], hi[ks], 0, 1, 2, 3));
+      }
+    } else {
+      lds_use(yr[sl][0]);
+      lds_use(yr[sl][1]);
+      yf[0] = yr[sl][0];
+      yf[1] = yr[sl][1];
+    }
+    V8 xf[2][ST];
+    if constexpr (XM == 2) {
+      i32x4 xv[2][ST];
+      static_for<2>([&](auto KS_) {
+        constexpr int ks = decltype(KS_)::value;
+        static_for<ST>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          xv[ks][t] = lds_read_b128<sl * SLOT + t * 2048>(xrd[ks]);
+        });
+      });
+      lds_wait<0>();
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int t = 0; t < ST; t++) {
+          lds_use(xv[ks][t]);
+          xf[ks][t] = __builtin_bit_cast(V8, xv[ks][t]);
+        }
+    } else if constexpr (XM == 1) {
+      i32x2 lo[2][ST], hi[2][ST];
+      static_for<2>([&](auto KS_) {
+        constexpr int ks = decltype(KS_)::value;
+        static_for<ST>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          lo[ks][t] = lds_read_tr16_b64<sl * SLOT + 16 * ks * XROW + t * 64>(tl);
+          hi[ks][t] = lds_read_tr16_b64<sl * SLOT + (16 * ks + 4) * XROW + t * 64>(tl);
+        });
+      });
+      lds_wait<0>();
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int t = 0; t < ST; t++) {
+          lds_use(lo[ks][t]);
+          lds_use(hi[ks][t]);
+          xf[ks][t] = __builtin_bit_cast(V8, (i32x4)__builtin_shufflevector(lo[ks][t], hi[ks][t], 0, 1, 2, 3));
+        }
+    } else {
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int t = 0; t < ST; t++) {
+          lds_use(xr[sl][ks][t]);
+          xf[ks][t] = xr[sl][ks][t];
+        }
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+      for (int t = 0; t < ST; t++) acc[t] = mfma32(yf[ks], xf[ks][t], acc[t]);
+  };
+
+  if (j_lo < j_hi) {
+    // past the end of the range the last stage is fetched again: the number of outstanding
+    // operations, and with it the partial wait, stays uniform
+    static_for<PD>([&](auto S_) { issue(min(j_lo + decltype(S_)::value, j_hi - 1), S_); });
+    for (int j = j_lo; j < j_hi; j += NS) {
+      static_for<NS>([&](auto U_) {
+        constexpr int u = decltype(U_)::value;
+        if (j + u < j_hi) {
+          issue(min(j + u + PD, j_hi - 1), std::integral_constant<int, (u + PD) % NS>{});
+          wait_vmcnt<PD * LPS>();
+          __builtin_amdgcn_sched_barrier(0);
+          compute(U_);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      });
+    }
+    wait_vmcnt<0>();
+  }
+
+  // ---- sum the waves' partial tiles through LDS (the rings are dead after the barrier)
+  __syncthreads();
+  LDS_PTR(float) const red = (LDS_PTR(float))lds;  // [NW][ST * 16][64]
+#pragma unroll
+  for (int t = 0; t < ST; t++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) red[(wave * ST * 16 + t * 16 + r) * 64 + lane] = acc[t][r];
+  __syncthreads();
+  float alpha = 1.f;
+  if (p.a_scale) alpha *= *p.a_scale;
+  if (p.b_scale) alpha *= *p.b_scale;
+  constexpr int RPW = ST * 16 / NW;  // accumulator registers finished by each wave
+  static_assert(RPW >= 1, "more waves than accumulator registers");
+#pragma unroll
+  for (int e = 0; e < RPW; e++) {
+    const int rr = wave * RPW + e, t = rr >> 4, r = rr & 15;
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < NW; w++) v += red[(w * ST * 16 + rr) * 64 + lane];
+    v *= alpha;
+    if (p.activation == 1) v = v >= 0.f ? v : 0.01f * v;
+    // register r of lane: row l = 8 (r / 4) + 4 g + r % 4 of the tile, column s = l32
+    const int s = 32 * t + l32, l = l0 + (r >> 2) * 8 + g * 4 + (r & 3);
+    if (s < p.S && l < p.L) {
+      const int64_t off = (int64_t)s * p.cs + (int64_t)l * p.cl;
+      if (p.out_dtype == 4) ((float*)p.C)[off] = v;
+      else if (p.out_dtype == 1) ((__bf16*)p.C)[off] = (__bf16)v;
+      else ((_Float16*)p.C)[off] = (_Float16)v;
+    }
+  }
+}
+
+template <typename V8, bool Y_LDS, int XM, int ST>
+static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
+  // four waves with three stages in flight each already saturate what this access pattern gets
+  // from HBM; the small LDS footprint lets several workgroups share a CU
+  constexpr int NW = 4, NS = 4;
+  constexpr int ring = NW * NS * ((Y_LDS ? 2048 : 0) + (XM ? 2048 * ST : 0)), red = NW * ST * 16 * 64 * 4;
+  constexpr int smem = ring > red ? ring : red;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm16_skinny_kernel<V8, Y_LDS, XM, ST, NW, NS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  gemm16_skinny_kernel<V8, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+// S <= 64, whole 32-row blocks of Y and whole 32-k stages; pitches in bytes, 16-byte aligned rows,
+// small enough that 64 rows of X / 32 rows of Y are reached with 32-bit offsets.  An S-contiguous
+// X (x_kmajor false) needs S = 32 or 64 and a K-contiguous Y.
+bool gemm16_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor) {
+  if (!x_kmajor && (!y_kmajor || (p.S != 32 && p.S != 64))) return false;
+  return p.S >= 1 && p.S <= 64 && p.L >= 32 && p.L % 32 == 0 && p.K >= 32 && p.K % 32 == 0 &&
+         p.x_pitch % 16 == 0 && p.y_pitch % 16 == 0 && p.x_pitch < (1 << 25) && p.y_pitch < (1 << 26);
+}
+
+template <typename V8>
+static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
+  const bool two = p.S > 32;
+  if (!x_kmajor) return two ? launch_skinny<V8, false, 1, 2>(p, stream) : launch_skinny<V8, false, 1, 1>(p, stream);
+  if (y_kmajor) return two ? launch_skinny<V8, false, 2, 2>(p, stream) : launch_skinny<V8, false, 2, 1>(p, stream);
+  return two ? launch_skinny<V8, true, 2, 2>(p, stream) : launch_skinny<V8, true, 2, 1>(p, stream);
+}
+
+int gemm16_skinny_launch(const SkinnyArgs& p, bool bf16, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
+  return bf16 ? launch_skinny_v<bf16x8>(p, y_kmajor, x_kmajor, stream) : launch_skinny_v<f16x8>(p, y_kmajor, x_kmajor, stream);
+}
+
+}  // namespace mi355

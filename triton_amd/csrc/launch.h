@@ -36,6 +36,21 @@ struct GemmStridedArgs {
   int activation, in_dtype, out_dtype;
 };
 
+// skinny 16-bit GEMM, out[s][l] = sum_k X[s][k] * Y[l][k]
+struct SkinnyArgs {
+  const char* X;    // small operand: S <= 64 rows, K contiguous or S contiguous
+  const char* Y;    // streamed operand: L rows, K contiguous or L contiguous
+  char* C;
+  int S, L, K;
+  int64_t x_pitch;  // bytes between rows s (K contiguous) or between k rows (S contiguous)
+  int64_t y_pitch;  // bytes between rows l (K contiguous) or between k rows (L contiguous)
+  int64_t cs, cl;   // element strides of the output along s and l
+  const float* a_scale;
+  const float* b_scale;
+  int activation;
+  int out_dtype;
+};
+
 struct AttnArgs {
   const char* q; const char* k; const char* v; char* o; float* lse;
   const char* d_o; const float* delta; char* dq; char* dk; char* dv;
@@ -62,6 +77,8 @@ int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStre
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
 bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
 int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
+bool gemm16_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor);
+int gemm16_skinny_launch(const SkinnyArgs& p, bool bf16, bool y_kmajor, bool x_kmajor, hipStream_t stream);
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
