@@ -932,7 +932,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     constexpr int nreads = decltype(NREADS_)::value, nloads = decltype(NLOADS_)::value;
     constexpr int ks = KSPLIT ? H : 0, aset = KSPLIT ? H : 0, bset = KSPLIT ? H : P, alo = KSPLIT ? 0 : H * AH;
     constexpr int half_slots = (kMfmas + 1) / 2;
-    constexpr int rper = (nreads + half_slots - 1) / half_slots;
+    constexpr int rper = nreads == 0 ? 1 : (nreads + half_slots - 1) / half_slots;
     constexpr int rslots = (nreads + rper - 1) / rper;
     constexpr int lper = nloads == 0 ? 1 : (nloads + (kMfmas - rslots) - 1) / (kMfmas - rslots);
     static_for<kMfmas>([&](auto N_) {
@@ -1014,6 +1014,40 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // nothing may still be writing this workgroup's LDS when it retires
   wait_all();
 
+  // Last, partial K step (unscaled types only): its 16-byte chunks past K are written as zeros (the
+  // reference masks them to 0, python/tutorials/03-matrix-multiplication.py:297-298).  Goes through
+  // registers into stage 0 and is multiplied without overlap: one step out of K / 32.
+  if constexpr (!Cfg::kScaled) {
+    if (p.k_bytes % RBK != 0) {
+      using Z = std::integral_constant<int, 0>;
+      using O = std::integral_constant<int, 1>;
+      __syncthreads();  // every wave is done reading the ring
+      const int kbase = nfull * RBK;
+#pragma unroll
+      for (int i = 0; i < ITA; i++) {
+        const int r = CopyA::row(wave, lane, i);
+        i32x4 v = {0, 0, 0, 0};
+        if (kbase + CopyA::chunk(lane, r) * 16 < p.k_bytes) v = *(const i32x4*)(baseA + nfull * stepA + offGA[i]);
+        *(LDS_PTR(i32x4))(lds + (i * NW + wave) * 1024 + lane * 16) = v;
+      }
+#pragma unroll
+      for (int i = 0; i < ITB; i++) {
+        bool ok;
+        if constexpr (B_KMAJOR) ok = kbase + CopyBk::chunk(lane, CopyBk::row(wave, lane, i)) * 16 < p.k_bytes;
+        else ok = nfull * KROWS + CopyBn::row(wave, lane, i) < p.K;
+        i32x4 v = {0, 0, 0, 0};
+        if (ok) v = *(const i32x4*)(baseB + nfull * stepB + offGB[i]);
+        *(LDS_PTR(i32x4))(lds + A_BYTES + (i * NW + wave) * 1024 + lane * 16) = v;
+      }
+      __syncthreads();
+      static_for<n_reads(0)>([&](auto R_) { read_one(R_, Z{}, Z{}, Z{}, 0u); });
+      settle(Z{}, Z{}, nfull);
+      half(Z{}, Z{}, std::integral_constant<int, n_reads(1)>{}, Z{}, [&](auto OP_) { read_one(OP_, O{}, Z{}, Z{}, 0u); });
+      settle(O{}, Z{}, nfull);
+      half(O{}, Z{}, Z{}, Z{}, [&](auto) {});
+    }
+  }
+
   gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
 }
 
@@ -1075,7 +1109,8 @@ template <typename Cfg, bool B_KMAJOR>
 static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
   {
     // whole K steps; block scales are fetched 16 bytes per row at a time
-    bool whole = p.k_bytes >= RBK && p.k_bytes % RBK == 0;
+    // (the unscaled pipelined kernels finish a partial last K step themselves)
+    bool whole = p.k_bytes >= RBK;
     if constexpr (Cfg::kScaled) {
       whole = p.k_bytes % (RBK * 4 * Cfg::kStepsPerScaleDword) == 0 && p.lds_a % 16 == 0 && p.lds_b % 16 == 0 &&
               ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0;
