@@ -93,6 +93,32 @@ int mi355_gemm(const void* A, const void* B, void* C,
                const float* a_scale, const float* b_scale,
                int activation, void* stream);
 
+/* mi355_gemm with the epilogues of the reference's dot test fused in:
+ *   C = softmax_rows?( act( (a_scale * b_scale) * A @ B + D ) )
+ *
+ * Stands in for the ADD_MATRIX / ADD_ROWS / ADD_COLS / DO_SOFTMAX branches of the kernel in
+ *   python/test/unit/language/test_core.py:3128-3141 (and its checks, :3226-3235)
+ * and keeps the ACTIVATION hook of python/tutorials/03-matrix-multiplication.py:304-307.
+ * D ("addend", NULL = none) is read as D[m * stride_dm + n * stride_dn]; a zero stride
+ * broadcasts: stride_dn = 0 is the reference's add-rows (one value per row of C), stride_dm = 0
+ * its add-cols (one value per column), both non-zero its add-matrix.  D is fp16, bf16 or fp32
+ * (addend_dtype) and is added to the fp32 accumulator before the activation and the one
+ * rounding to out_dtype.  The add-matrix form may alias C (the reference adds the previous
+ * contents of Z); a broadcast D must not overlap C.
+ * softmax = 1 then replaces every row of C by exp(c - max) / sum in a second launch on the
+ * same stream (fp32 arithmetic; the reference does it inside its single tile).
+ * CHAIN_DOT (:3142-3144) is two calls: the first with out_dtype = in_dtype, the second on its result.
+ */
+int mi355_gemm_epilogue(const void* A, const void* B, void* C,
+                        int M, int N, int K,
+                        int64_t stride_am, int64_t stride_ak,
+                        int64_t stride_bk, int64_t stride_bn,
+                        int64_t stride_cm, int64_t stride_cn,
+                        int in_dtype, int out_dtype,
+                        const float* a_scale, const float* b_scale,
+                        const void* addend, int64_t stride_dm, int64_t stride_dn, int addend_dtype,
+                        int activation, int softmax, void* stream);
+
 /*
  * Grouped GEMM: C_g[M_g,N_g] = A_g[M_g,K_g] @ B_g[K_g,N_g] for g = 0 .. group_size-1 in ONE launch.
  *

@@ -86,6 +86,35 @@ def matmul_closed_form(a: np.ndarray, b: np.ndarray, activation: str = "", out_d
     return formats.round_to(acc.astype(np.float32), out_dtype)
 
 
+def dot_epilogue(a: np.ndarray, b: np.ndarray, add: np.ndarray | None = None, activation: str = "",
+                 softmax: bool = False, chain_w: np.ndarray | None = None, mid_dtype: str = "fp16",
+                 out_dtype: str = "fp32", alpha: float = 1.0) -> np.ndarray:
+    """The epilogue chain of the reference's dot test kernel
+    (python/test/unit/language/test_core.py:3128-3145) on the fp32 accumulator z = a @ b:
+    `z += Z` with Z a matrix (ADD_MATRIX, :3129-3130), a per-row value broadcast along N (ADD_ROWS,
+    :3131-3133) or a per-column value broadcast along M (ADD_COLS, :3134-3135) - here one `add`
+    broadcastable to [M, N]; the ACTIVATION hook of the matmul tutorial
+    (python/tutorials/03-matrix-multiplication.py:304-307); row softmax `exp(z - max) / sum`
+    (DO_SOFTMAX, :3136-3141); `dot(z.to(w.dtype), w)` (CHAIN_DOT, :3142-3144: z is rounded to the
+    operand type `mid_dtype` first).  One rounding to `out_dtype` at the store (:3145).
+    Pinned by tests/test_oracle_gemm.py: zero addend = plain product, softmax rows sum to one and are
+    invariant under a per-row addend, identity chain = the rounded product, and the reference's own
+    z_ref formulas (:3226-3250) on integer data."""
+    z = (np.asarray(a, dtype=np.float64) @ np.asarray(b, dtype=np.float64)) * alpha
+    z = z.astype(np.float32)
+    if add is not None:
+        z = z + np.broadcast_to(np.asarray(add, dtype=np.float32), z.shape)
+    if activation == "leaky_relu":
+        z = leaky_relu(z)
+    if softmax:
+        num = np.exp(z - np.max(z, axis=1, keepdims=True))
+        z = (num / np.sum(num, axis=1, keepdims=True)).astype(np.float32)
+    if chain_w is not None:
+        zm = formats.round_to(z, mid_dtype)
+        z = (zm.astype(np.float64) @ np.asarray(chain_w, dtype=np.float64)).astype(np.float32)
+    return formats.round_to(z, out_dtype)
+
+
 def grouped_tile_walk(sizes, BM: int, BN: int, num_programs: int):
     """The tile schedule of `grouped_matmul_kernel` (python/tutorials/08-grouped-gemm.py:86-134):
     tiles are numbered problem after problem, row major inside a problem; program b visits

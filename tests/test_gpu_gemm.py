@@ -291,3 +291,47 @@ def test_skinny_16bit_decode_shapes_against_closed_form(gpu, dtype):
         assert np.allclose(c, ref, rtol=1e-2, atol=1e-2), (M, N, K, "row-major B")
         c = to_np(triton_amd.matmul(from_np(a, dtype, gpu), tb.t().contiguous().t(), activation=act))
         assert np.allclose(c, ref, rtol=1e-2, atol=1e-2), (M, N, K, "K-major B")
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512)])
+def test_fused_epilogues_of_the_reference_dot_test(gpu, dtype, shape):
+    # add-matrix / add-rows / add-cols / softmax / chain-dot (python/test/unit/language/test_core.py:3128-3145)
+    # through mi355_gemm_epilogue: MFMA tile kernels, the strided kernel (100, 70, 50) and a skinny
+    # shape (which takes the tile kernels when there is an addend).  Integer data: bit-exact.
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    z = rng.integers(-4, 5, size=(M, N)).astype(np.float32)
+    ta, tb = from_np(a, dtype, gpu), from_np(b, dtype, gpu)
+    for add_dt in ("fp32", dtype):
+        tz = from_np(z, add_dt, gpu)
+        for add_np, add_t in ((z, tz), (z[:, :1], tz[:, :1]), (z[:1, :], tz[:1, :]), (z[0], tz[0])):
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=add_t))
+            assert bits_equal(got, gemm.dot_epilogue(a, b, add=add_np)), (dtype, shape, add_dt, add_np.shape)
+    # in place: C holds the addend and receives the result (the reference adds to the old Z)
+    from triton_amd import _lib
+    tc = from_np(z, "fp32", gpu)
+    rc = _lib.load().mi355_gemm_epilogue(ta.data_ptr(), tb.data_ptr(), tc.data_ptr(), M, N, K, K, 1, N, 1, N, 1,
+                                         _lib.BF16 if dtype == "bf16" else _lib.F16, _lib.F32, 0, 0,
+                                         tc.data_ptr(), N, 1, _lib.F32, _lib.ACT_LEAKY_RELU, 0,
+                                         torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert np.allclose(to_np(tc), gemm.dot_epilogue(a, b, add=z, activation="leaky_relu"), rtol=1e-6, atol=0)
+    # softmax on small-magnitude data, output in the input type and in fp32
+    a2, b2 = randn_rounded(rng, (M, K), dtype, 0.3), randn_rounded(rng, (K, N), dtype, 0.3)
+    ta2, tb2 = from_np(a2, dtype, gpu), from_np(b2, dtype, gpu)
+    bias = randn_rounded(rng, (1, N), "fp32")
+    got = to_np(triton_amd.matmul(ta2, tb2, out_dtype=torch.float32, add=from_np(bias, "fp32", gpu), softmax=True))
+    ref = gemm.dot_epilogue(a2, b2, add=bias, softmax=True)
+    assert np.allclose(got, ref, rtol=1e-2, atol=1e-3) and np.allclose(got.sum(axis=1), 1.0, atol=1e-4)
+    got16 = to_np(triton_amd.matmul(ta2, tb2, softmax=True))
+    assert np.allclose(got16, gemm.dot_epilogue(a2, b2, softmax=True, out_dtype=dtype), rtol=1e-2, atol=1e-2)
+    # chain-dot: (A @ B) rounded to the input type, then @ W
+    w = rng.integers(-2, 3, size=(N, N)).astype(np.float32)
+    got = to_np(triton_amd.chain_dot(ta, tb, from_np(w, dtype, gpu), out_dtype=torch.float32))
+    assert bits_equal(got, gemm.dot_epilogue(a, b, chain_w=w, mid_dtype=dtype))
+    wr = randn_rounded(rng, (N, N), dtype, 0.3)
+    got = to_np(triton_amd.chain_dot(ta2, tb2, from_np(wr, dtype, gpu)))
+    assert np.allclose(got, gemm.dot_epilogue(a2, b2, chain_w=wr, mid_dtype=dtype, out_dtype=dtype), rtol=1e-2, atol=1e-2)

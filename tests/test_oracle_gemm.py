@@ -90,3 +90,38 @@ def test_linearity_and_identity():
     assert np.array_equal(gemm.matmul_tiled(a, eye, 32, 32, 16, 8, out_dtype="fp32"), a)
     perm = eye[:, rng.permutation(64)]
     assert np.array_equal(gemm.matmul_tiled(a, perm, 32, 32, 16, 8, out_dtype="fp32"), a @ perm)
+
+
+def test_dot_epilogue_pins():
+    # the epilogue chain of the reference's dot test (test_core.py:3128-3145) against what the
+    # mathematics fixes and against the reference's own z_ref formulas (:3226-3250) on integer data
+    rng = np.random.default_rng(17)
+    M, N, K = 48, 40, 24
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+    z0 = rng.integers(-5, 6, size=(M, N)).astype(np.float32)
+    plain = gemm.matmul_closed_form(a, b)
+    assert np.array_equal(gemm.dot_epilogue(a, b, add=np.zeros((M, N), np.float32)), plain)
+    # z_ref += z ; z_ref += z[:, 0][:, None] ; z_ref += z[0, :][None, :]   (exact in integers)
+    assert np.array_equal(gemm.dot_epilogue(a, b, add=z0), a @ b + z0)
+    assert np.array_equal(gemm.dot_epilogue(a, b, add=z0[:, :1]), a @ b + z0[:, 0][:, None])
+    assert np.array_equal(gemm.dot_epilogue(a, b, add=z0[:1, :]), a @ b + z0[0, :][None, :])
+    # a transposed broadcast (rows taken for columns) must fail the comparison above: M != N
+    # softmax: rows sum to one, invariant under a per-row addend, equal to the reference formula
+    s = gemm.dot_epilogue(0.1 * a, 0.1 * b, softmax=True)
+    assert np.allclose(s.sum(axis=1), 1.0, atol=1e-6) and np.all(s > 0)
+    assert np.allclose(gemm.dot_epilogue(0.1 * a, 0.1 * b, add=z0[:, :1], softmax=True), s, atol=1e-6)
+    zr = (0.1 * a) @ (0.1 * b)
+    num = np.exp(zr - np.max(zr, axis=-1, keepdims=True))
+    assert np.allclose(s, num / np.sum(num, axis=-1, keepdims=True), atol=1e-6)
+    assert not np.allclose(gemm.dot_epilogue(0.1 * a, 0.1 * b, add=z0[:1, :], softmax=True), s, atol=1e-3)
+    # chain-dot: identity W returns the rounded product; integer W is exact
+    eye = np.eye(N, dtype=np.float32)
+    assert np.array_equal(gemm.dot_epilogue(a, b, chain_w=eye), formats.round_to(plain, "fp16"))
+    w = rng.integers(-2, 3, size=(N, N)).astype(np.float32)
+    assert np.array_equal(gemm.dot_epilogue(a, b, chain_w=w), (a @ b) @ w)
+    # the intermediate rounding is visible: bf16 keeps 8 bits of 257
+    a1 = np.full((1, 1), 257.0, np.float32)
+    one = np.ones((1, 1), np.float32)
+    assert gemm.dot_epilogue(a1, one, chain_w=one, mid_dtype="bf16")[0, 0] == 256.0
+    assert gemm.dot_epilogue(a1, one, chain_w=one, mid_dtype="fp16")[0, 0] == 257.0

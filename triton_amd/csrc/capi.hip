@@ -86,11 +86,12 @@ const char* mi355_strerror(int code) {
   return "unknown error";
 }
 
-int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
-               int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
-               int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
-               int activation, void* stream_) {
+static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
+                     int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                     int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                     int activation, const void* aux, int64_t aux_sm, int64_t aux_sn, int aux_dtype, void* stream_) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
+  if (aux && aux_dtype != MI355_F16 && aux_dtype != MI355_BF16 && aux_dtype != MI355_F32) return MI355_EDTYPE;
   if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
   if (in_dtype < MI355_F16 || in_dtype > MI355_F8E5M2) return MI355_EDTYPE;
   if (out_dtype < MI355_F16 || out_dtype > MI355_F32) return MI355_EDTYPE;
@@ -109,7 +110,8 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && env_int("MI355_GEMM_FORCE_STRIDED", 0) == 0;
 
   if (!fast) {
-    GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype};
+    GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype,
+                      aux, aux_sm, aux_sn, aux_dtype};
     return gemm_strided_launch(s, stream);
   }
 
@@ -123,6 +125,7 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   p.activation = activation; p.out_dtype = out_dtype;
   p.group_m = env_int("MI355_GEMM_GROUP_M", 8);
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
+  p.aux = aux; p.aux_sm = aux_sm; p.aux_sn = aux_sn; p.aux_dtype = aux_dtype;
 
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   // 256x256 tiles once they fill three quarters of the CUs, 128x128 tiles (two workgroups per CU) below that
@@ -130,7 +133,8 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
   // large problems run the software-pipelined 8-wave kernel
   int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
-  if (!is8 && env_int("MI355_GEMM_SKINNY", 1)) {
+  // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
+  if (!is8 && !aux && env_int("MI355_GEMM_SKINNY", 1)) {
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
@@ -148,9 +152,30 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
     if (use && gemm16_skinny_ok(sk, y_kmajor, x_kmajor))
       return gemm16_skinny_launch(sk, in_dtype == MI355_BF16, y_kmajor, x_kmajor, stream);
   }
-  if (is8 && gemm8_skinny_ok(p) && env_int("MI355_GEMM_SKINNY", 1)) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && !aux && gemm8_skinny_ok(p) && env_int("MI355_GEMM_SKINNY", 1)) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
+}
+
+int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
+               int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+               int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+               int activation, void* stream_) {
+  return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
+                   activation, nullptr, 0, 0, 0, stream_);
+}
+
+int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int K,
+                        int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                        int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                        const void* addend, int64_t stride_dm, int64_t stride_dn, int addend_dtype,
+                        int activation, int softmax, void* stream_) {
+  if (softmax != 0 && softmax != 1) return MI355_EINVAL;
+  if (softmax && out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
+  int rc = gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
+                     activation, addend, stride_dm, stride_dn, addend_dtype, stream_);
+  if (rc || !softmax) return rc;
+  return softmax_rows_launch(C, M, N, scm, scn, out_dtype, (hipStream_t)stream_);
 }
 
 int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,

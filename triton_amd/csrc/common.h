@@ -195,6 +195,13 @@ __device__ __forceinline__ void block_barrier() {
 #endif
 }
 
+// One element of the epilogue addend (dtype codes of the C ABI: 0 fp16, 1 bf16, 4 fp32).
+__device__ __forceinline__ float load_aux(const void* aux, int64_t off, int dtype) {
+  if (dtype == 4) return ((const float*)aux)[off];
+  if (dtype == 1) return (float)((const __bf16*)aux)[off];
+  return (float)((const _Float16*)aux)[off];
+}
+
 // Map a hardware workgroup id to a logical one so that ids that are consecutive in the
 // logical order run on the same XCD (hardware deals workgroups round-robin over 8 XCDs,
 // each with its own L2).

@@ -99,6 +99,7 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmA
 #pragma unroll
         for (int e = 0; e < 4; e++) {
           float x = acc[i][j][rg * 4 + e] * alpha;
+          if (p.aux && n + e < p.N) x += load_aux(p.aux, (int64_t)m * p.aux_sm + (int64_t)(n + e) * p.aux_sn, p.aux_dtype);
           if (leaky) x = x >= 0.f ? x : 0.01f * x;
           v[e] = x;
         }

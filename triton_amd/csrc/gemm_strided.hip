@@ -69,6 +69,7 @@ __global__ __launch_bounds__(256) void gemm_strided_kernel(GemmStridedArgs p) {
       int m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
       if (m < p.M && n < p.N) {
         float x = acc[i][j] * alpha;
+        if (p.aux) x += load_aux(p.aux, (int64_t)m * p.aux_sm + (int64_t)n * p.aux_sn, p.aux_dtype);
         if (p.activation == 1) x = x >= 0.f ? x : 0.01f * x;
         store_elem(p.C, (int64_t)m * p.scm + (int64_t)n * p.scn, p.out_dtype, x);
       }

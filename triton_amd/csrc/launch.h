@@ -21,6 +21,11 @@ struct GemmArgs {
   int out_dtype;  // MI355_F16 / MI355_BF16 / MI355_F32 (fp8 kernels also MI355_F8E4M3)
   int group_m;
   int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
+  // optional addend of the epilogue: acc * alpha + aux[m * aux_sm + n * aux_sn] (a zero stride broadcasts
+  // a row or a column vector), added in fp32 before the activation; NULL = none
+  const void* aux;
+  int64_t aux_sm, aux_sn;  // element strides
+  int aux_dtype;           // MI355_F16 / MI355_BF16 / MI355_F32
   // block-scaled (MX) kernels only: e8m0 scale matrices [M, K/32], [N, K/32] and their row pitches
   const uint8_t* sA;
   const uint8_t* sB;
@@ -34,6 +39,7 @@ struct GemmStridedArgs {
   int64_t sam, sak, sbk, sbn, scm, scn;
   const float* a_scale; const float* b_scale;
   int activation, in_dtype, out_dtype;
+  const void* aux; int64_t aux_sm, aux_sn; int aux_dtype;  // as in GemmArgs
 };
 
 // skinny 16-bit GEMM, out[s][l] = sum_k X[s][k] * Y[l][k]
@@ -85,6 +91,7 @@ int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_fwd8_launch(const AttnArgs& p, bool e5m2, hipStream_t stream);  // fp8 inputs, V with N contiguous
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int softmax_rows_launch(void* C, int M, int N, int64_t scm, int64_t scn, int dtype, hipStream_t stream);
 int dequant_launch(const uint8_t* codes, float* out, int64_t n, int fmt, hipStream_t stream);
 
 }  // namespace mi355

@@ -76,14 +76,17 @@ def _scale_ptr(s, device):
     return s.data_ptr(), s
 
 
-def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None):
-    """C = act((a_scale*b_scale) * A @ B) with fp32 accumulation.
+def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, add=None, softmax=False):
+    """C = softmax_rows?(act((a_scale*b_scale) * A @ B + add)) with fp32 accumulation.
 
     Same contract as the reference wrapper (03:330-348): A must be contiguous, B may have any
     strides (the reference passes `b.T` for fp8, 03:378-382), the result is fp16 for fp16 / fp8
     inputs.  Extensions, all keyword-only and defaulting to the reference behaviour: bf16
     inputs give a bf16 result, `out_dtype` overrides the result type, `a_scale` / `b_scale`
-    are per-tensor fp32 dequantisation scales.
+    are per-tensor fp32 dequantisation scales; `add` (fp16 / bf16 / fp32, broadcastable to
+    [M, N]: a matrix, an [M, 1] column = the reference's add-rows, a [1, N] / [N] row = its
+    add-cols) and `softmax` are the fused epilogues of the reference's dot test
+    (python/test/unit/language/test_core.py:3128-3141).
     """
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
     assert _is_contiguous(a), "Matrix A must be contiguous"
@@ -105,13 +108,35 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None):
         return c.zero_()
     pa, keep_a = _scale_ptr(a_scale, device)
     pb, keep_b = _scale_ptr(b_scale, device)
-    rc = _lib.load().mi355_gemm(
+    act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
+    if add is None and not softmax:
+        rc = _lib.load().mi355_gemm(
+            a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+            a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+            in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, act, _stream())
+        _lib.check(rc, "mi355_gemm")
+        return c
+    d_ptr, d_sm, d_sn, d_dt = 0, 0, 0, 0
+    if add is not None:
+        _check_device(2, add)
+        if add.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+            raise TypeError(f"add must be fp16, bf16 or fp32, got {add.dtype}")
+        d = torch.broadcast_to(add, (M, N))  # zero strides on broadcast axes
+        d_ptr, d_sm, d_sn, d_dt = d.data_ptr(), d.stride(0), d.stride(1), _TORCH_TO_ABI[add.dtype]
+    rc = _lib.load().mi355_gemm_epilogue(
         a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
         a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
-        in_dt, _TORCH_TO_ABI[out_dtype], pa, pb,
-        _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE, _stream())
-    _lib.check(rc, "mi355_gemm")
+        in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, d_ptr, d_sm, d_sn, d_dt, act, int(bool(softmax)), _stream())
+    _lib.check(rc, "mi355_gemm_epilogue")
     return c
+
+
+def chain_dot(a, b, w, *, out_dtype=None):
+    """(A @ B) rounded to the input type, then @ W: the CHAIN_DOT branch of the reference's dot test
+    (python/test/unit/language/test_core.py:3142-3144, `tl.dot(z.to(w.dtype), w)`), as two launches."""
+    assert a.dtype == b.dtype == w.dtype, "Incompatible dtypes"
+    z = matmul(a, b, out_dtype=a.dtype)
+    return matmul(z, w, out_dtype=out_dtype)
 
 
 def matmul_like_input(a, b):
