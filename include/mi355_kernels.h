@@ -93,6 +93,25 @@ int mi355_gemm(const void* A, const void* B, void* C,
                const float* a_scale, const float* b_scale,
                int activation, void* stream);
 
+/* mi355_gemm with the kernel configuration chosen by the caller instead of the library's size
+ * heuristic: what the reference's autotuner does when it launches its best `Config`
+ * (python/triton/runtime/autotuner.py:146-179 `Autotuner.run`; the configs of the matmul
+ * tutorial, python/tutorials/03-matrix-multiplication.py:168-239, differ in tile shape,
+ * GROUP_SIZE_M, stages and warps).  tile: -1 = heuristic, 0 = 256x256 ping-pong, 1 = 128x128,
+ * 2 = 256x256 one barrier per K step, 3 / 4 = 256x256 software-pipelined with four / eight waves
+ * (a kernel that does not exist for the dtype falls back to the nearest one).  group_m: the
+ * reference's GROUP_SIZE_M (:265-273), 0 = default 8.  Operands without 16-byte rows run the
+ * strided kernel whatever `tile` says.
+ */
+int mi355_gemm_tuned(const void* A, const void* B, void* C,
+                     int M, int N, int K,
+                     int64_t stride_am, int64_t stride_ak,
+                     int64_t stride_bk, int64_t stride_bn,
+                     int64_t stride_cm, int64_t stride_cn,
+                     int in_dtype, int out_dtype,
+                     const float* a_scale, const float* b_scale,
+                     int activation, int tile, int group_m, void* stream);
+
 /* mi355_gemm with the epilogues of the reference's dot test fused in:
  *   C = softmax_rows?( act( (a_scale * b_scale) * A @ B + D ) )
  *

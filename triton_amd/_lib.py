@@ -26,6 +26,9 @@ SIGNATURES = {
     "mi355_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                            c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                            c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
+    "mi355_gemm_tuned": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                 c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                 c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "mi355_gemm_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int, c_int, c_void_p, c_void_p,

@@ -89,7 +89,8 @@ const char* mi355_strerror(int code) {
 static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
                      int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
                      int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
-                     int activation, const void* aux, int64_t aux_sm, int64_t aux_sn, int aux_dtype, void* stream_) {
+                     int activation, const void* aux, int64_t aux_sm, int64_t aux_sn, int aux_dtype,
+                     int tile_arg, int group_m_arg, void* stream_) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
   if (aux && aux_dtype != MI355_F16 && aux_dtype != MI355_BF16 && aux_dtype != MI355_F32) return MI355_EDTYPE;
   if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
@@ -123,7 +124,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.ldc = scm; p.scn = scn;
   p.a_scale = a_scale; p.b_scale = b_scale;
   p.activation = activation; p.out_dtype = out_dtype;
-  p.group_m = env_int("MI355_GEMM_GROUP_M", 8);
+  p.group_m = group_m_arg > 0 ? group_m_arg : env_int("MI355_GEMM_GROUP_M", 8);
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
   p.aux = aux; p.aux_sm = aux_sm; p.aux_sn = aux_sn; p.aux_dtype = aux_dtype;
 
@@ -132,9 +133,10 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
   // large problems run the software-pipelined 8-wave kernel
   int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
-  tile = env_int("MI355_GEMM_TILE", tile);
+  tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
   // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
-  if (!is8 && !aux && env_int("MI355_GEMM_SKINNY", 1)) {
+  const bool skinny_allowed = tile_arg < 0 && env_int("MI355_GEMM_SKINNY", 1);  // an explicit tile means a tile kernel
+  if (!is8 && !aux && skinny_allowed) {
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
@@ -152,7 +154,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     if (use && gemm16_skinny_ok(sk, y_kmajor, x_kmajor))
       return gemm16_skinny_launch(sk, in_dtype == MI355_BF16, y_kmajor, x_kmajor, stream);
   }
-  if (is8 && !aux && gemm8_skinny_ok(p) && env_int("MI355_GEMM_SKINNY", 1)) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
@@ -162,7 +164,16 @@ int mi355_gemm(const void* A, const void* B, void* C, int M, int N, int K,
                int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
                int activation, void* stream_) {
   return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
-                   activation, nullptr, 0, 0, 0, stream_);
+                   activation, nullptr, 0, 0, 0, -1, 0, stream_);
+}
+
+int mi355_gemm_tuned(const void* A, const void* B, void* C, int M, int N, int K,
+                     int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                     int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                     int activation, int tile, int group_m, void* stream_) {
+  if (tile < -1 || tile > 4 || group_m < 0) return MI355_EINVAL;
+  return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
+                   activation, nullptr, 0, 0, 0, tile, group_m, stream_);
 }
 
 int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int K,
@@ -173,7 +184,7 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int
   if (softmax != 0 && softmax != 1) return MI355_EINVAL;
   if (softmax && out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
   int rc = gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
-                     activation, addend, stride_dm, stride_dn, addend_dtype, stream_);
+                     activation, addend, stride_dm, stride_dn, addend_dtype, -1, 0, stream_);
   if (rc || !softmax) return rc;
   return softmax_rows_launch(C, M, N, scm, scn, out_dtype, (hipStream_t)stream_);
 }
