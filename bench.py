@@ -26,7 +26,7 @@ HBM_GBPS = 8000.0
 # HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc:
 # FETCH_SIZE 790628 KiB x 2.000 + WRITE_SIZE 196184 KiB x 1.000, the factors being what the same
 # counters read for a plain copy of known size (profiles/gemm_bf16_8192.md)
-MEASURED_TRAFFIC_BYTES = int((790628 * 2.000 + 196184 * 1.000) * 1024)
+MEASURED_TRAFFIC_BYTES = int((802145 * 2.000 + 200437 * 1.000) * 1024)
 
 
 def time_launches(fn, steps, warmup):
@@ -172,6 +172,22 @@ def main():
         byts = n * n + 16 * n + 2 * 16 * n
         extra["fp8_decode_m16"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1), "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
         del a8, a16
+        # 16-bit skinny shapes of the reference's regression table (test_performance.py:36-44): fp16, row-major B
+        for (sm, sn, sk) in ((16, n, n), (64, n, n), (n, 64, n)):
+            xa = torch.randn(sm, sk, device=dev, dtype=torch.float16)
+            xb = torch.randn(sk, sn, device=dev, dtype=torch.float16)
+            xc = torch.empty(sm, sn, device=dev, dtype=torch.float16)
+
+            def skinny():
+                rc = lib.mi355_gemm(xa.data_ptr(), xb.data_ptr(), xc.data_ptr(), sm, sn, sk, sk, 1, sn, 1, sn, 1,
+                                    _lib.F16, _lib.F16, None, None, 0, stream)
+                assert rc == 0, rc
+
+            ms = quick(skinny, iters=50, warmup=5)
+            byts = 2 * (sm * sk + sk * sn + sm * sn)
+            extra[f"fp16_skinny_{sm}x{sn}x{sk}"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1),
+                                                    "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
+            del xa, xb, xc
         # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch
         ga = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
         gb = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
