@@ -139,7 +139,7 @@ def main():
         "config": {"workload": f"bf16 GEMM M=N=K={n}, A row-major MxK, B row-major KxN, fp32 accumulate, bf16 out (BASELINE config 2)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK["bf16"], 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gemm_w4_kernel<Cfg16<bf16>, 8 waves, row-major B, 4 stages> (256x256 tile, software pipelined)", "launch_ms_avg": round(ev_ms, 5),
+                     "kernel": "gemm_w4_kernel<Cfg16<bf16>, 8 waves, row-major B, 4 stages, persistent> (256x256 tiles, software pipelined, one program per CU)", "launch_ms_avg": round(ev_ms, 5),
                      "launch_ms_min": round(min(per), 5), "algorithmic_flops": flops,
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),

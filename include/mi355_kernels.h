@@ -98,7 +98,10 @@ int mi355_gemm(const void* A, const void* B, void* C,
  * (python/triton/runtime/autotuner.py:146-179 `Autotuner.run`; the configs of the matmul
  * tutorial, python/tutorials/03-matrix-multiplication.py:168-239, differ in tile shape,
  * GROUP_SIZE_M, stages and warps).  tile: -1 = heuristic, 0 = 256x256 ping-pong, 1 = 128x128,
- * 2 = 256x256 one barrier per K step, 3 / 4 = 256x256 software-pipelined with four / eight waves
+ * 2 = 256x256 one barrier per K step, 3 / 4 = 256x256 software-pipelined with four / eight waves,
+ * 5 = the eight-wave pipelined kernel as persistent programs (one per CU, MI355_GEMM_PROGRAMS
+ * overrides) that walk their tiles as one stream of K steps, the schedule of
+ * python/tutorials/09-persistent-matmul.py:141-190
  * (a kernel that does not exist for the dtype falls back to the nearest one).  group_m: the
  * reference's GROUP_SIZE_M (:265-273), 0 = default 8.  Operands without 16-byte rows run the
  * strided kernel whatever `tile` says.

@@ -94,14 +94,17 @@ def test_exact_integers_on_mfma_path_bitwise_vs_tiled_oracle(gpu):
             assert bits_equal(got, ref)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
 def test_every_kernel_variant_is_bit_exact_on_integers(gpu, monkeypatch, tile):
-    # MI355_GEMM_TILE forces one MFMA kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves)
-    # for shapes the size heuristic would give to another; K = 520 has a partial last K step, which
-    # the ping-pong and pipelined kernels hand to the one-barrier kernel
+    # MI355_GEMM_TILE forces one MFMA kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves,
+    # persistent) for shapes the size heuristic would give to another; K = 520 has a
+    # partial last K step, which the ping-pong kernel hands to the one-barrier kernel and the
+    # pipelined kernels finish themselves; the persistent form takes whole tiles with K a multiple of
+    # 128 (512 x 768 x 512 with 3 programs: two tiles each, in one stream of K steps) and falls back otherwise
     monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
+    monkeypatch.setenv("MI355_GEMM_PROGRAMS", "3")
     rng = np.random.default_rng(11 + tile)
-    for (M, N, K) in [(512, 768, 512), (300, 264, 520), (256, 256, 64)]:
+    for (M, N, K) in [(512, 768, 512), (300, 264, 520), (256, 256, 64), (1280, 1024, 128)]:
         a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
         b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
         ref = gemm.matmul_closed_form(a, b, out_dtype="fp32")

@@ -40,7 +40,7 @@ class Config:
 
 def default_configs():
     """The kernels that exist for every MFMA dtype, with the GROUP_SIZE_M values worth trying."""
-    return [Config(1, 8), Config(2, 8), Config(3, 8), Config(4, 4), Config(4, 8), Config(4, 16)]
+    return [Config(1, 8), Config(2, 8), Config(3, 8), Config(4, 8), Config(5, 4), Config(5, 8), Config(5, 16)]
 
 
 def _launch(a, b, c, config: Config, activation: int = 0):

@@ -132,8 +132,10 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // 256x256 tiles once they fill three quarters of the CUs, 128x128 tiles (two workgroups per CU) below that
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
   // large problems run the software-pipelined 8-wave kernel
-  int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
+  // (5 = the persistent form of the pipelined kernel; it falls back to 4 for edge tiles or a K tail)
+  int tile = (tiles256 * 4 >= 3L * cus) ? 5 : 1;
   tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
+  p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent forms (tile 5 / 6): one workgroup per CU
   // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
   const bool skinny_allowed = tile_arg < 0 && env_int("MI355_GEMM_SKINNY", 1);  // an explicit tile means a tile kernel
   if (!is8 && !aux && skinny_allowed) {
@@ -171,7 +173,7 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C, int M, int N, int K,
                      int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
                      int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
                      int activation, int tile, int group_m, void* stream_) {
-  if (tile < -1 || tile > 4 || group_m < 0) return MI355_EINVAL;
+  if (tile < -1 || tile > 5 || group_m < 0) return MI355_EINVAL;
   return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
                    activation, nullptr, 0, 0, 0, tile, group_m, stream_);
 }

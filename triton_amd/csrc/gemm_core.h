@@ -80,57 +80,65 @@ struct TileCopyKN {
 // (i, j), the four consecutive columns `ncol0 + 32 j + 8 rg + 4 (l/32) ..`.
 template <int MT, int NT>
 __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l32, int g) {
-  // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3
+  // epilogue: lane owns row m = .. + l32 and, per register group rg, columns n .. n+3.
+  // The tile loops are compile-time recursions, not `#pragma unroll`: with a body this size the
+  // unroller may give up, and a runtime index into `acc` would move the accumulators to scratch memory.
   float alpha = 1.f;
   if (p.a_scale) alpha *= *p.a_scale;
   if (p.b_scale) alpha *= *p.b_scale;
   const bool leaky = p.activation == 1;
   const bool vec_ok = p.c_vec_ok;
+  const bool has_aux = p.aux != nullptr;
+  static_for<MT>([&](auto I_) {
+    constexpr int i = decltype(I_)::value;
+    const int m = mrow0 + i * 32 + l32;
+    if (m < p.M) {
+      static_for<NT>([&](auto J_) {
+        constexpr int j = decltype(J_)::value;
+        static_for<4>([&](auto RG_) {
+          constexpr int rg = decltype(RG_)::value;
+          const int n = ncol0 + j * 32 + rg * 8 + g * 4;
+          float v[4];
 #pragma unroll
-  for (int i = 0; i < MT; i++) {
-    int m = mrow0 + i * 32 + l32;
-    if (m >= p.M) continue;
+          for (int e = 0; e < 4; e++) v[e] = acc[i][j][rg * 4 + e] * alpha;
+          if (has_aux) {
 #pragma unroll
-    for (int j = 0; j < NT; j++) {
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        int n = ncol0 + j * 32 + rg * 8 + g * 4;
-        float v[4];
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          float x = acc[i][j][rg * 4 + e] * alpha;
-          if (p.aux && n + e < p.N) x += load_aux(p.aux, (int64_t)m * p.aux_sm + (int64_t)(n + e) * p.aux_sn, p.aux_dtype);
-          if (leaky) x = x >= 0.f ? x : 0.01f * x;
-          v[e] = x;
-        }
-        if (p.out_dtype == 4) {
-          float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
-          } else {
-#pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = v[e];
+            for (int e = 0; e < 4; e++)
+              if (n + e < p.N) v[e] += load_aux(p.aux, (int64_t)m * p.aux_sm + (int64_t)(n + e) * p.aux_sn, p.aux_dtype);
           }
-        } else if (p.out_dtype == 1) {
-          __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-          } else {
+          if (leaky) {
 #pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (__bf16)v[e];
+            for (int e = 0; e < 4; e++) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
           }
-        } else {
-          _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
-          if (vec_ok && n + 3 < p.N) {
-            *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
-          } else {
+          if (p.out_dtype == 4) {
+            float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+            if (vec_ok && n + 3 < p.N) {
+              *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
+            } else {
 #pragma unroll
-            for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (_Float16)v[e];
+              for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = v[e];
+            }
+          } else if (p.out_dtype == 1) {
+            __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+            if (vec_ok && n + 3 < p.N) {
+              *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (__bf16)v[e];
+            }
+          } else {
+            _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+            if (vec_ok && n + 3 < p.N) {
+              *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+            } else {
+#pragma unroll
+              for (int e = 0; e < 4; e++) if (n + e < p.N) c[e * p.scn] = (_Float16)v[e];
+            }
           }
-        }
-      }
+        });
+      });
     }
-  }
+  });
 }
 
 // One BM x BN tile of C (tile row pm, tile column pn) with a ring of NS LDS stages at `lds`
@@ -713,8 +721,9 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
 //   * one barrier per step, at its top: by then every wave holds tile kt in registers (so its
 //     stage may be overwritten) and has seen its own share of tile kt+1 arrive.
 // ---------------------------------------------------------------------------------------------
-template <typename Cfg, int WN, bool B_KMAJOR, int NS>
+template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
 __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
+  static_assert(!(PERSIST && Cfg::kScaled), "the persistent form exists for the unscaled types");
   using Operand = typename Cfg::Operand;
   constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   static_assert(WN == 2 || WN == 4, "four or eight waves");
@@ -740,15 +749,23 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // scalar: LDS destinations of the direct loads are scalar math
   const int wm = wave / WN, wn = wave % WN;
 
+  // One tile per workgroup, or (PERSIST, the schedule of python/tutorials/09-persistent-matmul.py:
+  // 141-190) gridDim.x workgroups that each walk tiles lid, lid + G, lid + 2G, ... of the grouped
+  // order as ONE stream of K steps: the direct loads run NS steps ahead across tile boundaries, so
+  // the ring never drains between tiles.  lid keeps the workgroups of one XCD on neighbouring tiles.
   const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
-  int pid = xcd_remap(blockIdx.x, num_m * num_n);
+  const int ntiles = num_m * num_n;
+  const int G = PERSIST ? (int)gridDim.x : ntiles;
+  const int lid = xcd_remap(blockIdx.x, G);
+  const int ntw = PERSIST ? (ntiles - lid + G - 1) / G : 1;  // tiles of this workgroup (the host keeps G <= ntiles)
   int pm, pn;
-  grouped_tile(pid, num_m, num_n, p.group_m, pm, pn);
-  const int m0 = pm * BM, n0 = pn * BN;
+  grouped_tile(lid, num_m, num_n, p.group_m, pm, pn);
+  int m0 = pm * BM, n0 = pn * BN;  // tile being multiplied
 
   // Sources of the direct loads: a scalar tile base that advances with kt plus a 32-bit per-lane
   // offset that never changes (the host keeps 256 rows of either operand within 2^31 bytes), so a
   // load costs no vector arithmetic.
+  // (PERSIST runs on whole tiles only, so the clamps below are neutral and the offsets serve every tile)
   const char* const baseA = p.A + (int64_t)m0 * p.lda;
   const char* const baseB = B_KMAJOR ? p.B + (int64_t)n0 * p.ldb : p.B + (int64_t)n0 * 2;
   unsigned offGA[ITA], offGB[ITB];
@@ -783,14 +800,33 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     if (NW == 8 && wave >= 4) srcSA = srcSB;
   }
 
-  // direct load number `i` of this wave's share of tile kt
-  auto issue_one = [&](auto I_, int kt, LDS_PTR(char) a) {
+  const int nfull = p.k_bytes / RBK;
+  // Fill cursor: the (tile, K step) the next direct loads fetch.  It runs NS positions ahead of the
+  // multiplication and stops on the last position of the workgroup's stream (which is then fetched
+  // again into a dead stage: the number of outstanding loads, and with it the partial waits, stays uniform).
+  int ftile = 0, fkt = 0;
+  const char* fillA = baseA;
+  const char* fillB = baseB;
+  auto fill_advance = [&]() {
+    if (fkt + 1 < nfull) {
+      fkt++;
+    } else if (PERSIST && ftile + 1 < ntw) {
+      ftile++;
+      fkt = 0;
+      int fm, fn;
+      grouped_tile(lid + ftile * G, num_m, num_n, p.group_m, fm, fn);
+      fillA = p.A + (int64_t)fm * BM * p.lda;
+      fillB = B_KMAJOR ? p.B + (int64_t)fn * BN * p.ldb : p.B + (int64_t)fn * BN * 2;
+    }
+  };
+  // direct load number `i` of this wave's share of the K step at (srcA, srcB)
+  auto issue_one = [&](auto I_, const char* srcA, const char* srcB, LDS_PTR(char) a) {
     constexpr int i = decltype(I_)::value;
     if constexpr (i < ITA) {
-      async_copy16_sbase(baseA + kt * stepA, offGA[i], lds_addr(a) + (i * NW + wave) * 1024);
+      async_copy16_sbase(srcA, offGA[i], lds_addr(a) + (i * NW + wave) * 1024);
     } else {
       constexpr int ib = i - ITA;
-      async_copy16_sbase(baseB + kt * stepB, offGB[ib], lds_addr(a) + A_BYTES + (ib * NW + wave) * 1024);
+      async_copy16_sbase(srcB, offGB[ib], lds_addr(a) + A_BYTES + (ib * NW + wave) * 1024);
     }
   };
   // scale group sg (the 16 scale bytes per row of K steps sg*SPG ..) into ring slot sg % 2: one
@@ -923,7 +959,6 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   };
 
   constexpr int kMfmas = AH * NT;  // per half
-  const int nfull = p.k_bytes / RBK;
 
   // MFMAs of half H with the memory instructions of the half in between: the `nreads` LDS reads
   // over the first MFMAs (they are needed at the top of the next half), then the `nloads`
@@ -959,15 +994,23 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // of outstanding loads - and with it the partial waits - uniform), first half of tile 0 requested
   issue_scales(0);
 #pragma unroll
-  for (int s = 0; s < NS; s++) static_for<kShare>([&](auto I_) { issue_one(I_, min(s, nfull - 1), lds + s * STAGE); });
+  for (int s = 0; s < NS; s++) {
+    const char* srcA = fillA + fkt * stepA;
+    const char* srcB = fillB + fkt * stepB;
+    static_for<kShare>([&](auto I_) { issue_one(I_, srcA, srcB, lds + s * STAGE); });
+    fill_advance();
+  }
   wait_vmcnt<(NS - 1) * kShare>();
   __builtin_amdgcn_sched_barrier(0);
   block_barrier();
   __builtin_amdgcn_sched_barrier(0);
   static_for<n_reads(0)>([&](auto R_) { read_one(R_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}, lds_addr(sc_ring)); });
 
-  // one K step of the tile in ring stage STG (its parity, for the one-sub-step types, is STG % 2)
-  auto step = [&](int kt, auto STG_) {
+  // one K step of the tile in ring stage STG (its parity, for the one-sub-step types, is STG % 2);
+  // kt = K step inside the current tile
+  int ckt = 0, ctile = 0;
+  auto step = [&](auto STG_) {
+    const int kt = ckt;
     constexpr int stage = decltype(STG_)::value, P = stage & 1;
     using H0 = std::integral_constant<int, 0>;
     using H1 = std::integral_constant<int, 1>;
@@ -997,20 +1040,48 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       const int ktn = kt + 1;
       const unsigned scbase = lds_addr(sc_ring) + ((ktn / SPG) & 1) * SC_SLOT + Cfg::scale_dword_offset(ktn % SPG);
       LDS_PTR(char) const fill = lds + stage * STAGE;
-      const int kfill = min(kt + NS, nfull - 1);
+      const char* srcA = fillA + fkt * stepA;
+      const char* srcB = fillB + fkt * stepB;
       constexpr int nr = n_reads(0);
       half(H1{}, P_{}, std::integral_constant<int, nr>{}, std::integral_constant<int, kShare>{}, [&](auto OP_) {
         constexpr int op = decltype(OP_)::value;
         if constexpr (op < nr) read_one(OP_, H0{}, PN{}, SN{}, scbase);
-        else issue_one(std::integral_constant<int, op - nr>{}, kfill, fill);
+        else issue_one(std::integral_constant<int, op - nr>{}, srcA, srcB, fill);
       });
+      fill_advance();
     }
+    ckt++;
   };
-  for (int kt = 0; kt < nfull; kt += NS) {
-    step(kt, std::integral_constant<int, 0>{});
-    if (kt + 1 < nfull) step(kt + 1, std::integral_constant<int, 1>{});
-    if (kt + 2 < nfull) step(kt + 2, std::integral_constant<int, 2>{});
-    if (kt + 3 < nfull) step(kt + 3, std::integral_constant<int, 3>{});
+  const int nsteps_all = ntw * nfull;
+  for (int s = 0; s < nsteps_all; s += NS) {
+    step(std::integral_constant<int, 0>{});
+    if (s + 1 < nsteps_all) step(std::integral_constant<int, 1>{});
+    if (s + 2 < nsteps_all) step(std::integral_constant<int, 2>{});
+    if (s + 3 < nsteps_all) step(std::integral_constant<int, 3>{});
+    if constexpr (PERSIST) {
+      // (the host launches this form only when a tile's K steps are a multiple of the ring length, so
+      //  tiles end here and the epilogue exists once in the loop body)
+      if (ckt == nfull) {
+        // tile finished: store it, start the next one.  The stores share the vector-memory counter
+        // with the direct loads and may complete out of order with them, so the counter is drained
+        // once per tile before the partial waits count again (the loads for the next tile's first
+        // steps were issued during the last steps of this one and have been in flight since).
+        gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+#pragma unroll
+        for (int i = 0; i < MT; i++)
+#pragma unroll
+          for (int j = 0; j < NT; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        ckt = 0;
+        ctile++;
+        grouped_tile(lid + min(ctile, ntw - 1) * G, num_m, num_n, p.group_m, pm, pn);
+        m0 = pm * BM;
+        n0 = pn * BN;
+        wait_vmcnt<0>();
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
   }
   // nothing may still be writing this workgroup's LDS when it retires
   wait_all();
@@ -1018,7 +1089,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // Last, partial K step (unscaled types only): its 16-byte chunks past K are written as zeros (the
   // reference masks them to 0, python/tutorials/03-matrix-multiplication.py:297-298).  Goes through
   // registers into stage 0 and is multiplied without overlap: one step out of K / 32.
-  if constexpr (!Cfg::kScaled) {
+  if constexpr (!Cfg::kScaled && !PERSIST) {
     if (p.k_bytes % RBK != 0) {
       using Z = std::integral_constant<int, 0>;
       using O = std::integral_constant<int, 1>;
@@ -1049,23 +1120,25 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     }
   }
 
-  gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+  if constexpr (!PERSIST) gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
 }
 
-template <typename Cfg, int WN, bool B_KMAJOR, int NS>
-static int launch_gemm_w4(const GemmArgs& p, hipStream_t stream) {
+template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
+static int launch_gemm_w4(const GemmArgs& p, hipStream_t stream, int num_programs = 0) {
   constexpr int BM = 256, BN = 256;
   constexpr int smem = NS * (BM + BN) * RBK + (Cfg::kScaled ? 2 * (BM + BN) * 16 : 0);
   static_assert(smem <= 160 * 1024, "LDS ring does not fit");
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
-  gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS><<<dim3(num_m * num_n), dim3(2 * WN * 64), smem, stream>>>(p);
+  int grid = num_m * num_n;
+  if (PERSIST && num_programs > 0 && num_programs < grid) grid = num_programs;
+  gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST><<<dim3(grid), dim3(2 * WN * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -1115,6 +1188,13 @@ static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
     if constexpr (Cfg::kScaled) {
       whole = p.k_bytes % (RBK * 4 * Cfg::kStepsPerScaleDword) == 0 && p.lds_a % 16 == 0 && p.lds_b % 16 == 0 &&
               ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0;
+    }
+    if constexpr (!Cfg::kScaled) {
+      // persistent form (5, eight waves; a four-wave persistent form spills): whole tiles, K steps in
+      // whole rings, one workgroup per CU; anything else runs the one-tile-per-workgroup form
+      const bool stream_ok = whole && p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % (4 * RBK) == 0 && p.num_programs > 0;
+      if (tile >= 5 && stream_ok) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4, true>(p, stream, p.num_programs);
+      if (tile >= 5) tile = 4;
     }
     if constexpr (Cfg::kSteps == 2) {  // the four-wave form of the one-sub-step types runs out of registers
       if (tile == 3 && whole) return launch_gemm_w4<Cfg, 2, B_KMAJOR, 4>(p, stream);

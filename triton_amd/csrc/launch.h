@@ -20,6 +20,7 @@ struct GemmArgs {
   int activation;
   int out_dtype;  // MI355_F16 / MI355_BF16 / MI355_F32 (fp8 kernels also MI355_F8E4M3)
   int group_m;
+  int num_programs;  // persistent kernels: workgroups to launch (0 = not persistent)
   int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
   // optional addend of the epilogue: acc * alpha + aux[m * aux_sm + n * aux_sn] (a zero stride broadcasts
   // a row or a column vector), added in fp32 before the activation; NULL = none

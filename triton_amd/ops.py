@@ -159,9 +159,10 @@ def matmul_like_input(a, b):
 
 
 def matmul_persistent(a, b):
-    """`matmul_persistent(a, b)` of the same tutorial (09:190-224): there, NUM_SMS programs walk the
-    tiles; here the schedule is the library's own (one workgroup per 256x256 tile fills the 256 CUs
-    in whole rounds at these sizes) and the result is the same `a @ b` in the input dtype."""
+    """`matmul_persistent(a, b)` of the same tutorial (09:190-224): NUM_SMS programs walk the tiles.
+    Here that is the library's default for large products with whole 256x256 tiles (one program per
+    CU, each walking its tiles as one stream of K steps), so this is the same call as
+    `matmul_like_input`; other shapes run one workgroup per tile.  Same `a @ b` in the input dtype."""
     return matmul_like_input(a, b)
 
 
