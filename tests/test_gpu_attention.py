@@ -63,9 +63,11 @@ def test_forward_variants_and_lse(gpu, causal, n_ctx, monkeypatch):
     (q, k, v, _), (tq, tk, tv, _) = _inputs(3, (2, 2, n_ctx, 128), "bf16", gpu)
     cf = A.attn_closed_form(q, k, v, causal, 0.125)
     # 0: 64 query rows per wave, 1: four waves of 32 rows, 2: eight waves of 32 rows (n_ctx = 384 leaves
-    # half of its second 256-row block empty)
-    for variant in ("0", "1", "2"):
+    # half of its second 256-row block empty), 3 and 4: 1 and 2 as persistent programs (two programs here, so
+    # that each walks several items)
+    for variant in ("0", "1", "2", "3", "4"):
         monkeypatch.setenv("MI355_ATTN_FWD_VARIANT", variant)
+        monkeypatch.setenv("MI355_ATTN_PROGRAMS", "1")
         o = torch.empty_like(tq)
         M = torch.empty(2, 2, n_ctx, dtype=torch.float32, device=gpu)
         I4 = _lib.I64x4

@@ -282,6 +282,318 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Persistent form: gridDim.x workgroups each walk several (head, query block) items as ONE stream
+// of K/V steps.  The direct loads of the next item's first K/V tile are issued during the last
+// step of the current one and its Q fragments a whole item ahead, so the per-item start-up (a
+// memory round trip for Q and for the first tile, worth about three K/V steps) is hidden.
+// Items are dealt round-robin in an order that keeps the workgroups of one XCD on one head; under
+// the causal mask odd rounds walk the query blocks short-to-long and even rounds long-to-short, so
+// every workgroup gets the same amount of work over two rounds.  One query tile (32 rows) per wave.
+// ---------------------------------------------------------------------------------------------
+template <typename V8, int D, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kernel(AttnArgs p) {
+  using S = typename Elem<V8>::type;
+  constexpr int BM = NW * 32, BN = 64;
+  constexpr int RB = D * 2;
+  using Tile = AttnTile<RB, BN, NW>;
+  constexpr int TILE = Tile::BYTES;
+  constexpr int INST = Tile::INST;
+  constexpr int KSQ = D / 16;
+  constexpr int DT = D / 32;
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][K tile | V tile]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
+
+  const int nqb = (p.N + BM - 1) / BM;
+  const int total = nqb * p.Z * p.H;
+  const int G = gridDim.x;
+  const int lid = xcd_remap(blockIdx.x, G);
+  const int nitems = (total - lid + G - 1) / G;  // the host keeps G <= total
+  const int heads_per_round = max(1, G / nqb);
+  const int64_t qpitch = p.sq[2] * 2, kpitch = p.sk[2] * 2, vpitch = p.sv[2] * 2, opitch = p.so[2] * 2;
+
+  // item r of this workgroup -> (head, query block)
+  auto item_of = [&](int r, int& hz, int& qb) {
+    const int L = r * G + lid;
+    hz = L / nqb;
+    const int j = L % nqb;
+    // direction by the round a head falls into (G / nqb heads per round): a bijection whatever G is,
+    // and equal to "even rounds long-to-short" when G is a multiple of nqb
+    qb = (p.causal && ((hz / heads_per_round) & 1) == 0) ? nqb - 1 - j : j;
+  };
+  auto steps_of = [&](int qb) {
+    const int kv_end = p.causal ? min(p.N, (qb + 1) * BM) : p.N;
+    return (kv_end + BN - 1) / BN;
+  };
+  auto head_ptr = [&](const char* base, const int64_t* st, int hz) {
+    return base + ((int64_t)(hz / p.H) * st[0] + (int64_t)(hz % p.H) * st[1]) * 2;
+  };
+  auto load_q = [&](V8 (&dst)[KSQ], int hz, int qb) {
+    const int r = min(qb * BM + wave * 32 + l32, p.N - 1);
+    const char* src = head_ptr(p.q, p.sq, hz) + (int64_t)r * qpitch + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) dst[ks] = *(const V8*)(src + ks * 32);
+  };
+
+  // ---- state of the item being multiplied
+  int c_item = 0, c_hz, c_qb, cj = 0;
+  item_of(0, c_hz, c_qb);
+  int nsteps = steps_of(c_qb);
+  int row0 = c_qb * BM + wave * 32;
+  int wave_last = p.causal ? (row0 + 31) / BN : nsteps - 1;
+  int wave_first_masked = p.causal ? row0 / BN : nsteps;
+  V8 qf[KSQ], qnext[KSQ];
+  load_q(qf, c_hz, c_qb);
+  {
+    int nhz, nqbk;
+    item_of(min(1, nitems - 1), nhz, nqbk);
+    load_q(qnext, nhz, nqbk);
+  }
+
+  // ---- fill cursor: the (item, K/V step) the next direct loads fetch; stops after the last one
+  int f_item = 0, fj = 0, f_steps = nsteps;
+  const char* f_k = head_ptr(p.k, p.sk, c_hz);
+  const char* f_v = head_ptr(p.v, p.sv, c_hz);
+  bool f_valid = true;
+  unsigned offK[INST], offV[INST];
+#pragma unroll
+  for (int i = 0; i < INST; i++) {
+    offK[i] = (unsigned)Tile::off(kpitch, wave, lane, i);
+    offV[i] = (unsigned)Tile::off(vpitch, wave, lane, i);
+  }
+  const unsigned lds_base = lds_addr(lds);
+  auto issue_fill = [&](int stage) {
+    if (!f_valid) return;
+    const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
+    const char* ksrc = f_k + (int64_t)fj * BN * kpitch;
+    const char* vsrc = f_v + (int64_t)fj * BN * vpitch;
+#pragma unroll
+    for (int i = 0; i < INST; i++) {
+      async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
+      async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+    }
+    if (++fj == f_steps) {
+      fj = 0;
+      if (++f_item < nitems) {
+        int hz, qb;
+        item_of(f_item, hz, qb);
+        f_steps = steps_of(qb);
+        f_k = head_ptr(p.k, p.sk, hz);
+        f_v = head_ptr(p.v, p.sv, hz);
+      } else {
+        f_valid = false;
+      }
+    }
+  };
+
+  const RowRead<RB> rk(l32, g);
+  const TrRead<RB> tv(i16, q4);
+  unsigned ka[KSQ], va[DT][2];
+#pragma unroll
+  for (int ks = 0; ks < KSQ; ks++) ka[ks] = lds_base + rk.rowb + (rk.xk ^ (ks * 32));
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int h2 = 0; h2 < 2; h2++) va[c][h2] = lds_base + (tv.tl ^ ((c << 6) | (h2 << 5)));
+
+  f32x16 oacc[DT];
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) oacc[c][r] = 0.f;
+  float m_i = -INFINITY, l_i = 0.f;
+  const float qk_scale = p.sm_scale * 1.44269504f;
+  constexpr float RESCALE_LOG2 = 8.f;  // lazy running maximum, as in attn_fwd_kernel
+
+  issue_fill(0);
+  wait_all();
+  __syncthreads();
+
+  // one K/V step of the stream in ring stage STAGE; false once the last item is stored
+  auto step = [&](auto STAGE_) -> bool {
+    constexpr int stage = decltype(STAGE_)::value;
+    constexpr int KOFF = stage * 2 * TILE, VOFF = KOFF + TILE;
+    const int j = cj;
+    issue_fill(stage ^ 1);
+    if (j <= wave_last && row0 < p.N) {
+      f32x16 s[2];
+#pragma unroll
+      for (int a = 0; a < 2; a++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s[a][r] = 0.f;
+      {
+        i32x4 kf[2][2];
+        kf[0][0] = lds_read_b128<KOFF>(ka[0]);
+        kf[0][1] = lds_read_b128<KOFF + 32 * RB>(ka[0]);
+        static_for<KSQ>([&](auto KS_) {
+          constexpr int ks = decltype(KS_)::value;
+          constexpr int cur = ks & 1, nxt = cur ^ 1;
+          if constexpr (ks + 1 < KSQ) {
+            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + 1]);
+            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + 1]);
+            lds_wait<2>();
+          } else {
+            lds_wait<0>();
+          }
+          lds_use(kf[cur][0]);
+          lds_use(kf[cur][1]);
+#pragma unroll
+          for (int a = 0; a < 2; a++) s[a] = mfma32(__builtin_bit_cast(V8, kf[cur][a]), qf[ks], s[a]);
+        });
+      }
+      V8 pf[4];
+      {
+        if (j >= wave_first_masked) {
+          const int qrow = row0 + l32;
+#pragma unroll
+          for (int a = 0; a < 2; a++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+              int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+              if (kv > qrow) s[a][r] = -INFINITY;
+            }
+        }
+        float mx = s[0][0];
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) mx = fmaxf(mx, s[a][r]);
+        mx = pair_max(mx);
+        const float m_new = fmaxf(m_i, mx * qk_scale);
+        if (__builtin_amdgcn_ballot_w64(m_new > m_i + RESCALE_LOG2) != 0) {
+          const float alpha = fast_exp2(m_i - m_new);
+          l_i *= alpha;
+          m_i = m_new;
+#pragma unroll
+          for (int c = 0; c < DT; c++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[c][r] *= alpha;
+        }
+        const float m_cur = m_i;
+        float rs = 0.f;
+#pragma unroll
+        for (int a = 0; a < 2; a++)
+#pragma unroll
+          for (int r = 0; r < 16; r++) {
+            float pv = fast_exp2(fmaf(s[a][r], qk_scale, -m_cur));
+            s[a][r] = pv;
+            rs += pv;
+          }
+        l_i += rs;
+#pragma unroll
+        for (int t = 0; t < 4; t++)
+#pragma unroll
+          for (int e = 0; e < 8; e++) pf[t][e] = (S)s[t >> 1][(t & 1) * 8 + e];
+      }
+      {
+        i32x2 vf[2][DT][2];
+        auto read_v = [&](auto T_, i32x2 (&dst)[DT][2]) {
+          constexpr int t = decltype(T_)::value;
+          static_for<DT>([&](auto C_) {
+            constexpr int c = decltype(C_)::value;
+            dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0]);
+            dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1]);
+          });
+        };
+        read_v(std::integral_constant<int, 0>{}, vf[0]);
+        static_for<4>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          constexpr int cur = t & 1, nxt = cur ^ 1;
+          if constexpr (t + 1 < 4) {
+            read_v(std::integral_constant<int, t + 1>{}, vf[nxt]);
+            lds_wait<2 * DT>();
+          } else {
+            lds_wait<0>();
+          }
+#pragma unroll
+          for (int c = 0; c < DT; c++) {
+            lds_use(vf[cur][c][0]);
+            lds_use(vf[cur][c][1]);
+            i32x4 both = __builtin_shufflevector(vf[cur][c][0], vf[cur][c][1], 0, 1, 2, 3);
+            oacc[c] = mfma32(__builtin_bit_cast(V8, both), pf[t], oacc[c]);
+          }
+        });
+      }
+    }
+    wait_all();
+    __syncthreads();
+    if (++cj < nsteps) return true;
+
+    // ---- item finished: O = acc / l, M = m + log2(l); then switch to the next item
+    {
+      float l = pair_sum(l_i);
+      const int row = row0 + l32;
+      if (row < p.N) {
+        const float inv = 1.f / l;
+        if (g == 0) p.lse[(int64_t)c_hz * p.N + row] = m_i + log2f(l);
+        char* dst = (char*)head_ptr(p.o, p.so, c_hz) + (int64_t)row * opitch;
+#pragma unroll
+        for (int c = 0; c < DT; c++)
+#pragma unroll
+          for (int rg = 0; rg < 4; rg++) {
+            int d = c * 32 + rg * 8 + g * 4;
+            typedef __attribute__((ext_vector_type(4))) S S4;
+            S4 v;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = (S)(oacc[c][rg * 4 + e] * inv);
+            *(S4*)(dst + d * 2) = v;
+          }
+      }
+    }
+    if (++c_item >= nitems) return false;
+    item_of(c_item, c_hz, c_qb);
+    cj = 0;
+    nsteps = steps_of(c_qb);
+    row0 = c_qb * BM + wave * 32;
+    wave_last = p.causal ? (row0 + 31) / BN : nsteps - 1;
+    wave_first_masked = p.causal ? row0 / BN : nsteps;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) qf[ks] = qnext[ks];
+    {
+      int nhz, nqbk;
+      item_of(min(c_item + 1, nitems - 1), nhz, nqbk);
+      load_q(qnext, nhz, nqbk);
+    }
+#pragma unroll
+    for (int c = 0; c < DT; c++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) oacc[c][r] = 0.f;
+    m_i = -INFINITY;
+    l_i = 0.f;
+    return true;
+  };
+
+  while (true) {
+    if (!step(std::integral_constant<int, 0>{})) break;
+    if (!step(std::integral_constant<int, 1>{})) break;
+  }
+  wait_all();
+}
+
+template <typename V8, int D, int NW>
+static int launch_fwd_stream(const AttnArgs& p, hipStream_t stream) {
+  constexpr int BM = NW * 32;
+  constexpr int smem = 2 * 2 * 64 * D * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_stream_kernel<V8, D, NW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int total = ((p.N + BM - 1) / BM) * p.Z * p.H;
+  // as many workgroups as are resident at once: two per CU with four waves, one with eight
+  int grid = p.num_programs > 0 ? p.num_programs * (NW == 4 ? 2 : 1) : total;
+  if (grid > total) grid = total;
+  attn_fwd_stream_kernel<V8, D, NW><<<dim3(grid), dim3(NW * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 template <typename V8, int D, int QT, int NW>
 static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
   constexpr int BM = NW * QT * 32;
@@ -300,6 +612,8 @@ static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
 
 template <typename V8>
 static int launch_fwd_d(const AttnArgs& p, int variant, hipStream_t stream) {
+  if (variant == 3) return p.D == 128 ? launch_fwd_stream<V8, 128, 4>(p, stream) : launch_fwd_stream<V8, 64, 4>(p, stream);
+  if (variant == 4) return p.D == 128 ? launch_fwd_stream<V8, 128, 8>(p, stream) : launch_fwd_stream<V8, 64, 8>(p, stream);
   if (p.D == 128) {
     if (variant == 2) return launch_fwd<V8, 128, 1, 8>(p, stream);
     return variant == 1 ? launch_fwd<V8, 128, 1, 4>(p, stream) : launch_fwd<V8, 128, 2, 4>(p, stream);

@@ -287,9 +287,11 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     return MI355_ESTRIDE;
   p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
   p.sm_scale = sm_scale; p.causal = causal != 0;
-  // eight waves (256 query rows) per K/V stream halve the L2 -> LDS traffic; under the causal mask
-  // the uneven row ranges of eight waves cost as much as that saves, so four waves stay
-  p.variant = env_int("MI355_ATTN_FWD_VARIANT", causal ? 1 : 2);
+  // eight waves (256 query rows) per K/V stream halve the L2 -> LDS traffic.  Under the causal mask
+  // their row ranges are uneven, which the persistent form (4) evens out by pairing long and short
+  // query blocks per program; without a mask the one-item-per-workgroup form (2) is the faster one.
+  p.variant = env_int("MI355_ATTN_FWD_VARIANT", causal ? 4 : 2);
+  p.num_programs = env_int("MI355_ATTN_PROGRAMS", device_info().cus > 0 ? device_info().cus : 256);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 

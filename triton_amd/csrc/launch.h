@@ -66,6 +66,7 @@ struct AttnArgs {
   float sm_scale;
   int causal;
   int variant;  // tiling variant (tuning knob)
+  int num_programs;  // persistent forward: CUs to fill (0 = one workgroup per item)
 };
 
 // Device-side tables of a grouped GEMM (layout of python/tutorials/08-grouped-gemm.py:66-77).
