@@ -36,7 +36,7 @@ def _code_distance(got_codes, ref_vals, fmt):
 
 @pytest.mark.parametrize("fmt", ["e5m2", "e4m3"])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("shape", [(1, 2, 128, 64), (1, 2, 256, 128), (2, 3, 512, 128), (1, 1, 384, 64)])
+@pytest.mark.parametrize("shape", [(1, 2, 128, 64), (1, 2, 256, 128), (2, 3, 512, 128), (1, 1, 384, 64), (1, 2, 384, 128)])
 def test_fp8_forward_against_oracle(gpu, fmt, causal, shape):
     (q, k, v), (tq, tk, tv) = _fp8_inputs(sum(shape), shape, fmt, gpu)
     sm_scale = shape[-1] ** -0.5
@@ -58,6 +58,18 @@ def test_fp8_forward_against_oracle(gpu, fmt, causal, shape):
     # against the unrounded fp64 result the fp8 rounding of P dominates (the oracle itself sits
     # 0.15 |o| + 0.035 away from it on these inputs)
     assert np.all(np.abs(got - cf["o"]) <= 0.15 * np.abs(cf["o"]) + 0.05)
+
+
+@pytest.mark.parametrize("causal", [True, False])
+def test_fp8_forward_eight_wave_variant_gives_the_same_codes(gpu, causal, monkeypatch):
+    # MI355_ATTN_FWD_VARIANT=2: 256 query rows per K/V stream (head_dim 128); N = 384 leaves half of
+    # the second block empty.  Same arithmetic per row, so the output codes are identical.
+    shape = (1, 2, 384, 128)
+    _, (tq, tk, tv) = _fp8_inputs(5, shape, "e5m2", gpu)
+    base = triton_amd.attention(tq, tk, tv, causal, 0.1).view(torch.uint8).cpu().numpy()
+    monkeypatch.setenv("MI355_ATTN_FWD_VARIANT", "2")
+    wide = triton_amd.attention(tq, tk, tv, causal, 0.1).view(torch.uint8).cpu().numpy()
+    assert np.array_equal(base, wide)
 
 
 def test_fp8_forward_exact_case_uniform_attention(gpu):

@@ -44,9 +44,9 @@ __device__ __forceinline__ f32x16 mfma_f8(i32x8 a, i32x8 b, f32x16 c) {
 #endif
 }
 
-template <int FMT, int D>
-__global__ __launch_bounds__(256, 2) void attn_fwd8_kernel(AttnArgs p) {
-  constexpr int NW = 4, BM = NW * 32, BN = 64;
+template <int FMT, int D, int NW>
+__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd8_kernel(AttnArgs p) {
+  constexpr int BM = NW * 32, BN = 64;
   constexpr int KSQ = D / 64;          // MFMA k-steps of S^T
   constexpr int DT = D / 32;           // 32-row tiles of O^T
   constexpr int KTILE = BN * D;        // K tile: 64 rows of D bytes
@@ -54,6 +54,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd8_kernel(AttnArgs p) {
   constexpr int STAGE = KTILE + VTILE;
   constexpr int KCH = D / 16;          // 16-byte chunks per K row
   constexpr int KINST = KTILE / 1024 / NW, VINST = VTILE / 1024 / NW;
+  static_assert(KINST >= 1 && VINST >= 1, "tiles too small for this wave count");
 
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
@@ -277,25 +278,31 @@ __global__ __launch_bounds__(256, 2) void attn_fwd8_kernel(AttnArgs p) {
   }
 }
 
-template <int FMT, int D>
+template <int FMT, int D, int NW>
 static int launch_fwd8(const AttnArgs& p, hipStream_t stream) {
-  constexpr int BM = 128;
+  constexpr int BM = NW * 32;
   constexpr int smem = 2 * 2 * 64 * D;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd8_kernel<FMT, D>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd8_kernel<FMT, D, NW>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int nqb = (p.N + BM - 1) / BM;
-  attn_fwd8_kernel<FMT, D><<<dim3(nqb * p.Z * p.H), dim3(256), smem, stream>>>(p);
+  attn_fwd8_kernel<FMT, D, NW><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
+template <int FMT>
+static int launch_fwd8_fmt(const AttnArgs& p, hipStream_t stream) {
+  // variant 2: eight waves (256 query rows per K/V stream), head_dim 128 only
+  if (p.D == 128) return p.variant == 2 ? launch_fwd8<FMT, 128, 8>(p, stream) : launch_fwd8<FMT, 128, 4>(p, stream);
+  return launch_fwd8<FMT, 64, 4>(p, stream);
+}
+
 int attn_fwd8_launch(const AttnArgs& p, bool e5m2, hipStream_t stream) {
-  if (e5m2) return p.D == 128 ? launch_fwd8<1, 128>(p, stream) : launch_fwd8<1, 64>(p, stream);
-  return p.D == 128 ? launch_fwd8<0, 128>(p, stream) : launch_fwd8<0, 64>(p, stream);
+  return e5m2 ? launch_fwd8_fmt<1>(p, stream) : launch_fwd8_fmt<0>(p, stream);
 }
 
 }  // namespace mi355
