@@ -49,7 +49,7 @@ def time_launches(fn, steps, warmup):
     return wall_ms, sum(per) / len(per), per
 
 
-def quick(fn, iters=10, warmup=2):
+def quick(fn, iters=30, warmup=10):
     _, ev_ms, _ = time_launches(fn, iters, warmup)
     return ev_ms
 
