@@ -723,7 +723,7 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
 // ---------------------------------------------------------------------------------------------
 template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
 __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
-  static_assert(!(PERSIST && Cfg::kScaled), "the persistent form exists for the unscaled types");
+  static_assert(!PERSIST || WN == 4, "the persistent form is the eight-wave one");
   using Operand = typename Cfg::Operand;
   constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   static_assert(WN == 2 || WN == 4, "four or eight waves");
@@ -791,13 +791,25 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
   const uint8_t* srcSA = nullptr;
   const uint8_t* srcSB = nullptr;
-  if constexpr (Cfg::kScaled) {
-    // four waves: every wave copies 64 A rows and 64 B rows; eight waves: waves 0-3 the A rows,
-    // waves 4-7 the B rows (the LDS side is A scales then B scales, 256 bytes per wave either way)
+  const uint8_t* nextSA = nullptr;  // PERSIST: the same lane's scale row in the workgroup's next tile
+  // scale rows of this lane in the tile at (tm, tn): four waves: every wave copies 64 A rows and 64 B
+  // rows; eight waves: waves 0-3 the A rows, waves 4-7 the B rows (the LDS side is A scales then B
+  // scales, 256 bytes per wave either way) - `sa` then holds the one pointer the wave needs
+  auto scale_rows = [&](int tm, int tn, const uint8_t*& sa, const uint8_t*& sb) {
     const int w4 = wave & 3;
-    srcSA = p.sA + (int64_t)min(m0 + w4 * 64 + lane, p.M - 1) * p.lds_a;
-    srcSB = p.sB + (int64_t)min(n0 + w4 * 64 + lane, p.N - 1) * p.lds_b;
-    if (NW == 8 && wave >= 4) srcSA = srcSB;
+    sa = p.sA + (int64_t)min(tm + w4 * 64 + lane, p.M - 1) * p.lds_a;
+    sb = p.sB + (int64_t)min(tn + w4 * 64 + lane, p.N - 1) * p.lds_b;
+    if (NW == 8 && wave >= 4) sa = sb;
+  };
+  auto next_tile_scale_rows = [&](int q) {  // q: index of a tile of this workgroup (clamped to the last)
+    int tm, tn;
+    const uint8_t* unused;
+    grouped_tile(lid + min(q, ntw - 1) * G, num_m, num_n, p.group_m, tm, tn);
+    scale_rows(tm * BM, tn * BN, nextSA, unused);
+  };
+  if constexpr (Cfg::kScaled) {
+    scale_rows(m0, n0, srcSA, srcSB);
+    if constexpr (PERSIST) next_tile_scale_rows(1);
   }
 
   const int nfull = p.k_bytes / RBK;
@@ -833,12 +845,20 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // direct load moves 64 rows; past the last group the last one is fetched again
   LDS_PTR(char) const sc_ring = lds + NS * STAGE;
   const int ngroups = p.k_bytes / (RBK * SPG);
-  auto issue_scales = [&](int sg) {
+  // Scale groups are numbered along the workgroup's whole stream of K steps (`gcount` = the group of
+  // the step being multiplied); group number n lives in ring slot n % 2.  `sg` = group inside the
+  // current tile; past its last group comes group 0 of the next tile (PERSIST) or the last group again.
+  int gcount = 0;
+  auto issue_scales = [&](int sg, int slot, int tile_index) {
     if constexpr (Cfg::kScaled) {
-      LDS_PTR(char) dst = sc_ring + (sg & 1) * SC_SLOT + wave * 1024;
-      const int off = min(sg, ngroups - 1) * 16;
-      async_copy16(srcSA + off, (LDS_PTR(void))dst);
-      if constexpr (NW == 4) async_copy16(srcSB + off, (LDS_PTR(void))(dst + BM * 16));
+      LDS_PTR(char) dst = sc_ring + slot * SC_SLOT + wave * 1024;
+      if (PERSIST && sg >= ngroups && tile_index + 1 < ntw) {
+        async_copy16(nextSA, (LDS_PTR(void))dst);
+      } else {
+        const int off = min(sg, ngroups - 1) * 16;
+        async_copy16(srcSA + off, (LDS_PTR(void))dst);
+        if constexpr (NW == 4) async_copy16(srcSB + off, (LDS_PTR(void))(dst + BM * 16));
+      }
     }
   };
 
@@ -992,7 +1012,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
 
   // prologue: NS tiles in flight (past the end of K the last tile again, which keeps the number
   // of outstanding loads - and with it the partial waits - uniform), first half of tile 0 requested
-  issue_scales(0);
+  issue_scales(0, 0, 0);
 #pragma unroll
   for (int s = 0; s < NS; s++) {
     const char* srcA = fillA + fkt * stepA;
@@ -1034,11 +1054,14 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     // ago, and the loads are older than the NS-2 shares the partial waits leave in flight by the
     // time the group is first read (SPG - 1 >= NS - 1 steps from now)
     if constexpr (Cfg::kScaled) {
-      if (kt % SPG == 0) issue_scales(kt / SPG + 1);
+      if (kt % SPG == 0) issue_scales(kt / SPG + 1, (gcount + 1) & 1, ctile);
     }
     {
       const int ktn = kt + 1;
-      const unsigned scbase = lds_addr(sc_ring) + ((ktn / SPG) & 1) * SC_SLOT + Cfg::scale_dword_offset(ktn % SPG);
+      // the next step's scales: same group, or the next one (whose first dword it then reads)
+      const bool new_group = ktn % SPG == 0;
+      const unsigned scbase = lds_addr(sc_ring) + ((gcount + (new_group ? 1 : 0)) & 1) * SC_SLOT + Cfg::scale_dword_offset(ktn % SPG);
+      if (new_group) gcount++;
       LDS_PTR(char) const fill = lds + stage * STAGE;
       const char* srcA = fillA + fkt * stepA;
       const char* srcB = fillB + fkt * stepB;
@@ -1078,6 +1101,10 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
         grouped_tile(lid + min(ctile, ntw - 1) * G, num_m, num_n, p.group_m, pm, pn);
         m0 = pm * BM;
         n0 = pn * BN;
+        if constexpr (Cfg::kScaled) {
+          srcSA = nextSA;
+          next_tile_scale_rows(ctile + 1);
+        }
         wait_vmcnt<0>();
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -1189,7 +1216,7 @@ static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
       whole = p.k_bytes % (RBK * 4 * Cfg::kStepsPerScaleDword) == 0 && p.lds_a % 16 == 0 && p.lds_b % 16 == 0 &&
               ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0;
     }
-    if constexpr (!Cfg::kScaled) {
+    {
       // persistent form (5, eight waves; a four-wave persistent form spills): whole tiles, K steps in
       // whole rings, one workgroup per CU; anything else runs the one-tile-per-workgroup form
       const bool stream_ok = whole && p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % (4 * RBK) == 0 && p.num_programs > 0;
