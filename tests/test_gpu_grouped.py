@@ -33,9 +33,14 @@ def test_reference_example_sizes(gpu, dtype):
         assert np.mean(c == ref) > 0.98
 
 
+@pytest.mark.parametrize("big_min", [None, 1])
 @pytest.mark.parametrize("nprog", [0, 1, 7, 100])
-def test_ragged_problems_are_bit_exact_on_integers(gpu, nprog):
-    # partial tiles, a single row, K tails (K % 32 != 0), and problems without 16-byte rows
+def test_ragged_problems_are_bit_exact_on_integers(gpu, nprog, big_min, monkeypatch):
+    # partial tiles, a single row, K tails (K % 32 != 0), and problems without 16-byte rows; once with
+    # the tile size the library picks for this group (128x128: fewer 256x256 tiles than CUs) and once
+    # with the 256x256 form forced (MI355_GROUPED_BIG_MIN=1)
+    if big_min is not None:
+        monkeypatch.setenv("MI355_GROUPED_BIG_MIN", str(big_min))
     rng = np.random.default_rng(nprog)
     shapes = [(256, 128, 64), (130, 72, 40), (1, 304, 8), (128, 128, 128), (100, 70, 50), (37, 19, 7), (300, 264, 520)]
     ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]

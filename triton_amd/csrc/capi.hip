@@ -205,7 +205,11 @@ int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d
   ga.sizes = d_sizes; ga.lds = d_lds; ga.group_size = group_size; ga.out_dtype = dtype;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const int nprog = num_programs > 0 ? num_programs : 2 * cus;
-  return gemm16_grouped_launch(ga, dtype == MI355_BF16, nprog, (hipStream_t)stream_);
+  // groups with at least one 256x256 tile per CU run 256x256 tiles, one program per CU (never more
+  // programs than the caller asked for); MI355_GROUPED_BIG_MIN moves the threshold (a huge value = never)
+  const int nprog_big = nprog < cus ? nprog : cus;
+  ga.big_tiles_min = env_int("MI355_GROUPED_BIG_MIN", cus);
+  return gemm16_grouped_launch(ga, dtype == MI355_BF16, nprog, nprog_big, (hipStream_t)stream_);
 }
 
 int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const uint8_t* sB, void* C,

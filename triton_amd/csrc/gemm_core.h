@@ -425,11 +425,23 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 // reference assumes full tiles), and a problem whose leading dimensions or N, K are not multiples
 // of 8 elements - no 16-byte rows - is computed by a plain dot-product loop instead.
 // ---------------------------------------------------------------------------------------------
-template <typename Cfg, typename T>
-__global__ __launch_bounds__(256, 1) void gemm_grouped_kernel(GroupedArgs ga) {
-  constexpr int BM = 128, BN = 128, NS = 4;
+// Two instantiations are launched back to back: 256x256 tiles (eight waves, one program per CU) and
+// 128x128 tiles (four waves, two programs per CU).  Both scan the size table first and only one of
+// them works: the large tiles when the group holds at least `big_tiles_min` of them (enough to give
+// every CU one), the small tiles otherwise - a decision every workgroup of both launches reaches
+// alike from the same table, so no host round trip is needed to see sizes that live on the device.
+template <typename Cfg, typename T, int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_grouped_kernel(GroupedArgs ga) {
+  constexpr int NS = 4;
+  constexpr bool BIG = BM == 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
+  {
+    long big_tiles = 0;
+    for (int gi = 0; gi < ga.group_size; gi++)
+      big_tiles += (long)((ga.sizes[gi * 3] + 255) / 256) * ((ga.sizes[gi * 3 + 1] + 255) / 256);
+    if ((big_tiles >= ga.big_tiles_min) != BIG) return;
+  }
   const int nprog = gridDim.x;
   int tile_idx = xcd_remap(blockIdx.x, nprog);
   int last_problem_end = 0;
@@ -450,7 +462,7 @@ __global__ __launch_bounds__(256, 1) void gemm_grouped_kernel(GroupedArgs ga) {
         const int t = tile_idx - last_problem_end;
         const int pm = t / num_n, pn = t % num_n;
         if (rows16) {
-          gemm_tile_body<Cfg, BM, BN, 2, 2, false, NS>(p, pm, pn, lds);
+          gemm_tile_body<Cfg, BM, BN, WM, WN, false, NS>(p, pm, pn, lds);
           // the next tile refills the ring: every wave must be done reading it
           wait_all();
           __syncthreads();
@@ -458,7 +470,7 @@ __global__ __launch_bounds__(256, 1) void gemm_grouped_kernel(GroupedArgs ga) {
           const T* A = (const T*)p.A;
           const T* B = (const T*)p.B;
           T* C = (T*)p.C;
-          for (int e = threadIdx.x; e < BM * BN; e += 256) {
+          for (int e = threadIdx.x; e < BM * BN; e += WM * WN * 64) {
             const int m = pm * BM + e / BN, n = pn * BN + e % BN;
             if (m < gm && n < gn) {
               float acc = 0.f;
@@ -474,18 +486,26 @@ __global__ __launch_bounds__(256, 1) void gemm_grouped_kernel(GroupedArgs ga) {
   }
 }
 
-template <typename Cfg, typename T>
-static int launch_gemm_grouped(const GroupedArgs& ga, int nprog, hipStream_t stream) {
-  constexpr int smem = 4 * (128 + 128) * RBK;
+template <typename Cfg, typename T, int BM, int BN, int WM, int WN>
+static int launch_gemm_grouped_one(const GroupedArgs& ga, int nprog, hipStream_t stream) {
+  constexpr int smem = 4 * (BM + BN) * RBK;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_grouped_kernel<Cfg, T>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_grouped_kernel<Cfg, T, BM, BN, WM, WN>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  gemm_grouped_kernel<Cfg, T><<<dim3(nprog), dim3(256), smem, stream>>>(ga);
+  gemm_grouped_kernel<Cfg, T, BM, BN, WM, WN><<<dim3(nprog), dim3(WM * WN * 64), smem, stream>>>(ga);
   return (int)hipGetLastError();
+}
+
+// nprog: programs of the 128x128 form; nprog_big: programs of the 256x256 form (one per CU)
+template <typename Cfg, typename T>
+static int launch_gemm_grouped(const GroupedArgs& ga, int nprog, int nprog_big, hipStream_t stream) {
+  int rc = launch_gemm_grouped_one<Cfg, T, 256, 256, 2, 4>(ga, nprog_big, stream);
+  if (rc) return rc;
+  return launch_gemm_grouped_one<Cfg, T, 128, 128, 2, 2>(ga, nprog, stream);
 }
 
 // ---------------------------------------------------------------------------------------------

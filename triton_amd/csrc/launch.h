@@ -78,9 +78,10 @@ struct GroupedArgs {
   const int* lds;          // [group_size][3] = lda, ldb, ldc in elements
   int group_size;
   int out_dtype;           // element type of A, B and C: 0 = fp16, 1 = bf16
+  int big_tiles_min;       // 256x256 tiles in the group from which the large-tile kernel takes the launch
 };
 
-int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hipStream_t stream);
+int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
 bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
