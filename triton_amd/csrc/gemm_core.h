@@ -739,7 +739,13 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
 //     tile kt issue; the reads and the direct loads of a step are spread over the first MFMAs of
 //     the step, one or two per MFMA, in program order (scheduling barriers keep them there);
 //   * one barrier per step, at its top: by then every wave holds tile kt in registers (so its
-//     stage may be overwritten) and has seen its own share of tile kt+1 arrive.
+//     stage may be overwritten) and has seen its own share of tile kt+1 arrive;
+//   * between the MFMAs of the K loop there are LDS reads, direct loads and scalar bookkeeping
+//     only: the loads take a scalar tile base plus a fixed 32-bit lane offset, the ring stage
+//     enters the LDS reads as an immediate (the loop is unrolled over the ring);
+//   * PERSIST: one workgroup per CU walks several tiles as one stream of K steps (see below);
+//     otherwise one tile per workgroup, and a partial last K step is finished through a masked
+//     register path.
 // ---------------------------------------------------------------------------------------------
 template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
 __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
