@@ -29,6 +29,34 @@ template <> struct ElemB<f16x8> { using type = _Float16; };
 // before and has seen its own share of the next one arrive; the stage before is refilled there,
 // three stages ahead.
 // ---------------------------------------------------------------------------------------------
+// S and dP MFMAs issued as inline assembly so that their results land in architectural VGPRs
+// while the compiler keeps the dK / dV accumulators (and, through the "a" constraint, the resident
+// K / V fragments) in AGPRs: the softmax and dS arithmetic then reads them directly instead of
+// through one v_accvgpr_read per value.  The compiler inserts no hazard waits for these: the
+// kernel's schedule provides them - a set of S / dP tiles is consumed one phase (at least sixteen
+// MFMAs) after the last MFMA that writes it, and the operands come from LDS reads and global
+// loads (waited for by count), never from VALU results.
+__device__ __forceinline__ void mfma32_first_v(f32x16& d, bf16x8 a, bf16x8 b) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+#endif
+}
+__device__ __forceinline__ void mfma32_first_v(f32x16& d, f16x8 a, f16x8 b) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+#endif
+}
+__device__ __forceinline__ void mfma32_acc_v(f32x16& d, bf16x8 a, bf16x8 b) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+#endif
+}
+__device__ __forceinline__ void mfma32_acc_v(f32x16& d, f16x8 a, f16x8 b) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+#endif
+}
+
 template <typename V8, int D, int NW>
 __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   using S = typename ElemB<V8>::type;
@@ -194,14 +222,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     static_for<KSQ>([&](auto KS_) {
       constexpr int ks = decltype(KS_)::value;
       if constexpr (ks == 0) {
-        f32x16 zero;
-#pragma unroll
-        for (int r = 0; r < 16; r++) zero[r] = 0.f;
-        sacc[par] = mfma32(__builtin_bit_cast(V8, rq[0]), kf[0], zero);
-        dpacc[par] = mfma32(__builtin_bit_cast(V8, rd[0]), vf[0], zero);
+        mfma32_first_v(sacc[par], __builtin_bit_cast(V8, rq[0]), kf[0]);
+        mfma32_first_v(dpacc[par], __builtin_bit_cast(V8, rd[0]), vf[0]);
       } else {
-        sacc[par] = mfma32(__builtin_bit_cast(V8, rq[ks]), kf[ks], sacc[par]);
-        dpacc[par] = mfma32(__builtin_bit_cast(V8, rd[ks]), vf[ks], dpacc[par]);
+        mfma32_acc_v(sacc[par], __builtin_bit_cast(V8, rq[ks]), kf[ks]);
+        mfma32_acc_v(dpacc[par], __builtin_bit_cast(V8, rd[ks]), vf[ks]);
       }
       if constexpr (do_x) {
         static_for<TRK>([&](auto O_) {
