@@ -815,27 +815,34 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     }
   }
   const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
-  const uint8_t* srcSA = nullptr;
-  const uint8_t* srcSB = nullptr;
-  const uint8_t* nextSA = nullptr;  // PERSIST: the same lane's scale row in the workgroup's next tile
-  // scale rows of this lane in the tile at (tm, tn): four waves: every wave copies 64 A rows and 64 B
-  // rows; eight waves: waves 0-3 the A rows, waves 4-7 the B rows (the LDS side is A scales then B
-  // scales, 256 bytes per wave either way) - `sa` then holds the one pointer the wave needs
-  auto scale_rows = [&](int tm, int tn, const uint8_t*& sa, const uint8_t*& sb) {
-    const int w4 = wave & 3;
-    sa = p.sA + (int64_t)min(tm + w4 * 64 + lane, p.M - 1) * p.lds_a;
-    sb = p.sB + (int64_t)min(tn + w4 * 64 + lane, p.N - 1) * p.lds_b;
-    if (NW == 8 && wave >= 4) sa = sb;
+  // Block scales: a scalar base per tile (first scale row of the tile's A rows / B rows) plus a
+  // fixed per-lane row offset, like the operand loads.  Four waves: every wave copies 64 A rows and
+  // 64 B rows; eight waves: waves 0-3 the A rows, waves 4-7 the B rows (the LDS side is A scales
+  // then B scales, 256 bytes per wave either way) - `scA` then is the one base the wave needs.
+  // (Edge tiles clamp rows onto the last one; PERSIST runs on whole tiles, where that is neutral.)
+  const uint8_t* scA = nullptr;
+  const uint8_t* scB = nullptr;
+  const uint8_t* scA_next = nullptr;  // PERSIST: the same base in the workgroup's next tile
+  unsigned scoffA = 0, scoffB = 0;
+  const bool second_half_wave = NW == 8 && wave >= 4;
+  auto scale_base = [&](int tm, int tn, const uint8_t*& a, const uint8_t*& b) {
+    a = p.sA + (int64_t)tm * p.lds_a;
+    b = p.sB + (int64_t)tn * p.lds_b;
+    if (second_half_wave) a = b;
   };
-  auto next_tile_scale_rows = [&](int q) {  // q: index of a tile of this workgroup (clamped to the last)
+  auto next_tile_scale_base = [&](int q) {  // q: index of a tile of this workgroup (clamped to the last)
     int tm, tn;
     const uint8_t* unused;
     grouped_tile(lid + min(q, ntw - 1) * G, num_m, num_n, p.group_m, tm, tn);
-    scale_rows(tm * BM, tn * BN, nextSA, unused);
+    scale_base(tm * BM, tn * BN, scA_next, unused);
   };
   if constexpr (Cfg::kScaled) {
-    scale_rows(m0, n0, srcSA, srcSB);
-    if constexpr (PERSIST) next_tile_scale_rows(1);
+    const int w4 = wave & 3;
+    scoffA = (unsigned)(min(m0 + w4 * 64 + lane, p.M - 1) - m0) * (unsigned)p.lds_a;
+    scoffB = (unsigned)(min(n0 + w4 * 64 + lane, p.N - 1) - n0) * (unsigned)p.lds_b;
+    if (second_half_wave) scoffA = scoffB;
+    scale_base(m0, n0, scA, scB);
+    if constexpr (PERSIST) next_tile_scale_base(1);
   }
 
   const int nfull = p.k_bytes / RBK;
@@ -877,13 +884,13 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   int gcount = 0;
   auto issue_scales = [&](int sg, int slot, int tile_index) {
     if constexpr (Cfg::kScaled) {
-      LDS_PTR(char) dst = sc_ring + slot * SC_SLOT + wave * 1024;
+      const unsigned dst = lds_addr(sc_ring) + slot * SC_SLOT + wave * 1024;
       if (PERSIST && sg >= ngroups && tile_index + 1 < ntw) {
-        async_copy16(nextSA, (LDS_PTR(void))dst);
+        async_copy16_sbase(scA_next, scoffA, dst);
       } else {
         const int off = min(sg, ngroups - 1) * 16;
-        async_copy16(srcSA + off, (LDS_PTR(void))dst);
-        if constexpr (NW == 4) async_copy16(srcSB + off, (LDS_PTR(void))(dst + BM * 16));
+        async_copy16_sbase(scA + off, scoffA, dst);
+        if constexpr (NW == 4) async_copy16_sbase(scB + off, scoffB, dst + BM * 16);
       }
     }
   };
@@ -1128,8 +1135,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
         m0 = pm * BM;
         n0 = pn * BN;
         if constexpr (Cfg::kScaled) {
-          srcSA = nextSA;
-          next_tile_scale_rows(ctile + 1);
+          scA = scA_next;
+          next_tile_scale_base(ctile + 1);
         }
         wait_vmcnt<0>();
         __builtin_amdgcn_sched_barrier(0);
