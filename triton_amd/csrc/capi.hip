@@ -234,8 +234,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  // (the persistent form, tile 5, exists for the scaled types too but measured 3-5 % slower at 8192^3)
-  int tile = (tiles256 * 4 >= 3L * cus) ? 4 : 1;
+  int tile = (tiles256 * 4 >= 3L * cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
   tile = env_int("MI355_GEMM_TILE", tile);
   p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);

@@ -853,11 +853,17 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   const char* fillA = baseA;
   const char* fillB = baseB;
   auto fill_advance = [&]() {
-    if (fkt + 1 < nfull) {
-      fkt++;
-    } else if (PERSIST && ftile + 1 < ntw) {
+    if constexpr (PERSIST) fkt++;  // (tile switches happen between groups of NS steps, below)
+    else if (fkt + 1 < nfull) fkt++;
+  };
+  // PERSIST: a tile's K steps are a multiple of NS and the cursor runs NS positions ahead, so it
+  // reaches the end of a tile exactly at the end of a group of NS steps: the switch to the next tile
+  // (integer divisions of the grouped order) stays out of the step bodies.  After the last tile
+  // the cursor wraps onto its first steps, whose re-fetch into dead stages is harmless.
+  auto fill_next_tile = [&]() {
+    fkt = 0;
+    if (ftile + 1 < ntw) {
       ftile++;
-      fkt = 0;
       int fm, fn;
       grouped_tile(lid + ftile * G, num_m, num_n, p.group_m, fm, fn);
       fillA = p.A + (int64_t)fm * BM * p.lda;
@@ -1053,6 +1059,9 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     static_for<kShare>([&](auto I_) { issue_one(I_, srcA, srcB, lds + s * STAGE); });
     fill_advance();
   }
+  if constexpr (PERSIST) {
+    if (fkt == nfull) fill_next_tile();
+  }
   wait_vmcnt<(NS - 1) * kShare>();
   __builtin_amdgcn_sched_barrier(0);
   block_barrier();
@@ -1115,6 +1124,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     if (s + 2 < nsteps_all) step(std::integral_constant<int, 2>{});
     if (s + 3 < nsteps_all) step(std::integral_constant<int, 3>{});
     if constexpr (PERSIST) {
+      if (fkt == nfull) fill_next_tile();
       // (the host launches this form only when a tile's K steps are a multiple of the ring length, so
       //  tiles end here and the epilogue exists once in the loop body)
       if (ckt == nfull) {
