@@ -338,3 +338,16 @@ def test_fused_epilogues_of_the_reference_dot_test(gpu, dtype, shape):
     wr = randn_rounded(rng, (N, N), dtype, 0.3)
     got = to_np(triton_amd.chain_dot(ta2, tb2, from_np(wr, dtype, gpu)))
     assert np.allclose(got, gemm.dot_epilogue(a2, b2, chain_w=wr, mid_dtype=dtype, out_dtype=dtype), rtol=1e-2, atol=1e-2)
+
+
+def test_skinny_16bit_full_decode_size(gpu):
+    # the table's largest decode shape, M = 16, N = K = 8192 fp16 with a row-major B, against the
+    # fp64 closed form; plus linearity in A (exact: the second operand doubles every product)
+    rng = np.random.default_rng(31)
+    a = randn_rounded(rng, (16, 8192), "fp16", 0.25)
+    b = randn_rounded(rng, (8192, 8192), "fp16", 0.25)
+    ta, tb = from_np(a, "fp16", gpu), from_np(b, "fp16", gpu)
+    c = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+    assert np.allclose(c, gemm.matmul_closed_form(a, b), rtol=1e-2, atol=1e-2)
+    c2 = to_np(triton_amd.matmul(ta * 2, tb, out_dtype=torch.float32))
+    assert bits_equal(c2, 2 * c)
