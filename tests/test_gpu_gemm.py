@@ -278,6 +278,12 @@ def test_skinny_16bit_kernel_is_bit_exact_on_integers(gpu, monkeypatch, dtype, s
         monkeypatch.setenv("MI355_GEMM_SKINNY", "0")      # the tile kernels on the same inputs
         assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), ref)
         monkeypatch.delenv("MI355_GEMM_SKINNY")
+    if dtype == "fp16":
+        # fp8 (K-major B, the `b.T` view): the same streaming kernel with one 32x32x64 MFMA per stage
+        for fmt, tdt in (("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)):
+            ca, cb = formats.encode_fp8(a, fmt), formats.encode_fp8(np.ascontiguousarray(b.T), fmt)
+            t8a, t8b = torch.from_numpy(ca).to(gpu).view(tdt), torch.from_numpy(cb).to(gpu).view(tdt).t()
+            assert bits_equal(to_np(triton_amd.matmul(t8a, t8b, out_dtype=torch.float32)), ref), (fmt, shape)
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])

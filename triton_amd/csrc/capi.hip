@@ -140,7 +140,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent forms (tile 5 / 6): one workgroup per CU
   // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
   const bool skinny_allowed = tile_arg < 0 && env_int("MI355_GEMM_SKINNY", 1);  // an explicit tile means a tile kernel
-  if (!is8 && !aux && skinny_allowed) {
+  if (!aux && skinny_allowed) {
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
@@ -155,8 +155,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       sk.x_pitch = p.ldb; sk.y_pitch = p.lda; sk.cs = scn; sk.cl = scm;
       y_kmajor = true; x_kmajor = b_kmajor; use = true;
     }
-    if (use && gemm16_skinny_ok(sk, y_kmajor, x_kmajor))
-      return gemm16_skinny_launch(sk, in_dtype == MI355_BF16, y_kmajor, x_kmajor, stream);
+    if (use && gemm_skinny_ok(sk, y_kmajor, x_kmajor, es))
+      return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);

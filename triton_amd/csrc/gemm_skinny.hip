@@ -1,4 +1,4 @@
-// Skinny fp16 / bf16 GEMM: one side of the product has at most 64 rows (decode-style M = 16..64,
+// Skinny GEMM (fp16 / bf16, and fp8 with both operands K-contiguous): one side of the product has at most 64 rows (decode-style M = 16..64,
 // or N <= 64), so the work is reading the other operand once from HBM
 // (shapes of python/test/regression/test_performance.py:36-44; kernel contract of
 // python/tutorials/03-matrix-multiplication.py:241-316).
@@ -19,8 +19,17 @@
 
 namespace mi355 {
 
-template <typename V8, bool Y_LDS, int XM, int ST, int NW, int NS>
+// Element families.  A stage is 64 BYTES of every operand row: 32 k of a 16-bit type (two
+// 32x32x16 MFMAs, lane-group g feeding bytes 32 ks + 16 g .. + 16) or 64 k of fp8 (one 32x32x64
+// MFMA, lane-group g feeding bytes 32 g .. + 32 as two 16-byte pieces).
+template <typename V8_> struct Skinny16 { using V = V8_; static constexpr bool kF8 = false; static constexpr int kFmt = 0; };
+template <int FMT> struct Skinny8 { using V = i32x4; static constexpr bool kF8 = true; static constexpr int kFmt = FMT; };  // 0 e4m3fn, 1 e5m2
+
+template <typename E, bool Y_LDS, int XM, int ST, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
+  using V8 = typename E::V;  // one 16-byte register group of an operand
+  constexpr bool F8 = E::kF8;
+  static_assert(!F8 || (!Y_LDS && XM == 2), "fp8: both operands K-contiguous, X through LDS");
   constexpr int PD = NS - 1;          // stages in flight
   constexpr int LPS = 2 + 2 * ST;     // vector-memory operations per stage: 2 of Y, 2 per 32 rows of X
   // X: 0 = K contiguous, straight into registers (32-byte pieces of 32 rows per instruction: slower,
@@ -42,7 +51,7 @@ __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
   // neighbouring 32-column blocks (the two halves of a 128-byte line of an L-contiguous Y) on one XCD
   const int l0 = xcd_remap(blockIdx.x, gridDim.x) * 32;
 
-  const int nstages = p.K / 32;
+  const int nstages = p.K / (F8 ? 64 : 32);
   const int per = (nstages + NW - 1) / NW;
   const int j_lo = wave * per, j_hi = min(nstages, j_lo + per);
 
@@ -71,15 +80,16 @@ __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
   const char* const ybase = Y_LDS ? p.Y + (int64_t)l0 * 2 : p.Y + (int64_t)l0 * p.y_pitch;
   // L-contiguous Y: direct load i of a stage moves k rows 16 i .. 16 i + 15, 64 bytes (32 l) each
   const unsigned yoff = Y_LDS ? (unsigned)(lane >> 2) * (unsigned)p.y_pitch + (lane & 3) * 16
-                              : (unsigned)l32 * (unsigned)p.y_pitch + g * 16;
+                              : (unsigned)l32 * (unsigned)p.y_pitch + g * (F8 ? 32 : 16);
   const unsigned ring = lds_addr(lds) + wave * (NS * SLOT);
   // transposed read: 16 lanes fetch 4 k rows x 16 l and receive 4 k values of one l each;
   // lane -> k row 8 g + i16 / 4 (+ 4 for the second read), l = 16 (q & 1) + i16
   const unsigned tl = ring + (8 * (q >> 1) + (i16 >> 2)) * (XM == 1 ? XROW : 64) + (q & 1) * 32 + (i16 & 3) * 8;
   // row-wise read of the K-contiguous X tile: row s = 32 t + l32, chunk (2 ks + g) ^ ((s >> 2) & 3)
+  // (fp8: the two pieces of the lane's 32 bytes, chunks 2 g and 2 g + 1)
   unsigned xrd[2];
 #pragma unroll
-  for (int ks = 0; ks < 2; ks++) xrd[ks] = ring + YSLOT + l32 * 64 + (((2 * ks + g) ^ ((l32 >> 2) & 3)) << 4);
+  for (int ks = 0; ks < 2; ks++) xrd[ks] = ring + YSLOT + l32 * 64 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 2) & 3)) << 4);
 
   V8 xr[NS][2][ST], yr[NS][2];
   auto issue = [&](int j, auto SLOT_) {
@@ -91,7 +101,7 @@ __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
     } else {
       const char* src = ybase + (int64_t)j * 64;
       load16_sbase<0>(yr[sl][0], src, yoff);
-      load16_sbase<32>(yr[sl][1], src, yoff);
+      load16_sbase<(F8 ? 16 : 32)>(yr[sl][1], src, yoff);
     }
     if constexpr (XM == 1) {
       const char* xsrc = p.X + (int64_t)j * 32 * p.x_pitch;
@@ -179,10 +189,21 @@ __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
           xf[ks][t] = xr[sl][ks][t];
         }
     }
+    if constexpr (F8) {
 #pragma unroll
-    for (int ks = 0; ks < 2; ks++)
+      for (int t = 0; t < ST; t++) {
+        const i32x8 a = __builtin_shufflevector(yf[0], yf[1], 0, 1, 2, 3, 4, 5, 6, 7);
+        const i32x8 b = __builtin_shufflevector(xf[0][t], xf[1][t], 0, 1, 2, 3, 4, 5, 6, 7);
+#if MI355_DEVICE_PASS
+        acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, acc[t], E::kFmt, E::kFmt, 0, 0, 0, 0);
+#endif
+      }
+    } else {
 #pragma unroll
-      for (int t = 0; t < ST; t++) acc[t] = mfma32(yf[ks], xf[ks][t], acc[t]);
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int t = 0; t < ST; t++) acc[t] = mfma32(yf[ks], xf[ks][t], acc[t]);
+    }
   };
 
   if (j_lo < j_hi) {
@@ -236,7 +257,7 @@ __global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
   }
 }
 
-template <typename V8, bool Y_LDS, int XM, int ST>
+template <typename E, bool Y_LDS, int XM, int ST>
 static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   // four waves with three stages in flight each already saturate what this access pattern gets
   // from HBM; the small LDS footprint lets several workgroups share a CU
@@ -245,34 +266,42 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm16_skinny_kernel<V8, Y_LDS, XM, ST, NW, NS>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm16_skinny_kernel<E, Y_LDS, XM, ST, NW, NS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  gemm16_skinny_kernel<V8, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
+  gemm16_skinny_kernel<E, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
-// S <= 64, whole 32-row blocks of Y and whole 32-k stages; pitches in bytes, 16-byte aligned rows,
+// S <= 64, whole 32-row blocks of Y and whole 64-byte stages; pitches in bytes, 16-byte aligned rows,
 // small enough that 64 rows of X / 32 rows of Y are reached with 32-bit offsets.  An S-contiguous
-// X (x_kmajor false) needs S = 32 or 64 and a K-contiguous Y.
-bool gemm16_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor) {
+// X (x_kmajor false) needs S = 32 or 64 and a K-contiguous Y.  elem_bytes = 2 or 1 (fp8: both
+// operands K-contiguous).
+bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_bytes) {
   if (!x_kmajor && (!y_kmajor || (p.S != 32 && p.S != 64))) return false;
-  return p.S >= 1 && p.S <= 64 && p.L >= 32 && p.L % 32 == 0 && p.K >= 32 && p.K % 32 == 0 &&
+  if (elem_bytes == 1 && !(x_kmajor && y_kmajor)) return false;
+  const int64_t kb = (int64_t)p.K * elem_bytes;
+  return p.S >= 1 && p.S <= 64 && p.L >= 32 && p.L % 32 == 0 && kb >= 64 && kb % 64 == 0 &&
          p.x_pitch % 16 == 0 && p.y_pitch % 16 == 0 && p.x_pitch < (1 << 25) && p.y_pitch < (1 << 26);
 }
 
 template <typename V8>
 static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
+  using E = Skinny16<V8>;
   const bool two = p.S > 32;
-  if (!x_kmajor) return two ? launch_skinny<V8, false, 1, 2>(p, stream) : launch_skinny<V8, false, 1, 1>(p, stream);
-  if (y_kmajor) return two ? launch_skinny<V8, false, 2, 2>(p, stream) : launch_skinny<V8, false, 2, 1>(p, stream);
-  return two ? launch_skinny<V8, true, 2, 2>(p, stream) : launch_skinny<V8, true, 2, 1>(p, stream);
+  if (!x_kmajor) return two ? launch_skinny<E, false, 1, 2>(p, stream) : launch_skinny<E, false, 1, 1>(p, stream);
+  if (y_kmajor) return two ? launch_skinny<E, false, 2, 2>(p, stream) : launch_skinny<E, false, 2, 1>(p, stream);
+  return two ? launch_skinny<E, true, 2, 2>(p, stream) : launch_skinny<E, true, 2, 1>(p, stream);
 }
 
-int gemm16_skinny_launch(const SkinnyArgs& p, bool bf16, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
-  return bf16 ? launch_skinny_v<bf16x8>(p, y_kmajor, x_kmajor, stream) : launch_skinny_v<f16x8>(p, y_kmajor, x_kmajor, stream);
+// kind: 0 fp16, 1 bf16, 2 fp8 e4m3fn, 3 fp8 e5m2 (the dtype codes of the C ABI)
+int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
+  const bool two = p.S > 32;
+  if (kind == 2) return two ? launch_skinny<Skinny8<0>, false, 2, 2>(p, stream) : launch_skinny<Skinny8<0>, false, 2, 1>(p, stream);
+  if (kind == 3) return two ? launch_skinny<Skinny8<1>, false, 2, 2>(p, stream) : launch_skinny<Skinny8<1>, false, 2, 1>(p, stream);
+  return kind == 1 ? launch_skinny_v<bf16x8>(p, y_kmajor, x_kmajor, stream) : launch_skinny_v<f16x8>(p, y_kmajor, x_kmajor, stream);
 }
 
 }  // namespace mi355

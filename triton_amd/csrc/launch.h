@@ -43,7 +43,7 @@ struct GemmStridedArgs {
   const void* aux; int64_t aux_sm, aux_sn; int aux_dtype;  // as in GemmArgs
 };
 
-// skinny 16-bit GEMM, out[s][l] = sum_k X[s][k] * Y[l][k]
+// skinny GEMM, out[s][l] = sum_k X[s][k] * Y[l][k]
 struct SkinnyArgs {
   const char* X;    // small operand: S <= 64 rows, K contiguous or S contiguous
   const char* Y;    // streamed operand: L rows, K contiguous or L contiguous
@@ -86,8 +86,8 @@ int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStre
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
 bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
 int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
-bool gemm16_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor);
-int gemm16_skinny_launch(const SkinnyArgs& p, bool bf16, bool y_kmajor, bool x_kmajor, hipStream_t stream);
+bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_bytes);
+int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmajor, hipStream_t stream);
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
