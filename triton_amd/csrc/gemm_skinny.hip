@@ -26,7 +26,7 @@ template <typename V8_> struct Skinny16 { using V = V8_; static constexpr bool k
 template <int FMT> struct Skinny8 { using V = i32x4; static constexpr bool kF8 = true; static constexpr int kFmt = FMT; };  // 0 e4m3fn, 1 e5m2
 
 template <typename E, bool Y_LDS, int XM, int ST, int NW, int NS>
-__global__ __launch_bounds__(NW * 64) void gemm16_skinny_kernel(SkinnyArgs p) {
+__global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   using V8 = typename E::V;  // one 16-byte register group of an operand
   constexpr bool F8 = E::kF8;
   static_assert(!F8 || (!Y_LDS && XM == 2), "fp8: both operands K-contiguous, X through LDS");
@@ -266,12 +266,12 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm16_skinny_kernel<E, Y_LDS, XM, ST, NW, NS>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<E, Y_LDS, XM, ST, NW, NS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  gemm16_skinny_kernel<E, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
+  gemm_skinny_kernel<E, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
