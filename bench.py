@@ -26,7 +26,7 @@ HBM_GBPS = 8000.0
 # HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc:
 # FETCH_SIZE 790628 KiB x 2.000 + WRITE_SIZE 196184 KiB x 1.000, the factors being what the same
 # counters read for a plain copy of known size (profiles/gemm_bf16_8192.md)
-MEASURED_TRAFFIC_BYTES = int((797506 * 2.000 + 182963 * 1.000) * 1024)
+MEASURED_TRAFFIC_BYTES = int((794679 * 2.000 + 186723 * 1.000) * 1024)
 
 
 def time_launches(fn, steps, warmup):
