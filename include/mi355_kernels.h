@@ -67,7 +67,8 @@ enum {
   MI355_Q_CU_COUNT = 1,
   MI355_Q_IS_GFX950 = 2,
   MI355_Q_LDS_BYTES = 3,
-  MI355_Q_CLOCK_KHZ = 4
+  MI355_Q_CLOCK_KHZ = 4,
+  MI355_Q_STREAMK_WORKSPACE_BYTES = 5 /* workspace mi355_gemm_streamk needs on this device */
 };
 
 /*
@@ -114,6 +115,27 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C,
                      int in_dtype, int out_dtype,
                      const float* a_scale, const float* b_scale,
                      int activation, int tile, int group_m, void* stream);
+
+/* mi355_gemm with a stream-K schedule: one program per CU, and the programs split ALL K steps of ALL
+ * 256x256 tiles evenly, so a tile count that is not a multiple of the CU count (or smaller than it:
+ * then this is split-K) still keeps every CU busy to the end.  The persistent schedule of
+ * python/tutorials/09-persistent-matmul.py:141-190 deals whole tiles; this deals their K steps.
+ * A program that covers only part of a tile leaves fp32 partial sums in `workspace` (caller-owned,
+ * at least mi355_query(MI355_Q_STREAMK_WORKSPACE_BYTES) bytes, 16-byte aligned, contents
+ * irrelevant before and after the call) and a second launch on the same stream adds the parts up
+ * in a fixed order: results do not depend on timing.  Nothing waits for another program, so
+ * the call is safe next to other work on the device.  Takes effect for fp16 / bf16 / fp8 operands on
+ * the MFMA path with M and N multiples of 256 and K a multiple of 128 elements (256 for fp8);
+ * any other call runs exactly as mi355_gemm.
+ */
+int mi355_gemm_streamk(const void* A, const void* B, void* C,
+                       int M, int N, int K,
+                       int64_t stride_am, int64_t stride_ak,
+                       int64_t stride_bk, int64_t stride_bn,
+                       int64_t stride_cm, int64_t stride_cn,
+                       int in_dtype, int out_dtype,
+                       const float* a_scale, const float* b_scale,
+                       int activation, void* workspace, size_t workspace_bytes, void* stream);
 
 /* mi355_gemm with the epilogues of the reference's dot test fused in:
  *   C = softmax_rows?( act( (a_scale * b_scale) * A @ B + D ) )

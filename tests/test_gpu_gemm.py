@@ -357,3 +357,35 @@ def test_skinny_16bit_full_decode_size(gpu):
     assert np.allclose(c, gemm.matmul_closed_form(a, b), rtol=1e-2, atol=1e-2)
     c2 = to_np(triton_amd.matmul(ta * 2, tb, out_dtype=torch.float32))
     assert bits_equal(c2, 2 * c)
+
+
+@pytest.mark.parametrize("nprog", [None, 7, 3])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3"])
+def test_stream_k_schedule_is_bit_exact_on_integers(gpu, monkeypatch, dtype, nprog):
+    # mi355_gemm_streamk: programs split all K steps of all 256x256 tiles evenly.  With the device's
+    # CU count (None) these small products are split-K (more programs than tiles); with 7 or 3
+    # programs ranges begin and end inside tiles and span whole tiles in between.  Integer data: the
+    # partial sums are exact, so any split gives the bits of the closed form.  Shapes the schedule
+    # does not take (partial tiles, K tails) run as plain calls.
+    if nprog is not None:
+        monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(nprog))
+    rng = np.random.default_rng(17 + (nprog or 0))
+    for (M, N, K) in [(512, 768, 1024), (256, 256, 4096), (1280, 256, 512), (300, 264, 520), (16, 512, 256)]:
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ref = gemm.matmul_closed_form(a, b, out_dtype="fp32")
+        if dtype == "e4m3":
+            ca, cb = formats.encode_fp8(a, "e4m3"), formats.encode_fp8(np.ascontiguousarray(b.T), "e4m3")
+            ta = torch.from_numpy(ca).to(gpu).view(torch.float8_e4m3fn)
+            tbs = [torch.from_numpy(cb).to(gpu).view(torch.float8_e4m3fn).t()]
+        else:
+            ta = from_np(a, dtype, gpu)
+            tbs = [from_np(b, dtype, gpu), from_np(np.ascontiguousarray(b.T), dtype, gpu).t()]
+        for tb in tbs:
+            got = to_np(triton_amd.matmul_streamk(ta, tb, out_dtype=torch.float32))
+            assert bits_equal(got, ref), (dtype, nprog, M, N, K, tb.stride())
+    # random data against the closed form, output in the input type
+    if dtype != "e4m3":
+        a2, b2 = randn_rounded(rng, (768, 1024), dtype), randn_rounded(rng, (1024, 512), dtype)
+        c = to_np(triton_amd.matmul_streamk(from_np(a2, dtype, gpu), from_np(b2, dtype, gpu)))
+        assert np.allclose(c, gemm.matmul_closed_form(a2, b2, out_dtype=dtype), rtol=1e-2, atol=1e-2)

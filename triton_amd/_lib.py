@@ -7,7 +7,7 @@ becomes a Python exception.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
+from ctypes import c_size_t, c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libmi355_kernels.so"
@@ -17,7 +17,7 @@ F16, BF16, F8E4M3, F8E5M2, F32 = 0, 1, 2, 3, 4
 MXFP4, MXFP8 = 0, 1
 ACT_NONE, ACT_LEAKY_RELU = 0, 1
 DEQ_E4M3, DEQ_E5M2, DEQ_E2M1, DEQ_E8M0 = 0, 1, 2, 3
-Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ = 0, 1, 2, 3, 4
+Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORKSPACE_BYTES = 0, 1, 2, 3, 4, 5
 
 I64x4 = c_int64 * 4
 
@@ -29,6 +29,9 @@ SIGNATURES = {
     "mi355_gemm_tuned": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                  c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mi355_gemm_streamk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                   c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                   c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
     "mi355_gemm_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int, c_int, c_void_p, c_void_p,

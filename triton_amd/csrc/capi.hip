@@ -68,6 +68,7 @@ int mi355_query(int what) {
     case MI355_Q_IS_GFX950: return d.gfx950;
     case MI355_Q_LDS_BYTES: return d.lds;
     case MI355_Q_CLOCK_KHZ: return d.clock_khz;
+    case MI355_Q_STREAMK_WORKSPACE_BYTES: return (d.cus > 0 ? d.cus : 256) * 2 * 256 * 256 * 4;
     default: return -1;
   }
 }
@@ -90,7 +91,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
                      int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
                      int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
                      int activation, const void* aux, int64_t aux_sm, int64_t aux_sn, int aux_dtype,
-                     int tile_arg, int group_m_arg, void* stream_) {
+                     int tile_arg, int group_m_arg, void* stream_, float* workspace = nullptr) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
   if (aux && aux_dtype != MI355_F16 && aux_dtype != MI355_BF16 && aux_dtype != MI355_F32) return MI355_EDTYPE;
   if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
@@ -137,7 +138,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // dynamic dispatch of one workgroup per tile balances better (6144^3: 1011 vs 942 TFLOP/s)
   int tile = (tiles256 * 4 >= 3L * cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
   tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
-  p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent forms (tile 5 / 6): one workgroup per CU
+  p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
+  if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
+  p.workspace = workspace;
   // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
   const bool skinny_allowed = tile_arg < 0 && env_int("MI355_GEMM_SKINNY", 1);  // an explicit tile means a tile kernel
   if (!aux && skinny_allowed) {
@@ -178,6 +181,18 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C, int M, int N, int K,
   if (tile < -1 || tile > 5 || group_m < 0) return MI355_EINVAL;
   return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
                    activation, nullptr, 0, 0, 0, tile, group_m, stream_);
+}
+
+int mi355_gemm_streamk(const void* A, const void* B, void* C, int M, int N, int K,
+                       int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                       int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                       int activation, void* workspace, size_t workspace_bytes, void* stream_) {
+  if (!workspace || !aligned(workspace, 16)) return MI355_EINVAL;
+  if (workspace_bytes < (size_t)mi355_query(MI355_Q_STREAMK_WORKSPACE_BYTES)) return MI355_EINVAL;
+  // partial 256x256 tiles, or fewer than 64 rows on a side (the streaming kernels): the plain call
+  const bool whole_tiles = M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0;
+  return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
+                   activation, nullptr, 0, 0, 0, whole_tiles ? 7 : -1, 0, stream_, (float*)workspace);
 }
 
 int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int K,

@@ -729,6 +729,58 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
   gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
 }
 
+// Stream-K partition: `ntiles * groups_per_tile` groups of K steps dealt evenly to `nprog` programs;
+// program `id` gets the half-open range [lo, hi) of global group indices (tile = index / groups_per_tile).
+struct StreamKRange { long lo, hi; };
+__host__ __device__ inline StreamKRange streamk_range(int ntiles, int groups_per_tile, int nprog, int id) {
+  const long total = (long)ntiles * groups_per_tile;
+  const long per = total / nprog, rem = total % nprog;
+  const long lo = id * per + (id < rem ? id : rem);
+  return {lo, lo + per + (id < rem ? 1 : 0)};
+}
+__host__ __device__ inline int streamk_owner(int ntiles, int groups_per_tile, int nprog, long group) {
+  const long total = (long)ntiles * groups_per_tile;
+  const long per = total / nprog, rem = total % nprog;
+  const long big = rem * (per + 1);
+  return group < big ? (int)(group / (per + 1)) : (int)(rem + (group - big) / per);
+}
+
+// Second kernel of stream-K: one 64-lane workgroup per 32x32 MFMA sub-tile of C (64 per 256x256 tile,
+// so that even a handful of split tiles spreads over the device).  A tile that several programs
+// covered in parts is summed from their workspace slots (in program order: deterministic) and
+// stored through the usual epilogue; tiles one program covered alone were stored by it already.
+// Workspace layout of a partial tile: [wave][i][j][lane][16 accumulator registers], i.e. 64 bytes per
+// lane and sub-tile, written and read with 16-byte accesses.
+template <int WN>
+__global__ __launch_bounds__(64) void gemm_streamk_fixup_kernel(GemmArgs p, int nprog, int groups_per_tile) {
+  constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
+  constexpr int SUB = NW * MT * NT;  // 32x32 sub-tiles per tile
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
+  const int t = blockIdx.x / SUB, sub = blockIdx.x % SUB;
+  const int first = streamk_owner(num_m * num_n, groups_per_tile, nprog, (long)t * groups_per_tile);
+  const int last = streamk_owner(num_m * num_n, groups_per_tile, nprog, (long)(t + 1) * groups_per_tile - 1);
+  if (first == last) return;
+  const int lane = threadIdx.x;
+  const int wave = sub / (MT * NT), i = (sub / NT) % MT, j = sub % NT;
+  const int wm = wave / WN, wn = wave % WN, l32 = lane & 31, g = lane >> 5;
+  f32x4 sum[4];
+#pragma unroll
+  for (int q = 0; q < 4; q++) sum[q] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int prog = first; prog <= last; prog++) {
+    const StreamKRange r = streamk_range(num_m * num_n, groups_per_tile, nprog, prog);
+    const int slot = (int)(r.lo / groups_per_tile) == t ? 0 : 1;
+    const f32x4* ws = (const f32x4*)(p.workspace + ((int64_t)prog * 2 + slot) * (BM * BN) + (int64_t)sub * 1024 + lane * 16);
+#pragma unroll
+    for (int q = 0; q < 4; q++) sum[q] += ws[q];
+  }
+  f32x16 acc[1][1];
+#pragma unroll
+  for (int r = 0; r < 16; r++) acc[0][0][r] = sum[r >> 2][r & 3];
+  int pm, pn;
+  grouped_tile(t, num_m, num_n, p.group_m, pm, pn);
+  gemm_epilogue<1, 1>(acc, p, pm * BM + wm * TM + i * 32, pn * BN + wn * TN + j * 32, l32, g);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Software-pipelined variant of the 256x256 tile, four or eight waves.  With four: one wave per SIMD, each owning a 128x128 quarter of C
 // (256 accumulator registers).  Per K step a wave reads (4 + 4) x 32 operand rows from LDS for
@@ -747,9 +799,10 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
 //     otherwise one tile per workgroup, and a partial last K step is finished through a masked
 //     register path.
 // ---------------------------------------------------------------------------------------------
-template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
+template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false, bool SK = false>
 __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   static_assert(!PERSIST || WN == 4, "the persistent form is the eight-wave one");
+  static_assert(!SK || (PERSIST && !Cfg::kScaled), "stream-K builds on the persistent form of the unscaled types");
   using Operand = typename Cfg::Operand;
   constexpr int BM = 256, BN = 256, WM = 2, NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   static_assert(WN == 2 || WN == 4, "four or eight waves");
@@ -779,13 +832,31 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   // 141-190) gridDim.x workgroups that each walk tiles lid, lid + G, lid + 2G, ... of the grouped
   // order as ONE stream of K steps: the direct loads run NS steps ahead across tile boundaries, so
   // the ring never drains between tiles.  lid keeps the workgroups of one XCD on neighbouring tiles.
+  // SK (stream-K): the G programs instead split ALL K steps of ALL tiles evenly (in groups of NS
+  // steps, tiles in the grouped order): program lid walks one contiguous range of the global step
+  // sequence, which may begin and end in the middle of a tile.  A tile it covers completely is
+  // stored as usual; of a tile it covers partly it leaves the fp32 partial sums in the workspace
+  // (slot 0 = the tile its range begins in, slot 1 = the tile it ends in) and a second kernel adds
+  // the partial tiles up.  No program ever waits for another one.
   const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
   const int ntiles = num_m * num_n;
   const int G = PERSIST ? (int)gridDim.x : ntiles;
   const int lid = xcd_remap(blockIdx.x, G);
-  const int ntw = PERSIST ? (ntiles - lid + G - 1) / G : 1;  // tiles of this workgroup (the host keeps G <= ntiles)
+  const int nfull = p.k_bytes / RBK;
+  int sk_first_tile = 0, sk_kt0 = 0, sk_steps = 0;
+  if constexpr (SK) {
+    const StreamKRange r = streamk_range(ntiles, nfull / NS, G, lid);
+    sk_first_tile = (int)(r.lo / (nfull / NS));
+    sk_kt0 = (int)(r.lo % (nfull / NS)) * NS;
+    sk_steps = (int)(r.hi - r.lo) * NS;
+    if (sk_steps == 0) return;  // more programs than groups of steps
+  }
+  const int sk_last_tile = SK ? sk_first_tile + (sk_kt0 + sk_steps - 1) / nfull : 0;
+  // tiles of this workgroup (PERSIST: the host keeps G <= ntiles) and the q-th of them
+  const int ntw = SK ? sk_last_tile - sk_first_tile + 1 : PERSIST ? (ntiles - lid + G - 1) / G : 1;
+  auto tile_id = [&](int q) { return SK ? sk_first_tile + q : lid + q * G; };
   int pm, pn;
-  grouped_tile(lid, num_m, num_n, p.group_m, pm, pn);
+  grouped_tile(tile_id(0), num_m, num_n, p.group_m, pm, pn);
   int m0 = pm * BM, n0 = pn * BN;  // tile being multiplied
 
   // Sources of the direct loads: a scalar tile base that advances with kt plus a 32-bit per-lane
@@ -833,7 +904,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   auto next_tile_scale_base = [&](int q) {  // q: index of a tile of this workgroup (clamped to the last)
     int tm, tn;
     const uint8_t* unused;
-    grouped_tile(lid + min(q, ntw - 1) * G, num_m, num_n, p.group_m, tm, tn);
+    grouped_tile(tile_id(min(q, ntw - 1)), num_m, num_n, p.group_m, tm, tn);
     scale_base(tm * BM, tn * BN, scA_next, unused);
   };
   if constexpr (Cfg::kScaled) {
@@ -845,11 +916,10 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     if constexpr (PERSIST) next_tile_scale_base(1);
   }
 
-  const int nfull = p.k_bytes / RBK;
   // Fill cursor: the (tile, K step) the next direct loads fetch.  It runs NS positions ahead of the
   // multiplication and stops on the last position of the workgroup's stream (which is then fetched
   // again into a dead stage: the number of outstanding loads, and with it the partial waits, stays uniform).
-  int ftile = 0, fkt = 0;
+  int ftile = 0, fkt = SK ? sk_kt0 : 0;
   const char* fillA = baseA;
   const char* fillB = baseB;
   auto fill_advance = [&]() {
@@ -865,7 +935,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     if (ftile + 1 < ntw) {
       ftile++;
       int fm, fn;
-      grouped_tile(lid + ftile * G, num_m, num_n, p.group_m, fm, fn);
+      grouped_tile(tile_id(ftile), num_m, num_n, p.group_m, fm, fn);
       fillA = p.A + (int64_t)fm * BM * p.lda;
       fillB = B_KMAJOR ? p.B + (int64_t)fn * BN * p.ldb : p.B + (int64_t)fn * BN * 2;
     }
@@ -1070,7 +1140,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
 
   // one K step of the tile in ring stage STG (its parity, for the one-sub-step types, is STG % 2);
   // kt = K step inside the current tile
-  int ckt = 0, ctile = 0;
+  int ckt = SK ? sk_kt0 : 0, ctile = 0;
+  int seg_kt0 = ckt;  // SK: K step at which this program entered the current tile
   auto step = [&](auto STG_) {
     const int kt = ckt;
     constexpr int stage = decltype(STG_)::value, P = stage & 1;
@@ -1117,7 +1188,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     }
     ckt++;
   };
-  const int nsteps_all = ntw * nfull;
+  const int nsteps_all = SK ? sk_steps : ntw * nfull;
   for (int s = 0; s < nsteps_all; s += NS) {
     step(std::integral_constant<int, 0>{});
     if (s + 1 < nsteps_all) step(std::integral_constant<int, 1>{});
@@ -1127,12 +1198,28 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       if (fkt == nfull) fill_next_tile();
       // (the host launches this form only when a tile's K steps are a multiple of the ring length, so
       //  tiles end here and the epilogue exists once in the loop body)
-      if (ckt == nfull) {
+      if (ckt == nfull || (SK && s + NS >= nsteps_all)) {
         // tile finished: store it, start the next one.  The stores share the vector-memory counter
         // with the direct loads and may complete out of order with them, so the counter is drained
         // once per tile before the partial waits count again (the loads for the next tile's first
         // steps were issued during the last steps of this one and have been in flight since).
-        gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+        if (SK && (seg_kt0 != 0 || ckt != nfull)) {
+          // part of a tile: raw partial sums, register order (the second kernel reads them back alike)
+          // ([wave][i][j][lane][16 registers]: 64 bytes per lane and 32x32 sub-tile)
+          float* ws = p.workspace + ((int64_t)lid * 2 + (ctile == 0 ? 0 : 1)) * (BM * BN) + lane * 16;
+          static_for<MT>([&](auto I_) {
+            static_for<NT>([&](auto J_) {
+              constexpr int i = decltype(I_)::value, j = decltype(J_)::value;
+              f32x4* dst = (f32x4*)(ws + ((wave * MT + i) * NT + j) * 1024);
+#pragma unroll
+              for (int q = 0; q < 4; q++)
+                dst[q] = f32x4{acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+            });
+          });
+        } else {
+          gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
+        }
+        seg_kt0 = 0;
 #pragma unroll
         for (int i = 0; i < MT; i++)
 #pragma unroll
@@ -1141,7 +1228,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
         ckt = 0;
         ctile++;
-        grouped_tile(lid + min(ctile, ntw - 1) * G, num_m, num_n, p.group_m, pm, pn);
+        grouped_tile(tile_id(min(ctile, ntw - 1)), num_m, num_n, p.group_m, pm, pn);
         m0 = pm * BM;
         n0 = pn * BN;
         if constexpr (Cfg::kScaled) {
@@ -1193,22 +1280,26 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   if constexpr (!PERSIST) gemm_epilogue<MT, NT>(acc, p, m0 + wm * TM, n0 + wn * TN, l32, g);
 }
 
-template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false>
+template <typename Cfg, int WN, bool B_KMAJOR, int NS, bool PERSIST = false, bool SK = false>
 static int launch_gemm_w4(const GemmArgs& p, hipStream_t stream, int num_programs = 0) {
   constexpr int BM = 256, BN = 256;
   constexpr int smem = NS * (BM + BN) * RBK + (Cfg::kScaled ? 2 * (BM + BN) * 16 : 0);
   static_assert(smem <= 160 * 1024, "LDS ring does not fit");
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST, SK>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN;
   int grid = num_m * num_n;
-  if (PERSIST && num_programs > 0 && num_programs < grid) grid = num_programs;
-  gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST><<<dim3(grid), dim3(2 * WN * 64), smem, stream>>>(p);
+  if (SK) grid = num_programs;
+  else if (PERSIST && num_programs > 0 && num_programs < grid) grid = num_programs;
+  gemm_w4_kernel<Cfg, WN, B_KMAJOR, NS, PERSIST, SK><<<dim3(grid), dim3(2 * WN * 64), smem, stream>>>(p);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess || !SK) return (int)e;
+  gemm_streamk_fixup_kernel<WN><<<dim3(num_m * num_n * 64), dim3(64), 0, stream>>>(p, grid, (p.k_bytes / RBK) / NS);
   return (int)hipGetLastError();
 }
 
@@ -1263,6 +1354,10 @@ static int launch_gemm_tile(const GemmArgs& p, int tile, hipStream_t stream) {
       // persistent form (5, eight waves; a four-wave persistent form spills): whole tiles, K steps in
       // whole rings, one workgroup per CU; anything else runs the one-tile-per-workgroup form
       const bool stream_ok = whole && p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % (4 * RBK) == 0 && p.num_programs > 0;
+      if constexpr (!Cfg::kScaled) {
+        // 7: stream-K (needs the caller's workspace: two 256x256 fp32 tiles per program)
+        if (tile == 7 && stream_ok && p.workspace != nullptr) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4, true, true>(p, stream, p.num_programs);
+      }
       if (tile >= 5 && stream_ok) return launch_gemm_w4<Cfg, 4, B_KMAJOR, 4, true>(p, stream, p.num_programs);
       if (tile >= 5) tile = 4;
     }

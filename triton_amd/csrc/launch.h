@@ -21,6 +21,7 @@ struct GemmArgs {
   int out_dtype;  // MI355_F16 / MI355_BF16 / MI355_F32 (fp8 kernels also MI355_F8E4M3)
   int group_m;
   int num_programs;  // persistent kernels: workgroups to launch (0 = not persistent)
+  float* workspace;  // stream-K: 2 * num_programs tiles of 256x256 fp32 (NULL = no stream-K)
   int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
   // optional addend of the epilogue: acc * alpha + aux[m * aux_sm + n * aux_sn] (a zero stride broadcasts
   // a row or a column vector), added in fp32 before the activation; NULL = none

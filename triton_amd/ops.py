@@ -131,6 +131,44 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     return c
 
 
+_streamk_workspace = {}
+
+
+def matmul_streamk(a, b, *, out_dtype=None):
+    """`matmul(a, b)` with the stream-K schedule: one program per CU, all K steps of all 256x256
+    tiles dealt evenly, so tile counts that are not a multiple of the CU count - or smaller than it,
+    where this becomes split-K - keep every CU busy.  The scheduling idea of the persistent
+    tutorial (python/tutorials/09-persistent-matmul.py:141-190) taken one step further; the
+    result is the same `a @ b` (partial tiles are added in a fixed order).  A per-device fp32
+    workspace is allocated on first use and kept."""
+    assert a.shape[1] == b.shape[0], "Incompatible dimensions"
+    assert _is_contiguous(a), "Matrix A must be contiguous"
+    in_dt = _abi_dtype(a)
+    assert in_dt == _abi_dtype(b), "Incompatible dtypes"
+    _check_device(0, a)
+    _check_device(1, b)
+    M, K = a.shape
+    _, N = b.shape
+    if out_dtype is None:
+        out_dtype = torch.bfloat16 if in_dt == _lib.BF16 else torch.float16
+    c = torch.empty((M, N), device=a.device, dtype=out_dtype)
+    if M == 0 or N == 0:
+        return c
+    if K == 0:
+        return c.zero_()
+    lib = _lib.load()
+    ws = _streamk_workspace.get(a.device)
+    if ws is None:
+        ws = torch.empty(lib.mi355_query(_lib.Q_STREAMK_WORKSPACE_BYTES), device=a.device, dtype=torch.uint8)
+        _streamk_workspace[a.device] = ws
+    rc = lib.mi355_gemm_streamk(
+        a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+        a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+        in_dt, _TORCH_TO_ABI[out_dtype], 0, 0, _lib.ACT_NONE, ws.data_ptr(), ws.numel(), _stream())
+    _lib.check(rc, "mi355_gemm_streamk")
+    return c
+
+
 def chain_dot(a, b, w, *, out_dtype=None):
     """(A @ B) rounded to the input type, then @ W: the CHAIN_DOT branch of the reference's dot test
     (python/test/unit/language/test_core.py:3142-3144, `tl.dot(z.to(w.dtype), w)`), as two launches."""
