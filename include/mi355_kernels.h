@@ -202,7 +202,8 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
  * Stands in for the launch of `_attn_fwd` by `_attention.forward`
  *   python/tutorials/06-fused-attention.py:98-187 (kernel), :25-75 (inner loop), :441-475 (host).
  * q,k,v,o are [Z,H,N_CTX,D] with the four element strides given per tensor (last stride must be 1);
- * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {64, 128}.
+ * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {64, 128, 256}
+ * (the backward entries take 64 and 128 only and return MI355_ESHAPE for 256).
  * fp8 forward (dtype MI355_F8E5M2 as in the reference's fp8 benchmark, :609-614, or MI355_F8E4M3):
  * q, k and o as above, v transposed in memory (stride 1 along N_CTX, a multiple of 16 along D:
  * what `v.permute(0,1,3,2).contiguous().permute(0,1,3,2)` yields); P is rounded to the fp8 type

@@ -121,3 +121,32 @@ def test_full_size_config3_sampled_heads(gpu, causal):
         gsl = lambda x: to_np(x[z:z + 1, h:h + 1])
         for name, got in (("o", gsl(o)), ("dq", gsl(tq.grad)), ("dk", gsl(tk.grad)), ("dv", gsl(tv.grad))):
             assert np.allclose(got, cf[name], atol=3e-2, rtol=1e-2), (name, z, h)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("causal", [True, False])
+def test_head_dim_256_forward(gpu, dtype, causal):
+    # the reference accepts HEAD_DIM 256 (06:447); here it exists for the forward (and its M) only:
+    # 512-byte K/V rows, 64 KiB LDS stages, one wave per SIMD.  The backward reports the shape.
+    shape = (1, 2, 384, 256)
+    (q, k, v, do), (tq, tk, tv, tdo) = _inputs(7, shape, dtype, gpu)
+    sm_scale = 256 ** -0.5
+    cf = A.attn_closed_form(q, k, v, causal, sm_scale)
+    from triton_amd import _lib
+    o = torch.empty_like(tq)
+    M = torch.empty(shape[:3], dtype=torch.float32, device=gpu)
+    I4 = _lib.I64x4
+    rc = _lib.load().mi355_attn_fwd(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(), M.data_ptr(),
+                                    *shape, I4(*tq.stride()), I4(*tk.stride()), I4(*tv.stride()), I4(*o.stride()),
+                                    sm_scale, int(causal), _lib.BF16 if dtype == "bf16" else _lib.F16,
+                                    torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert np.allclose(to_np(o), cf["o"], atol=1e-2, rtol=1e-2)
+    assert np.allclose(to_np(M), cf["M"], atol=2e-3, rtol=0)
+    if causal:
+        assert np.allclose(to_np(o)[:, :, 0], v[:, :, 0], atol=1e-3)   # the first query sees only the first key
+    tq.requires_grad_()
+    out = triton_amd.attention(tq, tk, tv, causal, sm_scale)
+    assert np.allclose(to_np(out.detach()), cf["o"], atol=1e-2, rtol=1e-2)
+    with pytest.raises(ValueError):
+        out.backward(tdo)

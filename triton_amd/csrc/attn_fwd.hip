@@ -1,4 +1,4 @@
-// Fused flash-attention forward for gfx950 (fp16 / bf16, head_dim 64 or 128).
+// Fused flash-attention forward for gfx950 (fp16 / bf16, head_dim 64, 128 or 256).
 //
 // Same algorithm as the reference `_attn_fwd` / `_attn_fwd_inner`
 // (python/tutorials/06-fused-attention.py:25-75, :98-187): a Q tile stays resident, K/V stream
@@ -136,7 +136,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
 
   auto step = [&](const int j, auto STAGE_) {
     constexpr int stage = decltype(STAGE_)::value;
-    constexpr int KOFF = stage * 2 * TILE, VOFF = KOFF + TILE;
+    // the stage offset rides in the instructions' 16-bit immediates where two stages fit below 64 KiB;
+    // with 512-byte rows (head_dim 256) a stage is 64 KiB and its offset is added to the addresses
+    constexpr bool kStageImm = 2 * 2 * TILE <= 65536;
+    constexpr int KOFF = kStageImm ? stage * 2 * TILE : 0, VOFF = KOFF + TILE;
+    const unsigned sreg = kStageImm ? 0u : (unsigned)(stage * 2 * TILE);
     if (j + 1 < nsteps) issue_kv(j + 1, stage ^ 1);
     if (j <= wave_last && row0 < p.N) {
       // ---- S^T = K Q^T : [2 kv tiles][QT q tiles]
@@ -149,14 +153,14 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           for (int r = 0; r < 16; r++) s[a][b][r] = 0.f;
       {
         i32x4 kf[2][2];
-        kf[0][0] = lds_read_b128<KOFF>(ka[0]);
-        kf[0][1] = lds_read_b128<KOFF + 32 * RB>(ka[0]);
+        kf[0][0] = lds_read_b128<KOFF>(ka[0] + sreg);
+        kf[0][1] = lds_read_b128<KOFF + 32 * RB>(ka[0] + sreg);
         static_for<KSQ>([&](auto KS_) {
           constexpr int ks = decltype(KS_)::value;
           constexpr int cur = ks & 1, nxt = cur ^ 1;
           if constexpr (ks + 1 < KSQ) {
-            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + 1]);
-            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + 1]);
+            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + 1] + sreg);
+            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + 1] + sreg);
             lds_wait<2>();
           } else {
             lds_wait<0>();
@@ -224,8 +228,8 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
           constexpr int t = decltype(T_)::value;
           static_for<DT>([&](auto C_) {
             constexpr int c = decltype(C_)::value;
-            dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0]);
-            dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1]);
+            dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0] + sreg);
+            dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1] + sreg);
           });
         };
         read_v(std::integral_constant<int, 0>{}, vf[0]);
@@ -612,8 +616,10 @@ static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
 
 template <typename V8>
 static int launch_fwd_d(const AttnArgs& p, int variant, hipStream_t stream) {
-  if (variant == 3) return p.D == 128 ? launch_fwd_stream<V8, 128, 4>(p, stream) : launch_fwd_stream<V8, 64, 4>(p, stream);
-  if (variant == 4) return p.D == 128 ? launch_fwd_stream<V8, 128, 8>(p, stream) : launch_fwd_stream<V8, 64, 8>(p, stream);
+  if (variant == 3 && p.D != 256) return p.D == 128 ? launch_fwd_stream<V8, 128, 4>(p, stream) : launch_fwd_stream<V8, 64, 4>(p, stream);
+  if (variant == 4 && p.D != 256) return p.D == 128 ? launch_fwd_stream<V8, 128, 8>(p, stream) : launch_fwd_stream<V8, 64, 8>(p, stream);
+  // head_dim 256: four waves of 32 query rows, one wave per SIMD (the O accumulator alone is 128 registers)
+  if (p.D == 256) return launch_fwd<V8, 256, 1, 4>(p, stream);
   if (p.D == 128) {
     if (variant == 2) return launch_fwd<V8, 128, 1, 8>(p, stream);
     return variant == 1 ? launch_fwd<V8, 128, 1, 4>(p, stream) : launch_fwd<V8, 128, 2, 4>(p, stream);

@@ -4,7 +4,7 @@
 //
 // One XOR swizzle of the 16-byte chunk index serves both patterns on the 64-bank (256 bytes per
 // sweep) LDS:
-//   D = 128 (256-byte rows):  chunk ^= ((row & 3) << 2) | ((row >> 2) & 3)
+//   D = 128, 256 (256- / 512-byte rows):  chunk ^= ((row & 3) << 2) | ((row >> 2) & 3)
 //   D =  64 (128-byte rows):  chunk ^= (((row >> 1) & 1) << 2) | ((row >> 2) & 3)
 // Row-wise reads are served 16 lanes (16 consecutive rows, one logical chunk) at a time: the XOR
 // value is a bijection of row & 15 (for 128-byte rows together with the half-sweep bit row & 1),
@@ -18,7 +18,8 @@ namespace mi355 {
 
 template <int RB>
 __device__ __forceinline__ int tile_swz(int row) {
-  if constexpr (RB == 256) return ((row & 3) << 2) | ((row >> 2) & 3);
+  // rows of 256 bytes or more start on a bank-sweep boundary: the same four XOR bits serve both
+  if constexpr (RB >= 256) return ((row & 3) << 2) | ((row >> 2) & 3);
   else return (((row >> 1) & 1) << 2) | ((row >> 2) & 3);
 }
 
@@ -75,7 +76,7 @@ struct TrRead {
   unsigned tl;
   __device__ TrRead(int i16, int q4) {
     const int g = q4 >> 1, x = i16 >> 2, e = 2 * (q4 & 1) + ((i16 & 3) >> 1);
-    const int xs = RB == 256 ? x : (x >> 1);
+    const int xs = RB >= 256 ? x : (x >> 1);
     tl = (4 * g + x) * RB + (xs << 6) + ((e ^ g) << 4) + (i16 & 1) * 8;
   }
   template <int C, int H>

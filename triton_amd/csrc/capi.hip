@@ -263,10 +263,12 @@ int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* st
   return dequant_launch(codes, out, n, fmt, (hipStream_t)stream_);
 }
 
-static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype) {
+static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype, bool allow_256 = false) {
   if (Z <= 0 || H <= 0 || N_CTX <= 0) return MI355_EINVAL;
   if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
-  if (D != 64 && D != 128) return MI355_ESHAPE;
+  // head_dim 256 exists for the 16-bit forward only (the backward kernels keep K, V and both
+  // accumulators of a key block in registers, which 256 columns do not fit)
+  if (D != 64 && D != 128 && !(allow_256 && D == 256)) return MI355_ESHAPE;
   if (N_CTX % 128 != 0) return MI355_ESHAPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
   p.Z = Z; p.H = H; p.N = N_CTX; p.D = D;
@@ -301,7 +303,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     p.variant = env_int("MI355_ATTN_FWD_VARIANT", 1);  // fp8: four waves, two workgroups per CU (eight waves measured 6-12 % slower)
     return attn_fwd8_launch(p, dtype == MI355_F8E5M2, (hipStream_t)stream_);
   }
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
   if (rc) return rc;
   if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))
     return MI355_EINVAL;
