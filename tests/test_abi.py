@@ -98,3 +98,26 @@ def test_dtype_names_of_reinterpreted_tensors():
             name = "fp8e4nv"
     assert ops._abi_dtype(Wrapped()) == _lib.F8E4M3
     assert ops._abi_dtype(torch.zeros(1, dtype=torch.bfloat16)) == _lib.BF16
+
+
+def test_launch_record_matches_the_tutorial_formulas():
+    # python/tutorials/09-persistent-matmul.py:34-45 and 06-fused-attention.py:630-634, evaluated lazily
+    from triton_amd import hooks
+
+    calls = []
+
+    def counted(*args):
+        calls.append(args)
+        return hooks.matmul_launch_metadata(*args)
+
+    md = hooks.LaunchMetadata({"name": "k", "stream": 7})
+    md.add(counted, ("k", 16, 8192, 8192, 1))
+    assert calls == []                       # nothing evaluated until a hook asks
+    rec = md.get()
+    assert rec == {"name": "k [M=16, N=8192, K=8192]", "stream": 7, "flops8": 2.0 * 16 * 8192 * 8192,
+                   "bytes": 16 * 8192 + 8192 * 8192}
+    md.get()
+    assert len(calls) == 1                   # and only once
+    rec = hooks.attention_launch_metadata("a", 4, 32, 4096, 128, False, 2)
+    assert rec["flops16"] == 2 * 2.0 * 4 * 32 * 4096 * 4096 * 128
+    assert hooks.enter("x", 0, hooks.matmul_launch_metadata, ("x", 1, 1, 1, 2)) is None   # no hook set

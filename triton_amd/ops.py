@@ -14,7 +14,7 @@ import math
 
 import torch
 
-from . import _lib
+from . import _lib, hooks
 
 _TORCH_TO_ABI = {
     torch.float16: _lib.F16,
@@ -29,6 +29,7 @@ _NAME_TO_ABI = {
     "float16": _lib.F16, "bfloat16": _lib.BF16, "float8_e4m3fn": _lib.F8E4M3, "float8_e5m2": _lib.F8E5M2,
 }
 _ABI_TO_TORCH = {v: k for k, v in _TORCH_TO_ABI.items()}
+_ELEM_BYTES = {_lib.F16: 2, _lib.BF16: 2, _lib.F8E4M3: 1, _lib.F8E5M2: 1, _lib.F32: 4}
 
 
 def _abi_dtype(t) -> int:
@@ -109,12 +110,15 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     pa, keep_a = _scale_ptr(a_scale, device)
     pb, keep_b = _scale_ptr(b_scale, device)
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
+    stream = _stream()
+    md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K, _ELEM_BYTES[in_dt]))
     if add is None and not softmax:
         rc = _lib.load().mi355_gemm(
             a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
             a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
-            in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, act, _stream())
+            in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, act, stream)
         _lib.check(rc, "mi355_gemm")
+        hooks.exit(md)
         return c
     d_ptr, d_sm, d_sn, d_dt = 0, 0, 0, 0
     if add is not None:
@@ -126,8 +130,9 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     rc = _lib.load().mi355_gemm_epilogue(
         a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
         a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
-        in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, d_ptr, d_sm, d_sn, d_dt, act, int(bool(softmax)), _stream())
+        in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, d_ptr, d_sm, d_sn, d_dt, act, int(bool(softmax)), stream)
     _lib.check(rc, "mi355_gemm_epilogue")
+    hooks.exit(md)
     return c
 
 
@@ -188,11 +193,14 @@ def matmul_like_input(a, b):
     M, K = a.shape
     K, N = b.shape
     c = torch.empty((M, N), device=a.device, dtype=a.dtype)
+    stream = _stream()
+    md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K, _ELEM_BYTES[in_dt]))
     rc = _lib.load().mi355_gemm(
         a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
         a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
-        in_dt, in_dt, None, None, _lib.ACT_NONE, _stream())
+        in_dt, in_dt, None, None, _lib.ACT_NONE, stream)
     _lib.check(rc, "mi355_gemm")
+    hooks.exit(md)
     return c
 
 
@@ -310,12 +318,16 @@ class _attention(torch.autograd.Function):
         Z, H, N_CTX = q.shape[0], q.shape[1], q.shape[2]
         M = torch.empty((Z, H, N_CTX), device=q.device, dtype=torch.float32)
         I4 = _lib.I64x4
+        stream = _stream()
+        md = hooks.enter("mi355_attn_fwd", stream, hooks.attention_launch_metadata,
+                         ("mi355_attn_fwd", Z, H, N_CTX, HEAD_DIM_K, causal, _ELEM_BYTES[dt]))
         rc = _lib.load().mi355_attn_fwd(
             q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr(),
             Z, H, N_CTX, HEAD_DIM_K,
             I4(*q.stride()), I4(*k.stride()), I4(*v.stride()), I4(*o.stride()),
-            float(sm_scale), int(bool(causal)), dt, _stream())
+            float(sm_scale), int(bool(causal)), dt, stream)
         _lib.check(rc, "mi355_attn_fwd")
+        hooks.exit(md)
         ctx.save_for_backward(q, k, v, o, M)
         ctx.sm_scale = sm_scale
         ctx.HEAD_DIM = HEAD_DIM_K
