@@ -99,8 +99,11 @@ def test_unsupported_configurations_raise(gpu):
     with pytest.raises(ValueError):          # N_CTX must be a multiple of 128 here (the reference asserts it in backward, 06:494)
         triton_amd.attention(q, q, q, True, 0.5)
     q32 = torch.zeros(1, 1, 128, 32, dtype=torch.float16, device=gpu)
-    with pytest.raises(ValueError):          # head_dim 32 passes the reference's assert (06:447) but has no kernel here
-        triton_amd.attention(q32, q32, q32, True, 0.5)
+    with pytest.raises(ValueError):          # the C ABI has no head_dim 32 kernel (the host wrapper pads to 64 instead)
+        triton_amd.ops._attention.apply(q32, q32, q32, True, 0.5)
+    q48 = torch.zeros(1, 1, 128, 48, dtype=torch.float16, device=gpu)
+    with pytest.raises(AssertionError):      # the reference's own assert (06:447)
+        triton_amd.attention(q48, q48, q48, True, 0.5)
 
 
 @pytest.mark.parametrize("causal", [True, False])
@@ -150,3 +153,24 @@ def test_head_dim_256_forward(gpu, dtype, causal):
     assert np.allclose(to_np(out.detach()), cf["o"], atol=1e-2, rtol=1e-2)
     with pytest.raises(ValueError):
         out.backward(tdo)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("D", [16, 32])
+@pytest.mark.parametrize("causal", [True, False])
+def test_head_dims_16_and_32_forward_and_backward(gpu, dtype, D, causal):
+    # HEAD_DIM 16 / 32 of the reference's assert (06:447): zero-padded to the 64-column kernels by the
+    # host wrapper; outputs and all three gradients against the closed form at the usual tolerance
+    shape = (2, 2, 256, D)
+    (q, k, v, do), (tq, tk, tv, tdo) = _inputs(11, shape, dtype, gpu)
+    sm_scale = D ** -0.5
+    cf = A.attn_closed_form(q, k, v, causal, sm_scale, do=do)
+    for t in (tq, tk, tv):
+        t.requires_grad_()
+    out = triton_amd.attention(tq, tk, tv, causal, sm_scale)
+    assert out.shape == tq.shape
+    out.backward(tdo)
+    assert np.allclose(to_np(out.detach()), cf["o"], atol=1e-2, rtol=1e-2)
+    for name, t in (("dq", tq), ("dk", tk), ("dv", tv)):
+        assert t.grad.shape == t.shape
+        assert np.allclose(to_np(t.grad), cf[name], atol=3e-2, rtol=1e-2), name
