@@ -94,10 +94,10 @@ def test_exact_integers_on_mfma_path_bitwise_vs_tiled_oracle(gpu):
             assert bits_equal(got, ref)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 def test_every_kernel_variant_is_bit_exact_on_integers(gpu, monkeypatch, tile):
     # MI355_GEMM_TILE forces one MFMA kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves,
-    # persistent) for shapes the size heuristic would give to another; K = 520 has a
+    # persistent, and 6 = four waves of 16x16x32 MFMAs for K-major B) for shapes the size heuristic would give to another; K = 520 has a
     # partial last K step, which the ping-pong kernel hands to the one-barrier kernel and the
     # pipelined kernels finish themselves; the persistent form takes whole tiles with K a multiple of
     # 128 (512 x 768 x 512 with 3 programs: two tiles each, in one stream of K steps) and falls back otherwise
@@ -130,6 +130,32 @@ def test_single_nonzero_locates_every_tile(gpu):
         c = triton_amd.matmul(a, b, out_dtype=torch.float32)
         nz = torch.nonzero(c)
         assert nz.tolist() == [[i, j]] and c[i, j].item() == -6.0
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
+    # the 128x128-per-wave kernel of 16x16x32 MFMAs (K-major B, whole 256x256 tiles, K bytes % 256 == 0):
+    # N(0,1) operands, every output type, alpha, the activation, a padded C, and the smallest K (two steps)
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    rng = np.random.default_rng(23)
+    for (M, N, K) in [(512, 256, 1152), (256, 768, 128)]:
+        a = randn_rounded(rng, (M, K), dtype)
+        b = randn_rounded(rng, (K, N), dtype)
+        ta = from_np(a, dtype, gpu)
+        tb = from_np(np.ascontiguousarray(b.T), dtype, gpu).t()
+        for out in ("fp32", dtype):
+            odt = torch.float32 if out == "fp32" else ta.dtype
+            c = to_np(triton_amd.matmul(ta, tb, out_dtype=odt))
+            assert np.allclose(c, gemm.matmul_closed_form(a, b, out_dtype=out), rtol=1e-2, atol=1e-2), (M, N, K, out)
+        c = to_np(triton_amd.matmul(ta, tb, activation="leaky_relu", a_scale=0.5, b_scale=4.0, out_dtype=torch.float32))
+        ref = gemm.matmul_closed_form(a, b, out_dtype="fp32") * 2.0
+        assert np.allclose(c, np.where(ref >= 0, ref, 0.01 * ref), rtol=1e-2, atol=1e-2)
+        # the same product through the autotuner entry into a C with padded rows
+        from triton_amd import autotune as at
+        cbuf = torch.zeros(M, N + 8, device=gpu, dtype=ta.dtype)
+        at._launch(ta, tb, cbuf[:, :N], at.Config(6, 4))
+        assert np.allclose(to_np(cbuf[:, :N]), gemm.matmul_closed_form(a, b, out_dtype=dtype), rtol=1e-2, atol=1e-2)
+        assert torch.count_nonzero(cbuf[:, N:]).item() == 0
 
 
 def test_leaky_relu_epilogue(gpu):

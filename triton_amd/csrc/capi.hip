@@ -163,6 +163,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
+  // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (K-major B, whole tiles, no addend)
+  if (tile == 6 && b_kmajor && !aux && gemm_wave128_ok(p)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 
@@ -178,7 +180,7 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C, int M, int N, int K,
                      int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
                      int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
                      int activation, int tile, int group_m, void* stream_) {
-  if (tile < -1 || tile > 5 || group_m < 0) return MI355_EINVAL;
+  if (tile < -1 || tile > 6 || group_m < 0) return MI355_EINVAL;
   return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
                    activation, nullptr, 0, 0, 0, tile, group_m, stream_);
 }

@@ -65,6 +65,19 @@ __device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned l
 #endif
 }
 
+// The same with an instruction offset, which the hardware adds to BOTH addresses (global and LDS):
+// several copies can then share one M0 value.  SETM0 = false reuses the M0 of the previous copy.
+template <int OFF, bool SETM0>
+__device__ __forceinline__ void async_copy16_sbase_off(const void* sbase, unsigned lane_off, unsigned lds_wave_base) {
+#if MI355_DEVICE_PASS
+  if constexpr (SETM0)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base), "i"(OFF) : "memory");
+  else
+    asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" :: "v"(lane_off), "s"(sbase), "i"(OFF) : "memory");
+#endif
+}
+
 // 16 bytes per lane from (wave-uniform 64-bit base + 32-bit lane offset + immediate) into
 // registers, issued as inline assembly so that the compiler neither counts it nor waits for it:
 // for loops that keep many loads in flight and wait with wait_vmcnt<> by hand.  The result may be

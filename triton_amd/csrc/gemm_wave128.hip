@@ -1,0 +1,230 @@
+// Four-wave GEMM with 128x128 of C per wave, built from 16x16x32 MFMAs (K-major A and B, 16-bit
+// types): one workgroup per 256x256 tile of C, one wave per SIMD, all 256 accumulator registers of
+// a lane in use.
+//
+// Why this shape: the GEMM runs at the board's power limit, and on N(0,1) operands a stream of
+// 16x16x32 MFMAs needs 11 % less energy per flop than a stream of 32x32x16 ones (16.9 vs 19.1 ns per
+// 32768 flop and SIMD, measured with nothing else running).  Against the eight-wave kernels of
+// gemm_core.h (128x64 per wave) every flop also needs a third fewer LDS fragment bytes.
+//
+// Loop: 128 bytes of every operand row per K step (two sub-steps of 64 MFMAs), two 64 KiB LDS
+// stages filled by direct global->LDS loads.  With a single wave per SIMD nothing else can issue
+// MFMAs while that wave is held up, so the memory instructions carry no scalar arithmetic: the
+// sixteen scalar bases of a wave's loads are fixed, the K position travels in the lane offset,
+// and the eight loads of one operand share one M0 value through their instruction offsets (which
+// the hardware adds to the global AND the LDS address).  Every fragment read is issued a sub-step
+// before its use.
+//
+// LDS tile of an operand: row r (128 bytes = eight 16-byte chunks) at r * 128, chunk c in slot
+// c ^ ((r >> 1) & 7): the 16 lanes of a ds_read_b128 pass (16 consecutive rows, one chunk) cover
+// all 64 banks once.  The direct loads write LDS linearly (lane i -> base + 16 i), so the
+// permutation is applied to the global address each lane fetches.
+#include "gemm_core.h"
+
+namespace mi355 {
+
+// D(16x16 fp32) += A(16x32) * B(32x16).  Lane l supplies A[l%16][8*(l/16) .. +8] and
+// B[8*(l/16) .. +8][l%16]; accumulator register r of lane l is D[4*(l/16) + r][l%16].
+__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+}
+__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+}
+
+// Epilogue for 16x16 tiles computed with the operands swapped (D[n][m]): lane l owns C row
+// `mrow0 + 16 i + l%16` and, of tile (i, j), the four consecutive columns `ncol0 + 16 j + 4 (l/16) ..`.
+template <int MT, int NT>
+__device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
+  float alpha = 1.f;
+  if (p.a_scale) alpha *= *p.a_scale;
+  if (p.b_scale) alpha *= *p.b_scale;
+  const bool leaky = p.activation == 1;
+  static_for<MT>([&](auto I_) {
+    constexpr int i = decltype(I_)::value;
+    const int m = mrow0 + i * 16 + l16;
+    static_for<NT>([&](auto J_) {
+      constexpr int j = decltype(J_)::value;
+      const int n = ncol0 + j * 16 + kg * 4;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        v[e] = acc[i][j][e] * alpha;
+        if (leaky) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
+      }
+      if (p.out_dtype == 4) {
+        float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+        if (p.c_vec_ok) *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
+        else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) c[e * p.scn] = v[e];
+        }
+      } else if (p.out_dtype == 1) {
+        __bf16* c = (__bf16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+        if (p.c_vec_ok) *(bf16x4*)c = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) c[e * p.scn] = (__bf16)v[e];
+        }
+      } else {
+        _Float16* c = (_Float16*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
+        if (p.c_vec_ok) *(f16x4*)c = f16x4{(_Float16)v[0], (_Float16)v[1], (_Float16)v[2], (_Float16)v[3]};
+        else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) c[e * p.scn] = (_Float16)v[e];
+        }
+      }
+    });
+  });
+}
+
+template <typename V8>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int MT = 8, NT = 8, KS = 2;                             // 16x16 tiles per wave, 16x16x32 sub-steps per stage
+  constexpr int NR = MT + NT, NM = MT * NT;                         // fragment reads and MFMAs per sub-step
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  int pm, pn;
+  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+
+  // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
+  // those rows is 4 (q & 1) + lane / 16, so the lane offset depends on the parity of j only
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
+  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  // load j (0..7: A, 8..15: B) of tile kt into the stage at `stage_base`.  M0 = middle of the wave's
+  // 8 KiB of that operand, instruction offsets -4096 .. 3072 (taken back out of the scalar base).
+  auto issue = [&](auto J_, int kt, unsigned stage_base) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
+  };
+
+  // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 4 ks + kg of row l16 (+ 16 t)
+  unsigned adrA[2][KS], adrB[2][KS];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const unsigned slot = ((4 * ks + kg) ^ s) * 16;
+      adrA[0][ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      adrB[0][ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+      adrA[1][ks] = adrA[0][ks] + STAGE;
+      adrB[1][ks] = adrB[0][ks] + STAGE;
+    }
+  }
+  struct Frags { V8 a[MT]; V8 b[NT]; };
+  Frags f[2];
+  auto read_one = [&](auto OP_, auto P_, auto KS_, Frags& dst) {
+    constexpr int op = decltype(OP_)::value, P = decltype(P_)::value, ks = decltype(KS_)::value;
+    if constexpr (op < MT) dst.a[op] = __builtin_bit_cast(V8, lds_read_b128<op * 16 * ROWB>(adrA[P][ks]));
+    else dst.b[op - MT] = __builtin_bit_cast(V8, lds_read_b128<(op - MT) * 16 * ROWB>(adrB[P][ks]));
+  };
+  auto pin = [&](Frags& x) {
+    static_for<MT>([&](auto T_) { lds_use(x.a[decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(x.b[decltype(T_)::value]); });
+  };
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue: both stages requested, first fragments of stage 0 read
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE); });
+  wait_vmcnt<16>();
+  block_barrier();
+  using Z = std::integral_constant<int, 0>;
+  static_for<NR>([&](auto OP_) { read_one(OP_, Z{}, Z{}, f[0]); });
+
+  // One sub-step: 64 MFMAs on f[ks]; the fragments of the next sub-step are requested over the first
+  // half of them (one read per two MFMAs).  The last sub-step of a stage first meets the other waves
+  // (every wave has then read all it needs of this stage, and the other stage has landed), reads the
+  // first fragments of the other stage and refills this one with the tile two steps ahead (one load
+  // per two MFMAs).
+  auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_, int kt) {
+    constexpr int P = decltype(P_)::value, ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
+    constexpr bool last = ks == KS - 1;
+    constexpr bool more = decltype(MORE_)::value;              // there is a next sub-step to read for
+    constexpr bool refill = last && decltype(REFILL_)::value;  // and a tile two steps ahead to request
+    lds_wait<0>();
+    pin(f[cur]);
+    if constexpr (last) {
+      wait_vmcnt<0>();
+      block_barrier();
+    }
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      acc[i][j] = mfma16(f[cur].b[j], f[cur].a[i], acc[i][j]);
+      if constexpr (more && n % 2 == 0 && n / 2 < NR)
+        read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, last ? (P ^ 1) : P>{},
+                 std::integral_constant<int, last ? 0 : ks + 1>{}, f[nxt]);
+      if constexpr (refill && n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, kt + 2, lds0 + P * STAGE);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  using T = std::true_type; using F = std::false_type;
+  auto stage = [&](auto P_, auto MORE_, auto REFILL_, int kt) {
+    substep(P_, I0{}, T{}, F{}, kt);
+    substep(P_, I1{}, MORE_, REFILL_, kt);
+  };
+  for (int kt = 0; kt < nk - 2; kt += 2) {
+    stage(I0{}, T{}, T{}, kt);
+    stage(I1{}, T{}, T{}, kt + 1);
+  }
+  stage(I0{}, T{}, F{}, nk - 2);
+  stage(I1{}, F{}, F{}, nk - 1);
+  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
+#endif
+}
+
+bool gemm_wave128_ok(const GemmArgs& p) {
+  // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
+}
+
+template <typename V8>
+static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = (p.M / 256) * (p.N / 256);
+  gemm_wave128_kernel<V8><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+// K-major B only (A is always K-major on the MFMA paths).
+int gemm_wave128_launch(const GemmArgs& p, bool bf16, hipStream_t stream) {
+  return bf16 ? launch_wave128<bf16x8>(p, stream) : launch_wave128<f16x8>(p, stream);
+}
+
+}  // namespace mi355
