@@ -163,8 +163,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
-  // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (K-major B, whole tiles, no addend)
-  if (tile == 6 && b_kmajor && !aux && gemm_wave128_ok(p)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, stream);
+  // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles, no addend)
+  if (tile == 6 && !aux && gemm_wave128_ok(p, b_kmajor)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 

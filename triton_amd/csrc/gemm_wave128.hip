@@ -25,11 +25,18 @@ namespace mi355 {
 
 // D(16x16 fp32) += A(16x32) * B(32x16).  Lane l supplies A[l%16][8*(l/16) .. +8] and
 // B[8*(l/16) .. +8][l%16]; accumulator register r of lane l is D[4*(l/16) + r][l%16].
-__device__ __forceinline__ f32x4 mfma16(bf16x8 a, bf16x8 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+// Issued as inline assembly with the accumulator constrained to the accumulation registers: left to
+// the register allocator, some of the 64 accumulator tuples of a lane end up in architectural
+// registers and get shuffled back and forth in every K step.
+__device__ __forceinline__ void mfma16(bf16x8 a, bf16x8 b, f32x4& c) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#endif
 }
-__device__ __forceinline__ f32x4 mfma16(f16x8 a, f16x8 b, f32x4 c) {
-  return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+__device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+#endif
 }
 
 // Epilogue for 16x16 tiles computed with the operands swapped (D[n][m]): lane l owns C row
@@ -78,13 +85,13 @@ __device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const Gemm
   });
 }
 
-template <typename V8>
+template <typename V8, bool B_KMAJOR>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
   constexpr int MT = 8, NT = 8, KS = 2;                             // 16x16 tiles per wave, 16x16x32 sub-steps per stage
-  constexpr int NR = MT + NT, NM = MT * NT;                         // fragment reads and MFMAs per sub-step
+  constexpr int NM = MT * NT;                                       // MFMAs per sub-step
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
@@ -101,45 +108,81 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
   // those rows is 4 (q & 1) + lane / 16, so the lane offset depends on the parity of j only
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[2], voffB[2];
+  unsigned voffA[2], voffB[B_KMAJOR ? 2 : 1];
 #pragma unroll
   for (int par = 0; par < 2; par++) {
     const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
     voffA[par] = drow * (unsigned)p.lda + chunk * 16;
-    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+    if constexpr (B_KMAJOR) voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  // Row-major B[K, N]: the stage holds 64 k rows of 512 bytes; instruction q = 8 * wave + j moves the k rows
+  // 2 q, 2 q + 1 (lane i: row i / 32, physical 16-byte chunk i % 32).  Element (k, n) lives in the 32-byte
+  // column group (n / 16) ^ 2 (k & 3) ^ ((k >> 3) & 1) of its row: a transpose read is served two 16-lane
+  // groups at a time - four consecutive k rows each, eight rows apart, the same 16 columns - and this
+  // spreads those 8 x 32 bytes over all banks.  With k = 16 wave + 2 j + i / 32 the XOR terms are
+  // 4 (j & 1) + 2 (i / 32) and (j >> 2) & 1: the j terms are XORed into the lane offset at each load.
+  if constexpr (!B_KMAJOR) {
+    const unsigned pg = (lane & 31) >> 1, half = lane & 1;
+    voffB[0] = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;   // j = 0; other j: XOR below
   }
   const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
-  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
-  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  const char* gB = B_KMAJOR ? p.B + ((int64_t)pn * BN + wave * 64) * p.ldb
+                            : p.B + (int64_t)pn * BN * 2 + (int64_t)(wave * 16) * p.ldb;
+  const int64_t stepA = 8 * p.lda, stepB = (B_KMAJOR ? 8 : 2) * p.ldb;
+  const unsigned kstepB = B_KMAJOR ? ROWB : 64 * (unsigned)p.ldb;   // bytes from one K step to the next
   // load j (0..7: A, 8..15: B) of tile kt into the stage at `stage_base`.  M0 = middle of the wave's
   // 8 KiB of that operand, instruction offsets -4096 .. 3072 (taken back out of the scalar base).
   auto issue = [&](auto J_, int kt, unsigned stage_base) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
     const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
     const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
-    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    unsigned lane_off;
+    if constexpr (j < 8) lane_off = voffA[j & 1] + (unsigned)kt * ROWB;
+    else if constexpr (B_KMAJOR) lane_off = voffB[j & 1] + (unsigned)kt * ROWB;
+    else lane_off = (voffB[0] ^ ((4 * (q & 1) + ((q >> 2) & 1)) * 32)) + (unsigned)kt * kstepB;
     async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
   };
 
   // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 4 ks + kg of row l16 (+ 16 t)
-  unsigned adrA[2][KS], adrB[2][KS];
+  unsigned adrA[KS], adrB[B_KMAJOR ? KS : NT];   // stage 0; stage 1 is 64 KiB further (added at the read)
   {
     const unsigned s = (l16 >> 1) & 7;
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       const unsigned slot = ((4 * ks + kg) ^ s) * 16;
-      adrA[0][ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
-      adrB[0][ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
-      adrA[1][ks] = adrA[0][ks] + STAGE;
-      adrB[1][ks] = adrB[0][ks] + STAGE;
+      adrA[ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      if constexpr (B_KMAJOR) adrB[ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+    // row-major B: lane i of the 16-lane group kg addresses k row 8 kg + i / 4 (+ 32 ks, + 4 for the second
+    // read) and the 8 bytes (i & 3) of the 16-column group of tile t; (k & 3) = i / 4 and (k >> 3) & 1 = kg & 1
+    // for every ks and both reads
+    if constexpr (!B_KMAJOR) {
+      const unsigned k = 8 * kg + (l16 >> 2), m = (2 * (l16 >> 2)) ^ (kg & 1);
+#pragma unroll
+      for (int t = 0; t < NT; t++) adrB[t] = lds0 + A_BYTES + k * (BN * 2) + ((wn * 8 + (t ^ m)) * 32) + (l16 & 3) * 8;
     }
   }
+  static_assert(STAGE == 65536, "stage 1 = stage 0 + 64 KiB");
   struct Frags { V8 a[MT]; V8 b[NT]; };
   Frags f[2];
+  constexpr int NRD = MT + NT;  // fragment reads per sub-step (a row-major B fragment takes two instructions)
   auto read_one = [&](auto OP_, auto P_, auto KS_, Frags& dst) {
     constexpr int op = decltype(OP_)::value, P = decltype(P_)::value, ks = decltype(KS_)::value;
-    if constexpr (op < MT) dst.a[op] = __builtin_bit_cast(V8, lds_read_b128<op * 16 * ROWB>(adrA[P][ks]));
-    else dst.b[op - MT] = __builtin_bit_cast(V8, lds_read_b128<(op - MT) * 16 * ROWB>(adrB[P][ks]));
+    constexpr unsigned so = P * STAGE;
+    if constexpr (op < MT) {
+      dst.a[op] = __builtin_bit_cast(V8, lds_read_b128<op * 16 * ROWB>(adrA[ks] + so));
+    } else if constexpr (B_KMAJOR) {
+      dst.b[op - MT] = __builtin_bit_cast(V8, lds_read_b128<(op - MT) * 16 * ROWB>(adrB[ks] + so));
+    } else {
+      // two transpose reads per fragment: k .. k + 3 into the low, k + 4 .. k + 7 into the high half
+      constexpr int t = op - MT, imm = ks * 32 * BN * 2;
+      // (the compiler's own builtin, not inline assembly: it can then place the two halves directly in
+      // the four-register operand; its wait-count bookkeeping only ever adds to the explicit waits)
+      const unsigned ad = adrB[t] + so + imm;
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(uintptr_t)ad);
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(uintptr_t)(ad + 4 * BN * 2));
+      dst.b[t] = __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    }
   };
   auto pin = [&](Frags& x) {
     static_for<MT>([&](auto T_) { lds_use(x.a[decltype(T_)::value]); });
@@ -158,7 +201,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   wait_vmcnt<16>();
   block_barrier();
   using Z = std::integral_constant<int, 0>;
-  static_for<NR>([&](auto OP_) { read_one(OP_, Z{}, Z{}, f[0]); });
+  static_for<NRD>([&](auto OP_) { read_one(OP_, Z{}, Z{}, f[0]); });
 
   // One sub-step: 64 MFMAs on f[ks]; the fragments of the next sub-step are requested over the first
   // half of them (one read per two MFMAs).  The last sub-step of a stage first meets the other waves
@@ -178,8 +221,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
     }
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
-      acc[i][j] = mfma16(f[cur].b[j], f[cur].a[i], acc[i][j]);
-      if constexpr (more && n % 2 == 0 && n / 2 < NR)
+      mfma16(f[cur].b[j], f[cur].a[i], acc[i][j]);
+      if constexpr (more && n % 2 == 0 && n / 2 < NRD)
         read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, last ? (P ^ 1) : P>{},
                  std::integral_constant<int, last ? 0 : ks + 1>{}, f[nxt]);
       if constexpr (refill && n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, kt + 2, lds0 + P * STAGE);
@@ -198,33 +241,37 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   }
   stage(I0{}, T{}, F{}, nk - 2);
   stage(I1{}, F{}, F{}, nk - 1);
+  // the compiler does not know that the assembly above are MFMAs: let the last ones retire before their
+  // results are read
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
   gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
 #endif
 }
 
-bool gemm_wave128_ok(const GemmArgs& p) {
+bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
   // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
-  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256 &&
-         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
+  if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
+  return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (int64_t)p.K * p.ldb + 512 < (1ll << 31);
 }
 
-template <typename V8>
+template <typename V8, bool B_KMAJOR>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int grid = (p.M / 256) * (p.N / 256);
-  gemm_wave128_kernel<V8><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_kernel<V8, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
-// K-major B only (A is always K-major on the MFMA paths).
-int gemm_wave128_launch(const GemmArgs& p, bool bf16, hipStream_t stream) {
-  return bf16 ? launch_wave128<bf16x8>(p, stream) : launch_wave128<f16x8>(p, stream);
+int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream) {
+  if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true>(p, stream) : launch_wave128<f16x8, true>(p, stream);
+  return bf16 ? launch_wave128<bf16x8, false>(p, stream) : launch_wave128<f16x8, false>(p, stream);
 }
 
 }  // namespace mi355
