@@ -158,6 +158,27 @@ def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
         assert torch.count_nonzero(cbuf[:, N:]).item() == 0
 
 
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_four_wave_16x16_fp8_kernel_against_dequantised_closed_form(gpu, monkeypatch, fmt, tdt):
+    # the fp8 form of the same kernel (16x16x128 MFMAs; K-major B, whole tiles, K % 256 == 0): every finite
+    # code as input, per-tensor scales, fp32 and bf16 outputs
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    rng = np.random.default_rng(29)
+    table = formats.fp8_table(fmt)
+    finite = np.array([c for c in range(256) if np.isfinite(table[c])], dtype=np.uint8)
+    for (M, N, K) in [(256, 512, 768), (512, 256, 256)]:
+        ca = rng.choice(finite, size=(M, K)); cb = rng.choice(finite, size=(N, K))
+        a = table[ca].astype(np.float64); b = table[cb].astype(np.float64)
+        # keep the products in range: scale both operands down by their largest magnitude
+        sa, sb = 1.0 / np.abs(a).max(), 1.0 / np.abs(b).max()
+        ref = (a @ b.T) * (sa * sb)
+        ta = torch.from_numpy(ca).to(gpu).view(tdt); tb = torch.from_numpy(cb).to(gpu).view(tdt).t()
+        got = to_np(triton_amd.matmul(ta, tb, a_scale=float(sa), b_scale=float(sb), out_dtype=torch.float32))
+        assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max()), (fmt, M, N, K)
+        got = to_np(triton_amd.matmul(ta, tb, a_scale=float(sa), b_scale=float(sb), out_dtype=torch.bfloat16))
+        assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max()), (fmt, M, N, K, "bf16")
+
+
 def test_leaky_relu_epilogue(gpu):
     rng = np.random.default_rng(6)
     a = randn_rounded(rng, (256, 128), "fp16"); b = randn_rounded(rng, (128, 264), "fp16")

@@ -248,6 +248,157 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #endif
 }
 
+// ---------------------------------------------------------------------------------------------
+// The same kernel for fp8 (e4m3fn / e5m2, both operands K-major): 16x16x128 f8f6f4 MFMAs, one per
+// accumulator tile and K step (128 bytes of K = one whole LDS row).  A fragment is 32 bytes per
+// lane (two 16-byte chunks, eight registers), so a K step's sixteen fragments fill 128 registers;
+// the step is split in two halves by rows of A: the first uses A fragments 0..3, the second 4..7
+// (read during the first), while the B fragments and the first four A fragments of the next
+// stage are read during the second half into a second set.  Any assignment of K positions to the
+// bytes of a lane works as long as A and B use the same one: lane (r, kg) takes the chunks
+// 2 kg and 2 kg + 1 of its row.  The fragment reads are ordinary LDS loads here (the compiler then
+// places the two halves directly in the eight-register operand and waits for each fragment just
+// before its first use); the direct global->LDS loads stay invisible to its bookkeeping.
+// ---------------------------------------------------------------------------------------------
+template <int FMT>
+__device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4& c) {
+#if MI355_DEVICE_PASS
+  if constexpr (FMT == 0) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:1 blgp:1" : "+a"(c) : "v"(a), "v"(b));
+#endif
+}
+
+template <int FMT>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int MT = 8, NT = 8, MH = MT / 2;
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  int pm, pn;
+  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+
+  // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
+  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  auto issue = [&](auto J_, int kt, unsigned stage_base) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
+  };
+
+  // ---- fragment reads: lane (l16, kg) wants the chunks 2 kg, 2 kg + 1 of row l16 (+ 16 t)
+  LDS_PTR(const char) fragA[2];
+  LDS_PTR(const char) fragB[2];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const unsigned slot = ((2 * kg + c) ^ s) * 16;
+      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * 128 + l16) * ROWB + slot;
+      fragB[c] = (LDS_PTR(const char))lds_raw + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+  }
+  auto read_frag = [&](LDS_PTR(const char) (&base)[2], int off) {
+    i32x4 lo = *(LDS_PTR(const i32x4))(base[0] + off);
+    i32x4 hi = *(LDS_PTR(const i32x4))(base[1] + off);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  i32x8 a0[MH], a1[MH], b[2][NT];
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE); });
+  wait_vmcnt<16>();
+  block_barrier();
+#pragma unroll
+  for (int t = 0; t < NT; t++) b[0][t] = read_frag(fragB, t * 16 * ROWB);
+#pragma unroll
+  for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
+
+  // One K step on stage P with the B fragments of set `cur`.
+  auto step = [&](auto P_, auto CUR_, auto MORE_, auto REFILL_, int kt) {
+    constexpr int P = decltype(P_)::value, cur = decltype(CUR_)::value, nxt = cur ^ 1;
+    constexpr bool more = decltype(MORE_)::value, refill = decltype(REFILL_)::value;
+    constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
+    // first half: rows 0..3 of A; the A fragments 4..7 of this stage are read meanwhile
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_f8<FMT>(b[cur][j], a0[i], acc[i][j]);
+      if constexpr (n % 4 == 0 && n / 4 < MH) a1[n / 4] = read_frag(fragA, so + (MH + n / 4) * 16 * ROWB);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    // every wave has now requested all it needs of stage P: once those reads are back and the other
+    // stage has landed, meet, then read the next fragments from the other stage and refill this one
+    lds_wait<0>();
+    wait_vmcnt<0>();
+    block_barrier();
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
+      if constexpr (more && n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
+      if constexpr (more && n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
+      if constexpr (refill && n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, kt + 2, lds0 + P * STAGE);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+  };
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  using T = std::true_type; using F = std::false_type;
+  for (int kt = 0; kt < nk - 2; kt += 2) {
+    step(I0{}, I0{}, T{}, T{}, kt);
+    step(I1{}, I1{}, T{}, T{}, kt + 1);
+  }
+  step(I0{}, I0{}, T{}, F{}, nk - 2);
+  step(I1{}, I1{}, F{}, F{}, nk - 1);
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
+#endif
+}
+
+template <int FMT>
+static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = (p.M / 256) * (p.N / 256);
+  gemm_wave128_f8_kernel<FMT><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
+  return e5m2 ? launch_wave128_f8<1>(p, stream) : launch_wave128_f8<0>(p, stream);
+}
+
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
   // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
   if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
