@@ -33,7 +33,7 @@ def test_key_follows_the_reference_layout():
 def test_first_call_benchmarks_every_config_then_the_table_answers(monkeypatch, tmp_path, capsys):
     launches = []
     _stub(monkeypatch, launches)
-    cost = {1: 3.0, 2: 2.0, 3: 0.5, 4: 1.0, 5: 0.9}
+    cost = {1: 3.0, 2: 2.0, 3: 0.5, 4: 1.0, 5: 0.9, 6: 0.8}
     benched = []
 
     def bench(fn):
@@ -57,7 +57,7 @@ def test_first_call_benchmarks_every_config_then_the_table_answers(monkeypatch, 
     assert len(benched) == 2 * len(t.configs) and len(t.cache) == 2
     # a single row of tiles: GROUP_SIZE_M cannot matter, duplicates are pruned
     assert [(c.tile, c.group_m) for c in t.prune_configs(_FakeTensor((128, 64), None), _FakeTensor((64, 4096), None))] == \
-        [(1, 8), (2, 8), (3, 8), (4, 8), (5, 4)]
+        [(1, 8), (2, 8), (3, 8), (4, 8), (5, 4), (6, 4)]
     # the table survives a restart
     doc = json.load(open(path))
     assert doc["version"] == 1 and len(doc["entries"]) == 2

@@ -39,8 +39,10 @@ class Config:
 
 
 def default_configs():
-    """The kernels that exist for every MFMA dtype, with the GROUP_SIZE_M values worth trying."""
-    return [Config(1, 8), Config(2, 8), Config(3, 8), Config(4, 8), Config(5, 4), Config(5, 8), Config(5, 16)]
+    """The kernels that exist for every MFMA dtype (6 falls back to 5 where its shape conditions do not hold),
+    with the GROUP_SIZE_M values worth trying."""
+    return [Config(1, 8), Config(2, 8), Config(3, 8), Config(4, 8), Config(5, 4), Config(5, 8), Config(5, 16),
+            Config(6, 4), Config(6, 8)]
 
 
 def _launch(a, b, c, config: Config, activation: int = 0):
