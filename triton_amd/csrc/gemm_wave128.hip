@@ -101,8 +101,14 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   const int l16 = lane & 15, kg = lane >> 4;
 
   const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid is either one workgroup per tile or, when
+  // that divides evenly, one per CU) as ONE stream of K steps: the loads of the last two steps of a tile
+  // already fetch the first two K steps of the next one, so its first fragments are in registers when the
+  // finished tile is stored.
+  int tile = blockIdx.x;
   int pm, pn;
-  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
 
   // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
@@ -125,9 +131,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
     const unsigned pg = (lane & 31) >> 1, half = lane & 1;
     voffB[0] = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;   // j = 0; other j: XOR below
   }
-  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
-  const char* gB = B_KMAJOR ? p.B + ((int64_t)pn * BN + wave * 64) * p.ldb
-                            : p.B + (int64_t)pn * BN * 2 + (int64_t)(wave * 16) * p.ldb;
+  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
+  const char* gA;
+  const char* gB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb
+                  : p.B + (int64_t)fn * BN * 2 + (int64_t)(wave * 16) * p.ldb;
+  };
+  set_fill_tile(pm, pn);
   const int64_t stepA = 8 * p.lda, stepB = (B_KMAJOR ? 8 : 2) * p.ldb;
   const unsigned kstepB = B_KMAJOR ? ROWB : 64 * (unsigned)p.ldb;   // bytes from one K step to the next
   // load j (0..7: A, 8..15: B) of tile kt into the stage at `stage_base`.  M0 = middle of the wave's
@@ -190,10 +202,13 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   };
 
   f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < MT; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
-    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
 
   // ---- prologue: both stages requested, first fragments of stage 0 read
   static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
@@ -231,20 +246,50 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   using T = std::true_type; using F = std::false_type;
-  auto stage = [&](auto P_, auto MORE_, auto REFILL_, int kt) {
-    substep(P_, I0{}, T{}, F{}, kt);
-    substep(P_, I1{}, MORE_, REFILL_, kt);
+  // A K step: `fk` is the K step (of the tile the scalar bases point at) that its loads fetch.
+  auto stage = [&](auto P_, int fk) {
+    substep(P_, I0{}, T{}, F{}, fk - 2);
+    substep(P_, I1{}, T{}, T{}, fk - 2);
   };
-  for (int kt = 0; kt < nk - 2; kt += 2) {
-    stage(I0{}, T{}, T{}, kt);
-    stage(I1{}, T{}, T{}, kt + 1);
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;   // next K step to fetch, and the tile it belongs to
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  if (nk == 2) { fk = 1; advance(); }   // (two steps per tile: the prologue fetched both, the cursor is on the next tile)
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 2) {
+      stage(I0{}, fk); advance();
+      stage(I1{}, fk); advance();
+    }
+    // The next tile's first fragments were requested by reads the compiler cannot see: have them landed
+    // before the epilogue's register traffic could move their registers.  Nor does it know that the assembly
+    // above are MFMAs: let the last ones retire before their results are read.
+    lds_wait<0>();
+    pin(f[0]);
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    // (the tile and lane coordinates pass through an empty assembly statement so that none of the
+    // epilogue's address arithmetic is hoisted out of the tile loop, where it would occupy - and spill -
+    // registers throughout the K loop)
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
   }
-  stage(I0{}, T{}, F{}, nk - 2);
-  stage(I1{}, F{}, F{}, nk - 1);
-  // the compiler does not know that the assembly above are MFMAs: let the last ones retire before their
-  // results are read
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 #endif
 }
 
@@ -415,7 +460,10 @@ static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int grid = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / 256) * (p.N / 256);
+  // one program per CU when that deals the tiles evenly, else one workgroup per tile (the hardware's
+  // dynamic dispatch then balances the ragged last round)
+  const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
   gemm_wave128_kernel<V8, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
