@@ -107,18 +107,19 @@ def test_full_size_8192_sampled_rows(gpu, fmt):
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max() / 64)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
 def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile):
     # MI355_GEMM_TILE forces one kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves,
     # persistent) for shapes the size heuristic would give to another; K = 1536 covers three 16-byte
     # scale groups per row in the pipelined kernels (an odd number: the two-slot scale ring changes
     # parity from tile to tile in the persistent form, two programs for six and twelve tiles),
-    # K = 1056 (not a multiple of 512) their fall-back.
+    # K = 1056 (not a multiple of 512) their fall-back.  6 = MXFP4 on four waves of scaled 16x16x128 MFMAs: whole
+    # 256x256 tiles and K a multiple of 1024 (the last two shapes: one and two groups of four K steps), else 5.
     monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
     monkeypatch.setenv("MI355_GEMM_PROGRAMS", "2")
     rng = np.random.default_rng(tile)
-    for (M, N, K) in [(512, 256, 1536), (300, 520, 1056), (768, 512, 1536), (768, 1024, 1024)]:
+    for (M, N, K) in [(512, 256, 1536), (300, 520, 1056), (768, 512, 1536), (768, 1024, 1024), (512, 256, 2048)]:
         if fmt == "mxfp4":
             a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
         else:

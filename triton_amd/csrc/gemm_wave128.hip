@@ -444,6 +444,207 @@ int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
   return e5m2 ? launch_wave128_f8<1>(p, stream) : launch_wave128_f8<0>(p, stream);
 }
 
+// ---------------------------------------------------------------------------------------------
+// MXFP4 (e2m1 codes, one e8m0 scale per 32 elements of K) on the same skeleton: scaled 16x16x128
+// f8f6f4 MFMAs, two per accumulator tile and K step (128 bytes of a row = 256 elements = 8 scale
+// blocks of 16 bytes).  Lane (r, kg) of sub-step ks multiplies block 2 kg + ks of its row, so the two
+// scale bytes a lane needs in a K step are neighbours: shifted down once, the byte selector of the MFMA
+// is the compile-time ks.  (Which K positions a lane takes is free as long as A, B and the scales
+// agree.)  The scales travel like the operands: 16 bytes per row (two K steps) per direct load into a
+// two-slot LDS ring (row r at 16 r), one `ds_read_b32` per fragment and K step from there.
+// ---------------------------------------------------------------------------------------------
+// Scaled fp4 MFMA with the accumulator pinned to the accumulation registers (see mfma16): byte SEL of the two
+// scale dwords applies; fp4 operands are four registers.
+template <int SEL>
+__device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32x4& c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+  if constexpr (SEL == 0)
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                 : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+  else
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                 : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+#endif
+}
+
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
+  constexpr int MT = 8, NT = 8, KS = 2, NM = MT * NT, NRD = MT + NT;
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  int pm, pn;
+  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+
+  // ---- operand loads, as in the 16-bit kernel
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
+  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  auto issue = [&](auto J_, int kt, unsigned stage_base) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
+  };
+  // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of rows 64 w .. 64 w + 63 of A and of B
+  const char* gSA = (const char*)p.sA + ((int64_t)pm * BM + wave * 64) * p.lds_a;
+  const char* gSB = (const char*)p.sB + ((int64_t)pn * BN + wave * 64) * p.lds_b;
+  const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
+  auto issue_scales = [&](int h) {   // pair h of K steps -> slot h & 1 (past the end of K: the last pair again)
+    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT + wave * 1024;
+    const int hd = h < nk / 2 ? h : nk / 2 - 1;
+    async_copy16_sbase(gSA, voffSA + (unsigned)hd * 16, slot);
+    async_copy16_sbase(gSB, voffSB + (unsigned)hd * 16, slot + BM * 16);
+  };
+  // Past the end of K the last tile is requested again (into a stage nobody reads any more), which keeps
+  // the loop uniform: one code path, no special last steps.
+  auto tile_at = [&](int t) { return t < nk ? t : nk - 1; };
+
+  // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 2 kg + ks of row l16 (+ 16 t)
+  unsigned adrA[KS], adrB[KS];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const unsigned slot = ((2 * kg + ks) ^ s) * 16;
+      adrA[ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      adrB[ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+  }
+  struct Frags { i32x4 a[MT]; i32x4 b[NT]; };
+  Frags f[2];
+  auto read_one = [&](auto OP_, auto P_, auto KS_, Frags& dst) {
+    constexpr int op = decltype(OP_)::value, P = decltype(P_)::value, ks = decltype(KS_)::value;
+    constexpr unsigned so = P * STAGE;
+    if constexpr (op < MT) dst.a[op] = lds_read_b128<op * 16 * ROWB>(adrA[ks] + so);
+    else dst.b[op - MT] = lds_read_b128<(op - MT) * 16 * ROWB>(adrB[ks] + so);
+  };
+  auto pin = [&](Frags& x) {
+    static_for<MT>([&](auto T_) { lds_use(x.a[decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(x.b[decltype(T_)::value]); });
+  };
+  // scales of a K step: the dword holding this lane's two bytes, shifted so that they sit in bytes 0 and 1
+  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + (kg >> 1) * 4;
+  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + (kg >> 1) * 4;
+  const int sshift = 16 * (kg & 1);
+  int sa[2][MT], sb[2][NT];
+  auto read_scales = [&](auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 1) * 8
+    constexpr int set = decltype(SET_)::value, off = decltype(OFF_)::value;
+    static_for<MT>([&](auto T_) { constexpr int t = decltype(T_)::value; sa[set][t] = lds_read_b32<off + t * 256>(adrSA); });
+    static_for<NT>([&](auto T_) { constexpr int t = decltype(T_)::value; sb[set][t] = lds_read_b32<off + t * 256>(adrSB); });
+  };
+  auto fix_scales = [&](auto SET_) {
+    constexpr int set = decltype(SET_)::value;
+    static_for<MT>([&](auto T_) { constexpr int t = decltype(T_)::value; lds_use(sa[set][t]); sa[set][t] = (int)((unsigned)sa[set][t] >> sshift); });
+    static_for<NT>([&](auto T_) { constexpr int t = decltype(T_)::value; lds_use(sb[set][t]); sb[set][t] = (int)((unsigned)sb[set][t] >> sshift); });
+  };
+
+  f32x4 acc[MT][NT];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  using T = std::true_type; using F = std::false_type;
+  issue_scales(0);
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE); });
+  wait_vmcnt<16>();
+  block_barrier();
+  static_for<NRD>([&](auto OP_) { read_one(OP_, I0{}, I0{}, f[0]); });
+  read_scales(I0{}, I0{});
+  lds_wait<0>();
+  fix_scales(I0{});
+
+  // K step U (0..3 within a group of four: stage U & 1, scale slot U >> 1, scale set U & 1)
+  auto step = [&](auto U_, int kt) {
+    constexpr int U = decltype(U_)::value, P = U & 1, set = U & 1;
+    // sub-step 0
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp4<0>(f[0].b[j], f[0].a[i], acc[i][j], sb[set][j], sa[set][i]);
+      if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P>{}, I1{}, f[1]);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    // sub-step 1: meet, then read the next step's first fragments and scales and refill this stage
+    lds_wait<0>();
+    pin(f[1]);
+    wait_vmcnt<0>();
+    block_barrier();
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp4<1>(f[1].b[j], f[1].a[i], acc[i][j], sb[set][j], sa[set][i]);
+      if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
+      if constexpr (n == 32)
+        read_scales(std::integral_constant<int, set ^ 1>{}, std::integral_constant<int, (((U + 1) & 3) >> 1) * SC_SLOT + ((U + 1) & 1) * 8>{});
+      if constexpr (n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, tile_at(kt + 2), lds0 + P * STAGE);
+      // (the scales of the K steps kt + 2, kt + 3 are requested in the even step kt, into the slot the steps
+      // kt - 2, kt - 1 used: its last reader was the read for step kt - 1, issued during step kt - 2)
+      if constexpr (P == 0 && n == 34) issue_scales((kt + 2) >> 1);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    // everything requested above has landed before the registers are touched again
+    lds_wait<0>();
+    pin(f[0]);
+    fix_scales(std::integral_constant<int, set ^ 1>{});
+  };
+  using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
+  lds_wait<0>();
+  pin(f[0]);
+  for (int kt = 0; kt < nk; kt += 4) {
+    step(I0{}, kt);
+    step(I1{}, kt + 1);
+    step(I2{}, kt + 2);
+    step(I3{}, kt + 3);
+  }
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
+#endif
+}
+
+bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
+  // whole tiles, K steps in groups of four (K a multiple of 1024 elements), scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 512 == 0 && p.k_bytes >= 512 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
+         p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
+         p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
+}
+
+int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = (p.M / 256) * (p.N / 256);
+  gemm_wave128_mxfp4_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
   // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
   if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
