@@ -328,8 +328,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   const int l16 = lane & 15, kg = lane >> 4;
 
   const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
   int pm, pn;
-  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
 
   // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
@@ -341,8 +343,14 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     voffA[par] = drow * (unsigned)p.lda + chunk * 16;
     voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
   }
-  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
-  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
+  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
+  const char* gA;
+  const char* gB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+  };
+  set_fill_tile(pm, pn);
   const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
   auto issue = [&](auto J_, int kt, unsigned stage_base) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
@@ -372,10 +380,13 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   i32x8 a0[MH], a1[MH], b[2][NT];
 
   f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < MT; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
-    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
   static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
@@ -387,10 +398,9 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #pragma unroll
   for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
 
-  // One K step on stage P with the B fragments of set `cur`.
-  auto step = [&](auto P_, auto CUR_, auto MORE_, auto REFILL_, int kt) {
+  // One K step on stage P with the B fragments of set `cur`; its loads fetch K step `fk` of the fill tile.
+  auto step = [&](auto P_, auto CUR_, int fk) {
     constexpr int P = decltype(P_)::value, cur = decltype(CUR_)::value, nxt = cur ^ 1;
-    constexpr bool more = decltype(MORE_)::value, refill = decltype(REFILL_)::value;
     constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
     // first half: rows 0..3 of A; the A fragments 4..7 of this stage are read meanwhile
     static_for<MH * NT>([&](auto N_) {
@@ -407,22 +417,44 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     static_for<MH * NT>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
       mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
-      if constexpr (more && n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
-      if constexpr (more && n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
-      if constexpr (refill && n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, kt + 2, lds0 + P * STAGE);
+      if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
+      if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
+      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE);
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
-  using T = std::true_type; using F = std::false_type;
-  for (int kt = 0; kt < nk - 2; kt += 2) {
-    step(I0{}, I0{}, T{}, T{}, kt);
-    step(I1{}, I1{}, T{}, T{}, kt + 1);
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  if (nk == 2) { fk = 1; advance(); }
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 2) {
+      step(I0{}, I0{}, fk); advance();
+      step(I1{}, I1{}, fk); advance();
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
   }
-  step(I0{}, I0{}, T{}, F{}, nk - 2);
-  step(I1{}, I1{}, F{}, F{}, nk - 1);
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 #endif
 }
 
@@ -435,7 +467,8 @@ static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int grid = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / 256) * (p.N / 256);
+  const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
   gemm_wave128_f8_kernel<FMT><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
