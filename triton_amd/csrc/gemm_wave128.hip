@@ -515,8 +515,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   const int l16 = lane & 15, kg = lane >> 4;
 
   const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
   int pm, pn;
-  grouped_tile(xcd_remap(blockIdx.x, num_m * num_n), num_m, num_n, p.group_m, pm, pn);
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
 
   // ---- operand loads, as in the 16-bit kernel
@@ -528,8 +530,18 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     voffA[par] = drow * (unsigned)p.lda + chunk * 16;
     voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
   }
-  const char* gA = p.A + ((int64_t)pm * BM + wave * 64) * p.lda;
-  const char* gB = p.B + ((int64_t)pn * BN + wave * 64) * p.ldb;
+  // scalar bases (operands and scales) of the tile the loads are fetching, two K steps ahead of the MFMAs
+  const char* gA;
+  const char* gB;
+  const char* gSA;
+  const char* gSB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
+  };
+  set_fill_tile(pm, pn);
   const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
   auto issue = [&](auto J_, int kt, unsigned stage_base) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
@@ -539,18 +551,12 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
   };
   // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of rows 64 w .. 64 w + 63 of A and of B
-  const char* gSA = (const char*)p.sA + ((int64_t)pm * BM + wave * 64) * p.lds_a;
-  const char* gSB = (const char*)p.sB + ((int64_t)pn * BN + wave * 64) * p.lds_b;
   const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
-  auto issue_scales = [&](int h) {   // pair h of K steps -> slot h & 1 (past the end of K: the last pair again)
-    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT + wave * 1024;
-    const int hd = h < nk / 2 ? h : nk / 2 - 1;
-    async_copy16_sbase(gSA, voffSA + (unsigned)hd * 16, slot);
-    async_copy16_sbase(gSB, voffSB + (unsigned)hd * 16, slot + BM * 16);
+  auto issue_scales = [&](int h) {   // pair h of K steps of the fill tile -> slot h & 1 (K steps come in fours, so
+    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT + wave * 1024;   // the slots alternate across tiles too)
+    async_copy16_sbase(gSA, voffSA + (unsigned)h * 16, slot);
+    async_copy16_sbase(gSB, voffSB + (unsigned)h * 16, slot + BM * 16);
   };
-  // Past the end of K the last tile is requested again (into a stage nobody reads any more), which keeps
-  // the loop uniform: one code path, no special last steps.
-  auto tile_at = [&](int t) { return t < nk ? t : nk - 1; };
 
   // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 2 kg + ks of row l16 (+ 16 t)
   unsigned adrA[KS], adrB[KS];
@@ -592,10 +598,13 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   };
 
   f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
 #pragma unroll
-  for (int i = 0; i < MT; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
-    for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
 
   // ---- prologue
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
@@ -611,7 +620,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   fix_scales(I0{});
 
   // K step U (0..3 within a group of four: stage U & 1, scale slot U >> 1, scale set U & 1)
-  auto step = [&](auto U_, int kt) {
+  auto step = [&](auto U_, int fk) {   // fk: the K step (of the fill tile) that this step's loads fetch
     constexpr int U = decltype(U_)::value, P = U & 1, set = U & 1;
     // sub-step 0
     static_for<NM>([&](auto N_) {
@@ -631,10 +640,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
       if constexpr (n == 32)
         read_scales(std::integral_constant<int, set ^ 1>{}, std::integral_constant<int, (((U + 1) & 3) >> 1) * SC_SLOT + ((U + 1) & 1) * 8>{});
-      if constexpr (n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, tile_at(kt + 2), lds0 + P * STAGE);
-      // (the scales of the K steps kt + 2, kt + 3 are requested in the even step kt, into the slot the steps
-      // kt - 2, kt - 1 used: its last reader was the read for step kt - 1, issued during step kt - 2)
-      if constexpr (P == 0 && n == 34) issue_scales((kt + 2) >> 1);
+      if constexpr (n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE);
+      // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
+      // two steps back used: its last reader was the read for the previous step, issued a step ago)
+      if constexpr (P == 0 && n == 34) issue_scales(fk >> 1);
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     // everything requested above has landed before the registers are touched again
@@ -645,15 +654,38 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
   lds_wait<0>();
   pin(f[0]);
-  for (int kt = 0; kt < nk; kt += 4) {
-    step(I0{}, kt);
-    step(I1{}, kt + 1);
-    step(I2{}, kt + 2);
-    step(I3{}, kt + 3);
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 4) {
+      step(I0{}, fk); advance();
+      step(I1{}, fk); advance();
+      step(I2{}, fk); advance();
+      step(I3{}, fk); advance();
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
   }
   wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
-  asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
-  gemm_epilogue16<MT, NT>(acc, p, pm * BM + wm * 128, pn * BN + wn * 128, l16, kg);
 #endif
 }
 
@@ -673,7 +705,8 @@ int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int grid = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / 256) * (p.N / 256);
+  const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
   gemm_wave128_mxfp4_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
