@@ -114,7 +114,7 @@ def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile
     # persistent) for shapes the size heuristic would give to another; K = 1536 covers three 16-byte
     # scale groups per row in the pipelined kernels (an odd number: the two-slot scale ring changes
     # parity from tile to tile in the persistent form, two programs for six and twelve tiles),
-    # K = 1056 (not a multiple of 512) their fall-back.  6 = MXFP4 on four waves of scaled 16x16x128 MFMAs: whole
+    # K = 1056 (not a multiple of 512) their fall-back.  6 = four waves of scaled 16x16x128 MFMAs (both formats): whole
     # 256x256 tiles and K a multiple of 1024 (the last two shapes: one and two groups of four K steps), else 5.
     monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
     monkeypatch.setenv("MI355_GEMM_PROGRAMS", "2")

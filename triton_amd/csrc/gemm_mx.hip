@@ -105,6 +105,7 @@ int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
   }
   // 6: MXFP4 on four waves of scaled 16x16x128 MFMAs (whole tiles, K a multiple of 1024)
   if (tile == 6 && fmt == 0 && gemm_wave128_mxfp4_ok(p)) return gemm_wave128_mxfp4_launch(p, stream);
+  if (tile == 6 && fmt != 0 && gemm_wave128_mxfp8_ok(p)) return gemm_wave128_mxfp8_launch(p, stream);
   return fmt == 0 ? launch_gemm_tile<CfgMxfp4, true>(p, tile, stream) : launch_gemm_tile<CfgMxfp8, true>(p, tile, stream);
 }
 

@@ -458,6 +458,223 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #endif
 }
 
+// Scaled fp8 (e4m3) MFMA with the accumulator pinned to the accumulation registers; byte 0 of the scale dwords.
+__device__ __forceinline__ void mfma16_mxfp8(const i32x8& a, const i32x8& b, f32x4& c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]"
+               : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+#endif
+}
+#ifndef MXFP8_CHUNK
+#define MXFP8_CHUNK(kg, c) ((kg) + 4 * (c))
+#endif
+
+// MXFP8 (e4m3 codes, one e8m0 scale per 32 elements): the fp8 kernel above with scaled MFMAs; a K step is
+// 128 elements = four scale blocks, the scales travel 16 bytes per row (four K steps) per direct load into a
+// two-slot LDS ring like those of the MXFP4 kernel below.
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int MT = 8, NT = 8, MH = MT / 2;
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
+  int pm, pn;
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+
+  // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
+  const char* gA;
+  const char* gB;
+  const char* gSA;
+  const char* gSB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
+  };
+  set_fill_tile(pm, pn);
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  auto issue = [&](auto J_, int kt, unsigned stage_base) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0>(src, lane_off, dst);
+  };
+
+  // ---- scale loads: wave w fetches the 16 scale bytes (four K steps) of rows 64 w .. 64 w + 63 of A and of B
+  const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
+  auto issue_scales = [&](int g) {   // group g of four K steps of the fill tile -> slot g & 1 (K steps come in eights)
+    const unsigned slot = lds0 + SC_BASE + (g & 1) * SC_SLOT + wave * 1024;
+    async_copy16_sbase(gSA, voffSA + (unsigned)g * 16, slot);
+    async_copy16_sbase(gSB, voffSB + (unsigned)g * 16, slot + BM * 16);
+  };
+  // scales of a K step: the dword of the step's four blocks, shifted so that this lane group's byte is byte 0
+  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16;
+  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16;
+  const int sshift = 8 * kg;
+  int sa[2][MT], sb[2][NT];
+  auto read_scales = [&](auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 3) * 4
+    constexpr int set = decltype(SET_)::value, off = decltype(OFF_)::value;
+    static_for<MT>([&](auto T_) { constexpr int t = decltype(T_)::value; sa[set][t] = lds_read_b32<off + t * 256>(adrSA); });
+    static_for<NT>([&](auto T_) { constexpr int t = decltype(T_)::value; sb[set][t] = lds_read_b32<off + t * 256>(adrSB); });
+  };
+  auto fix_scales = [&](auto SET_) {
+    constexpr int set = decltype(SET_)::value;
+    static_for<MT>([&](auto T_) { constexpr int t = decltype(T_)::value; lds_use(sa[set][t]); sa[set][t] = (int)((unsigned)sa[set][t] >> sshift); });
+    static_for<NT>([&](auto T_) { constexpr int t = decltype(T_)::value; lds_use(sb[set][t]); sb[set][t] = (int)((unsigned)sb[set][t] >> sshift); });
+  };
+
+  // ---- fragment reads.  The 8-bit forms of the scaled MFMA split a lane's 32 bytes: registers 0-3 of the lane
+  // groups 2 b, 2 b + 1 together are scale block b, registers 4-7 block 2 + b, and block b takes its scale from
+  // lane group b.  So lane (l16, kg) reads chunk kg into its low and chunk 4 + kg into its high registers and
+  // supplies the scale of block kg.
+  LDS_PTR(const char) fragA[2];
+  LDS_PTR(const char) fragB[2];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const unsigned slot = ((MXFP8_CHUNK(kg, c)) ^ s) * 16;
+      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * 128 + l16) * ROWB + slot;
+      fragB[c] = (LDS_PTR(const char))lds_raw + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+  }
+  auto read_frag = [&](LDS_PTR(const char) (&base)[2], int off) {
+    i32x4 lo = *(LDS_PTR(const i32x4))(base[0] + off);
+    i32x4 hi = *(LDS_PTR(const i32x4))(base[1] + off);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  i32x8 a0[MH], a1[MH], b[2][NT];
+
+  f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
+
+  // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
+  issue_scales(0);
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE); });
+  wait_vmcnt<16>();
+  block_barrier();
+  read_scales(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+  lds_wait<0>();
+  fix_scales(std::integral_constant<int, 0>{});
+#pragma unroll
+  for (int t = 0; t < NT; t++) b[0][t] = read_frag(fragB, t * 16 * ROWB);
+#pragma unroll
+  for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
+
+  // K step U (0..7 within a group of eight: stage and register sets U & 1, scale slot U >> 2); its loads fetch
+  // K step `fk` of the fill tile.
+  auto step = [&](auto U_, int fk) {
+    constexpr int U = decltype(U_)::value, P = U & 1, cur = U & 1, nxt = cur ^ 1, UN = (U + 1) & 7;
+    constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp8(b[cur][j], a0[i], acc[i][j], sb[cur][j], sa[cur][i]);
+      if constexpr (n % 4 == 0 && n / 4 < MH) a1[n / 4] = read_frag(fragA, so + (MH + n / 4) * 16 * ROWB);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    lds_wait<0>();
+    wait_vmcnt<0>();
+    block_barrier();
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp8(b[cur][j], a1[i], acc[MH + i][j], sb[cur][j], sa[cur][MH + i]);
+      if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
+      if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
+      if constexpr (n == 14) read_scales(std::integral_constant<int, nxt>{}, std::integral_constant<int, (UN >> 2) * SC_SLOT + (UN & 3) * 4>{});
+      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE);
+      // (the scales of the K steps fk .. fk + 3 are requested in the third step of every four, into the slot whose
+      // last reader was the read for the step before this one)
+      if constexpr ((U & 3) == 2 && n == 16) issue_scales(fk >> 2);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    lds_wait<0>();
+    fix_scales(std::integral_constant<int, nxt>{});
+  };
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 8) {
+      static_for<8>([&](auto U_) { step(U_, fk); advance(); });
+    }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
+  }
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+#endif
+}
+
+bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
+  // whole tiles, K steps in groups of eight (K a multiple of 1024), scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 1024 == 0 && p.k_bytes >= 1024 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
+         p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
+         p.lds_a * 64 + p.k_bytes / 32 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 32 < (1ll << 31);
+}
+
+int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int tiles = (p.M / 256) * (p.N / 256);
+  const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
+  gemm_wave128_mxfp8_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 template <int FMT>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128;

@@ -90,6 +90,8 @@ int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
 bool gemm_wave128_mxfp4_ok(const GemmArgs& p);
 int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream);
+bool gemm_wave128_mxfp8_ok(const GemmArgs& p);
+int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream);
 bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
 int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
 bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_bytes);
