@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   // half of them (one read per two MFMAs).  The last sub-step of a stage first meets the other waves
   // (every wave has then read all it needs of this stage, and the other stage has landed), reads the
   // first fragments of the other stage and refills this one with the tile two steps ahead (one load
-  // per two MFMAs).
+  // per four MFMAs).
   auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_, int kt) {
     constexpr int P = decltype(P_)::value, ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
     constexpr bool last = ks == KS - 1;
@@ -237,10 +237,13 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
       mfma16(f[cur].b[j], f[cur].a[i], acc[i][j]);
+      // one fragment read per two MFMAs over the first half, one direct load per four MFMAs (64 cycles) over the
+      // whole sub-step: loads issued faster than the memory pipeline takes them hold up the MFMAs behind them
+      // (one per two MFMAs: -3.5 %)
       if constexpr (more && n % 2 == 0 && n / 2 < NRD)
         read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, last ? (P ^ 1) : P>{},
                  std::integral_constant<int, last ? 0 : ks + 1>{}, f[nxt]);
-      if constexpr (refill && n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, kt + 2, lds0 + P * STAGE);
+      if constexpr (refill && n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, kt + 2, lds0 + P * STAGE);
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -277,7 +280,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
     // above are MFMAs: let the last ones retire before their results are read.
     lds_wait<0>();
     pin(f[0]);
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     // (the tile and lane coordinates pass through an empty assembly statement so that none of the
     // epilogue's address arithmetic is hoisted out of the tile loop, where it would occupy - and spill -
     // registers throughout the K loop)
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       step(I0{}, I0{}, fk); advance();
       step(I1{}, I1{}, fk); advance();
     }
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
@@ -640,7 +643,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
     for (int kt = 0; kt < nk; kt += 8) {
       static_for<8>([&](auto U_) { step(U_, fk); advance(); });
     }
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
@@ -857,10 +860,11 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
       if constexpr (n == 32)
         read_scales(std::integral_constant<int, set ^ 1>{}, std::integral_constant<int, (((U + 1) & 3) >> 1) * SC_SLOT + ((U + 1) & 1) * 8>{});
-      if constexpr (n % 2 == 1 && n / 2 < 16) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE);
+      if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fk, lds0 + P * STAGE);   // one per 64 cycles
       // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
       // two steps back used: its last reader was the read for the previous step, issued a step ago)
-      if constexpr (P == 0 && n == 34) issue_scales(fk >> 1);
+      // (after the last operand load: the eight loads of an operand share the M0 value that the first one sets)
+      if constexpr (P == 0 && n == 62) issue_scales(fk >> 1);
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     // everything requested above has landed before the registers are touched again
@@ -893,7 +897,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       step(I2{}, fk); advance();
       step(I3{}, fk); advance();
     }
-    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
