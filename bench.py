@@ -24,9 +24,9 @@ PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4":
 HBM_GBPS = 8000.0
 
 # HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc:
-# FETCH_SIZE 788311 KiB x 2.000 + WRITE_SIZE 131235 KiB x 1.000, the factors being what the same
+# FETCH_SIZE 820374 KiB x 2.000 + WRITE_SIZE 143130 KiB x 1.000, the factors being what the same
 # counters read for a plain copy of known size (profiles/gemm_bf16_8192.md)
-MEASURED_TRAFFIC_BYTES = int((788311 * 2.000 + 131235 * 1.000) * 1024)
+MEASURED_TRAFFIC_BYTES = int((820374 * 2.000 + 143130 * 1.000) * 1024)
 
 
 def time_launches(fn, steps, warmup):
@@ -139,7 +139,7 @@ def main():
         "config": {"workload": f"bf16 GEMM M=N=K={n}, A row-major MxK, B row-major KxN, fp32 accumulate, bf16 out (BASELINE config 2)"},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 2), "peak": PEAK["bf16"], "unit": "TFLOP/s",
                      "frac": round(achieved / PEAK["bf16"], 4), "traffic": MEASURED_TRAFFIC_BYTES,
-                     "kernel": "gemm_wave128_kernel<bf16, row-major B> (256x256 tile per workgroup, four waves of 128x128 from 16x16x32 MFMAs, two 64 KiB LDS stages)", "launch_ms_avg": round(ev_ms, 5),
+                     "kernel": "gemm_wave128_kernel<bf16, row-major B> (256x256 tiles, four waves of 128x128 from 16x16x32 MFMAs, two 64 KiB LDS stages, one program per CU)", "launch_ms_avg": round(ev_ms, 5),
                      "launch_ms_min": round(min(per), 5), "algorithmic_flops": flops,
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
