@@ -66,7 +66,9 @@ __device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned l
 }
 
 // The same with an instruction offset, which the hardware adds to BOTH addresses (global and LDS):
-// several copies can then share one M0 value.  SETM0 = false reuses the M0 of the previous copy.
+// several copies can then share one M0 value.  SETM0 = false reuses the M0 of the previous copy: nothing in
+// between may write M0 (compiler-generated code does so only for indirect register indexing, message and GWS
+// instructions and its own LDS-direct loads, none of which the kernels using this have).
 template <int OFF, bool SETM0>
 __device__ __forceinline__ void async_copy16_sbase_off(const void* sbase, unsigned lane_off, unsigned lds_wave_base) {
 #if MI355_DEVICE_PASS

@@ -253,6 +253,11 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   auto stage = [&](auto P_, int fk) {
     substep(P_, I0{}, T{}, F{}, fk - 2);
     substep(P_, I1{}, T{}, T{}, fk - 2);
+    // The fragment reads above are invisible to the compiler: have them landed before control reaches a loop
+    // edge, where the register allocator may copy the registers they write.  (They were issued over the first
+    // half of the sub-step, so this does not wait.)
+    lds_wait<0>();
+    pin(f[0]);
   };
   // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
   // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
