@@ -156,6 +156,10 @@ def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
         at._launch(ta, tb, cbuf[:, :N], at.Config(6, 4))
         assert np.allclose(to_np(cbuf[:, :N]), gemm.matmul_closed_form(a, b, out_dtype=dtype), rtol=1e-2, atol=1e-2)
         assert torch.count_nonzero(cbuf[:, N:]).item() == 0
+        # and into a column-major C (unit stride along M: the epilogue falls back to single stores), row-major B
+        ct = torch.zeros(N, M, device=gpu, dtype=torch.float32)
+        at._launch(ta, from_np(b, dtype, gpu), ct.t(), at.Config(6, 8))
+        assert np.allclose(to_np(ct.t()), gemm.matmul_closed_form(a, b, out_dtype="fp32"), rtol=1e-2, atol=1e-2)
 
 
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
