@@ -296,6 +296,24 @@ def test_full_size_8192_bf16_sampled_rows_and_exact_permutation(gpu):
     del c, cp
 
 
+def test_full_size_8192_fp8_sampled_rows_and_k_major_bf16(gpu):
+    # BASELINE config 4 at full size (e4m3fn codes with per-tensor scales, bf16 out), sampled rows against the
+    # dequantised fp64 product; and config 2 with B stored K-major (the `b.T` view), sampled rows
+    n = 8192
+    g = torch.Generator(device="cpu").manual_seed(1)
+    x = torch.randn(n, n, generator=g); y = torch.randn(n, n, generator=g)
+    sx = (x.abs().amax() / 448).item(); sy = (y.abs().amax() / 448).item()
+    qa = (x / sx).clamp(-448, 448).to(torch.float8_e4m3fn); qb = (y / sy).clamp(-448, 448).to(torch.float8_e4m3fn)   # qb is [N, K]
+    c = triton_amd.matmul(qa.to(gpu), qb.to(gpu).t(), a_scale=sx, b_scale=sy, out_dtype=torch.bfloat16)
+    rows = [0, 255, 256, 4097, 8191]
+    ref = (qa[rows].double().numpy() @ qb.double().numpy().T) * (sx * sy)
+    assert np.allclose(to_np(c[rows]), ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max() / 16)
+    a16 = x.bfloat16(); b16 = y.bfloat16()                       # b16 is [N, K]: K-major B
+    c16 = triton_amd.matmul(a16.to(gpu), b16.to(gpu).t())
+    ref16 = formats.round_bf16((a16[rows].double().numpy() @ b16.double().numpy().T).astype(np.float32))
+    assert np.allclose(to_np(c16[rows]), ref16, rtol=1e-2, atol=1e-2)
+
+
 def test_decode_shape_m16(gpu):
     # config 4 decode variant: M = 16, N = K = 8192 (bandwidth bound)
     rng = np.random.default_rng(3)
