@@ -130,13 +130,14 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.aux = aux; p.aux_sm = aux_sm; p.aux_sn = aux_sn; p.aux_dtype = aux_dtype;
 
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
-  // 256x256 tiles once they fill three quarters of the CUs, 128x128 tiles (two workgroups per CU) below that
+  // 256x256 tiles once they fill half of the CUs, 128x128 tiles (two workgroups per CU) below that
+  // (bf16, 144 tiles: 912 vs 651 TFLOP/s; 100 tiles: 654 vs 715)
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
   // large problems run the software-pipelined 8-wave kernel
   // (5 = the persistent form of the pipelined kernel; it falls back to 4 for edge tiles or a K tail)
   // persistent only when every program gets the same number of tiles: with a remainder the hardware's
   // dynamic dispatch of one workgroup per tile balances better (6144^3: 1011 vs 942 TFLOP/s)
-  int tile = (tiles256 * 4 >= 3L * cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
+  int tile = (tiles256 * 2 >= cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
   // 16-bit operands, whole 256x256 tiles and K steps, at least half a round of tiles: four waves of
   // 16x16x32 MFMAs, one workgroup per tile (at 8192^3 bf16 +5 % over the persistent form with a row-major
   // B, +14 % with a K-major B; at 3072^3, 144 tiles, 790 vs 660 TFLOP/s for the 128x128 tiles)
@@ -257,7 +258,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
-  int tile = (tiles256 * 4 >= 3L * cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
+  int tile = (tiles256 * 2 >= cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
   // MXFP4 with whole 256x256 tiles, K a multiple of 1024 and at least half a round of tiles: four waves of
   // scaled 16x16x128 MFMAs (8192^3: 4000-4050 vs 3340-3640 TFLOP/s for the persistent eight-wave kernel)
   if (fmt == MI355_MXFP4 && tiles256 * 2 >= cus && gemm_wave128_mxfp4_ok(p)) tile = 6;
