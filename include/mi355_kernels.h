@@ -177,7 +177,9 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C,
  * `num_programs` workgroups walk the tiles of all problems (the reference's NUM_SM); 0 picks two
  * per compute unit.  Any sizes are accepted (partial tiles are handled; the reference assumes
  * full tiles); problems whose lda, ldb, N or K are not multiples of 8 elements, or whose A / B
- * are not 16-byte aligned, run a slower loop inside the same kernel.  Nothing about the device
+ * are not 16-byte aligned, run a slower loop inside the same kernel.  Groups in which every problem
+ * is whole 256x256 tiles with K a multiple of 128 (and ldb a multiple of 256 elements) run a faster
+ * kernel from one tile per compute unit and K >= 1024 on.  Nothing about the device
  * arrays can be checked on the host: they must hold `group_size` valid entries.
  */
 int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,

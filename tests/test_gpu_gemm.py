@@ -160,6 +160,12 @@ def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
         ct = torch.zeros(N, M, device=gpu, dtype=torch.float32)
         at._launch(ta, from_np(b, dtype, gpu), ct.t(), at.Config(6, 8))
         assert np.allclose(to_np(ct.t()), gemm.matmul_closed_form(a, b, out_dtype="fp32"), rtol=1e-2, atol=1e-2)
+        # row-major B as a column slice of wider matrices: a pitch that is a multiple of 512 bytes (this kernel)
+        # and one that is not (its column-group XOR needs that multiple: another kernel takes the product)
+        for pad in (256, 8):
+            wide = from_np(np.pad(b, ((0, 0), (pad, pad))), dtype, gpu)
+            c = to_np(triton_amd.matmul(ta, wide[:, pad:pad + N], out_dtype=torch.float32))
+            assert np.allclose(c, gemm.matmul_closed_form(a, b, out_dtype="fp32"), rtol=1e-2, atol=1e-2), pad
 
 
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])

@@ -62,3 +62,47 @@ def test_strided_rows_and_empty_group(gpu):
     assert triton_amd.group_gemm_fn([], []) == []
     with pytest.raises(AssertionError):
         triton_amd.group_gemm_fn([a], [b, b])
+
+
+@pytest.mark.parametrize("nprog", [0, 7, 100])
+def test_groups_of_whole_256_tiles(gpu, nprog, monkeypatch):
+    # every problem whole 256x256 tiles and K % 128 == 0: the four-wave 16x16-MFMA kernel takes the group
+    # (thresholds lowered so that 20 tiles and K = 128 are enough); exact sums of small integers, rounded
+    # once; K from one pair of stages up to several, M != N, problems of one tile between larger ones
+    monkeypatch.setenv("MI355_GROUPED_BIG_MIN", "1")
+    monkeypatch.setenv("MI355_GROUPED_WAVE128_MIN_K", "128")
+    rng = np.random.default_rng(40 + nprog)
+    shapes = [(256, 256, 128), (512, 256, 256), (256, 256, 1024), (256, 768, 384), (1024, 512, 128), (256, 256, 256), (512, 512, 640)]
+    ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]
+    gb = [rng.integers(-2, 3, size=(k, n)).astype(np.float32) for m, n, k in shapes]
+    ref = [a @ b for a, b in zip(ga, gb)]
+    for dtype in ("fp16", "bf16"):
+        outs = _run(gpu, ga, gb, dtype, num_programs=nprog)
+        for c, r in zip(outs, ref):
+            assert bits_equal(c, formats.round_to(r, dtype))   # (K = 1024 reaches beyond bf16's exact integers)
+    # the same group through the eight-wave kernels
+    monkeypatch.setenv("MI355_GROUPED_WAVE128_MIN_K", "0")
+    for c, r in zip(_run(gpu, ga, gb, "fp16", num_programs=nprog), ref):
+        assert bits_equal(c, r)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_whole_tile_groups_at_the_default_thresholds_against_closed_form(gpu, dtype):
+    # 256 tiles of 256x256 with K = 2048 select the four-wave kernel without any knob: N(0,1) operands, padded
+    # rows of A and C-sized B pitch of 512-byte multiples in the second problem.  A B pitch that is no such
+    # multiple (third case) sends the group to the eight-wave kernels.
+    rng = np.random.default_rng(5)
+    mk = lambda shape: formats.round_to(rng.standard_normal(shape).astype(np.float32), dtype)
+    a = [mk((2048, 2048)) for _ in range(4)]
+    b = [mk((2048, 2048)) for _ in range(4)]
+    ref = [gemm.matmul_closed_form(x, y, out_dtype=dtype) for x, y in zip(a, b)]
+    ta = [from_np(x, dtype, gpu) for x in a]
+    tb = [from_np(y, dtype, gpu) for y in b]
+    ta[1] = from_np(np.pad(a[1], ((0, 0), (0, 64))), dtype, gpu)[:, :2048]
+    for pad in (0, 256, 8):
+        if pad:
+            tb[1] = from_np(np.pad(b[1], ((0, 0), (pad, 0))), dtype, gpu)[:, pad:]
+        outs = triton_amd.group_gemm_fn(ta, tb)
+        for c, r in zip(outs, ref):
+            assert np.allclose(to_np(c), r, rtol=1e-2, atol=1e-2), pad
+            assert np.mean(to_np(c) == r) > 0.98

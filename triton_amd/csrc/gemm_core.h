@@ -430,18 +430,38 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 // them works: the large tiles when the group holds at least `big_tiles_min` of them (enough to give
 // every CU one), the small tiles otherwise - a decision every workgroup of both launches reaches
 // alike from the same table, so no host round trip is needed to see sizes that live on the device.
+//
+// A third launch (gemm_wave128.hip) takes groups made of whole 256x256 tiles only, see grouped_plan.
+
+// Which grouped kernel computes this group: 2 = the four-wave 16x16-MFMA kernel (every problem whole
+// 256x256 tiles, K a multiple of 128 and at least `wave128_min_k`, 16-byte rows of A, 512-byte multiples
+// as pitch of B, 32-bit lane offsets, and at least `big_tiles_min` tiles), 1 = 256x256 tiles,
+// 0 = 128x128 tiles.  (That kernel restarts its two-stage pipeline at every tile and fetches two K steps
+// too many per tile; measured against the other two on fp16 groups of 256 to 1024 tiles it gains 10-25 %
+// on problems of 2048^2 and 4096^2 with K from 1024 to 4096, is even at K = 512 and loses 10 % on 64
+// problems of 1024^3.)
+__device__ __forceinline__ int grouped_plan(const GroupedArgs& ga) {
+  long big_tiles = 0;
+  bool whole = ga.wave128_min_k > 0;
+  for (int gi = 0; gi < ga.group_size; gi++) {
+    const int gm = ga.sizes[gi * 3], gn = ga.sizes[gi * 3 + 1], gk = ga.sizes[gi * 3 + 2];
+    const int lda = ga.lds[gi * 3], ldb = ga.lds[gi * 3 + 1];
+    big_tiles += (long)((gm + 255) / 256) * ((gn + 255) / 256);
+    whole = whole && gm % 256 == 0 && gn % 256 == 0 && gk % 128 == 0 && gk >= 128 && gk >= ga.wave128_min_k && lda % 8 == 0 && ldb % 256 == 0 &&
+            lda > 0 && ldb > 0 && (ga.a_ptrs[gi] | ga.b_ptrs[gi]) % 16 == 0 &&
+            (int64_t)lda * 16 + gk * 2 < (1ll << 31) && (int64_t)gk * ldb * 2 + 512 < (1ll << 31);
+  }
+  if (whole && big_tiles >= ga.big_tiles_min) return 2;
+  return big_tiles >= ga.big_tiles_min ? 1 : 0;
+}
+
 template <typename Cfg, typename T, int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_grouped_kernel(GroupedArgs ga) {
   constexpr int NS = 4;
   constexpr bool BIG = BM == 256;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   LDS_PTR(char) const lds = (LDS_PTR(char))smem;
-  {
-    long big_tiles = 0;
-    for (int gi = 0; gi < ga.group_size; gi++)
-      big_tiles += (long)((ga.sizes[gi * 3] + 255) / 256) * ((ga.sizes[gi * 3 + 1] + 255) / 256);
-    if ((big_tiles >= ga.big_tiles_min) != BIG) return;
-  }
+  if (grouped_plan(ga) != (BIG ? 1 : 0)) return;
   const int nprog = gridDim.x;
   int tile_idx = xcd_remap(blockIdx.x, nprog);
   int last_problem_end = 0;
@@ -503,7 +523,9 @@ static int launch_gemm_grouped_one(const GroupedArgs& ga, int nprog, hipStream_t
 // nprog: programs of the 128x128 form; nprog_big: programs of the 256x256 form (one per CU)
 template <typename Cfg, typename T>
 static int launch_gemm_grouped(const GroupedArgs& ga, int nprog, int nprog_big, hipStream_t stream) {
-  int rc = launch_gemm_grouped_one<Cfg, T, 256, 256, 2, 4>(ga, nprog_big, stream);
+  int rc = gemm_wave128_grouped_launch(ga, std::is_same<T, __bf16>::value, nprog_big, stream);
+  if (rc) return rc;
+  rc = launch_gemm_grouped_one<Cfg, T, 256, 256, 2, 4>(ga, nprog_big, stream);
   if (rc) return rc;
   return launch_gemm_grouped_one<Cfg, T, 128, 128, 2, 2>(ga, nprog, stream);
 }

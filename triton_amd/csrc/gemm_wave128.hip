@@ -85,15 +85,35 @@ __device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const Gemm
   });
 }
 
-template <typename V8, bool B_KMAJOR>
-__global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
+// The same for a plain C = A @ B in the operands' own 16-bit type with unit column stride (the grouped GEMM).
+template <int MT, int NT, typename OutT>
+__device__ __forceinline__ void gemm_epilogue16_plain(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
+  typedef OutT Out4 __attribute__((ext_vector_type(4)));
+  static_for<MT>([&](auto I_) {
+    constexpr int i = decltype(I_)::value;
+    OutT* row = (OutT*)p.C + (int64_t)(mrow0 + i * 16 + l16) * p.ldc + ncol0 + kg * 4;
+    static_for<NT>([&](auto J_) {
+      constexpr int j = decltype(J_)::value;
+      const f32x4 v = acc[i][j];
+      if (p.c_vec_ok) *(Out4*)(row + j * 16) = Out4{(OutT)v[0], (OutT)v[1], (OutT)v[2], (OutT)v[3]};
+      else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) row[j * 16 + e] = (OutT)v[e];
+      }
+    });
+  });
+}
+
+// The tiles `tile`, `tile + tile_step`, ... (< M/256 * N/256) of one problem, computed by the calling workgroup
+// with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  PLAIN: C has
+// the type of the operands, no scales, no activation.
+template <typename V8, bool B_KMAJOR, bool XCD, bool PLAIN = false>
+__device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
   constexpr int MT = 8, NT = 8, KS = 2;                             // 16x16 tiles per wave, 16x16x32 sub-steps per stage
   constexpr int NM = MT * NT;                                       // MFMAs per sub-step
-  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -102,13 +122,12 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 
   const int num_m = p.M / BM, num_n = p.N / BN;
   const int ntiles = num_m * num_n;
-  // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid is either one workgroup per tile or, when
-  // that divides evenly, one per CU) as ONE stream of K steps: the loads of the last two steps of a tile
-  // already fetch the first two K steps of the next one, so its first fragments are in registers when the
-  // finished tile is stored.
-  int tile = blockIdx.x;
+  // The tiles are computed as ONE stream of K steps: the loads of the last two steps of a tile already
+  // fetch the first two K steps of the next one, so its first fragments are in registers when the finished
+  // tile is stored.
+  auto tile_at = [&](int t, int& tm, int& tn) { grouped_tile(XCD ? xcd_remap(t, ntiles) : t, num_m, num_n, p.group_m, tm, tn); };
   int pm, pn;
-  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+  tile_at(tile, pm, pn);
   const int nk = p.k_bytes / ROWB;
 
   // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
@@ -129,7 +148,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   // 4 (j & 1) + 2 (i / 32) and (j >> 2) & 1: the j terms are XORed into the lane offset at each load.
   if constexpr (!B_KMAJOR) {
     const unsigned pg = (lane & 31) >> 1, half = lane & 1;
-    voffB[0] = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;   // j = 0; other j: XOR below
+    // j = 0; other j: XOR below (which needs a pitch that is a multiple of 512 bytes)
+    voffB[0] = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;
   }
   // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
   const char* gA;
@@ -266,10 +286,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
   auto advance = [&]() {
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) {
-        ftile += gridDim.x;
+      if (ftile + tile_step < ntiles) {
+        ftile += tile_step;
         int fm, fn;
-        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        tile_at(ftile, fm, fn);
         set_fill_tile(fm, fn);
       }
     }
@@ -291,13 +311,61 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
     // registers throughout the K loop)
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
-    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
-    tile += gridDim.x;
+    if constexpr (PLAIN) gemm_epilogue16_plain<MT, NT, std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>>(acc, p, em, en, el, ek);
+    else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += tile_step;
     if (tile >= ntiles) break;
-    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    tile_at(tile, pm, pn);
     zero_acc();
   }
   wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+#endif
+}
+
+// Workgroup b computes the tiles b, b + gridDim.x, ... (the grid is either one workgroup per tile or, when
+// that divides evenly, one per CU).
+template <typename V8, bool B_KMAJOR>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  gemm_wave128_tiles<V8, B_KMAJOR, true>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
+#endif
+}
+
+// Grouped GEMM (python/tutorials/08-grouped-gemm.py:64-140: pointers, sizes and leading dimensions of the
+// problems in device arrays, row-major B) for groups made of whole 256x256 tiles: gridDim.x workgroups walk
+// the tiles of all problems, numbered problem after problem; a tile is one run of the stream above (its
+// loads wrap around to the tile's own first steps at the end), so consecutive tiles of a workgroup may
+// belong to different problems.  Every workgroup first reads the tables and returns unless this kernel is
+// the one that the group's shapes select (grouped_plan).
+template <typename V8>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_grouped_kernel(GroupedArgs ga) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+  if (grouped_plan(ga) != 2) return;
+  const int nprog = gridDim.x;
+  int tile_idx = xcd_remap(blockIdx.x, nprog);
+  int first = 0;   // number of the first tile of problem gi
+  for (int gi = 0; gi < ga.group_size; gi++) {
+    const int gm = ga.sizes[gi * 3], gn = ga.sizes[gi * 3 + 1], gk = ga.sizes[gi * 3 + 2];
+    const int num_tiles = (gm / 256) * (gn / 256);
+    if (tile_idx < first + num_tiles) {
+      const int ldc = ga.lds[gi * 3 + 2];
+      GemmArgs p{};
+      p.A = (const char*)ga.a_ptrs[gi]; p.B = (const char*)ga.b_ptrs[gi]; p.C = (char*)ga.c_ptrs[gi];
+      p.M = gm; p.N = gn; p.K = gk; p.k_bytes = gk * 2;
+      p.lda = (int64_t)ga.lds[gi * 3] * 2; p.ldb = (int64_t)ga.lds[gi * 3 + 1] * 2; p.ldc = ldc; p.scn = 1;
+      p.out_dtype = ga.out_dtype; p.group_m = 8;
+      p.c_vec_ok = (ldc % 4 == 0) && (((uintptr_t)p.C) % 16 == 0);
+      while (tile_idx < first + num_tiles) {
+        gemm_wave128_tiles<V8, false, false, true>(p, tile_idx - first, num_tiles, lds0);
+        block_barrier();   // the next tile's loads overwrite the stages: every wave must be done reading them
+        tile_idx += nprog;
+      }
+    }
+    first += num_tiles;
+  }
 #endif
 }
 
@@ -941,7 +1009,9 @@ bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
   // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
   if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
   if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
-  return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (int64_t)p.K * p.ldb + 512 < (1ll << 31);
+  // (row-major B: the per-load XOR of the column group acts on the whole lane offset, so the row term
+  // in it - a multiple of the pitch - must leave the bits of the 512-byte tile row alone)
+  return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
 template <typename V8, bool B_KMAJOR>
@@ -959,6 +1029,23 @@ static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
   gemm_wave128_kernel<V8, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
+}
+
+template <typename V8>
+static int launch_wave128_grouped(const GroupedArgs& ga, int nprog, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_grouped_kernel<V8>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  gemm_wave128_grouped_kernel<V8><<<dim3(nprog), dim3(256), smem, stream>>>(ga);
+  return (int)hipGetLastError();
+}
+
+int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hipStream_t stream) {
+  return bf16 ? launch_wave128_grouped<bf16x8>(ga, nprog, stream) : launch_wave128_grouped<f16x8>(ga, nprog, stream);
 }
 
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream) {

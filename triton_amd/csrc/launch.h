@@ -80,7 +80,10 @@ struct GroupedArgs {
   int group_size;
   int out_dtype;           // element type of A, B and C: 0 = fp16, 1 = bf16
   int big_tiles_min;       // 256x256 tiles in the group from which the large-tile kernel takes the launch
+  int wave128_min_k;       // groups of whole 256x256 tiles with every K >= this go to the four-wave 16x16-MFMA kernel (0 = never)
 };
+
+int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hipStream_t stream);
 
 int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
