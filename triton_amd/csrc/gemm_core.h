@@ -440,19 +440,24 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 // too many per tile; measured against the other two on fp16 groups of 256 to 1024 tiles it gains 10-25 %
 // on problems of 2048^2 and 4096^2 with K from 1024 to 4096, is even at K = 512 and loses 10 % on 64
 // problems of 1024^3.)
+// Every wave reads the tables with one problem per lane (all loads in flight at once: a serial scan of 16
+// problems took 4-8 us in each of the three launches) and combines the lanes' findings.
 __device__ __forceinline__ int grouped_plan(const GroupedArgs& ga) {
-  long big_tiles = 0;
-  bool whole = ga.wave128_min_k > 0;
-  for (int gi = 0; gi < ga.group_size; gi++) {
+  long long big_tiles = 0;
+  bool whole = true;
+  for (int gi = threadIdx.x & 63; gi < ga.group_size; gi += 64) {
     const int gm = ga.sizes[gi * 3], gn = ga.sizes[gi * 3 + 1], gk = ga.sizes[gi * 3 + 2];
     const int lda = ga.lds[gi * 3], ldb = ga.lds[gi * 3 + 1];
-    big_tiles += (long)((gm + 255) / 256) * ((gn + 255) / 256);
+    big_tiles += (long long)((gm + 255) / 256) * ((gn + 255) / 256);
     whole = whole && gm % 256 == 0 && gn % 256 == 0 && gk % 128 == 0 && gk >= 128 && gk >= ga.wave128_min_k && lda % 8 == 0 && ldb % 256 == 0 &&
             lda > 0 && ldb > 0 && (ga.a_ptrs[gi] | ga.b_ptrs[gi]) % 16 == 0 &&
             (int64_t)lda * 16 + gk * 2 < (1ll << 31) && (int64_t)gk * ldb * 2 + 512 < (1ll << 31);
   }
-  if (whole && big_tiles >= ga.big_tiles_min) return 2;
-  return big_tiles >= ga.big_tiles_min ? 1 : 0;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) big_tiles += __shfl_xor(big_tiles, off);
+  const bool all_whole = ga.wave128_min_k > 0 && __all(whole);
+  const int plan = (all_whole && big_tiles >= ga.big_tiles_min) ? 2 : (big_tiles >= ga.big_tiles_min ? 1 : 0);
+  return __builtin_amdgcn_readfirstlane(plan);
 }
 
 template <typename Cfg, typename T, int BM, int BN, int WM, int WN>
