@@ -378,6 +378,51 @@ def test_skinny_16bit_decode_shapes_against_closed_form(gpu, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_fused_addends_in_the_four_wave_kernel(gpu, dtype, monkeypatch):
+    # the add-matrix / add-rows / add-cols forms (python/test/unit/language/test_core.py:3128-3145) in the
+    # addend instantiation of the 16x16-MFMA kernel: integer data, bit-exact; both B layouts, addend in fp32
+    # and in the input type, with scales and the activation, result in fp32 and in the input type
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    M, N, K = 512, 768, 256
+    rng = np.random.default_rng(77)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    z = rng.integers(-4, 5, size=(M, N)).astype(np.float32)
+    ta = from_np(a, dtype, gpu)
+    for tb in (from_np(b, dtype, gpu), from_np(np.ascontiguousarray(b.T), dtype, gpu).t()):
+        for add_dt in ("fp32", dtype):
+            tz = from_np(z, add_dt, gpu)
+            for add_np, add_t in ((z, tz), (z[:, :1], tz[:, :1]), (z[:1, :], tz[:1, :]), (z[0], tz[0])):
+                got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=add_t))
+                assert bits_equal(got, gemm.dot_epilogue(a, b, add=add_np)), (dtype, add_dt, add_np.shape)
+        got = to_np(triton_amd.matmul(ta, tb, add=from_np(z, "fp32", gpu), activation="leaky_relu", a_scale=0.5, b_scale=0.25))
+        ref = a @ b * 0.125 + z
+        ref = formats.round_to(np.where(ref >= 0, ref, np.float32(0.01) * ref).astype(np.float32), dtype)
+        assert np.allclose(got, ref, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_fused_addends_in_the_four_wave_fp8_kernel(gpu, monkeypatch, fmt, tdt):
+    # the same addend forms in the fp8 kernel of 16x16x128 MFMAs: codes of small integers (exact products
+    # and sums), addend in fp32 and bf16, bit-exact in fp32
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    M, N, K = 512, 256, 512
+    rng = np.random.default_rng(78)
+    table = formats.fp8_table(fmt)
+    small = np.array([c for c in range(256) if table[c] in (-2.0, -1.0, 0.0, 1.0, 2.0) and not (c == 0x80)], dtype=np.uint8)
+    ca = rng.choice(small, size=(M, K)); cb = rng.choice(small, size=(N, K))
+    a = table[ca].astype(np.float32); b = table[cb].astype(np.float32).T
+    z = rng.integers(-4, 5, size=(M, N)).astype(np.float32)
+    ta = torch.from_numpy(ca).to(gpu).view(tdt)
+    tb = torch.from_numpy(cb).to(gpu).view(tdt).t()
+    for add_dt in ("fp32", "bf16"):
+        tz = from_np(z, add_dt, gpu)
+        for add_np, add_t in ((z, tz), (z[:, :1], tz[:, :1]), (z[:1, :], tz[:1, :])):
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=add_t))
+            assert bits_equal(got, gemm.dot_epilogue(a, b, add=add_np)), (fmt, add_dt, add_np.shape)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512)])
 def test_fused_epilogues_of_the_reference_dot_test(gpu, dtype, shape):
     # add-matrix / add-rows / add-cols / softmax / chain-dot (python/test/unit/language/test_core.py:3128-3145)

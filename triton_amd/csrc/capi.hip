@@ -142,7 +142,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // 16x16x32 MFMAs, one workgroup per tile (at 8192^3 bf16 +5 % over the persistent form with a row-major
   // B, +14 % with a K-major B; at 3072^3, 144 tiles, 790 vs 660 TFLOP/s for the 128x128 tiles)
   // (fp8, K-major B: 16x16x128 MFMAs, 8192^3 e4m3 2790-2810 vs 2570-2600 TFLOP/s)
-  if (!aux && tiles256 * 2 >= cus && gemm_wave128_ok(p, b_kmajor)) tile = 6;
+  // (an epilogue addend: instantiations of their own)
+  if (tiles256 * 2 >= cus && gemm_wave128_ok(p, b_kmajor)) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
   p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
@@ -168,10 +169,10 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && !aux && gemm_wave128_ok(p, true)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && tile == 6 && gemm_wave128_ok(p, true)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
-  // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles, no addend)
-  if (tile == 6 && !aux && gemm_wave128_ok(p, b_kmajor)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
+  // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
+  if (tile == 6 && gemm_wave128_ok(p, b_kmajor)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 

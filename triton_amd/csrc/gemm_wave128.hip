@@ -41,12 +41,19 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 
 // Epilogue for 16x16 tiles computed with the operands swapped (D[n][m]): lane l owns C row
 // `mrow0 + 16 i + l%16` and, of tile (i, j), the four consecutive columns `ncol0 + 16 j + 4 (l/16) ..`.
-template <int MT, int NT>
-__device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
+// AuxT: element type of the addend of the fused epilogues (void = none).  With an addend the kernels are
+// separate instantiations: its arguments cost the plain kernels scalar registers that they need for their
+// load bases.  `aux_vec`: the four addend elements of a lane are consecutive and aligned (one load).
+template <int MT, int NT, typename AuxT>
+__device__ __forceinline__ void gemm_epilogue16_impl(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
+  constexpr bool AUX = !std::is_void<AuxT>::value;
+  using AuxE = std::conditional_t<AUX, AuxT, float>;
+  typedef AuxE Aux4 __attribute__((ext_vector_type(4)));
   float alpha = 1.f;
   if (p.a_scale) alpha *= *p.a_scale;
   if (p.b_scale) alpha *= *p.b_scale;
   const bool leaky = p.activation == 1;
+  const bool aux_vec = AUX && p.aux_sn == 1 && p.aux_sm % 4 == 0 && (uintptr_t)p.aux % 16 == 0;
   static_for<MT>([&](auto I_) {
     constexpr int i = decltype(I_)::value;
     const int m = mrow0 + i * 16 + l16;
@@ -55,9 +62,21 @@ __device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const Gemm
       const int n = ncol0 + j * 16 + kg * 4;
       float v[4];
 #pragma unroll
-      for (int e = 0; e < 4; e++) {
-        v[e] = acc[i][j][e] * alpha;
-        if (leaky) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
+      for (int e = 0; e < 4; e++) v[e] = acc[i][j][e] * alpha;
+      if constexpr (AUX) {
+        const AuxE* ax = (const AuxE*)p.aux + (int64_t)m * p.aux_sm + (int64_t)n * p.aux_sn;
+        if (aux_vec) {
+          const Aux4 t = *(const Aux4*)ax;
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)t[e];
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; e++) v[e] += (float)ax[e * p.aux_sn];
+        }
+      }
+      if (leaky) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
       }
       if (p.out_dtype == 4) {
         float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
@@ -85,6 +104,14 @@ __device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const Gemm
   });
 }
 
+template <int MT, int NT, bool AUX = false>
+__device__ __forceinline__ void gemm_epilogue16(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
+  if constexpr (!AUX) gemm_epilogue16_impl<MT, NT, void>(acc, p, mrow0, ncol0, l16, kg);
+  else if (p.aux_dtype == 4) gemm_epilogue16_impl<MT, NT, float>(acc, p, mrow0, ncol0, l16, kg);
+  else if (p.aux_dtype == 1) gemm_epilogue16_impl<MT, NT, __bf16>(acc, p, mrow0, ncol0, l16, kg);
+  else gemm_epilogue16_impl<MT, NT, _Float16>(acc, p, mrow0, ncol0, l16, kg);
+}
+
 // The same for a plain C = A @ B in the operands' own 16-bit type with unit column stride (the grouped GEMM).
 template <int MT, int NT, typename OutT>
 __device__ __forceinline__ void gemm_epilogue16_plain(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
@@ -105,9 +132,9 @@ __device__ __forceinline__ void gemm_epilogue16_plain(f32x4 (&acc)[MT][NT], cons
 }
 
 // The tiles `tile`, `tile + tile_step`, ... (< M/256 * N/256) of one problem, computed by the calling workgroup
-// with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  PLAIN: C has
-// the type of the operands, no scales, no activation.
-template <typename V8, bool B_KMAJOR, bool XCD, bool PLAIN = false>
+// with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  EPI: 0 = scales,
+// activation, any output type; 1 = C has the type of the operands, no scales, no activation; 2 = 0 plus the addend.
+template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0>
 __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -311,8 +338,8 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     // registers throughout the K loop)
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
-    if constexpr (PLAIN) gemm_epilogue16_plain<MT, NT, std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>>(acc, p, em, en, el, ek);
-    else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>>(acc, p, em, en, el, ek);
+    else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
     tile += tile_step;
     if (tile >= ntiles) break;
     tile_at(tile, pm, pn);
@@ -324,11 +351,11 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 
 // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid is either one workgroup per tile or, when
 // that divides evenly, one per CU).
-template <typename V8, bool B_KMAJOR>
+template <typename V8, bool B_KMAJOR, bool AUX>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-  gemm_wave128_tiles<V8, B_KMAJOR, true>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
+  gemm_wave128_tiles<V8, B_KMAJOR, true, AUX ? 2 : 0>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
 #endif
 }
 
@@ -359,7 +386,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_grouped_kernel(GroupedArg
       p.out_dtype = ga.out_dtype; p.group_m = 8;
       p.c_vec_ok = (ldc % 4 == 0) && (((uintptr_t)p.C) % 16 == 0);
       while (tile_idx < first + num_tiles) {
-        gemm_wave128_tiles<V8, false, false, true>(p, tile_idx - first, num_tiles, lds0);
+        gemm_wave128_tiles<V8, false, false, 1>(p, tile_idx - first, num_tiles, lds0);
         block_barrier();   // the next tile's loads overwrite the stages: every wave must be done reading them
         tile_idx += nprog;
       }
@@ -389,7 +416,7 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 #endif
 }
 
-template <int FMT>
+template <int FMT, bool AUX>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -524,7 +551,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
-    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    gemm_epilogue16<MT, NT, AUX>(acc, p, em, en, el, ek);
     tile += gridDim.x;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
@@ -751,23 +778,24 @@ int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-template <int FMT>
+template <int FMT, bool AUX>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, AUX>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
-  gemm_wave128_f8_kernel<FMT><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_f8_kernel<FMT, AUX><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
-  return e5m2 ? launch_wave128_f8<1>(p, stream) : launch_wave128_f8<0>(p, stream);
+  if (p.aux) return e5m2 ? launch_wave128_f8<1, true>(p, stream) : launch_wave128_f8<0, true>(p, stream);
+  return e5m2 ? launch_wave128_f8<1, false>(p, stream) : launch_wave128_f8<0, false>(p, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -1014,12 +1042,12 @@ bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
   return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
-template <typename V8, bool B_KMAJOR>
+template <typename V8, bool B_KMAJOR, bool AUX>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, AUX>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
@@ -1027,7 +1055,7 @@ static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   // one program per CU when that deals the tiles evenly, else one workgroup per tile (the hardware's
   // dynamic dispatch then balances the ragged last round)
   const int grid = (p.num_programs > 0 && tiles > p.num_programs && tiles % p.num_programs == 0) ? p.num_programs : tiles;
-  gemm_wave128_kernel<V8, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_kernel<V8, B_KMAJOR, AUX><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -1049,8 +1077,12 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 }
 
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream) {
-  if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true>(p, stream) : launch_wave128<f16x8, true>(p, stream);
-  return bf16 ? launch_wave128<bf16x8, false>(p, stream) : launch_wave128<f16x8, false>(p, stream);
+  if (p.aux) {
+    if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, true>(p, stream) : launch_wave128<f16x8, true, true>(p, stream);
+    return bf16 ? launch_wave128<bf16x8, false, true>(p, stream) : launch_wave128<f16x8, false, true>(p, stream);
+  }
+  if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, false>(p, stream) : launch_wave128<f16x8, true, false>(p, stream);
+  return bf16 ? launch_wave128<bf16x8, false, false>(p, stream) : launch_wave128<f16x8, false, false>(p, stream);
 }
 
 }  // namespace mi355
