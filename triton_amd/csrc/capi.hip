@@ -143,7 +143,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // B, +14 % with a K-major B; at 3072^3, 144 tiles, 790 vs 660 TFLOP/s for the 128x128 tiles)
   // (fp8, K-major B: 16x16x128 MFMAs, 8192^3 e4m3 2790-2810 vs 2570-2600 TFLOP/s)
   // (an epilogue addend: instantiations of their own)
-  if (tiles256 * 2 >= cus && gemm_wave128_ok(p, b_kmajor)) tile = 6;
+  // (fp8 from three quarters of a round: at 144 tiles the eight-wave kernel is 4-7 % ahead - 3072^3 1520 vs
+  // 1450, 3072x3072x8192 2040 vs 1890 TFLOP/s -, at 196 tiles the four-wave one by 2 %, at 225 by 13 %)
+  if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && gemm_wave128_ok(p, b_kmajor)) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
   p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
