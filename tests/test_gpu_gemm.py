@@ -401,6 +401,31 @@ def test_fused_addends_in_the_four_wave_kernel(gpu, dtype, monkeypatch):
         assert np.allclose(got, ref, rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("programs", [2, 3, 4])
+def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, programs):
+    # five tiles (1280 x 256) on at most 2 / 3 / 4 programs: 3 rounds on 2 programs (2 + 2 + 1 tiles), 2 rounds
+    # on 3 (2 + 2 + 1) - with 4 CUs also 2 rounds, so again 3 programs; a program with fewer tiles than the others
+    # wraps its loads earlier.  bf16 with both B layouts and fp8, sums of small integers: bit-exact.
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(programs))
+    rng = np.random.default_rng(90 + programs)
+    M, N = 1280, 256
+    for K in (128, 384):
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ref = a @ b
+        ta = from_np(a, "bf16", gpu)
+        for tb in (from_np(b, "bf16", gpu), from_np(np.ascontiguousarray(b.T), "bf16", gpu).t()):
+            assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), ref), (K, programs)
+    K = 512
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    ca, cb = formats.encode_fp8(a, "e4m3"), formats.encode_fp8(np.ascontiguousarray(b.T), "e4m3")
+    t8a = torch.from_numpy(ca).to(gpu).view(torch.float8_e4m3fn)
+    t8b = torch.from_numpy(cb).to(gpu).view(torch.float8_e4m3fn).t()
+    assert bits_equal(to_np(triton_amd.matmul(t8a, t8b, out_dtype=torch.float32)), a @ b), programs
+
+
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
 def test_fused_addends_in_the_four_wave_fp8_kernel(gpu, monkeypatch, fmt, tdt):
     # the same addend forms in the fp8 kernel of 16x16x128 MFMAs: codes of small integers (exact products

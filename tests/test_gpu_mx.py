@@ -131,3 +131,24 @@ def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile
             sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
         ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
         assert bits_equal(_run(gpu, a, sa, b, sb, fmt, torch.float32), ref32), (fmt, tile, M, N, K)
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
+@pytest.mark.parametrize("programs", [2, 3])
+def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, fmt, programs):
+    # five tiles on at most 2 / 3 programs of the scaled 16x16x128 kernels (2 + 2 + 1 tiles either way, in three or
+    # two rounds); K of one and of two groups of four K steps (the scale ring's parity at the tile switch)
+    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(programs))
+    rng = np.random.default_rng(60 + programs)
+    for (M, N, K) in [(1280, 256, 1024), (256, 1280, 2048)]:
+        if fmt == "mxfp4":
+            a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
+        else:
+            vals = np.array([0x00, 0x30, 0x38, 0x3C, 0x40, 0xB0, 0xB8, 0xC0], dtype=np.uint8)  # 0, .5, 1, 1.5, 2, -.5, -1, -2
+            a = vals[rng.integers(0, len(vals), size=(M, K))]
+            b = vals[rng.integers(0, len(vals), size=(N, K))]
+            sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+            sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
+        assert bits_equal(_run(gpu, a, sa, b, sb, fmt, torch.float32), ref32), (fmt, programs, M, N, K)
