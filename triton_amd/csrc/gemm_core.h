@@ -528,7 +528,7 @@ static int launch_gemm_grouped_one(const GroupedArgs& ga, int nprog, hipStream_t
 // nprog: programs of the 128x128 form; nprog_big: programs of the 256x256 form (one per CU)
 template <typename Cfg, typename T>
 static int launch_gemm_grouped(const GroupedArgs& ga, int nprog, int nprog_big, hipStream_t stream) {
-  int rc = gemm_wave128_grouped_launch(ga, std::is_same<T, __bf16>::value, nprog_big, stream);
+  int rc = ga.wave128_min_k > 0 ? gemm_wave128_grouped_launch(ga, std::is_same<T, __bf16>::value, nprog_big, stream) : 0;
   if (rc) return rc;
   rc = launch_gemm_grouped_one<Cfg, T, 256, 256, 2, 4>(ga, nprog_big, stream);
   if (rc) return rc;
