@@ -181,7 +181,7 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C,
  * full tiles); problems whose lda, ldb, N or K are not multiples of 8 elements, or whose A / B
  * are not 16-byte aligned, run a slower loop inside the same kernel.  Groups in which every problem
  * is whole 256x256 tiles with K a multiple of 128 (and ldb a multiple of 256 elements) run a faster
- * kernel from one tile per compute unit and K >= 1024 on.  Nothing about the device
+ * kernel from one tile per compute unit and K >= 512 on.  Nothing about the device
  * arrays can be checked on the host: they must hold `group_size` valid entries.
  */
 int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,

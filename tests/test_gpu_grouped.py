@@ -64,13 +64,17 @@ def test_strided_rows_and_empty_group(gpu):
         triton_amd.group_gemm_fn([a], [b, b])
 
 
+@pytest.mark.parametrize("chunk", [4, 1, 3])
 @pytest.mark.parametrize("nprog", [0, 7, 100])
-def test_groups_of_whole_256_tiles(gpu, nprog, monkeypatch):
+def test_groups_of_whole_256_tiles(gpu, nprog, chunk, monkeypatch):
     # every problem whole 256x256 tiles and K % 128 == 0: the four-wave 16x16-MFMA kernel takes the group
     # (thresholds lowered so that 20 tiles and K = 128 are enough); exact sums of small integers, rounded
     # once; K from one pair of stages up to several, M != N, problems of one tile between larger ones
     monkeypatch.setenv("MI355_GROUPED_BIG_MIN", "1")
     monkeypatch.setenv("MI355_GROUPED_WAVE128_MIN_K", "128")
+    # a program's tiles: chunks of up to 4 / 1 / 3 consecutive tiles (7 programs, 20 tiles: chunks of 3, runs that
+    # cross from one problem into the next and runs of several tiles inside one problem)
+    monkeypatch.setenv("MI355_GROUPED_CHUNK", str(chunk))
     rng = np.random.default_rng(40 + nprog)
     shapes = [(256, 256, 128), (512, 256, 256), (256, 256, 1024), (256, 768, 384), (1024, 512, 128), (256, 256, 256), (512, 512, 640)]
     ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]

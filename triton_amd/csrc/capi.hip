@@ -237,7 +237,9 @@ int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d
   const int nprog_big = nprog < cus ? nprog : cus;
   ga.big_tiles_min = env_int("MI355_GROUPED_BIG_MIN", cus);
   // smallest K of a group of whole 256x256 tiles that the four-wave 16x16-MFMA kernel takes (0 = never)
-  ga.wave128_min_k = env_int("MI355_GROUPED_WAVE128_MIN_K", 1024);
+  ga.wave128_min_k = env_int("MI355_GROUPED_WAVE128_MIN_K", 512);
+  ga.chunk = env_int("MI355_GROUPED_CHUNK", 4);
+  if (ga.chunk < 1) ga.chunk = 1;
   return gemm16_grouped_launch(ga, dtype == MI355_BF16, nprog, nprog_big, (hipStream_t)stream_);
 }
 

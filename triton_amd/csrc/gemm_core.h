@@ -436,13 +436,12 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
 // Which grouped kernel computes this group: 2 = the four-wave 16x16-MFMA kernel (every problem whole
 // 256x256 tiles, K a multiple of 128 and at least `wave128_min_k`, 16-byte rows of A, 512-byte multiples
 // as pitch of B, 32-bit lane offsets, and at least `big_tiles_min` tiles), 1 = 256x256 tiles,
-// 0 = 128x128 tiles.  (That kernel restarts its two-stage pipeline at every tile and fetches two K steps
-// too many per tile; measured against the other two on fp16 groups of 256 to 1024 tiles it gains 10-25 %
-// on problems of 2048^2 and 4096^2 with K from 1024 to 4096, is even at K = 512 and loses 10 % on 64
-// problems of 1024^3.)
+// 0 = 128x128 tiles.  (That kernel restarts its two-stage pipeline at every run of tiles and fetches two K steps
+// too many per run; measured against the other two on fp16 groups of 256 to 2048 tiles of 1024^2 to 4096^2
+// problems it gains 5-25 % with K from 512 to 4096.)
 // Every wave reads the tables with one problem per lane (all loads in flight at once: a serial scan of 16
 // problems took 4-8 us in each of the three launches) and combines the lanes' findings.
-__device__ __forceinline__ int grouped_plan(const GroupedArgs& ga) {
+__device__ __forceinline__ int grouped_plan(const GroupedArgs& ga, long long* total_tiles = nullptr) {
   long long big_tiles = 0;
   bool whole = true;
   for (int gi = threadIdx.x & 63; gi < ga.group_size; gi += 64) {
@@ -455,6 +454,7 @@ __device__ __forceinline__ int grouped_plan(const GroupedArgs& ga) {
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) big_tiles += __shfl_xor(big_tiles, off);
+  if (total_tiles) *total_tiles = __builtin_amdgcn_readfirstlane((int)big_tiles);   // (256x256 tiles of all problems)
   const bool all_whole = ga.wave128_min_k > 0 && __all(whole);
   const int plan = (all_whole && big_tiles >= ga.big_tiles_min) ? 2 : (big_tiles >= ga.big_tiles_min ? 1 : 0);
   return __builtin_amdgcn_readfirstlane(plan);

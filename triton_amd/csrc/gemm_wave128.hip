@@ -41,6 +41,26 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 
 // Epilogue for 16x16 tiles computed with the operands swapped (D[n][m]): lane l owns C row
 // `mrow0 + 16 i + l%16` and, of tile (i, j), the four consecutive columns `ncol0 + 16 j + 4 (l/16) ..`.
+// The MFMAs of these kernels are inline assembly, so the compiler neither knows that they are MFMAs nor waits
+// for the last ones before it reads their results.  Waiting alone is not enough: nothing ties a plain
+// `s_nop` statement to the accumulators, and the compiler has moved accumulator reads (spills and moves of the
+// epilogue's register shuffle) in front of it, where they see registers that the last MFMAs have yet to write.
+// So every accumulator passes through an (empty) assembly statement behind the wait: volatile statements keep
+// their order, and a value read after its statement is read after the wait.
+__device__ __forceinline__ void mfma_drain_row(f32x4 (&r)[8]) {
+#if MI355_DEVICE_PASS
+  asm volatile("" : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]), "+a"(r[7]));
+#endif
+}
+template <int MT>
+__device__ __forceinline__ void mfma_drain(f32x4 (&acc)[MT][8]) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+#endif
+#pragma unroll
+  for (int i = 0; i < MT; i++) mfma_drain_row(acc[i]);
+}
+
 // Workgroups for `tiles` tiles on at most `cap` CUs.  More tiles than CUs need r = ceil(tiles / cap) rounds
 // however they are dealt: ceil(tiles / r) programs walk r tiles each (the last ones r - 1) as one stream of K
 // steps, without the restart that a fresh workgroup per tile pays, and the CUs left without a program leave
@@ -145,11 +165,11 @@ __device__ __forceinline__ void gemm_epilogue16_plain(f32x4 (&acc)[MT][NT], cons
   });
 }
 
-// The tiles `tile`, `tile + tile_step`, ... (< M/256 * N/256) of one problem, computed by the calling workgroup
+// The tiles `tile`, `tile + tile_step`, ... (< `tile_stop`, by default M/256 * N/256) of one problem, computed by the calling workgroup
 // with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  EPI: 0 = scales,
 // activation, any output type; 1 = C has the type of the operands, no scales, no activation; 2 = 0 plus the addend.
 template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0>
-__device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0) {
+__device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0, const int tile_stop = -1) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
@@ -163,6 +183,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 
   const int num_m = p.M / BM, num_n = p.N / BN;
   const int ntiles = num_m * num_n;
+  const int tend = tile_stop < 0 ? ntiles : tile_stop;   // the walk ends before this tile
   // The tiles are computed as ONE stream of K steps: the loads of the last two steps of a tile already
   // fetch the first two K steps of the next one, so its first fragments are in registers when the finished
   // tile is stored.
@@ -327,7 +348,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   auto advance = [&]() {
     if (++fk == nk) {
       fk = 0;
-      if (ftile + tile_step < ntiles) {
+      if (ftile + tile_step < tend) {
         ftile += tile_step;
         int fm, fn;
         tile_at(ftile, fm, fn);
@@ -346,7 +367,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     // above are MFMAs: let the last ones retire before their results are read.
     lds_wait<0>();
     pin(f[0]);
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    mfma_drain(acc);
     // (the tile and lane coordinates pass through an empty assembly statement so that none of the
     // epilogue's address arithmetic is hoisted out of the tile loop, where it would occupy - and spill -
     // registers throughout the K loop)
@@ -355,7 +376,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
     tile += tile_step;
-    if (tile >= ntiles) break;
+    if (tile >= tend) break;
     tile_at(tile, pm, pn);
     zero_acc();
   }
@@ -383,14 +404,27 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_grouped_kernel(GroupedArg
 #if MI355_DEVICE_PASS
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
-  if (grouped_plan(ga) != 2) return;
+  long long total = 0;
+  if (grouped_plan(ga, &total) != 2) return;
+  // The tiles of all problems, numbered problem after problem, are dealt in chunks of c consecutive tiles:
+  // program w (renumbered so that the programs of one XCD are neighbours) takes the chunks w, w + nprog, ...
+  // The part of a chunk inside one problem is one stream of K steps (tile after tile down a column of C
+  // tiles: the B panel is fetched once); the stream restarts at the next chunk and where a chunk crosses into
+  // the next problem.  c = tiles per program, at most `chunk` (4): longer runs save more restarts, but all
+  // programs together then work on nprog * c tiles at a time, and with 256 programs on 2048^3 problems eight
+  // tiles each already spread over 32 problems, more operands than the last-level cache holds (-8 % there,
+  // against +8 to +17 % for four tiles each on 16 such problems).
   const int nprog = gridDim.x;
-  int tile_idx = xcd_remap(blockIdx.x, nprog);
+  const int w = xcd_remap(blockIdx.x, nprog);
+  const int tot = (int)total;
+  const int c = max(1, min(ga.chunk, (tot + nprog - 1) / nprog));
+  int chunk = w;
+  int cur = chunk * c, limit = min(cur + c, tot);
   int first = 0;   // number of the first tile of problem gi
-  for (int gi = 0; gi < ga.group_size; gi++) {
+  for (int gi = 0; gi < ga.group_size && cur < tot; gi++) {
     const int gm = ga.sizes[gi * 3], gn = ga.sizes[gi * 3 + 1], gk = ga.sizes[gi * 3 + 2];
     const int num_tiles = (gm / 256) * (gn / 256);
-    if (tile_idx < first + num_tiles) {
+    if (cur < first + num_tiles) {
       const int ldc = ga.lds[gi * 3 + 2];
       GemmArgs p{};
       p.A = (const char*)ga.a_ptrs[gi]; p.B = (const char*)ga.b_ptrs[gi]; p.C = (char*)ga.c_ptrs[gi];
@@ -398,10 +432,16 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_grouped_kernel(GroupedArg
       p.lda = (int64_t)ga.lds[gi * 3] * 2; p.ldb = (int64_t)ga.lds[gi * 3 + 1] * 2; p.ldc = ldc; p.scn = 1;
       p.out_dtype = ga.out_dtype; p.group_m = 8;
       p.c_vec_ok = (ldc % 4 == 0) && (((uintptr_t)p.C) % 16 == 0);
-      while (tile_idx < first + num_tiles) {
-        gemm_wave128_tiles<V8, false, false, 1>(p, tile_idx - first, num_tiles, lds0);
-        block_barrier();   // the next tile's loads overwrite the stages: every wave must be done reading them
-        tile_idx += nprog;
+      while (cur < tot && cur < first + num_tiles) {
+        const int stop = min(limit, first + num_tiles) - first;
+        gemm_wave128_tiles<V8, false, false, 1>(p, cur - first, 1, lds0, stop);
+        block_barrier();   // the next run's loads overwrite the stages: every wave must be done reading them
+        cur = first + stop;
+        if (cur == limit) {
+          chunk += nprog;
+          cur = chunk * c;
+          limit = min(cur + c, tot);
+        }
       }
     }
     first += num_tiles;
@@ -561,7 +601,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       step(I0{}, I0{}, fk); advance();
       step(I1{}, I1{}, fk); advance();
     }
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT, AUX>(acc, p, em, en, el, ek);
@@ -755,8 +795,12 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   while (true) {
     for (int kt = 0; kt < nk; kt += 8) {
       static_for<8>([&](auto U_) { step(U_, fk); advance(); });
+      // The last MFMAs must have retired before control leaves this loop: behind it the compiler moves every
+      // accumulator (its register shuffle for the epilogue) and, not knowing that the assembly above are
+      // MFMAs, does so without waiting; a wait placed behind the loop can end up behind those moves.
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     }
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
@@ -1010,8 +1054,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       step(I1{}, fk); advance();
       step(I2{}, fk); advance();
       step(I3{}, fk); advance();
+      // (the last MFMAs retire inside the loop: see the MXFP8 kernel)
+      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
     }
-    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+    mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);

@@ -80,6 +80,7 @@ struct GroupedArgs {
   int group_size;
   int out_dtype;           // element type of A, B and C: 0 = fp16, 1 = bf16
   int big_tiles_min;       // 256x256 tiles in the group from which the large-tile kernel takes the launch
+  int chunk;               // four-wave kernel: most consecutive tiles that a program takes as one run (1 = every nprog-th tile)
   int wave128_min_k;       // groups of whole 256x256 tiles with every K >= this go to the four-wave 16x16-MFMA kernel (0 = never)
 };
 
