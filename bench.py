@@ -23,10 +23,14 @@ if ROOT not in sys.path:
 PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4": 10100.0}
 HBM_GBPS = 8000.0
 
-# HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel measured with rocprofv3 --pmc:
-# FETCH_SIZE 820374 KiB x 2.000 + WRITE_SIZE 143130 KiB x 1.000, the factors being what the same
-# counters read for a plain copy of known size (profiles/gemm_bf16_8192.md)
-MEASURED_TRAFFIC_BYTES = int((820374 * 2.000 + 143130 * 1.000) * 1024)
+# HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel.  NOT read in this run (hardware counters need
+# rocprofv3 around the process): taken from the two rocprofv3 --pmc runs of this same command that
+# profiles/gemm_bf16_8192.md records - FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what
+# the same counter reads for a plain device copy of known size (--copy-calibration).
+MEASURED_TRAFFIC_KIB = {"FETCH_SIZE": 820374, "FETCH_scale": 2.000, "WRITE_SIZE": 143130, "WRITE_scale": 1.000}
+MEASURED_TRAFFIC_BYTES = int((MEASURED_TRAFFIC_KIB["FETCH_SIZE"] * MEASURED_TRAFFIC_KIB["FETCH_scale"]
+                              + MEASURED_TRAFFIC_KIB["WRITE_SIZE"] * MEASURED_TRAFFIC_KIB["WRITE_scale"]) * 1024)
+TRAFFIC_SOURCE = "profiles/gemm_bf16_8192.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs of this command; not measured in this run)"
 
 
 def time_launches(fn, steps, warmup):
@@ -56,13 +60,89 @@ def quick(fn, iters=60, warmup=20):
     return ev_ms
 
 
+def observed_clock_mhz(lib, fn, rounds=12, launches_per_round=4, window_us=15):
+    """Shader clock while `fn` runs back to back (an untimed leg of its own).  After every few launches a
+    one-wave probe kernel on the SAME stream reads the shader-clock counter and the constant-rate real-time
+    counter over `window_us`: the board's power management moves the clock on a millisecond scale, so
+    the clock in the microseconds behind a kernel is the clock that kernel ran at.  (A probe that lives next
+    to the kernels on a second stream would hold one SIMD slot and cost a one-workgroup-per-CU kernel a
+    whole round of tiles - and so raise the very clock it reads.)"""
+    import torch
+
+    from triton_amd import _lib
+
+    wall_khz = lib.mi355_query(_lib.Q_WALL_CLOCK_KHZ)
+    if wall_khz <= 0:
+        return None
+    ticks = torch.zeros(rounds, 2, dtype=torch.int64, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    for _ in range(3 * launches_per_round):
+        fn()
+    for r in range(rounds):
+        for _ in range(launches_per_round):
+            fn()
+        rc = lib.mi355_clock_probe(ticks[r].data_ptr(), window_us, stream)
+        assert rc == 0, rc
+    torch.cuda.synchronize()
+    t = ticks.cpu()
+    c, r = int(t[:, 0].sum()), int(t[:, 1].sum())
+    return round(c / r * wall_khz / 1e3, 1) if r > 0 else None
+
+
+def _median_of_3(fn):
+    """1 warm + median of 3 passes, seconds."""
+    fn()
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[1]
+
+
+def cpu_baselines_other(threads):
+    """The other CPU legs: config 1 in full under the interpreter's execution model, the attention
+    oracle on a (Z, H) = (1, 1) slice of config 3 (flagged: a slice, not the whole job), and plain
+    multithreaded fp32 torch.matmul on the host as the best-CPU line."""
+    import numpy as np
+    import torch
+
+    from oracle import attention as OA
+    from oracle import formats, gemm
+
+    out = {}
+    rng = np.random.default_rng(0)
+    a = formats.round_fp16(rng.standard_normal((512, 512)).astype(np.float32))
+    b = formats.round_fp16(rng.standard_normal((512, 512)).astype(np.float32))
+    dt = _median_of_3(lambda: gemm.matmul_tiled(a, b, 64, 64, 32, 8, out_dtype="fp16"))
+    out["config1_fp16_512_tiles_64x64x32"] = {
+        "value": round(2.0 * 512 ** 3 / dt / 1e12, 6), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": f"oracle.gemm.matmul_tiled 512^3 fp16 in full (64 programs x 16 K steps, serial grid loop), 1 warm + median of 3, {dt * 1e3:.1f} ms"}
+    Z, H, N, D = 1, 1, 4096, 128
+    q, k, v = (formats.round_bf16(rng.normal(0, 0.5, (Z, H, N, D)).astype(np.float32)) for _ in range(3))
+    for causal in (True, False):
+        dt = _median_of_3(lambda: OA.attn_fwd_tiled(q, k, v, causal, D ** -0.5, "bf16"))
+        fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
+        out[f"attn_fwd_{'causal' if causal else 'noncausal'}"] = {
+            "value": round(fl / dt / 1e12, 5), "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"oracle.attention.attn_fwd_tiled bf16 on the (Z, H) = (1, 1) slice of config 3 (N=4096, D=128; 1/128 of the job, flagged: slice), "
+                      f"1 warm + median of 3, {dt:.2f} s"}
+    n = 4096
+    ta, tb = torch.randn(n, n), torch.randn(n, n)
+    dt = _median_of_3(lambda: torch.matmul(ta, tb))
+    out["torch_matmul_fp32_best_cpu"] = {
+        "value": round(2.0 * n ** 3 / dt / 1e12, 4), "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "library",
+        "sample": f"torch.matmul fp32 {n}^3 on the host (not the reference's path: the best-CPU line), 1 warm + median of 3, {dt:.2f} s"}
+    return out
+
+
 def cpu_baseline_gemm(budget_s=20.0):
     """The CPU oracle (a port of the reference's interpreter execution model: serial grid loop,
     one fp32 np.matmul per K chunk, python/triton/runtime/interpreter.py:1088-1092, :542-549) on a
     bounded sample of the GEMM workload: same tile program, size reduced until it fits the budget."""
     import numpy as np
 
-    from oracle import gemm
+    from oracle import formats, gemm
 
     try:
         from threadpoolctl import threadpool_info
@@ -70,24 +150,29 @@ def cpu_baseline_gemm(budget_s=20.0):
     except Exception:
         threads = os.cpu_count() or 1
     rng = np.random.default_rng(0)
+    # size: the largest power of two whose four passes (1 warm + 3 timed) fit the budget, found by doubling
     n = 1024
-    best = None
     while True:
-        a = rng.standard_normal((n, n)).astype(np.float32)
-        b = rng.standard_normal((n, n)).astype(np.float32)
+        a = formats.round_bf16(rng.standard_normal((n, n)).astype(np.float32))
+        b = formats.round_bf16(rng.standard_normal((n, n)).astype(np.float32))
         t0 = time.perf_counter()
-        gemm.matmul_tiled(a, b, 128, 256, 64, 8, out_dtype="fp32")
+        gemm.matmul_tiled(a, b, 128, 256, 64, 8, out_dtype="bf16")
         dt = time.perf_counter() - t0
-        best = (n, dt)
-        if dt * 8 > budget_s or n >= 8192:
+        if dt * 8 * 4 > budget_s or n >= 8192:
             break
         n *= 2
-    n, dt = best
-    return {
+    dt = _median_of_3(lambda: gemm.matmul_tiled(a, b, 128, 256, 64, 8, out_dtype="bf16"))
+    base = {
         "value": round(2.0 * n ** 3 / dt / 1e12, 5), "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
-        "sample": f"oracle.gemm.matmul_tiled {n}^3 (tiles 128x256x64, GROUP_M 8, fp32 accumulate), one pass, {dt:.2f} s; "
-                  f"host has {os.cpu_count()} logical cpus",
+        "sample": f"oracle.gemm.matmul_tiled {n}^3 bf16 values (tiles 128x256x64, GROUP_M 8, fp32 accumulate, bf16 out): the {n}^3 "
+                  f"sub-problem of the 8192^3 workload (1/{(8192 // n) ** 3} of its flop; throughput, not extrapolated time), "
+                  f"1 warm + median of 3, {dt:.2f} s per pass; BLAS threads {threads}, host has {os.cpu_count()} logical cpus",
     }
+    try:
+        base["other_legs"] = cpu_baselines_other(int(threads))
+    except Exception as e:   # a baseline leg must never take the GPU numbers down with it
+        base["other_legs"] = {"error": repr(e)}
+    return base
 
 
 def main():
@@ -145,8 +230,10 @@ def main():
                      "launch_ms_min": round(min(per), 5), "algorithmic_flops": flops,
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
-                   "clock_khz": lib.mi355_query(_lib.Q_CLOCK_KHZ)},
+                   "nominal_clock_khz": lib.mi355_query(_lib.Q_CLOCK_KHZ),
+                   "observed_sclk_mhz_during_headline_gemm": observed_clock_mhz(lib, step)},
     }
+    out["roofline"]["traffic_source"] = TRAFFIC_SOURCE
 
     if not args.no_extra:
         from triton_amd import testing
@@ -157,12 +244,19 @@ def main():
         extra["bf16_gemm_do_bench"] = {"ms_median": round(med, 4), "ms_p20": round(p20, 4), "ms_p80": round(p80, 4),
                                        "tflops_median": round(testing.matmul_tflops(n, n, n, med), 1)}
         # fp8 e4m3 GEMM, K-major B, per-tensor scales, bf16 out (config 4) and its decode shape
-        a8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
-        b8 = torch.randn(n, n, device=dev).to(torch.float8_e4m3fn)
-        sc = torch.tensor([0.01], device=dev)
-        ms = quick(lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sc, b_scale=sc))
-        extra["fp8_e4m3_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK["fp8"], 4)}
-        a16 = torch.randn(16, n, device=dev).to(torch.float8_e4m3fn)
+        # operands as config 4 states them: N(0, 1) scaled to a per-tensor amax of 448, clamped, cast; the scales
+        # that undo it go to the epilogue
+        def quantize_e4m3(x):
+            scale = (x.abs().amax() / 448.0).float().reshape(1)
+            return (x / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn), scale
+
+        a8, sa8 = quantize_e4m3(torch.randn(n, n, device=dev))
+        b8, sb8 = quantize_e4m3(torch.randn(n, n, device=dev))
+        fp8_fn = lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sa8, b_scale=sb8)
+        ms = quick(fp8_fn)
+        extra["fp8_e4m3_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK["fp8"], 4),
+                                       "sclk_mhz": observed_clock_mhz(lib, fp8_fn), "data": "N(0,1) scaled to amax 448, e4m3fn, per-tensor fp32 scales"}
+        a16, _ = quantize_e4m3(torch.randn(16, n, device=dev))
         c16 = torch.empty(16, n, device=dev, dtype=torch.bfloat16)
 
         def decode():  # straight through the C ABI: at ~20 us per launch the Python wrapper would dominate
@@ -212,12 +306,22 @@ def main():
         del ga, gb
         # MX GEMMs (config 5)
         for fmt, kb in (("mxfp4", n // 2), ("mxfp8", n)):
-            pa = torch.randint(0, 120, (n, kb), device=dev, dtype=torch.uint8)
-            pb = torch.randint(0, 120, (n, kb), device=dev, dtype=torch.uint8)
+            # config 5: fp4 codes uniform over all 16 values (every byte value), e4m3 codes uniform over the 254
+            # finite ones (0x7F / 0xFF are NaN), scales uniform over 2^-4 .. 2^4
+            def codes():
+                if fmt == "mxfp4":
+                    return torch.randint(0, 256, (n, kb), device=dev, dtype=torch.uint8)
+                r = torch.randint(0, 254, (n, kb), device=dev, dtype=torch.uint8)
+                return r + (r >= 127).to(torch.uint8)      # 0..126 -> 0x00..0x7E, 127..253 -> 0x80..0xFE
+
+            pa, pb = codes(), codes()
             sa = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
             sb = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
-            ms = quick(lambda: triton_amd.mx_matmul(pa, sa, pb, sb, fmt))
-            extra[f"{fmt}_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK[fmt], 4)}
+            mx_fn = lambda: triton_amd.mx_matmul(pa, sa, pb, sb, fmt)
+            ms = quick(mx_fn)
+            extra[f"{fmt}_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK[fmt], 4),
+                                         "sclk_mhz": observed_clock_mhz(lib, mx_fn),
+                                         "data": "codes uniform over all finite values, e8m0 scales uniform over 2^-4 .. 2^4"}
         del b8
         # flash attention (config 3), flops by the reference formula (06:630-636)
         Z, H, N, D = 4, 32, 4096, 128
@@ -227,9 +331,12 @@ def main():
         sm = D ** -0.5
         for causal in (True, False):
             fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
-            ms = quick(lambda: triton_amd.attention(q, k, v, causal, sm))
+            qd, kd, vd = q.detach(), k.detach(), v.detach()
+            fwd_fn = lambda: triton_amd.attention(qd, kd, vd, causal, sm)
+            ms = quick(fwd_fn)
             tag = "causal" if causal else "noncausal"
-            extra[f"attn_fwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["bf16"], 4)}
+            extra[f"attn_fwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["bf16"], 4),
+                                        "sclk_mhz": observed_clock_mhz(lib, fwd_fn)}
             o = triton_amd.attention(q, k, v, causal, sm)
             do = torch.randn_like(o)
             # gradients returned, not accumulated into .grad (that would add three elementwise kernels)

@@ -68,7 +68,8 @@ enum {
   MI355_Q_IS_GFX950 = 2,
   MI355_Q_LDS_BYTES = 3,
   MI355_Q_CLOCK_KHZ = 4,
-  MI355_Q_STREAMK_WORKSPACE_BYTES = 5 /* workspace mi355_gemm_streamk needs on this device */
+  MI355_Q_STREAMK_WORKSPACE_BYTES = 5, /* workspace mi355_gemm_streamk needs on this device */
+  MI355_Q_WALL_CLOCK_KHZ = 6           /* rate of the constant real-time counter (mi355_clock_probe) */
 };
 
 /*
@@ -255,9 +256,26 @@ int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
  */
 int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* stream);
 
+/*
+ * Shader clock under load: a one-wave kernel that lives for `duration_us` (at most 2 s) of real time on
+ * `stream` and then writes ticks[0] = shader-clock cycles and ticks[1] = real-time counter ticks that
+ * passed (device memory, two uint64, 8-byte aligned).  Launched on a second stream next to the kernels
+ * under study, clock = ticks[0] / ticks[1] * mi355_query(MI355_Q_WALL_CLOCK_KHZ) is the clock they ran at:
+ * the board lowers the clock of MFMA-heavy kernels to hold its power limit, so peak fractions computed
+ * from the nominal clock (as python/triton/testing.py:404-426 `get_max_tensorcore_tflops` does from a
+ * clock argument) need the observed one.  Asynchronous like every other entry.
+ */
+int mi355_clock_probe(uint64_t* ticks, int duration_us, void* stream);
+
 /* Device facts needed by callers (analogue of get_device_properties,
  * third_party/amd/backend/driver.c:125-141).  Returns -1 for an unknown selector. */
 int mi355_query(int what);
+
+/* The library reads its MI355_* tuning variables from the environment once, at the first call that
+ * needs one (the reference reads its own per call or per import: python/triton/runtime/jit.py:717,
+ * :848, python/triton/runtime/autotuner.py:166); this reads them again, for a caller that changed
+ * them afterwards.  Not to be called while another thread is inside the library. */
+void mi355_refresh_env(void);
 
 /* Static string for a return code of the functions above (never NULL). */
 const char* mi355_strerror(int code);

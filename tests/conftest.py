@@ -25,3 +25,14 @@ def gpu():
     _lib.load()  # raises ImportError if the HIP library has not been built
     assert _lib.load().mi355_query(_lib.Q_IS_GFX950) == 1, "these kernels are gfx950-only"
     return torch.device("cuda", 0)
+
+
+@pytest.fixture(autouse=True)
+def _library_rereads_environment():
+    """Autouse fixtures are set up first and torn down last: after monkeypatch has restored the MI355_*
+    variables a test changed (util.set_knob), the library (if built and loaded) reads them again."""
+    yield
+    from triton_amd import _lib
+
+    if _lib._lib is not None:
+        _lib._lib.mi355_refresh_env()

@@ -7,7 +7,7 @@ import torch
 
 import triton_amd
 from oracle import attention as A
-from util import from_np, randn_rounded, to_np
+from util import from_np, randn_rounded, to_np, set_knob
 
 pytestmark = pytest.mark.gpu
 
@@ -39,6 +39,27 @@ def test_reference_test_op_configuration_fp16(gpu):
         assert np.allclose(got, cf[name], atol=1e-2, rtol=0), name
 
 
+def _max_err(got, ref):
+    """(max absolute error, max of |got - ref| / (atol + rtol |ref|) at rtol = atol = 1e-2)."""
+    d = np.abs(got - ref)
+    return float(d.max()), float((d / (1e-2 + 1e-2 * np.abs(ref))).max())
+
+
+def _check_against_tiled_and_closed_form(tag, got, tiled, cf, dtype):
+    """The stated bar - rtol = atol = 1e-2 for fp16 / bf16 outputs - is held against the restated tile
+    programs, which round P, dS and the pre-scaled K where the kernels' own type does (the causal
+    backward is the reference program verbatim, 06:308-435).  The fp64 closed form, which rounds
+    nowhere, is a second and for bf16 looser check (3e-2: three fewer mantissa bits through P, dS
+    and the outputs).  Both maxima are printed (pytest -s / on failure)."""
+    cf_tol = 1e-2 if dtype == "fp16" else 3e-2
+    for name in ("o", "dq", "dk", "dv"):
+        e_t, r_t = _max_err(got[name], tiled[name])
+        e_c, _ = _max_err(got[name], cf[name])
+        print(f"{tag} {dtype} {name}: max |err| vs tiled oracle {e_t:.3e} ({r_t:.2f} of the 1e-2 bound), vs fp64 closed form {e_c:.3e}")
+        assert np.allclose(got[name], tiled[name], atol=1e-2, rtol=1e-2), (name, "tiled oracle", e_t)
+        assert np.allclose(got[name], cf[name], atol=cf_tol, rtol=1e-2), (name, "closed form", e_c)
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("causal", [True, False])
 @pytest.mark.parametrize("shape", [(1, 2, 128, 64), (1, 2, 256, 128), (2, 3, 512, 128), (1, 1, 384, 128), (1, 1, 640, 64)])
@@ -47,12 +68,11 @@ def test_forward_backward_against_oracle(gpu, dtype, causal, shape):
     sm_scale = shape[-1] ** -0.5
     o, dq, dk, dv = _fwd_bwd(tq, tk, tv, tdo, causal, sm_scale)
     cf = A.attn_closed_form(q, k, v, causal, sm_scale, do)
-    tol = 1e-2 if dtype == "fp16" else 3e-2   # bf16 carries 3 fewer mantissa bits through P, dS and the outputs
-    for name, got in (("o", o), ("dq", dq), ("dk", dk), ("dv", dv)):
-        assert np.allclose(got, cf[name], atol=tol, rtol=1e-2), name
-    # and against the restated tile programs (non-causal backward is the build's extension there too)
+    # the restated tile programs in the kernels' own type (non-causal backward: the build's extension there too)
     ro, rM = A.attn_fwd_tiled(q, k, v, causal, sm_scale, dtype)
-    assert np.allclose(o, ro, atol=tol, rtol=1e-2)
+    rdq, rdk, rdv, _ = A.attn_bwd_tiled(q, k, v, ro, do, rM, sm_scale, causal, dtype)
+    _check_against_tiled_and_closed_form(f"{shape} causal={causal}", dict(o=o, dq=dq, dk=dk, dv=dv),
+                                         dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, dtype)
 
 
 @pytest.mark.parametrize("n_ctx", [512, 384])
@@ -66,8 +86,8 @@ def test_forward_variants_and_lse(gpu, causal, n_ctx, monkeypatch):
     # half of its second 256-row block empty), 3 and 4: 1 and 2 as persistent programs (two programs here, so
     # that each walks several items)
     for variant in ("0", "1", "2", "3", "4"):
-        monkeypatch.setenv("MI355_ATTN_FWD_VARIANT", variant)
-        monkeypatch.setenv("MI355_ATTN_PROGRAMS", "1")
+        set_knob(monkeypatch, "MI355_ATTN_FWD_VARIANT", variant)
+        set_knob(monkeypatch, "MI355_ATTN_PROGRAMS", "1")
         o = torch.empty_like(tq)
         M = torch.empty(2, 2, n_ctx, dtype=torch.float32, device=gpu)
         I4 = _lib.I64x4
@@ -109,7 +129,8 @@ def test_unsupported_configurations_raise(gpu):
 @pytest.mark.parametrize("causal", [True, False])
 def test_full_size_config3_sampled_heads(gpu, causal):
     # BASELINE config 3: Z=4, H=32, N=4096, D=128 bf16, sm_scale = 1/sqrt(128); two heads are checked
-    # in full against the fp64 closed form (forward, M and all three gradients)
+    # in full against the restated tile programs in bf16 at rtol = atol = 1e-2 and the fp64 closed form
+    # (forward and all three gradients)
     Z, H, N, D = 4, 32, 4096, 128
     g = torch.Generator(device="cpu").manual_seed(20)
     q, k, v = (torch.empty(Z, H, N, D).normal_(0, 0.5, generator=g).bfloat16() for _ in range(3))
@@ -121,9 +142,12 @@ def test_full_size_config3_sampled_heads(gpu, causal):
     for (z, h) in [(0, 0), (3, 17)]:
         sl = lambda x: x[z:z + 1, h:h + 1].float().numpy()
         cf = A.attn_closed_form(sl(q), sl(k), sl(v), causal, sm_scale, sl(do))
+        ro, rM = A.attn_fwd_tiled(sl(q), sl(k), sl(v), causal, sm_scale, "bf16")
+        rdq, rdk, rdv, _ = A.attn_bwd_tiled(sl(q), sl(k), sl(v), ro, sl(do), rM, sm_scale, causal, "bf16")
         gsl = lambda x: to_np(x[z:z + 1, h:h + 1])
-        for name, got in (("o", gsl(o)), ("dq", gsl(tq.grad)), ("dk", gsl(tk.grad)), ("dv", gsl(tv.grad))):
-            assert np.allclose(got, cf[name], atol=3e-2, rtol=1e-2), (name, z, h)
+        _check_against_tiled_and_closed_form(f"config 3 head ({z}, {h}) causal={causal}",
+                                             dict(o=gsl(o), dq=gsl(tq.grad), dk=gsl(tk.grad), dv=gsl(tv.grad)),
+                                             dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, "bf16")
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
@@ -170,7 +194,10 @@ def test_head_dims_16_and_32_forward_and_backward(gpu, dtype, D, causal):
     out = triton_amd.attention(tq, tk, tv, causal, sm_scale)
     assert out.shape == tq.shape
     out.backward(tdo)
-    assert np.allclose(to_np(out.detach()), cf["o"], atol=1e-2, rtol=1e-2)
-    for name, t in (("dq", tq), ("dk", tk), ("dv", tv)):
+    for t in (tq, tk, tv):
         assert t.grad.shape == t.shape
-        assert np.allclose(to_np(t.grad), cf[name], atol=3e-2, rtol=1e-2), name
+    ro, rM = A.attn_fwd_tiled(q, k, v, causal, sm_scale, dtype, BLOCK_N=16 if D == 16 else 32)   # (06:111: BLOCK_N <= HEAD_DIM)
+    rdq, rdk, rdv, _ = A.attn_bwd_tiled(q, k, v, ro, do, rM, sm_scale, causal, dtype)
+    _check_against_tiled_and_closed_form(f"{shape} causal={causal}",
+                                         dict(o=to_np(out.detach()), dq=to_np(tq.grad), dk=to_np(tk.grad), dv=to_np(tv.grad)),
+                                         dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, dtype)

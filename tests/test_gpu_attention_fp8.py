@@ -12,6 +12,8 @@ import triton_amd
 from oracle import attention as A
 from oracle import formats
 
+from util import set_knob
+
 pytestmark = pytest.mark.gpu
 TDT = {"e5m2": torch.float8_e5m2, "e4m3": torch.float8_e4m3fn}
 
@@ -67,7 +69,7 @@ def test_fp8_forward_eight_wave_variant_gives_the_same_codes(gpu, causal, monkey
     shape = (1, 2, 384, 128)
     _, (tq, tk, tv) = _fp8_inputs(5, shape, "e5m2", gpu)
     base = triton_amd.attention(tq, tk, tv, causal, 0.1).view(torch.uint8).cpu().numpy()
-    monkeypatch.setenv("MI355_ATTN_FWD_VARIANT", "2")
+    set_knob(monkeypatch, "MI355_ATTN_FWD_VARIANT", "2")
     wide = triton_amd.attention(tq, tk, tv, causal, 0.1).view(torch.uint8).cpu().numpy()
     assert np.array_equal(base, wide)
 

@@ -13,7 +13,7 @@ import torch
 
 import triton_amd
 from oracle import formats, gemm
-from util import bits_equal, from_np, randn_rounded, to_np
+from util import bits_equal, from_np, randn_rounded, to_np, set_knob
 
 pytestmark = pytest.mark.gpu
 HERE = os.path.dirname(os.path.abspath(__file__))
@@ -101,8 +101,8 @@ def test_every_kernel_variant_is_bit_exact_on_integers(gpu, monkeypatch, tile):
     # partial last K step, which the ping-pong kernel hands to the one-barrier kernel and the
     # pipelined kernels finish themselves; the persistent form takes whole tiles with K a multiple of
     # 128 (512 x 768 x 512 with 3 programs: two tiles each, in one stream of K steps) and falls back otherwise
-    monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
-    monkeypatch.setenv("MI355_GEMM_PROGRAMS", "3")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", str(tile))
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", "3")
     rng = np.random.default_rng(11 + tile)
     for (M, N, K) in [(512, 768, 512), (300, 264, 520), (256, 256, 64), (1280, 1024, 128)]:
         a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
@@ -136,7 +136,7 @@ def test_single_nonzero_locates_every_tile(gpu):
 def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
     # the 128x128-per-wave kernel of 16x16x32 MFMAs (K-major B, whole 256x256 tiles, K bytes % 256 == 0):
     # N(0,1) operands, every output type, alpha, the activation, a padded C, and the smallest K (two steps)
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
     rng = np.random.default_rng(23)
     for (M, N, K) in [(512, 256, 1152), (256, 768, 128)]:
         a = randn_rounded(rng, (M, K), dtype)
@@ -172,7 +172,7 @@ def test_four_wave_16x16_kernel_against_closed_form(gpu, monkeypatch, dtype):
 def test_four_wave_16x16_fp8_kernel_against_dequantised_closed_form(gpu, monkeypatch, fmt, tdt):
     # the fp8 form of the same kernel (16x16x128 MFMAs; K-major B, whole tiles, K % 256 == 0): every finite
     # code as input, per-tensor scales, fp32 and bf16 outputs
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
     rng = np.random.default_rng(29)
     table = formats.fp8_table(fmt)
     finite = np.array([c for c in range(256) if np.isfinite(table[c])], dtype=np.uint8)
@@ -236,7 +236,7 @@ def test_fp8_raw_code_inputs_like_reference_test(gpu):
     assert np.allclose(c, ref, rtol=0.01, atol=0.01)
 
 
-def test_fp8_row_major_b_and_fp8_output_use_the_strided_kernel(gpu):
+def test_fp8_row_major_b_uses_the_strided_kernel_and_fp8_output(gpu):
     rng = np.random.default_rng(8)
     ca = formats.encode_fp8(rng.standard_normal((64, 96)).astype(np.float32), "e4m3")
     cb = formats.encode_fp8(rng.standard_normal((96, 80)).astype(np.float32), "e4m3")    # [K, N] row-major
@@ -251,6 +251,70 @@ def test_fp8_row_major_b_and_fp8_output_use_the_strided_kernel(gpu):
     assert np.array_equal(out8.view(torch.uint8).cpu().numpy(), formats.encode_fp8(ref, "e4m3"))
     a16 = from_np(tab[ca], "fp16", gpu); b16 = from_np(tab[cb], "fp16", gpu)
     assert triton_amd.matmul_like_input(a16, b16).dtype == torch.float16
+
+
+@pytest.mark.parametrize("tile", [None, 6])
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_fp8_output_of_the_mfma_epilogues_rounds_like_the_oracle(gpu, monkeypatch, fmt, tdt, tile):
+    # fp8 outputs (tutorial 09: c has the dtype of a, 09:93-96, :124) are stored by the MFMA kernels' own
+    # epilogues.  A zero product plus an fp32 addend puts chosen fp32 values through that conversion: every
+    # code value, every midpoint between neighbouring codes (ties to even), values just off the midpoints,
+    # sub-normal results, finite overflow (saturates to the largest finite code) and NaN.
+    if tile is not None:
+        set_knob(monkeypatch, "MI355_GEMM_TILE", tile)     # 6: four-wave kernel (its own epilogue); default here: 128x128 tiles
+    n = 512
+    tab = formats.fp8_table(fmt).astype(np.float64)
+    _, _, _, max_code = formats.FP8_FORMATS[fmt]
+    pos = tab[: max_code + 1]
+    mids = (pos[:-1] + pos[1:]) / 2
+    vals = np.concatenate([pos, mids, mids * (1 + 2.0 ** -20), mids * (1 - 2.0 ** -20), [pos[-1] * 1.01, pos[-1] * 1.07, 1e9, 3e38],
+                           [pos[1] / 2, pos[1] / 4, pos[1] * 0.75, 1e-30]])
+    vals = np.concatenate([vals, -vals]).astype(np.float32)
+    rng = np.random.default_rng(3)
+    d = np.concatenate([vals, (rng.standard_normal(n * n - len(vals) - 2) * 30).astype(np.float32), [np.nan, -np.nan]]).astype(np.float32)
+    d = d.reshape(n, n)
+    z = torch.zeros(n, n, dtype=torch.bfloat16, device=gpu)
+    out = triton_amd.matmul(z, z, add=torch.from_numpy(d).to(gpu), out_dtype=tdt)
+    got = out.view(torch.uint8).cpu().numpy()
+    want = formats.encode_fp8(d, fmt)
+    finite = ~np.isnan(d)
+    assert np.array_equal(got[finite] & 0x7F, want[finite] & 0x7F)
+    nz = finite & (want & 0x7F != 0)
+    assert np.array_equal(got[nz] >> 7, want[nz] >> 7)                      # sign (of non-zero results)
+    assert np.all(np.isnan(formats.fp8_table(fmt)[got[~finite]]))           # NaN stays NaN
+
+
+def test_full_size_fp8_to_fp8_runs_an_mfma_kernel(gpu):
+    # tutorial 09's matmul on e4m3fn operands returns e4m3fn (09:105-138): at 8192^3 that must be the
+    # four-wave MFMA kernel, not the one-thread-per-output strided kernel - told apart by time (the strided
+    # kernel needs seconds for this product)
+    n = 8192
+    g = torch.Generator(device="cpu").manual_seed(9)
+    a = (torch.randn(n, n, generator=g) * 0.25).to(torch.float8_e4m3fn)
+    b = (torch.randn(n, n, generator=g) * 0.25).to(torch.float8_e4m3fn)     # [N, K]
+    ta, tb = a.to(gpu), b.to(gpu).t()
+    out = triton_amd.matmul_like_input(ta, tb)
+    assert out.dtype == torch.float8_e4m3fn
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(3):
+        out = triton_amd.matmul_like_input(ta, tb)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / 3
+    print(f"fp8 -> fp8 8192^3: {ms:.3f} ms per call")
+    assert ms < 5.0, ms
+    rows = [0, 255, 4096, 8191]
+    ref = a[rows].double().numpy() @ b.double().numpy().T
+    tab = formats.fp8_table("e4m3")
+    got = tab[out[rows].view(torch.uint8).cpu().numpy()]
+    want = tab[formats.encode_fp8(ref.astype(np.float32), "e4m3")]
+    # the fp8 MFMA's accumulation error (about 6e-5 relative) may move a value across a rounding boundary:
+    # equal codes almost everywhere, never more than one code apart (e4m3 spacing: 2^-3 relative)
+    assert np.mean(got == want) > 0.98
+    assert np.allclose(got, want, rtol=0.13, atol=2.0 ** -9)
+    assert np.allclose(got, ref, rtol=0.07, atol=2.0 ** -9)                  # half a code spacing (plus slack) from the exact product
 
 
 @pytest.mark.parametrize("fmt", ["e4m3", "e5m2", "e2m1", "e8m0"])
@@ -302,6 +366,55 @@ def test_full_size_8192_bf16_sampled_rows_and_exact_permutation(gpu):
     del c, cp
 
 
+def _sampled_rows_check(gpu, M, N, K, dtype, seed, layout="row_major_b"):
+    """C = A @ B at full size on N(0, 1) operands; rows at tile edges and a few inside are compared with the
+    fp64 product rounded to the output type at rtol = atol = 1e-2, and one signed-permutation product
+    (every output a single exactly representable term) bitwise."""
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    a = torch.randn(M, K, generator=g).to(tdt)
+    b = torch.randn(K, N, generator=g).to(tdt)
+    tb = b.to(gpu)
+    if layout == "k_major_b":
+        tb = tb.t().contiguous().t()
+    c = triton_amd.matmul(a.to(gpu), tb)
+    assert c.dtype == tdt and c.shape == (M, N)
+    rows = sorted({0, 1, 255, 256, M // 2 - 1, M // 2, M - 257, M - 256, M - 1, (5 * M) // 8 + 3})
+    ref = formats.round_to((a[rows].double().numpy() @ b.double().numpy()).astype(np.float32), dtype)
+    got = to_np(c[rows])
+    print(f"{M}x{N}x{K} {dtype} {layout}: max |err| {np.abs(got - ref).max():.3e} on {len(rows)} rows")
+    assert np.allclose(got, ref, rtol=1e-2, atol=1e-2)
+    if K <= N:
+        perm = torch.randperm(N, generator=g)[:K] if K < N else torch.randperm(N, generator=g)
+        sign = (torch.randint(0, 2, (K,), generator=g) * 2 - 1).to(tdt)
+        pb = torch.zeros(K, N, dtype=tdt)
+        pb[torch.arange(K), perm] = sign                 # row k of B has its one entry in column perm[k]
+        cp = triton_amd.matmul(a.to(gpu), pb.to(gpu)).cpu()
+        want = torch.zeros(M, N, dtype=tdt)
+        want[:, perm] = a * sign[None, :]
+        assert torch.equal(cp, want)
+
+
+@pytest.mark.parametrize("n", [2048, 3072, 4096, 5120, 6144, 7168])
+def test_config2_sweep_sizes_bf16(gpu, n):
+    # BASELINE config 2 sweeps square sizes 1024 .. 8192 (1024 and 8192 have tests of their own): 5120, 6144
+    # and 7168 are the sizes whose tiles do not divide by the CU count, so the persistent programs walk ragged
+    # rounds of tiles as one stream of K steps
+    _sampled_rows_check(gpu, n, n, n, "bf16", seed=n)
+
+
+def test_full_size_8192_fp16_sampled_rows(gpu):
+    # config 2 names fp16 next to bf16
+    _sampled_rows_check(gpu, 8192, 8192, 8192, "fp16", seed=5)
+
+
+@pytest.mark.parametrize("layout", ["row_major_b", "k_major_b"])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_uneven_k_8192x8192x8176(gpu, dtype, layout):
+    # the reference's own EVEN_K == False performance shape (python/test/regression/test_performance.py:46)
+    _sampled_rows_check(gpu, 8192, 8192, 8176, dtype, seed=46, layout=layout)
+
+
 def test_full_size_8192_fp8_sampled_rows_and_k_major_bf16(gpu):
     # BASELINE config 4 at full size (e4m3fn codes with per-tensor scales, bf16 out), sampled rows against the
     # dequantised fp64 product; and config 2 with B stored K-major (the `b.T` view), sampled rows
@@ -350,7 +463,7 @@ def test_skinny_16bit_kernel_is_bit_exact_on_integers(gpu, monkeypatch, dtype, s
     for tb in (from_np(b, dtype, gpu), from_np(np.ascontiguousarray(b.T), dtype, gpu).t()):
         got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
         assert bits_equal(got, ref), (dtype, shape, tb.stride())
-        monkeypatch.setenv("MI355_GEMM_SKINNY", "0")      # the tile kernels on the same inputs
+        set_knob(monkeypatch, "MI355_GEMM_SKINNY", "0")      # the tile kernels on the same inputs
         assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), ref)
         monkeypatch.delenv("MI355_GEMM_SKINNY")
     if dtype == "fp16":
@@ -382,7 +495,7 @@ def test_fused_addends_in_the_four_wave_kernel(gpu, dtype, monkeypatch):
     # the add-matrix / add-rows / add-cols forms (python/test/unit/language/test_core.py:3128-3145) in the
     # addend instantiation of the 16x16-MFMA kernel: integer data, bit-exact; both B layouts, addend in fp32
     # and in the input type, with scales and the activation, result in fp32 and in the input type
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
     M, N, K = 512, 768, 256
     rng = np.random.default_rng(77)
     a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
@@ -406,8 +519,8 @@ def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, program
     # five tiles (1280 x 256) on at most 2 / 3 / 4 programs: 3 rounds on 2 programs (2 + 2 + 1 tiles), 2 rounds
     # on 3 (2 + 2 + 1) - with 4 CUs also 2 rounds, so again 3 programs; a program with fewer tiles than the others
     # wraps its loads earlier.  bf16 with both B layouts and fp8, sums of small integers: bit-exact.
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
-    monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(programs))
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", str(programs))
     rng = np.random.default_rng(90 + programs)
     M, N = 1280, 256
     for K in (128, 384):
@@ -430,7 +543,7 @@ def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, program
 def test_fused_addends_in_the_four_wave_fp8_kernel(gpu, monkeypatch, fmt, tdt):
     # the same addend forms in the fp8 kernel of 16x16x128 MFMAs: codes of small integers (exact products
     # and sums), addend in fp32 and bf16, bit-exact in fp32
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
     M, N, K = 512, 256, 512
     rng = np.random.default_rng(78)
     table = formats.fp8_table(fmt)
@@ -513,7 +626,7 @@ def test_stream_k_schedule_is_bit_exact_on_integers(gpu, monkeypatch, dtype, npr
     # partial sums are exact, so any split gives the bits of the closed form.  Shapes the schedule
     # does not take (partial tiles, K tails) run as plain calls.
     if nprog is not None:
-        monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(nprog))
+        set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", str(nprog))
     rng = np.random.default_rng(17 + (nprog or 0))
     for (M, N, K) in [(512, 768, 1024), (256, 256, 4096), (1280, 256, 512), (300, 264, 520), (16, 512, 256)]:
         a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)

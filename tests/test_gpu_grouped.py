@@ -7,7 +7,7 @@ import torch
 
 import triton_amd
 from oracle import formats, gemm
-from util import bits_equal, from_np, to_np
+from util import bits_equal, from_np, to_np, set_knob
 
 pytestmark = pytest.mark.gpu
 
@@ -40,7 +40,7 @@ def test_ragged_problems_are_bit_exact_on_integers(gpu, nprog, big_min, monkeypa
     # the tile size the library picks for this group (128x128: fewer 256x256 tiles than CUs) and once
     # with the 256x256 form forced (MI355_GROUPED_BIG_MIN=1)
     if big_min is not None:
-        monkeypatch.setenv("MI355_GROUPED_BIG_MIN", str(big_min))
+        set_knob(monkeypatch, "MI355_GROUPED_BIG_MIN", str(big_min))
     rng = np.random.default_rng(nprog)
     shapes = [(256, 128, 64), (130, 72, 40), (1, 304, 8), (128, 128, 128), (100, 70, 50), (37, 19, 7), (300, 264, 520)]
     ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]
@@ -70,11 +70,11 @@ def test_groups_of_whole_256_tiles(gpu, nprog, chunk, monkeypatch):
     # every problem whole 256x256 tiles and K % 128 == 0: the four-wave 16x16-MFMA kernel takes the group
     # (thresholds lowered so that 20 tiles and K = 128 are enough); exact sums of small integers, rounded
     # once; K from one pair of stages up to several, M != N, problems of one tile between larger ones
-    monkeypatch.setenv("MI355_GROUPED_BIG_MIN", "1")
-    monkeypatch.setenv("MI355_GROUPED_WAVE128_MIN_K", "128")
+    set_knob(monkeypatch, "MI355_GROUPED_BIG_MIN", "1")
+    set_knob(monkeypatch, "MI355_GROUPED_WAVE128_MIN_K", "128")
     # a program's tiles: chunks of up to 4 / 1 / 3 consecutive tiles (7 programs, 20 tiles: chunks of 3, runs that
     # cross from one problem into the next and runs of several tiles inside one problem)
-    monkeypatch.setenv("MI355_GROUPED_CHUNK", str(chunk))
+    set_knob(monkeypatch, "MI355_GROUPED_CHUNK", str(chunk))
     rng = np.random.default_rng(40 + nprog)
     shapes = [(256, 256, 128), (512, 256, 256), (256, 256, 1024), (256, 768, 384), (1024, 512, 128), (256, 256, 256), (512, 512, 640)]
     ga = [rng.integers(-2, 3, size=(m, k)).astype(np.float32) for m, n, k in shapes]
@@ -85,7 +85,7 @@ def test_groups_of_whole_256_tiles(gpu, nprog, chunk, monkeypatch):
         for c, r in zip(outs, ref):
             assert bits_equal(c, formats.round_to(r, dtype))   # (K = 1024 reaches beyond bf16's exact integers)
     # the same group through the eight-wave kernels
-    monkeypatch.setenv("MI355_GROUPED_WAVE128_MIN_K", "0")
+    set_knob(monkeypatch, "MI355_GROUPED_WAVE128_MIN_K", "0")
     for c, r in zip(_run(gpu, ga, gb, "fp16", num_programs=nprog), ref):
         assert bits_equal(c, r)
 

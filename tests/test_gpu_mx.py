@@ -7,7 +7,7 @@ import torch
 
 import triton_amd
 from oracle import formats, mx
-from util import bits_equal, to_np
+from util import bits_equal, to_np, set_knob
 
 pytestmark = pytest.mark.gpu
 
@@ -116,8 +116,8 @@ def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile
     # parity from tile to tile in the persistent form, two programs for six and twelve tiles),
     # K = 1056 (not a multiple of 512) their fall-back.  6 = four waves of scaled 16x16x128 MFMAs (both formats): whole
     # 256x256 tiles and K a multiple of 1024 (the last two shapes: one and two groups of four K steps), else 5.
-    monkeypatch.setenv("MI355_GEMM_TILE", str(tile))
-    monkeypatch.setenv("MI355_GEMM_PROGRAMS", "2")
+    set_knob(monkeypatch, "MI355_GEMM_TILE", str(tile))
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", "2")
     rng = np.random.default_rng(tile)
     for (M, N, K) in [(512, 256, 1536), (300, 520, 1056), (768, 512, 1536), (768, 1024, 1024), (512, 256, 2048)]:
         if fmt == "mxfp4":
@@ -138,8 +138,8 @@ def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile
 def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, fmt, programs):
     # five tiles on at most 2 / 3 programs of the scaled 16x16x128 kernels (2 + 2 + 1 tiles either way, in three or
     # two rounds); K of one and of two groups of four K steps (the scale ring's parity at the tile switch)
-    monkeypatch.setenv("MI355_GEMM_TILE", "6")
-    monkeypatch.setenv("MI355_GEMM_PROGRAMS", str(programs))
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", str(programs))
     rng = np.random.default_rng(60 + programs)
     for (M, N, K) in [(1280, 256, 1024), (256, 1280, 2048)]:
         if fmt == "mxfp4":

@@ -27,3 +27,13 @@ def bits_equal(a: np.ndarray, b: np.ndarray) -> bool:
     a = np.ascontiguousarray(a, dtype=np.float32)
     b = np.ascontiguousarray(b, dtype=np.float32)
     return a.shape == b.shape and np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+def set_knob(monkeypatch, name: str, value) -> None:
+    """Set one of the library's MI355_* environment knobs for the rest of the test.  The library reads
+    the environment once per process, so it is told to read it again (conftest does the same after
+    every test, when monkeypatch has restored the variables)."""
+    from triton_amd import _lib
+
+    monkeypatch.setenv(name, str(value))
+    _lib.load().mi355_refresh_env()

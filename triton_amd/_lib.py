@@ -17,7 +17,7 @@ F16, BF16, F8E4M3, F8E5M2, F32 = 0, 1, 2, 3, 4
 MXFP4, MXFP8 = 0, 1
 ACT_NONE, ACT_LEAKY_RELU = 0, 1
 DEQ_E4M3, DEQ_E5M2, DEQ_E2M1, DEQ_E8M0 = 0, 1, 2, 3
-Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORKSPACE_BYTES = 0, 1, 2, 3, 4, 5
+Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORKSPACE_BYTES, Q_WALL_CLOCK_KHZ = 0, 1, 2, 3, 4, 5, 6
 
 I64x4 = c_int64 * 4
 
@@ -50,7 +50,9 @@ SIGNATURES = {
                                c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                POINTER(c_int64), c_float, c_int, c_int, c_void_p]),
     "mi355_dequant": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "mi355_clock_probe": (c_int, [c_void_p, c_int, c_void_p]),
     "mi355_query": (c_int, [c_int]),
+    "mi355_refresh_env": (None, []),
     "mi355_strerror": (c_char_p, [c_int]),
 }
 

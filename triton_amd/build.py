@@ -31,6 +31,10 @@ HIPCC_FLAGS = [
 EXTRA_FLAGS = {
     "attn_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "attn_bwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    # keeps the device assembly next to the object file: this file issues its MFMAs as inline assembly, so the
+    # compiler inserts no wait before reads of their results, and tests/test_isa_mfma_hazard.py checks on the
+    # generated code that every such read comes late enough
+    "gemm_wave128.hip": ["-save-temps=obj"],
 }
 
 

@@ -18,23 +18,6 @@
 
 namespace mi355 {
 
-template <int FMT>  // 0 = e4m3fn, 1 = e5m2
-__device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
-#if MI355_DEVICE_PASS
-  int w = 0;
-  if constexpr (FMT == 1) {
-    w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, w, false);
-    w = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
-  } else {
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
-    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
-  }
-  return w;
-#else
-  return 0;
-#endif
-}
-
 template <int FMT>
 __device__ __forceinline__ f32x16 mfma_f8(i32x8 a, i32x8 b, f32x16 c) {
 #if MI355_DEVICE_PASS

@@ -5,6 +5,8 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 #include <string.h>
+#include <atomic>
+#include <climits>
 #include <mutex>
 #include "../../include/mi355_kernels.h"
 #include "launch.h"
@@ -14,7 +16,7 @@ using namespace mi355;
 namespace {
 
 struct DeviceInfo {
-  int ok = 0, cus = 0, gfx950 = 0, lds = 0, clock_khz = 0;
+  int ok = 0, cus = 0, gfx950 = 0, lds = 0, clock_khz = 0, wall_clock_khz = 0;
 };
 
 const DeviceInfo& device_info() {
@@ -29,15 +31,55 @@ const DeviceInfo& device_info() {
     info.gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
     info.lds = (int)prop.sharedMemPerBlock;
     info.clock_khz = prop.clockRate;
+    if (hipDeviceGetAttribute(&info.wall_clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) info.wall_clock_khz = 0;
     info.ok = 1;
   });
   return info;
 }
 
-int env_int(const char* name, int dflt) {
+// Tuning knobs from the environment (the reference's third configuration mechanism: environment
+// variables read by the runtime, python/triton/runtime/jit.py:717, :848).  Read ONCE per process, at the
+// first call that needs them, and again only when mi355_refresh_env() is called: a launch costs no getenv.
+// UNSET = the variable is absent or empty and the call site's own default applies.
+constexpr int UNSET = INT_MIN;
+struct Knobs {
+  int force_strided, group_m, tile, programs, skinny, grouped_big_min, grouped_wave128_min_k, grouped_chunk,
+      attn_fwd_variant, attn_programs;
+};
+Knobs g_knobs;
+std::atomic<int> g_knobs_ready{0};
+std::mutex g_knobs_mutex;
+
+int read_env(const char* name, int lo) {
   const char* s = getenv(name);
-  return s && *s ? atoi(s) : dflt;
+  if (!s || !*s) return UNSET;
+  const int v = atoi(s);
+  return v < lo ? lo : v;   // (out-of-range values are clamped, never passed on to a kernel)
 }
+
+void load_knobs() {
+  std::lock_guard<std::mutex> lock(g_knobs_mutex);
+  Knobs k;
+  k.force_strided = read_env("MI355_GEMM_FORCE_STRIDED", 0);
+  k.group_m = read_env("MI355_GEMM_GROUP_M", 1);
+  k.tile = read_env("MI355_GEMM_TILE", 0);
+  k.programs = read_env("MI355_GEMM_PROGRAMS", 1);
+  k.skinny = read_env("MI355_GEMM_SKINNY", 0);
+  k.grouped_big_min = read_env("MI355_GROUPED_BIG_MIN", 1);
+  k.grouped_wave128_min_k = read_env("MI355_GROUPED_WAVE128_MIN_K", 0);
+  k.grouped_chunk = read_env("MI355_GROUPED_CHUNK", 1);
+  k.attn_fwd_variant = read_env("MI355_ATTN_FWD_VARIANT", 0);
+  k.attn_programs = read_env("MI355_ATTN_PROGRAMS", 1);
+  g_knobs = k;
+  g_knobs_ready.store(1, std::memory_order_release);
+}
+
+const Knobs& knobs() {
+  if (!g_knobs_ready.load(std::memory_order_acquire)) load_knobs();
+  return g_knobs;
+}
+
+int knob(int value, int dflt) { return value == UNSET ? dflt : value; }
 
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
@@ -68,10 +110,13 @@ int mi355_query(int what) {
     case MI355_Q_IS_GFX950: return d.gfx950;
     case MI355_Q_LDS_BYTES: return d.lds;
     case MI355_Q_CLOCK_KHZ: return d.clock_khz;
+    case MI355_Q_WALL_CLOCK_KHZ: return d.wall_clock_khz;
     case MI355_Q_STREAMK_WORKSPACE_BYTES: return (d.cus > 0 ? d.cus : 256) * 2 * 256 * 256 * 4;
     default: return -1;
   }
 }
+
+void mi355_refresh_env(void) { load_knobs(); }
 
 const char* mi355_strerror(int code) {
   switch (code) {
@@ -103,13 +148,13 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const bool is8 = es == 1;
   const int vec = 16 / es;  // elements per 16-byte chunk
 
-  const bool out_ok = out_dtype == MI355_F16 || out_dtype == MI355_BF16 || out_dtype == MI355_F32;
+  const bool out_ok = true;   // every output type of the ABI has a store in the MFMA epilogues (fp8: hardware conversion, saturating)
   const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
   const bool b_nmajor = !is8 && sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
   // the tile copies address 256 rows of an operand with 32-bit byte offsets from a 64-bit tile base
   const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
-  const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && env_int("MI355_GEMM_FORCE_STRIDED", 0) == 0;
+  const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && knob(knobs().force_strided, 0) == 0;
 
   if (!fast) {
     GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype,
@@ -125,7 +170,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.ldc = scm; p.scn = scn;
   p.a_scale = a_scale; p.b_scale = b_scale;
   p.activation = activation; p.out_dtype = out_dtype;
-  p.group_m = group_m_arg > 0 ? group_m_arg : env_int("MI355_GEMM_GROUP_M", 8);
+  p.group_m = group_m_arg > 0 ? group_m_arg : knob(knobs().group_m, 8);
+  // four consecutive C elements as one store: rows of 16-bit / fp32 elements 16-byte aligned (for fp8 that
+  // makes every group of four 4-byte aligned)
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
   p.aux = aux; p.aux_sm = aux_sm; p.aux_sn = aux_sn; p.aux_dtype = aux_dtype;
 
@@ -146,12 +193,12 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // (fp8 from three quarters of a round: at 144 tiles the eight-wave kernel is 4-7 % ahead - 3072^3 1520 vs
   // 1450, 3072x3072x8192 2040 vs 1890 TFLOP/s -, at 196 tiles the four-wave one by 2 %, at 225 by 13 %)
   if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && gemm_wave128_ok(p, b_kmajor)) tile = 6;
-  tile = tile_arg >= 0 ? tile_arg : env_int("MI355_GEMM_TILE", tile);
-  p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
+  tile = tile_arg >= 0 ? tile_arg : knob(knobs().tile, tile);
+  p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;
   // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
-  const bool skinny_allowed = tile_arg < 0 && env_int("MI355_GEMM_SKINNY", 1);  // an explicit tile means a tile kernel
+  const bool skinny_allowed = tile_arg < 0 && knob(knobs().skinny, 1);  // an explicit tile means a tile kernel
   if (!aux && skinny_allowed) {
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
@@ -235,10 +282,10 @@ int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d
   // groups with at least one 256x256 tile per CU run 256x256 tiles, one program per CU (never more
   // programs than the caller asked for); MI355_GROUPED_BIG_MIN moves the threshold (a huge value = never)
   const int nprog_big = nprog < cus ? nprog : cus;
-  ga.big_tiles_min = env_int("MI355_GROUPED_BIG_MIN", cus);
+  ga.big_tiles_min = knob(knobs().grouped_big_min, cus);
   // smallest K of a group of whole 256x256 tiles that the four-wave 16x16-MFMA kernel takes (0 = never)
-  ga.wave128_min_k = env_int("MI355_GROUPED_WAVE128_MIN_K", 512);
-  ga.chunk = env_int("MI355_GROUPED_CHUNK", 4);
+  ga.wave128_min_k = knob(knobs().grouped_wave128_min_k, 512);
+  ga.chunk = knob(knobs().grouped_chunk, 4);
   if (ga.chunk < 1) ga.chunk = 1;
   return gemm16_grouped_launch(ga, dtype == MI355_BF16, nprog, nprog_big, (hipStream_t)stream_);
 }
@@ -260,7 +307,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.M = M; p.N = N; p.K = K; p.k_bytes = (int)row_bytes;
   p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.scn = 1;
   p.out_dtype = out_dtype;
-  p.group_m = env_int("MI355_GEMM_GROUP_M", 8);
+  p.group_m = knob(knobs().group_m, 8);
   p.c_vec_ok = ldc % 4 == 0 && aligned(C, 16);
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
@@ -271,9 +318,16 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   if (fmt == MI355_MXFP4 && tiles256 * 2 >= cus && gemm_wave128_mxfp4_ok(p)) tile = 6;
   // (MXFP8 likewise: 2530-2570 vs 2110-2240)
   if (fmt == MI355_MXFP8 && tiles256 * 2 >= cus && gemm_wave128_mxfp8_ok(p)) tile = 6;
-  tile = env_int("MI355_GEMM_TILE", tile);
-  p.num_programs = env_int("MI355_GEMM_PROGRAMS", cus);
+  tile = knob(knobs().tile, tile);
+  p.num_programs = knob(knobs().programs, cus);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
+}
+
+int mi355_clock_probe(uint64_t* ticks, int duration_us, void* stream_) {
+  if (!ticks || !aligned(ticks, 8) || duration_us <= 0 || duration_us > 2000000) return MI355_EINVAL;
+  if (!device_info().gfx950 || device_info().wall_clock_khz <= 0) return MI355_EDEVICE;
+  const unsigned long long real_ticks = (unsigned long long)duration_us * (unsigned long long)device_info().wall_clock_khz / 1000ull;
+  return clock_probe_launch((unsigned long long*)ticks, real_ticks, (hipStream_t)stream_);
 }
 
 int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* stream_) {
@@ -321,7 +375,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
       return MI355_ESTRIDE;
     p.q = (const char*)q; p.k = (const char*)k; p.v = (const char*)v; p.o = (char*)o; p.lse = Mlse;
     p.sm_scale = sm_scale; p.causal = causal != 0;
-    p.variant = env_int("MI355_ATTN_FWD_VARIANT", 1);  // fp8: four waves, two workgroups per CU (eight waves measured 6-12 % slower)
+    p.variant = knob(knobs().attn_fwd_variant, 1);  // fp8: four waves, two workgroups per CU (eight waves measured 6-12 % slower)
     return attn_fwd8_launch(p, dtype == MI355_F8E5M2, (hipStream_t)stream_);
   }
   int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
@@ -336,8 +390,8 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
   // eight waves (256 query rows) per K/V stream halve the L2 -> LDS traffic.  Under the causal mask
   // their row ranges are uneven, which the persistent form (4) evens out by pairing long and short
   // query blocks per program; without a mask the one-item-per-workgroup form (2) is the faster one.
-  p.variant = env_int("MI355_ATTN_FWD_VARIANT", causal ? 4 : 2);
-  p.num_programs = env_int("MI355_ATTN_PROGRAMS", device_info().cus > 0 ? device_info().cus : 256);
+  p.variant = knob(knobs().attn_fwd_variant, causal ? 4 : 2);
+  p.num_programs = knob(knobs().attn_programs, device_info().cus > 0 ? device_info().cus : 256);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 

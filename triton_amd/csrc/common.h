@@ -210,6 +210,48 @@ __device__ __forceinline__ void block_barrier() {
 #endif
 }
 
+// Four fp32 values -> four fp8 codes in one dword (value 0 in the low byte), round to nearest even, by the
+// hardware conversion (OCP e4m3fn / e5m2 on gfx950).  Values beyond the largest finite code come out as
+// NaN (e4m3fn) / infinity (e5m2): callers that need saturation clamp first (pack4_fp8_sat).
+template <int FMT>  // 0 = e4m3fn, 1 = e5m2
+__device__ __forceinline__ int pack4_fp8(float a, float b, float c, float d) {
+#if MI355_DEVICE_PASS
+  int w = 0;
+  if constexpr (FMT == 1) {
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_bf8_f32(c, d, w, true);
+  } else {
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, w, false);
+    w = __builtin_amdgcn_cvt_pk_fp8_f32(c, d, w, true);
+  }
+  return w;
+#else
+  return 0;
+#endif
+}
+
+// The same with finite overflow saturating to the largest finite code (448 / 57344, the downcast maxima of
+// python/test/unit/language/test_conversions.py:307-329); NaN stays NaN.
+template <int FMT>
+__device__ __forceinline__ int pack4_fp8_sat(float a, float b, float c, float d) {
+  constexpr float MAXV = FMT == 1 ? 57344.f : 448.f;
+  auto sat = [](float x) { return x != x ? x : fminf(fmaxf(x, -MAXV), MAXV); };
+  return pack4_fp8<FMT>(sat(a), sat(b), sat(c), sat(d));
+}
+
+// Store of four consecutive C elements as fp8 (out_dtype 2 = e4m3fn, 3 = e5m2): one dword when `vec`
+// (unit column stride, 4-byte aligned), else `count` single bytes `scn` apart.
+__device__ __forceinline__ void store4_fp8(char* C, int64_t off, int64_t scn, int out_dtype, const float (&v)[4], bool vec, int count) {
+  const int w = out_dtype == 3 ? pack4_fp8_sat<1>(v[0], v[1], v[2], v[3]) : pack4_fp8_sat<0>(v[0], v[1], v[2], v[3]);
+  if (vec && count == 4) {
+    *(int*)(C + off) = w;
+  } else {
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+      if (e < count) C[off + e * scn] = (char)(w >> (8 * e));
+  }
+}
+
 // One element of the epilogue addend (dtype codes of the C ABI: 0 fp16, 1 bf16, 4 fp32).
 __device__ __forceinline__ float load_aux(const void* aux, int64_t off, int dtype) {
   if (dtype == 4) return ((const float*)aux)[off];

@@ -3,6 +3,7 @@
 // `matmul(a, b.T)` with b stored [N, K], python/tutorials/03-matrix-multiplication.py:378-382,
 // python/tutorials/09-persistent-matmul.py:396-407).
 #include "gemm_core.h"
+#include "formats.h"
 
 namespace mi355 {
 
@@ -107,6 +108,8 @@ __global__ __launch_bounds__(256) void gemm8_skinny_kernel(GemmArgs p) {
     if (m < p.M && n < p.N) {
       const int64_t off = (int64_t)m * p.ldc + (int64_t)n * p.scn;
       if (p.out_dtype == 4) ((float*)p.C)[off] = v;
+      else if (p.out_dtype == 2) ((uint8_t*)p.C)[off] = f32_to_e4m3(v);
+      else if (p.out_dtype == 3) ((uint8_t*)p.C)[off] = f32_to_e5m2(v);
       else if (p.out_dtype == 1) ((__bf16*)p.C)[off] = (__bf16)v;
       else ((_Float16*)p.C)[off] = (_Float16)v;
     }

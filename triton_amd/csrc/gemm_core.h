@@ -110,7 +110,10 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmA
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
           }
-          if (p.out_dtype == 4) {
+          if (p.out_dtype == 2 || p.out_dtype == 3) {
+            const int count = p.N - n < 4 ? p.N - n : 4;
+            if (count > 0) store4_fp8(p.C, (int64_t)m * p.ldc + (int64_t)n * p.scn, p.scn, p.out_dtype, v, vec_ok, count);
+          } else if (p.out_dtype == 4) {
             float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
             if (vec_ok && n + 3 < p.N) {
               *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};

@@ -16,6 +16,7 @@
 //     product with N = 32 or 64).
 #include "common.h"
 #include "launch.h"
+#include "formats.h"
 
 namespace mi355 {
 
@@ -251,6 +252,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
     if (s < p.S && l < p.L) {
       const int64_t off = (int64_t)s * p.cs + (int64_t)l * p.cl;
       if (p.out_dtype == 4) ((float*)p.C)[off] = v;
+      else if (p.out_dtype == 2) ((uint8_t*)p.C)[off] = f32_to_e4m3(v);
+      else if (p.out_dtype == 3) ((uint8_t*)p.C)[off] = f32_to_e5m2(v);
       else if (p.out_dtype == 1) ((__bf16*)p.C)[off] = (__bf16)v;
       else ((_Float16*)p.C)[off] = (_Float16)v;
     }

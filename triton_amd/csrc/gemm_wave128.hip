@@ -47,6 +47,21 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 // epilogue's register shuffle) in front of it, where they see registers that the last MFMAs have yet to write.
 // So every accumulator passes through an (empty) assembly statement behind the wait: volatile statements keep
 // their order, and a value read after its statement is read after the wait.
+//
+// The wait itself (mfma_retire) stands INSIDE the K loop, at the end of the body of a tile's last iteration:
+// whatever the register allocator does with the accumulators on the edge that leaves the loop (its register
+// shuffle for the epilogue, spills), it does behind the loop's last basic block, hence behind the wait.  A
+// wait placed behind the loop can end up behind those moves (a block-scaled fp8 product once came out wrong
+// that way, in one run of many).  A read of an MFMA result has to come (passes + 3) issue slots behind the
+// MFMA - 7 for the 4-pass 16x16x32 16-bit and 16x16x128 fp4 forms, 11 for the 8-pass 16x16x128 fp8 form -;
+// `s_nop 15` is 16 slots of 4 cycles, once per tile.
+// The loop compares with a copy of the step count that went through an empty assembly statement: told that
+// the test equals the loop's own exit test, the compiler sinks the wait out of the loop again.
+__device__ __forceinline__ void mfma_retire() {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 15" ::: "memory");
+#endif
+}
 __device__ __forceinline__ void mfma_drain_row(f32x4 (&r)[8]) {
 #if MI355_DEVICE_PASS
   asm volatile("" : "+a"(r[0]), "+a"(r[1]), "+a"(r[2]), "+a"(r[3]), "+a"(r[4]), "+a"(r[5]), "+a"(r[6]), "+a"(r[7]));
@@ -55,7 +70,7 @@ __device__ __forceinline__ void mfma_drain_row(f32x4 (&r)[8]) {
 template <int MT>
 __device__ __forceinline__ void mfma_drain(f32x4 (&acc)[MT][8]) {
 #if MI355_DEVICE_PASS
-  asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  asm volatile("s_nop 15" ::: "memory");
 #endif
 #pragma unroll
   for (int i = 0; i < MT; i++) mfma_drain_row(acc[i]);
@@ -112,7 +127,9 @@ __device__ __forceinline__ void gemm_epilogue16_impl(f32x4 (&acc)[MT][NT], const
 #pragma unroll
         for (int e = 0; e < 4; e++) v[e] = v[e] >= 0.f ? v[e] : 0.01f * v[e];
       }
-      if (p.out_dtype == 4) {
+      if (p.out_dtype == 2 || p.out_dtype == 3) {
+        store4_fp8(p.C, (int64_t)m * p.ldc + (int64_t)n * p.scn, p.scn, p.out_dtype, v, p.c_vec_ok, 4);
+      } else if (p.out_dtype == 4) {
         float* c = (float*)p.C + (int64_t)m * p.ldc + (int64_t)n * p.scn;
         if (p.c_vec_ok) *(f32x4*)c = f32x4{v[0], v[1], v[2], v[3]};
         else {
@@ -191,6 +208,8 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   int pm, pn;
   tile_at(tile, pm, pn);
   const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
 
   // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
   // those rows is 4 (q & 1) + lane / 16, so the lane offset depends on the parity of j only
@@ -361,6 +380,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     for (int kt = 0; kt < nk; kt += 2) {
       stage(I0{}, fk); advance();
       stage(I1{}, fk); advance();
+      if (kt + 2 >= nk_last) mfma_retire();
     }
     // The next tile's first fragments were requested by reads the compiler cannot see: have them landed
     // before the epilogue's register traffic could move their registers.  Nor does it know that the assembly
@@ -489,6 +509,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
 
   // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
   const unsigned drow = lane >> 3, dslot = lane & 7;
@@ -600,6 +622,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     for (int kt = 0; kt < nk; kt += 2) {
       step(I0{}, I0{}, fk); advance();
       step(I1{}, I1{}, fk); advance();
+      if (kt + 2 >= nk_last) mfma_retire();
     }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
@@ -648,6 +671,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
 
   // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
   const unsigned drow = lane >> 3, dslot = lane & 7;
@@ -795,10 +820,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   while (true) {
     for (int kt = 0; kt < nk; kt += 8) {
       static_for<8>([&](auto U_) { step(U_, fk); advance(); });
-      // The last MFMAs must have retired before control leaves this loop: behind it the compiler moves every
-      // accumulator (its register shuffle for the epilogue) and, not knowing that the assembly above are
-      // MFMAs, does so without waiting; a wait placed behind the loop can end up behind those moves.
-      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+      if (kt + 8 >= nk_last) mfma_retire();
     }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
@@ -898,6 +920,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
 
   // ---- operand loads, as in the 16-bit kernel
   const unsigned drow = lane >> 3, dslot = lane & 7;
@@ -1054,8 +1078,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       step(I1{}, fk); advance();
       step(I2{}, fk); advance();
       step(I3{}, fk); advance();
-      // (the last MFMAs retire inside the loop: see the MXFP8 kernel)
-      asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+      if (kt + 4 >= nk_last) mfma_retire();
     }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;

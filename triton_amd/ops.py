@@ -66,12 +66,23 @@ def _is_contiguous(t) -> bool:
     return True
 
 
+_scale_cache = {}
+
+
 def _scale_ptr(s, device):
-    """None, a python float or a 1-element fp32 device tensor -> (pointer or None, keep-alive)."""
+    """None, a python float or a 1-element fp32 device tensor -> (pointer or None, keep-alive).
+    A python float becomes a device scalar once per (device, value): repeated calls with the same
+    scale pay no host-to-device copy."""
     if s is None:
         return None, None
     if not isinstance(s, torch.Tensor):
-        s = torch.tensor([float(s)], dtype=torch.float32, device=device)
+        key = (str(device), float(s))
+        t = _scale_cache.get(key)
+        if t is None:
+            if len(_scale_cache) >= 256:
+                _scale_cache.clear()
+            t = _scale_cache[key] = torch.tensor([float(s)], dtype=torch.float32, device=device)
+        s = t
     assert s.dtype == torch.float32 and s.numel() == 1, "scales are one fp32 value per tensor"
     _check_device(-1, s)
     return s.data_ptr(), s
@@ -144,8 +155,9 @@ def matmul_streamk(a, b, *, out_dtype=None):
     tiles dealt evenly, so tile counts that are not a multiple of the CU count - or smaller than it,
     where this becomes split-K - keep every CU busy.  The scheduling idea of the persistent
     tutorial (python/tutorials/09-persistent-matmul.py:141-190) taken one step further; the
-    result is the same `a @ b` (partial tiles are added in a fixed order).  A per-device fp32
-    workspace is allocated on first use and kept."""
+    result is the same `a @ b` (partial tiles are added in a fixed order).  An fp32 workspace per
+    (device, stream) is allocated on first use and kept: calls on different streams may overlap, so
+    they must not share partial-tile slots."""
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
     assert _is_contiguous(a), "Matrix A must be contiguous"
     in_dt = _abi_dtype(a)
@@ -162,14 +174,15 @@ def matmul_streamk(a, b, *, out_dtype=None):
     if K == 0:
         return c.zero_()
     lib = _lib.load()
-    ws = _streamk_workspace.get(a.device)
+    stream = _stream()
+    ws = _streamk_workspace.get((a.device, stream))
     if ws is None:
         ws = torch.empty(lib.mi355_query(_lib.Q_STREAMK_WORKSPACE_BYTES), device=a.device, dtype=torch.uint8)
-        _streamk_workspace[a.device] = ws
+        _streamk_workspace[(a.device, stream)] = ws
     rc = lib.mi355_gemm_streamk(
         a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
         a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
-        in_dt, _TORCH_TO_ABI[out_dtype], 0, 0, _lib.ACT_NONE, ws.data_ptr(), ws.numel(), _stream())
+        in_dt, _TORCH_TO_ABI[out_dtype], 0, 0, _lib.ACT_NONE, ws.data_ptr(), ws.numel(), stream)
     _lib.check(rc, "mi355_gemm_streamk")
     return c
 
