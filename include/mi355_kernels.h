@@ -58,7 +58,8 @@ enum {
   MI355_EDTYPE = -2,   /* dtype combination not supported                         */
   MI355_ESHAPE = -3,   /* shape constraint of the kernel family violated          */
   MI355_ESTRIDE = -4,  /* stride / alignment constraint violated                  */
-  MI355_EDEVICE = -5   /* no gfx950 device current                                */
+  MI355_EDEVICE = -5,  /* no gfx950 device current                                */
+  MI355_ESCRATCH = -6  /* the call needs more than the library's static scratch   */
 };
 
 /* mi355_query selectors */
@@ -141,6 +142,26 @@ int mi355_gemm_streamk(const void* A, const void* B, void* C,
                        int in_dtype, int out_dtype,
                        const float* a_scale, const float* b_scale,
                        int activation, void* workspace, size_t workspace_bytes, void* stream);
+
+/* mi355_gemm_streamk for callers that cannot allocate (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc): the same kernels, with the partial-tile workspace in a static device
+ * array of the library instead of a caller's buffer.  No counterpart in the reference.  The call performs
+ * no hipMalloc / hipFree and calls no allocating routine.  Limit: the array is 128 MiB per GPU (two
+ * 256x256 fp32 tiles for each of at most 256 programs, one program per compute unit; every GPU the library
+ * runs on holds it until the process ends); a device or MI355_GEMM_PROGRAMS setting that would need more
+ * programs returns MI355_ESCRATCH.  The first call on a device looks the array's address up (do it once
+ * before capturing a graph).  All calls on one GPU share that GPU's array: two calls that overlap in time
+ * on one GPU (different streams, or threads) race and give wrong results - serialise them.  Its contents are
+ * irrelevant before and after a call (every slot a call reads, the same call wrote), so nothing is cleared.
+ */
+int mi355_gemm_streamk_static(const void* A, const void* B, void* C,
+                              int M, int N, int K,
+                              int64_t stride_am, int64_t stride_ak,
+                              int64_t stride_bk, int64_t stride_bn,
+                              int64_t stride_cm, int64_t stride_cn,
+                              int in_dtype, int out_dtype,
+                              const float* a_scale, const float* b_scale,
+                              int activation, void* stream);
 
 /* mi355_gemm with the epilogues of the reference's dot test fused in:
  *   C = softmax_rows?( act( (a_scale * b_scale) * A @ B + D ) )

@@ -32,6 +32,9 @@ SIGNATURES = {
     "mi355_gemm_streamk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                    c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),
+    "mi355_gemm_streamk_static": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                          c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                          c_int, c_int, c_void_p, c_void_p, c_int, c_void_p]),
     "mi355_gemm_epilogue": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int, c_int, c_void_p, c_void_p,

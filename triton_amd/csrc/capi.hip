@@ -126,6 +126,7 @@ const char* mi355_strerror(int code) {
     case MI355_ESHAPE: return "shape not supported by this kernel family";
     case MI355_ESTRIDE: return "stride or alignment not supported by this kernel family";
     case MI355_EDEVICE: return "current device is not a gfx950 GPU";
+    case MI355_ESCRATCH: return "the library's static scratch array is too small for this call (more than 256 programs)";
     default: break;
   }
   if (code > 0) return hipGetErrorString((hipError_t)code);
@@ -252,6 +253,54 @@ int mi355_gemm_streamk(const void* A, const void* B, void* C, int M, int N, int 
   const bool whole_tiles = M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0;
   return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
                    activation, nullptr, 0, 0, 0, whole_tiles ? 7 : -1, 0, stream_, (float*)workspace);
+}
+
+// ---- stream-K without an allocation anywhere: the partial-tile workspace is a static device array.
+// Host code must never use the array's NAME as an address (there it is a host-side stand-in; a kernel
+// handed it would fault): the address on each device comes from hipGetSymbolAddress, once per device,
+// and only that pointer is passed on.
+constexpr int kStaticStreamKPrograms = 256;                                   // one program per CU of an MI355X
+constexpr size_t kStaticStreamKBytes = (size_t)kStaticStreamKPrograms * 2 * 256 * 256 * 4;   // 128 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticStreamKBytes];
+
+namespace {
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices];          // per device: each GPU holds its own copy of the array
+std::mutex g_scratch_mutex;
+
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return MI355_EDEVICE;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // with device `dev` current: that device's copy
+    if (e != hipSuccess) return (int)e;
+    if (!ptr) return MI355_EDEVICE;
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MI355_OK;
+}
+}  // namespace
+
+int mi355_gemm_streamk_static(const void* A, const void* B, void* C, int M, int N, int K,
+                              int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                              int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                              int activation, void* stream_) {
+  if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
+  // the static array holds two partial tiles for each of at most 256 programs (one per CU)
+  const int cus = device_info().cus > 0 ? device_info().cus : 256;
+  const int programs = knob(knobs().programs, cus) < cus ? knob(knobs().programs, cus) : cus;
+  if (programs > kStaticStreamKPrograms) return MI355_ESCRATCH;
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc) return rc;
+  const bool whole_tiles = M > 0 && N > 0 && M % 256 == 0 && N % 256 == 0;
+  return gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
+                   activation, nullptr, 0, 0, 0, whole_tiles ? 7 : -1, 0, stream_, (float*)ws);
 }
 
 int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int K,
