@@ -60,33 +60,57 @@ def quick(fn, iters=60, warmup=20):
     return ev_ms
 
 
-def observed_clock_mhz(lib, fn, rounds=12, launches_per_round=4, window_us=15):
-    """Shader clock while `fn` runs back to back (an untimed leg of its own).  After every few launches a
-    one-wave probe kernel on the SAME stream reads the shader-clock counter and the constant-rate real-time
-    counter over `window_us`: the board's power management moves the clock on a millisecond scale, so
-    the clock in the microseconds behind a kernel is the clock that kernel ran at.  (A probe that lives next
-    to the kernels on a second stream would hold one SIMD slot and cost a one-workgroup-per-CU kernel a
-    whole round of tiles - and so raise the very clock it reads.)"""
+def observed_clock_mhz(fn, seconds=1.0):
+    """Shader clock while `fn` runs back to back (an untimed leg of its own): the driver's current-clock
+    reading (the starred line of /sys/class/drm/card*/device/pp_dpm_sclk, what rocm-smi --showclocks
+    prints) sampled every 10 ms by a host thread over `seconds` of sustained launches; the median of the
+    samples taken after the first quarter.  None where the file is not readable.  (The board holds its
+    power limit by lowering the clock of MFMA-heavy kernels, so the nominal clock says little.  The
+    library's own mi355_clock_probe reads the counters on the device, but a probe wave next to a kernel
+    that fills every SIMD costs that kernel a round of tiles, and the clock is back up within
+    microseconds of a kernel's end - so it suits kernels that leave a wave slot free, not these.)"""
+    import glob
+    import re
+    import threading
+
     import torch
 
-    from triton_amd import _lib
-
-    wall_khz = lib.mi355_query(_lib.Q_WALL_CLOCK_KHZ)
-    if wall_khz <= 0:
+    paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    if not paths:
         return None
-    ticks = torch.zeros(rounds, 2, dtype=torch.int64, device="cuda")
-    stream = torch.cuda.current_stream().cuda_stream
-    for _ in range(3 * launches_per_round):
+    samples, stop = [], [False]
+
+    def poll():
+        while not stop[0]:
+            best = None
+            for path in paths:   # (one GPU per box; with several cards, the busiest one is the one under test)
+                try:
+                    m = re.search(r"(\d+)\s*Mhz\s*\*", open(path).read(), re.I)
+                except OSError:
+                    m = None
+                if m:
+                    best = max(best or 0, int(m.group(1)))
+            if best is not None:
+                samples.append(best)
+            time.sleep(0.01)
+
+    for _ in range(5):
         fn()
-    for r in range(rounds):
-        for _ in range(launches_per_round):
-            fn()
-        rc = lib.mi355_clock_probe(ticks[r].data_ptr(), window_us, stream)
-        assert rc == 0, rc
     torch.cuda.synchronize()
-    t = ticks.cpu()
-    c, r = int(t[:, 0].sum()), int(t[:, 1].sum())
-    return round(c / r * wall_khz / 1e3, 1) if r > 0 else None
+    th = threading.Thread(target=poll)
+    th.start()
+    t0 = time.perf_counter()
+    done = torch.cuda.Event()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            fn()
+        done.record()
+        done.synchronize()
+    stop[0] = True
+    th.join()
+    torch.cuda.synchronize()
+    tail = sorted(samples[len(samples) // 4:])
+    return float(tail[len(tail) // 2]) if tail else None
 
 
 def _median_of_3(fn):
@@ -175,6 +199,146 @@ def cpu_baseline_gemm(budget_s=20.0):
     return base
 
 
+def secondary_workloads(lib, dev, n):
+    """name -> builder of the other workloads of the path.  A builder allocates its inputs (synthetic, on the
+    distributions the configurations state) and returns (launch function, algorithmic flop or bytes per
+    launch, "flops" | "bytes", {"peak": ..., "data": ..., "clock": bool}, launches to time)."""
+    import torch
+
+    import triton_amd
+    from triton_amd import _lib
+
+    stream = torch.cuda.current_stream().cuda_stream
+    flops = 2.0 * n ** 3
+    W = {}
+
+    # config 4: N(0, 1) scaled to a per-tensor amax of 448, clamped, cast to e4m3fn; the fp32 scales that undo
+    # it go to the epilogue; K-major B, bf16 out
+    def quantize_e4m3(x):
+        scale = (x.abs().amax() / 448.0).float().reshape(1)
+        return (x / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn), scale
+
+    def fp8_gemm():
+        a8, sa8 = quantize_e4m3(torch.randn(n, n, device=dev))
+        b8, sb8 = quantize_e4m3(torch.randn(n, n, device=dev))
+        fn = lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sa8, b_scale=sb8)
+        return fn, flops, "flops", {"peak": "fp8", "clock": True, "data": "N(0,1) scaled to amax 448, e4m3fn, per-tensor fp32 scales"}, 60
+    W["fp8_e4m3_gemm_8192"] = fp8_gemm
+
+    def fp8_decode():
+        b8, _ = quantize_e4m3(torch.randn(n, n, device=dev))
+        a16, _ = quantize_e4m3(torch.randn(16, n, device=dev))
+        c16 = torch.empty(16, n, device=dev, dtype=torch.bfloat16)
+
+        def fn():  # straight through the C ABI: at ~20 us per launch the Python wrapper would dominate
+            rc = lib.mi355_gemm(a16.data_ptr(), b8.data_ptr(), c16.data_ptr(), 16, n, n, n, 1, 1, n, n, 1,
+                                _lib.F8E4M3, _lib.BF16, None, None, 0, stream)
+            assert rc == 0, rc
+
+        return fn, n * n + 16 * n + 2 * 16 * n, "bytes", {}, 50
+    W["fp8_decode_m16"] = fp8_decode
+
+    # 16-bit skinny shapes of the reference's regression table (test_performance.py:36-44): fp16, row-major B
+    def skinny(sm, sn, sk):
+        def build():
+            xa = torch.randn(sm, sk, device=dev, dtype=torch.float16)
+            xb = torch.randn(sk, sn, device=dev, dtype=torch.float16)
+            xc = torch.empty(sm, sn, device=dev, dtype=torch.float16)
+
+            def fn():
+                rc = lib.mi355_gemm(xa.data_ptr(), xb.data_ptr(), xc.data_ptr(), sm, sn, sk, sk, 1, sn, 1, sn, 1,
+                                    _lib.F16, _lib.F16, None, None, 0, stream)
+                assert rc == 0, rc
+
+            return fn, 2 * (sm * sk + sk * sn + sm * sn), "bytes", {}, 50
+        return build
+    for (sm, sn, sk) in ((16, n, n), (64, n, n), (n, 64, n)):
+        W[f"fp16_skinny_{sm}x{sn}x{sk}"] = skinny(sm, sn, sk)
+
+    # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch; launch only, device tables prepared
+    # once (like `triton_perf_fn`, 08:217-228)
+    def grouped():
+        ga = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        gb = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        gc = [torch.empty(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
+        i64 = lambda xs: torch.tensor([x.data_ptr() for x in xs], device=dev, dtype=torch.int64)
+        d_a, d_b, d_c = i64(ga), i64(gb), i64(gc)
+        d_sz = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
+        d_ld = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
+
+        def fn(keep=(ga, gb, gc)):
+            rc = lib.mi355_grouped_gemm(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr(), d_sz.data_ptr(), d_ld.data_ptr(),
+                                        16, _lib.F16, 0, stream)
+            assert rc == 0, rc
+
+        return fn, 16 * 2.0 * 2048 ** 3, "flops", {"peak": "fp16"}, 60
+    W["grouped_gemm_16x2048"] = grouped
+
+    # config 5: fp4 codes uniform over all 16 values (every byte value), e4m3 codes uniform over the 254 finite
+    # ones (0x7F / 0xFF are NaN), e8m0 scales uniform over 2^-4 .. 2^4
+    def mx(fmt):
+        def build():
+            kb = n // 2 if fmt == "mxfp4" else n
+
+            def codes():
+                if fmt == "mxfp4":
+                    return torch.randint(0, 256, (n, kb), device=dev, dtype=torch.uint8)
+                r = torch.randint(0, 254, (n, kb), device=dev, dtype=torch.uint8)
+                return r + (r >= 127).to(torch.uint8)      # 0..126 -> 0x00..0x7E, 127..253 -> 0x80..0xFE
+
+            pa, pb = codes(), codes()
+            sa = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
+            sb = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
+            fn = lambda: triton_amd.mx_matmul(pa, sa, pb, sb, fmt)
+            return fn, flops, "flops", {"peak": fmt, "clock": True,
+                                        "data": "codes uniform over all finite values, e8m0 scales uniform over 2^-4 .. 2^4"}, 60
+        return build
+    W["mxfp4_gemm_8192"] = mx("mxfp4")
+    W["mxfp8_gemm_8192"] = mx("mxfp8")
+
+    # flash attention (config 3), flops by the reference formula (06:630-636)
+    Z, H, N, D = 4, 32, 4096, 128
+    sm_scale = D ** -0.5
+
+    def qkv():
+        return tuple(torch.empty(Z, H, N, D, device=dev, dtype=torch.bfloat16).normal_(0, 0.5) for _ in range(3))
+
+    def attn_fwd(causal):
+        def build():
+            q, k, v = qkv()
+            fn = lambda: triton_amd.attention(q, k, v, causal, sm_scale)
+            return fn, 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0), "flops", {"peak": "bf16", "clock": True}, 60
+        return build
+
+    def attn_bwd(causal):
+        def build():
+            q, k, v = (t.requires_grad_() for t in qkv())
+            o = triton_amd.attention(q, k, v, causal, sm_scale)
+            do = torch.randn_like(o)
+            # gradients returned, not accumulated into .grad (that would add three elementwise kernels)
+            fn = lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True)
+            return fn, 2.5 * 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0), "flops", {"peak": "bf16", "clock": True}, 8
+        return build
+
+    # fp8 forward (06:609-614): e5m2 inputs, V transposed in memory
+    def attn_fwd8(causal):
+        def build():
+            q, k, v = qkv()
+            q8, k8 = q.to(torch.float8_e5m2), k.to(torch.float8_e5m2)
+            v8 = v.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2).to(torch.float8_e5m2)
+            fn = lambda: triton_amd.attention(q8, k8, v8, causal, sm_scale)
+            return fn, 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0), "flops", {"peak": "fp8"}, 60
+        return build
+
+    for causal in (True, False):
+        tag = "causal" if causal else "noncausal"
+        W[f"attn_fwd_{tag}"] = attn_fwd(causal)
+        W[f"attn_bwd_{tag}"] = attn_bwd(causal)
+    for causal in (True, False):
+        W[f"attn_fwd_fp8_{'causal' if causal else 'noncausal'}"] = attn_fwd8(causal)
+    return W
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -183,6 +347,9 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--size", type=int, default=8192)
+    ap.add_argument("--only", default=None,
+                    help="run just this secondary workload (a key of the 'extra' object) for --steps launches and print its "
+                         "record: the command line to put under rocprofv3 for that workload's kernels")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also launch plain device copies of the A matrix (a kernel of known traffic, for scaling PMC byte counters)")
     args = ap.parse_args()
@@ -200,6 +367,16 @@ def main():
     dev = torch.device("cuda", 0)
     torch.manual_seed(0)
     n = args.size
+    if args.only:
+        table = secondary_workloads(lib, dev, n)
+        if args.only not in table:
+            print("bench.py: --only takes one of " + ", ".join(table), file=sys.stderr)
+            sys.exit(2)
+        fn, work, kind, info, _ = table[args.only]()
+        wall_ms, ev_ms, _ = time_launches(fn, args.steps, args.warmup)
+        print(json.dumps({"workload": args.only, "steps": args.steps, "ms_per_launch": round(ev_ms, 5),
+                          ("tflops" if kind == "flops" else "gbps"): round(work / ev_ms / (1e9 if kind == "flops" else 1e6), 1)}))
+        return
     a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
     b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
     c = torch.empty(n, n, device=dev, dtype=torch.bfloat16)
@@ -231,7 +408,7 @@ def main():
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
                    "nominal_clock_khz": lib.mi355_query(_lib.Q_CLOCK_KHZ),
-                   "observed_sclk_mhz_during_headline_gemm": observed_clock_mhz(lib, step)},
+                   "observed_sclk_mhz_during_headline_gemm": observed_clock_mhz(step)},
     }
     out["roofline"]["traffic_source"] = TRAFFIC_SOURCE
 
@@ -243,113 +420,20 @@ def main():
         med, p20, p80 = testing.do_bench(step, warmup=25, rep=100, quantiles=[0.5, 0.2, 0.8])
         extra["bf16_gemm_do_bench"] = {"ms_median": round(med, 4), "ms_p20": round(p20, 4), "ms_p80": round(p80, 4),
                                        "tflops_median": round(testing.matmul_tflops(n, n, n, med), 1)}
-        # fp8 e4m3 GEMM, K-major B, per-tensor scales, bf16 out (config 4) and its decode shape
-        # operands as config 4 states them: N(0, 1) scaled to a per-tensor amax of 448, clamped, cast; the scales
-        # that undo it go to the epilogue
-        def quantize_e4m3(x):
-            scale = (x.abs().amax() / 448.0).float().reshape(1)
-            return (x / scale).clamp(-448.0, 448.0).to(torch.float8_e4m3fn), scale
-
-        a8, sa8 = quantize_e4m3(torch.randn(n, n, device=dev))
-        b8, sb8 = quantize_e4m3(torch.randn(n, n, device=dev))
-        fp8_fn = lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sa8, b_scale=sb8)
-        ms = quick(fp8_fn)
-        extra["fp8_e4m3_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK["fp8"], 4),
-                                       "sclk_mhz": observed_clock_mhz(lib, fp8_fn), "data": "N(0,1) scaled to amax 448, e4m3fn, per-tensor fp32 scales"}
-        a16, _ = quantize_e4m3(torch.randn(16, n, device=dev))
-        c16 = torch.empty(16, n, device=dev, dtype=torch.bfloat16)
-
-        def decode():  # straight through the C ABI: at ~20 us per launch the Python wrapper would dominate
-            rc = lib.mi355_gemm(a16.data_ptr(), b8.data_ptr(), c16.data_ptr(), 16, n, n, n, 1, 1, n, n, 1,
-                                _lib.F8E4M3, _lib.BF16, None, None, 0, stream)
-            assert rc == 0, rc
-
-        ms = quick(decode, iters=50, warmup=5)
-        byts = n * n + 16 * n + 2 * 16 * n
-        extra["fp8_decode_m16"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1), "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
-        del a8, a16
-        # 16-bit skinny shapes of the reference's regression table (test_performance.py:36-44): fp16, row-major B
-        for (sm, sn, sk) in ((16, n, n), (64, n, n), (n, 64, n)):
-            xa = torch.randn(sm, sk, device=dev, dtype=torch.float16)
-            xb = torch.randn(sk, sn, device=dev, dtype=torch.float16)
-            xc = torch.empty(sm, sn, device=dev, dtype=torch.float16)
-
-            def skinny():
-                rc = lib.mi355_gemm(xa.data_ptr(), xb.data_ptr(), xc.data_ptr(), sm, sn, sk, sk, 1, sn, 1, sn, 1,
-                                    _lib.F16, _lib.F16, None, None, 0, stream)
-                assert rc == 0, rc
-
-            ms = quick(skinny, iters=50, warmup=5)
-            byts = 2 * (sm * sk + sk * sn + sm * sn)
-            extra[f"fp16_skinny_{sm}x{sn}x{sk}"] = {"us": round(ms * 1e3, 2), "gbps": round(byts / ms / 1e6, 1),
-                                                    "frac_of_hbm": round(byts / ms / 1e6 / HBM_GBPS, 4)}
-            del xa, xb, xc
-        # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch
-        ga = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
-        gb = [torch.randn(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
-        gc = [torch.empty(2048, 2048, device=dev, dtype=torch.float16) for _ in range(16)]
-        # launch only, device tables prepared once (like `triton_perf_fn`, 08:217-228)
-        i64 = lambda xs: torch.tensor([x.data_ptr() for x in xs], device=dev, dtype=torch.int64)
-        d_a, d_b, d_c = i64(ga), i64(gb), i64(gc)
-        d_sz = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
-        d_ld = torch.tensor([2048] * 48, device=dev, dtype=torch.int32)
-
-        def grouped():
-            rc = lib.mi355_grouped_gemm(d_a.data_ptr(), d_b.data_ptr(), d_c.data_ptr(), d_sz.data_ptr(), d_ld.data_ptr(),
-                                        16, _lib.F16, 0, stream)
-            assert rc == 0, rc
-
-        ms = quick(grouped)
-        gfl = 16 * 2.0 * 2048 ** 3
-        extra["grouped_gemm_16x2048"] = {"ms": round(ms, 4), "tflops": round(gfl / ms / 1e9, 1), "frac_of_peak": round(gfl / ms / 1e9 / PEAK["fp16"], 4)}
-        del gc
-        del ga, gb
-        # MX GEMMs (config 5)
-        for fmt, kb in (("mxfp4", n // 2), ("mxfp8", n)):
-            # config 5: fp4 codes uniform over all 16 values (every byte value), e4m3 codes uniform over the 254
-            # finite ones (0x7F / 0xFF are NaN), scales uniform over 2^-4 .. 2^4
-            def codes():
-                if fmt == "mxfp4":
-                    return torch.randint(0, 256, (n, kb), device=dev, dtype=torch.uint8)
-                r = torch.randint(0, 254, (n, kb), device=dev, dtype=torch.uint8)
-                return r + (r >= 127).to(torch.uint8)      # 0..126 -> 0x00..0x7E, 127..253 -> 0x80..0xFE
-
-            pa, pb = codes(), codes()
-            sa = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
-            sb = torch.randint(123, 132, (n, n // 32), device=dev, dtype=torch.uint8)
-            mx_fn = lambda: triton_amd.mx_matmul(pa, sa, pb, sb, fmt)
-            ms = quick(mx_fn)
-            extra[f"{fmt}_gemm_8192"] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_of_peak": round(flops / ms / 1e9 / PEAK[fmt], 4),
-                                         "sclk_mhz": observed_clock_mhz(lib, mx_fn),
-                                         "data": "codes uniform over all finite values, e8m0 scales uniform over 2^-4 .. 2^4"}
-        del b8
-        # flash attention (config 3), flops by the reference formula (06:630-636)
-        Z, H, N, D = 4, 32, 4096, 128
-        q = torch.empty(Z, H, N, D, device=dev, dtype=torch.bfloat16).normal_(0, 0.5).requires_grad_()
-        k = torch.empty_like(q).normal_(0, 0.5).requires_grad_()
-        v = torch.empty_like(q).normal_(0, 0.5).requires_grad_()
-        sm = D ** -0.5
-        for causal in (True, False):
-            fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
-            qd, kd, vd = q.detach(), k.detach(), v.detach()
-            fwd_fn = lambda: triton_amd.attention(qd, kd, vd, causal, sm)
-            ms = quick(fwd_fn)
-            tag = "causal" if causal else "noncausal"
-            extra[f"attn_fwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["bf16"], 4),
-                                        "sclk_mhz": observed_clock_mhz(lib, fwd_fn)}
-            o = triton_amd.attention(q, k, v, causal, sm)
-            do = torch.randn_like(o)
-            # gradients returned, not accumulated into .grad (that would add three elementwise kernels)
-            ms = quick(lambda: torch.autograd.grad(o, (q, k, v), do, retain_graph=True), iters=5)
-            extra[f"attn_bwd_{tag}"] = {"ms": round(ms, 4), "tflops": round(2.5 * fl / ms / 1e9, 1), "frac_of_peak": round(2.5 * fl / ms / 1e9 / PEAK["bf16"], 4)}
-        # fp8 forward (06:609-614): e5m2 inputs, V transposed in memory
-        q8, k8 = q.detach().to(torch.float8_e5m2), k.detach().to(torch.float8_e5m2)
-        v8 = v.detach().permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2).to(torch.float8_e5m2)
-        for causal in (True, False):
-            fl = 4.0 * Z * H * N * N * D * (0.5 if causal else 1.0)
-            ms = quick(lambda: triton_amd.attention(q8, k8, v8, causal, sm))
-            tag = "causal" if causal else "noncausal"
-            extra[f"attn_fwd_fp8_{tag}"] = {"ms": round(ms, 4), "tflops": round(fl / ms / 1e9, 1), "frac_of_peak": round(fl / ms / 1e9 / PEAK["fp8"], 4)}
+        del a, b, c
+        for name, build in secondary_workloads(lib, dev, n).items():
+            fn, work, kind, info, iters = build()
+            ms = quick(fn, iters=iters, warmup=max(5, iters // 3))
+            if kind == "flops":
+                rec = {"ms": round(ms, 4), "tflops": round(work / ms / 1e9, 1), "frac_of_peak": round(work / ms / 1e9 / PEAK[info["peak"]], 4)}
+                if info.get("clock"):
+                    rec["sclk_mhz"] = observed_clock_mhz(fn)
+            else:
+                rec = {"us": round(ms * 1e3, 2), "gbps": round(work / ms / 1e6, 1), "frac_of_hbm": round(work / ms / 1e6 / HBM_GBPS, 4)}
+            if info.get("data"):
+                rec["data"] = info["data"]
+            extra[name] = rec
+            del fn
         out["extra"] = extra
 
     if not args.no_cpu:
