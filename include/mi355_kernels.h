@@ -231,7 +231,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
  *   python/tutorials/06-fused-attention.py:98-187 (kernel), :25-75 (inner loop), :441-475 (host).
  * q,k,v,o are [Z,H,N_CTX,D] with the four element strides given per tensor (last stride must be 1);
  * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {64, 128, 256}
- * (the backward entries take 64 and 128 only and return MI355_ESHAPE for 256).
+ * (forward and backward entries alike).
  * fp8 forward (dtype MI355_F8E5M2 as in the reference's fp8 benchmark, :609-614, or MI355_F8E4M3):
  * q, k and o as above, v transposed in memory (stride 1 along N_CTX, a multiple of 16 along D:
  * what `v.permute(0,1,3,2).contiguous().permute(0,1,3,2)` yields); P is rounded to the fp8 type
@@ -256,7 +256,9 @@ int mi355_attn_bwd_preprocess(const void* o, const void* d_o, float* delta,
  * Flash-attention backward: dq, dk, dv from q, k, v, do, Mlse (from the forward) and delta.
  * Stands in for the launch of `_attn_bwd` by `_attention.backward`
  *   python/tutorials/06-fused-attention.py:308-435 (kernel), :208-305 (inner loops), :478-517 (host).
- * All of q,k,v,do,dq,dk,dv share one stride set (HOST array of 4, last = 1), as in the reference (:481).
+ * All of q,k,v,do,dq,dk,dv share one stride set (HOST array of 4, last = 1), as in the reference (:481):
+ * only that one array is passed and validated, every tensor is addressed with it and must be 16-byte aligned;
+ * a caller whose tensors differ in strides must make them alike first (the reference asserts it, :481).
  * k is the ORIGINAL key tensor: the pre-scaling `k * (sm_scale / ln 2)` the reference does on the
  * host (:490-492) is folded into the kernel.  causal = 0 gives the full (non-causal) backward,
  * which the reference kernel cannot produce.  N_CTX must be a multiple of 128 (:494).

@@ -152,13 +152,15 @@ def test_full_size_config3_sampled_heads(gpu, causal):
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("causal", [True, False])
-def test_head_dim_256_forward(gpu, dtype, causal):
-    # the reference accepts HEAD_DIM 256 (06:447); here it exists for the forward (and its M) only:
-    # 512-byte K/V rows, 64 KiB LDS stages, one wave per SIMD.  The backward reports the shape.
-    shape = (1, 2, 384, 256)
+@pytest.mark.parametrize("shape", [(1, 2, 384, 256), (2, 1, 128, 256)])
+def test_head_dim_256_forward_and_backward(gpu, dtype, causal, shape):
+    # the reference accepts HEAD_DIM 256 (06:447) and its backward is generic in it (06:308-435).  Forward:
+    # 512-byte K/V rows, 64 KiB LDS stages, one wave per SIMD; backward: the dQ kernel at this width, and a
+    # dK/dV kernel whose programs own half of the output columns each.  M through the C ABI, then the
+    # outputs and all three gradients against the tile oracle and the closed form.
     (q, k, v, do), (tq, tk, tv, tdo) = _inputs(7, shape, dtype, gpu)
     sm_scale = 256 ** -0.5
-    cf = A.attn_closed_form(q, k, v, causal, sm_scale)
+    cf = A.attn_closed_form(q, k, v, causal, sm_scale, do)
     from triton_amd import _lib
     o = torch.empty_like(tq)
     M = torch.empty(shape[:3], dtype=torch.float32, device=gpu)
@@ -172,11 +174,11 @@ def test_head_dim_256_forward(gpu, dtype, causal):
     assert np.allclose(to_np(M), cf["M"], atol=2e-3, rtol=0)
     if causal:
         assert np.allclose(to_np(o)[:, :, 0], v[:, :, 0], atol=1e-3)   # the first query sees only the first key
-    tq.requires_grad_()
-    out = triton_amd.attention(tq, tk, tv, causal, sm_scale)
-    assert np.allclose(to_np(out.detach()), cf["o"], atol=1e-2, rtol=1e-2)
-    with pytest.raises(ValueError):
-        out.backward(tdo)
+    go, gdq, gdk, gdv = _fwd_bwd(tq, tk, tv, tdo, causal, sm_scale)
+    ro, rM = A.attn_fwd_tiled(q, k, v, causal, sm_scale, dtype)
+    rdq, rdk, rdv, _ = A.attn_bwd_tiled(q, k, v, ro, do, rM, sm_scale, causal, dtype)
+    _check_against_tiled_and_closed_form(f"{shape} causal={causal}", dict(o=go, dq=gdq, dk=gdk, dv=gdv),
+                                         dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])

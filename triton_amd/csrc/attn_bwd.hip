@@ -1,4 +1,4 @@
-// Flash-attention backward for gfx950 (fp16 / bf16, head_dim 64 or 128): delta = rowsum(O*dO),
+// Flash-attention backward for gfx950 (fp16 / bf16, head_dim 64, 128 or 256): delta = rowsum(O*dO),
 // then dK/dV with the K/V tile stationary and dQ with the Q tile stationary - the same
 // atomics-free split as the reference (`_attn_bwd_preprocess`, `_attn_bwd_dkdv`, `_attn_bwd_dq`,
 // python/tutorials/06-fused-attention.py:190-204, :208-257, :261-305, driver :308-435), as
@@ -271,7 +271,8 @@ int attn_bwd_dkdv_launch(const AttnArgs& p, bool bf16, hipStream_t stream);  // 
 
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
   int rc;
-  if (bf16) rc = p.D == 128 ? launch_bwd_d<bf16x8, 128>(p, stream) : launch_bwd_d<bf16x8, 64>(p, stream);
+  if (p.D == 256) rc = bf16 ? launch_bwd_d<bf16x8, 256>(p, stream) : launch_bwd_d<f16x8, 256>(p, stream);
+  else if (bf16) rc = p.D == 128 ? launch_bwd_d<bf16x8, 128>(p, stream) : launch_bwd_d<bf16x8, 64>(p, stream);
   else rc = p.D == 128 ? launch_bwd_d<f16x8, 128>(p, stream) : launch_bwd_d<f16x8, 64>(p, stream);
   if (rc) return rc;
   return attn_bwd_dkdv_launch(p, bf16, stream);
@@ -279,7 +280,11 @@ int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
 
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
   dim3 grid, block(256);
-  if (p.D == 128) {
+  if (p.D == 256) {
+    grid = dim3((p.N + 7) / 8, p.Z * p.H);
+    if (bf16) attn_bwd_pre_kernel<bf16x8, 256><<<grid, block, 0, stream>>>(p);
+    else attn_bwd_pre_kernel<f16x8, 256><<<grid, block, 0, stream>>>(p);
+  } else if (p.D == 128) {
     grid = dim3((p.N + 15) / 16, p.Z * p.H);
     if (bf16) attn_bwd_pre_kernel<bf16x8, 128><<<grid, block, 0, stream>>>(p);
     else attn_bwd_pre_kernel<f16x8, 128><<<grid, block, 0, stream>>>(p);

@@ -324,6 +324,201 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   }
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// dK/dV for head_dim 256.  K, V fragments (128 registers) plus both accumulators (256 more at this
+// width) do not fit one wave, so a workgroup owns 128 key rows and HALF of the output columns:
+// program 2 i + h computes dK[:, 128 h .. 128 h + 127] and dV[:, same] of key block i.  S and dP
+// need the whole head dimension and are computed by both programs (6 products' worth of MFMAs
+// for the 4 that count per output half - the price of keeping every accumulator in registers
+// and of needing no workspace and no atomics).  Plain structure, two LDS stages of a Q and a dO
+// tile (64 rows x 512 bytes each), one barrier per stage: this width is about coverage of the
+// reference surface (python/tutorials/06-fused-attention.py:447 admits HEAD_DIM 256), not speed.
+// ---------------------------------------------------------------------------------------------
+template <typename V8, int D, int NW>
+__global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_split_kernel(AttnArgs p) {
+  using S = typename ElemB<V8>::type;
+  typedef __attribute__((ext_vector_type(4))) S S4;
+  constexpr int BN = NW * 32, BM = 64, RB = D * 2, KSQ = D / 16, DH = D / 2, DT = DH / 32;
+  using Tile = AttnTile<RB, BM, NW>;
+  constexpr int TILE = Tile::BYTES;
+
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  LDS_PTR(char) const lds = (LDS_PTR(char))smem;  // [stage][Q tile | dO tile]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q4 = lane >> 4;
+
+  const int nkb = (p.N + BN - 1) / BN;
+  const int dhalf = blockIdx.x & 1;
+  const int pid = blockIdx.x >> 1;
+  const int hz = pid / nkb, kbk = pid % nkb;
+  const int z = hz / p.H, h = hz % p.H;
+  const int n0 = kbk * BN, nrow0 = n0 + wave * 32;
+  const int ncol = nrow0 + l32;   // this lane's key row
+
+  const int64_t head_off = ((int64_t)z * p.sq[0] + (int64_t)h * p.sq[1]) * 2;
+  const int64_t pitch = p.sq[2] * 2;
+  const char* qbase = p.q + head_off;
+  const char* dobase = p.d_o + head_off;
+  const float* lse = p.lse + (int64_t)hz * p.N;
+  const float* delta = p.delta + (int64_t)hz * p.N;
+
+  V8 kf[KSQ], vf[KSQ];
+  {
+    const int r = min(ncol, p.N - 1);
+    const char* sk = p.k + head_off + (int64_t)r * pitch + g * 16;
+    const char* sv = p.v + head_off + (int64_t)r * pitch + g * 16;
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) {
+      kf[ks] = *(const V8*)(sk + ks * 32);
+      vf[ks] = *(const V8*)(sv + ks * 32);
+    }
+  }
+
+  const int m_begin = p.causal ? (n0 / BM) * BM : 0;
+  const int nsteps = (p.N - m_begin + BM - 1) / BM;
+
+  unsigned offQD[Tile::INST];
+#pragma unroll
+  for (int i = 0; i < Tile::INST; i++) offQD[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+  const unsigned lds_base = lds_addr(lds);
+  auto issue = [&](int j, int stage) {
+    const unsigned qd = lds_base + stage * (2 * TILE), dd = qd + TILE;
+    const char* qsrc = qbase + (int64_t)(m_begin + j * BM) * pitch;
+    const char* dsrc = dobase + (int64_t)(m_begin + j * BM) * pitch;
+#pragma unroll
+    for (int i = 0; i < Tile::INST; i++) {
+      async_copy16_sbase(qsrc, offQD[i], qd + (i * NW + wave) * 1024);
+      async_copy16_sbase(dsrc, offQD[i], dd + (i * NW + wave) * 1024);
+    }
+  };
+
+  const RowRead<RB> rr(l32, g);
+  TrRead<RB> tt(i16, q4);
+  tt.tl ^= (unsigned)dhalf << 8;   // column blocks 4 h .. 4 h + 3: 256 bytes further, and the swizzle XOR leaves bit 8 alone
+
+  f32x16 dk[DT], dv[DT];
+#pragma unroll
+  for (int c = 0; c < DT; c++)
+#pragma unroll
+    for (int r = 0; r < 16; r++) { dk[c][r] = 0.f; dv[c][r] = 0.f; }
+
+  const float qk_scale = p.sm_scale * 1.4426950408889634f;
+
+  issue(0, 0);
+  wait_all();
+  __syncthreads();
+
+  for (int j = 0; j < nsteps; j++) {
+    const int stage = j & 1;
+    if (j + 1 < nsteps) issue(j + 1, stage ^ 1);
+    const unsigned qb = lds_base + stage * (2 * TILE), db = qb + TILE;
+    const int ms = m_begin + j * BM;
+    static_for<2>([&](auto A_) {
+      constexpr int a = decltype(A_)::value;
+      const int mt0 = ms + a * 32;   // first query row of this 32-row tile
+      // under the causal mask a tile whose rows all lie above this wave's key rows contributes nothing
+      if (!p.causal || mt0 + 31 >= nrow0) {
+        f32x16 s, dp;
+#pragma unroll
+        for (int r = 0; r < 16; r++) { s[r] = 0.f; dp[r] = 0.f; }
+        i32x4 qf[2], df[2];
+        qf[0] = lds_read_b128<a * 32 * RB>(rr.template addr<0>(qb));
+        df[0] = lds_read_b128<a * 32 * RB>(rr.template addr<0>(db));
+        static_for<KSQ>([&](auto KS_) {
+          constexpr int ks = decltype(KS_)::value;
+          constexpr int cur = ks & 1, nxt = cur ^ 1;
+          if constexpr (ks + 1 < KSQ) {
+            qf[nxt] = lds_read_b128<a * 32 * RB>(rr.template addr<ks + 1>(qb));
+            df[nxt] = lds_read_b128<a * 32 * RB>(rr.template addr<ks + 1>(db));
+            lds_wait<2>();
+          } else {
+            lds_wait<0>();
+          }
+          lds_use(qf[cur]);
+          lds_use(df[cur]);
+          s = mfma32(__builtin_bit_cast(V8, qf[cur]), kf[ks], s);      // S[q][key] = Q K^T
+          dp = mfma32(__builtin_bit_cast(V8, df[cur]), vf[ks], dp);    // dP[q][key] = dO V^T
+        });
+        V8 pf[2], dsf[2];
+        const bool masked = p.causal && mt0 < nrow0 + 32;
+#pragma unroll
+        for (int rg = 0; rg < 4; rg++) {
+          const int mrow = min(mt0 + rg * 8 + g * 4, p.N - 4);
+          const f32x4 mv = *(const f32x4*)(lse + mrow);
+          const f32x4 dl = *(const f32x4*)(delta + mrow);
+#pragma unroll
+          for (int e = 0; e < 4; e++) {
+            const int r = rg * 4 + e;
+            float pv = fast_exp2(fmaf(s[r], qk_scale, -mv[e]));
+            if (masked && mt0 + rg * 8 + g * 4 + e < ncol) pv = 0.f;
+            const float dsv = pv * (dp[r] - dl[e]);
+            pf[r >> 3][r & 7] = (S)pv;
+            dsf[r >> 3][r & 7] = (S)dsv;
+          }
+        }
+        // dV^T += dO^T p and dK^T += Q^T ds over the two k-steps of 16 query rows
+        static_for<2>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          static_for<DT>([&](auto C_) {
+            constexpr int c = decltype(C_)::value;
+            constexpr int imm0 = (a * 32 + 16 * t) * RB, imm1 = (a * 32 + 16 * t + 8) * RB;
+            i32x2 q0 = lds_read_tr16_b64<imm0>(tt.template addr<c, 0>(qb));
+            i32x2 q1 = lds_read_tr16_b64<imm1>(tt.template addr<c, 1>(qb));
+            i32x2 d0 = lds_read_tr16_b64<imm0>(tt.template addr<c, 0>(db));
+            i32x2 d1 = lds_read_tr16_b64<imm1>(tt.template addr<c, 1>(db));
+            lds_wait<0>();
+            lds_use(q0); lds_use(q1); lds_use(d0); lds_use(d1);
+            const i32x4 qt = __builtin_shufflevector(q0, q1, 0, 1, 2, 3);
+            const i32x4 dt = __builtin_shufflevector(d0, d1, 0, 1, 2, 3);
+            dv[c] = mfma32(__builtin_bit_cast(V8, dt), pf[t], dv[c]);
+            dk[c] = mfma32(__builtin_bit_cast(V8, qt), dsf[t], dk[c]);
+          });
+        });
+      }
+    });
+    wait_all();
+    __syncthreads();
+  }
+
+  if (ncol < p.N) {
+    char* dkd = p.dk + head_off + (int64_t)ncol * pitch;
+    char* dvd = p.dv + head_off + (int64_t)ncol * pitch;
+#pragma unroll
+    for (int c = 0; c < DT; c++)
+#pragma unroll
+      for (int rg = 0; rg < 4; rg++) {
+        const int d = dhalf * DH + c * 32 + rg * 8 + g * 4;
+        S4 a, b;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          a[e] = (S)(dk[c][rg * 4 + e] * p.sm_scale);
+          b[e] = (S)dv[c][rg * 4 + e];
+        }
+        *(S4*)(dkd + d * 2) = a;
+        *(S4*)(dvd + d * 2) = b;
+      }
+  }
+}
+
+template <typename V8>
+static int launch_dkdv_256(const AttnArgs& p, hipStream_t stream) {
+  constexpr int NW = 4, BN = NW * 32, D = 256;
+  constexpr int smem = 2 * 2 * 64 * D * 2;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_split_kernel<V8, D, NW>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int nkb = (p.N + BN - 1) / BN;
+  attn_bwd_dkdv_split_kernel<V8, D, NW><<<dim3(2 * nkb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
 template <typename V8, int D>
 static int launch_dkdv(const AttnArgs& p, hipStream_t stream) {
   constexpr int NW = 4, BN = NW * 32;
@@ -341,6 +536,7 @@ static int launch_dkdv(const AttnArgs& p, hipStream_t stream) {
 }
 
 int attn_bwd_dkdv_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
+  if (p.D == 256) return bf16 ? launch_dkdv_256<bf16x8>(p, stream) : launch_dkdv_256<f16x8>(p, stream);
   if (bf16) return p.D == 128 ? launch_dkdv<bf16x8, 128>(p, stream) : launch_dkdv<bf16x8, 64>(p, stream);
   return p.D == 128 ? launch_dkdv<f16x8, 128>(p, stream) : launch_dkdv<f16x8, 64>(p, stream);
 }

@@ -390,8 +390,7 @@ int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* st
 static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype, bool allow_256 = false) {
   if (Z <= 0 || H <= 0 || N_CTX <= 0) return MI355_EINVAL;
   if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
-  // head_dim 256 exists for the 16-bit forward only (the backward kernels keep K, V and both
-  // accumulators of a key block in registers, which 256 columns do not fit)
+  // head_dim 256: 16-bit forward and backward (not the fp8 forward)
   if (D != 64 && D != 128 && !(allow_256 && D == 256)) return MI355_ESHAPE;
   if (N_CTX % 128 != 0) return MI355_ESHAPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
@@ -448,7 +447,7 @@ int mi355_attn_bwd_preprocess(const void* o, const void* d_o, float* delta,
                               int Z, int H, int N_CTX, int D, const int64_t* stride, int dtype, void* stream_) {
   if (!o || !d_o || !delta) return MI355_EINVAL;
   AttnArgs p{};
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
   if (rc) return rc;
   if (!copy_strides(stride, p.so)) return MI355_EINVAL;
   if (!attn_stride_ok(p.so, o, D) || !aligned(d_o, 16)) return MI355_ESTRIDE;
@@ -464,7 +463,7 @@ int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
                    float sm_scale, int causal, int dtype, void* stream_) {
   if (!q || !k || !v || !d_o || !Mlse || !delta || !dq || !dk || !dv) return MI355_EINVAL;
   AttnArgs p{};
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
   if (rc) return rc;
   if (!copy_strides(stride, p.sq)) return MI355_EINVAL;
   if (!attn_stride_ok(p.sq, q, D) || !aligned(k, 16) || !aligned(v, 16) || !aligned(d_o, 16) ||

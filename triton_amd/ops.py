@@ -377,7 +377,7 @@ class _attention(torch.autograd.Function):
 def attention(q, k, v, causal, sm_scale):
     """`attention(q, k, v, causal, sm_scale)` of the reference (06:520, `_attention.apply`).
 
-    Head dims 64 and 128 run the kernels directly (256: forward only).  The reference also admits 16
+    Head dims 64, 128 and 256 run the kernels directly, forward and backward.  The reference also admits 16
     and 32 (06:447): for those q, k and v are zero-padded to 64 columns - the scores, the softmax and
     the first HEAD_DIM columns of every output and gradient are unchanged by zero columns - and the
     result is sliced back; autograd carries the gradients through the padding."""
