@@ -152,3 +152,29 @@ def test_four_wave_kernels_deal_tiles_in_ragged_rounds(gpu, monkeypatch, fmt, pr
             sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
         ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
         assert bits_equal(_run(gpu, a, sa, b, sb, fmt, torch.float32), ref32), (fmt, programs, M, N, K)
+
+
+def test_mxfp8_with_freshly_uploaded_operands_is_bit_exact_every_time(gpu, monkeypatch):
+    # Regression: a tile base that the compiler had spilled was restored by a VALU instruction right in front of an
+    # inline-assembly load of the four-wave MXFP8 kernel's prologue, which then - in a few per cent of launches, and
+    # only with cold caches - fetched eight rows of A from a stale address.  Fresh uploads before every launch (cold
+    # operands, as in the other tests' helper) and exact sums: every launch must give the bits of the oracle.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", "5")
+    rng = np.random.default_rng(65)
+    M, N, K = 1280, 256, 2048
+    vals = np.array([0x00, 0x30, 0x38, 0x3C, 0x40, 0xB0, 0xB8, 0xC0], dtype=np.uint8)  # 0, .5, 1, 1.5, 2, -.5, -1, -2
+    cases = []
+    for _ in range(3):
+        a = vals[rng.integers(0, len(vals), size=(M, K))]
+        b = vals[rng.integers(0, len(vals), size=(N, K))]
+        sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+        sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        cases.append((a, sa, b, sb, mx.mx_matmul(a, sa, b, sb, "mxfp8", out_dtype="fp32")))
+    churn = []
+    for rep in range(60):
+        a, sa, b, sb, ref = cases[rep % 3]
+        churn.append(torch.empty(int(rng.integers(1, 64)) * 4096, device=gpu, dtype=torch.uint8))   # moves the upload addresses around
+        if len(churn) > 8:
+            churn.pop(0)
+        assert bits_equal(_run(gpu, a, sa, b, sb, "mxfp8", torch.float32), ref), rep

@@ -7,10 +7,12 @@ becomes a Python exception.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_size_t, c_char_p, c_float, c_int, c_int64, c_void_p, POINTER
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "csrc" / "libmi355_kernels.so"
+# MI355_KERNELS_LIB: another build of the same library (a variant under test); default: the in-tree build
+LIB_PATH = Path(os.environ.get("MI355_KERNELS_LIB") or Path(__file__).resolve().parent / "csrc" / "libmi355_kernels.so")
 
 # enums of include/mi355_kernels.h
 F16, BF16, F8E4M3, F8E5M2, F32 = 0, 1, 2, 3, 4

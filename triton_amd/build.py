@@ -22,6 +22,10 @@ HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument", "-Wno-ignored-attributes",
+    # keeps the device assembly (<stem>-hip-amdgcn-amd-amdhsa-gfx950.s) next to the object files: the kernels issue
+    # MFMAs, LDS reads and direct global->LDS loads as inline assembly, which the compiler's hazard recogniser cannot
+    # see into, so tests/test_isa_hazards.py checks the generated code of every kernel instead
+    "-save-temps=obj",
 ]
 
 # Per-file additions.  The attention kernels rescale their MFMA accumulators with VALU code every
@@ -31,10 +35,6 @@ HIPCC_FLAGS = [
 EXTRA_FLAGS = {
     "attn_fwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
     "attn_bwd.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
-    # keeps the device assembly next to the object file: this file issues its MFMAs as inline assembly, so the
-    # compiler inserts no wait before reads of their results, and tests/test_isa_mfma_hazard.py checks on the
-    # generated code that every such read comes late enough
-    "gemm_wave128.hip": ["-save-temps=obj"],
 }
 
 

@@ -57,11 +57,22 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds
 // and a 32-bit per-lane byte offset: the address add happens in the memory pipeline instead of
 // costing a 64-bit vector add per load.  `lds_wave_base` must be wave-uniform.  The load is
 // invisible to the compiler's wait-count bookkeeping: callers wait with wait_vmcnt<>.
+//
+// SETTLE: a vector-memory instruction must not read a scalar register within 5 issue slots of a VALU
+// instruction writing it - and that is how the compiler restores a SPILLED scalar register (v_readlane_b32),
+// possibly right in front of this statement, whose contents it cannot see.  Inside the K loops the bases are
+// produced by scalar arithmetic (checked on the generated code by tests/test_isa_hazards.py); the loads of a
+// kernel's prologue, where restored spills do occur, are issued with SETTLE = true: five idle slots first.
+template <bool SETTLE = false>
 __device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned lane_off, unsigned lds_wave_base) {
 #if MI355_DEVICE_PASS
   // one idle issue slot between the M0 write and the LDS-DMA instruction that reads it
-  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
-               :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base) : "memory");
+  if constexpr (SETTLE)
+    asm volatile("s_nop 4\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base) : "memory");
+  else
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                 :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base) : "memory");
 #endif
 }
 
@@ -69,12 +80,18 @@ __device__ __forceinline__ void async_copy16_sbase(const void* sbase, unsigned l
 // several copies can then share one M0 value.  SETM0 = false reuses the M0 of the previous copy: nothing in
 // between may write M0 (compiler-generated code does so only for indirect register indexing, message and GWS
 // instructions and its own LDS-direct loads, none of which the kernels using this have).
-template <int OFF, bool SETM0>
+template <int OFF, bool SETM0, bool SETTLE = false>
 __device__ __forceinline__ void async_copy16_sbase_off(const void* sbase, unsigned lane_off, unsigned lds_wave_base) {
 #if MI355_DEVICE_PASS
-  if constexpr (SETM0)
+  // (SETTLE: see async_copy16_sbase; the idle slots stand inside the statement, behind any restore of its inputs)
+  if constexpr (SETM0 && SETTLE)
+    asm volatile("s_nop 4\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
+                 :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base), "i"(OFF) : "memory");
+  else if constexpr (SETM0)
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1 offset:%3"
                  :: "v"(lane_off), "s"(sbase), "s"(lds_wave_base), "i"(OFF) : "memory");
+  else if constexpr (SETTLE)
+    asm volatile("s_nop 4\n\tglobal_load_lds_dwordx4 %0, %1 offset:%2" :: "v"(lane_off), "s"(sbase), "i"(OFF) : "memory");
   else
     asm volatile("global_load_lds_dwordx4 %0, %1 offset:%2" :: "v"(lane_off), "s"(sbase), "i"(OFF) : "memory");
 #endif
@@ -156,6 +173,14 @@ __device__ __forceinline__ int lds_read_b32(unsigned addr) {
   int v = 0;
 #if MI355_DEVICE_PASS
   asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int OFF>
+__device__ __forceinline__ int lds_read_u8(unsigned addr) {   // one byte, zero-extended
+  int v = 0;
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_u8 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
 #endif
   return v;
 }

@@ -1,0 +1,475 @@
+// Block-scaled (MXFP8 / MXFP4) forms of the four-wave GEMM of gemm_wave128.hip: the same skeleton - one workgroup
+// per 256x256 tile of C, four waves of 128x128 from 16x16 MFMAs, 128 bytes of every operand row per K step, two
+// 64 KiB LDS stages filled by direct global->LDS loads with fixed scalar bases - with scaled 16x16x128 f8f6f4
+// MFMAs and the e8m0 block scales travelling through a small LDS ring of their own.
+#include "gemm_wave128.h"
+
+namespace mi355 {
+
+// Scaled fp8 (e4m3) MFMA with the accumulator pinned to the accumulation registers; byte 0 of the scale dwords.
+__device__ __forceinline__ void mfma16_mxfp8(const i32x8& a, const i32x8& b, f32x4& c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+  asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0]"
+               : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+#endif
+}
+#ifndef MXFP8_CHUNK
+#define MXFP8_CHUNK(kg, c) ((kg) + 4 * (c))
+#endif
+
+// MXFP8 (e4m3 codes, one e8m0 scale per 32 elements): the fp8 kernel above with scaled MFMAs; a K step is
+// 128 elements = four scale blocks, the scales travel 16 bytes per row (four K steps) per direct load into a
+// two-slot LDS ring like those of the MXFP4 kernel below.
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int MT = 8, NT = 8, MH = MT / 2;
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
+  int pm, pn;
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
+
+  // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
+  const char* gA;
+  const char* gB;
+  const char* gSA;
+  const char* gSB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
+  };
+  set_fill_tile(pm, pn);
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+  };
+
+  // ---- scale loads: wave w fetches the 16 scale bytes (four K steps) of rows 64 w .. 64 w + 63 of A and of B
+  const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
+  auto issue_scales = [&](int g, auto SETTLE_) {   // group g of four K steps of the fill tile -> slot g & 1 (K steps come in eights)
+    const unsigned slot = lds0 + SC_BASE + (g & 1) * SC_SLOT + wave * 1024;
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)g * 16, slot);
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)g * 16, slot + BM * 16);
+  };
+  // scales of a K step: lane group kg supplies block kg of its row, fetched as one byte (ds_read_u8: it arrives in
+  // byte 0, the position the MFMA's selector names, so no shift), one read per two MFMAs
+  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + kg;
+  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + kg;
+  int sa[2][MT], sb[2][NT];
+  auto read_scale = [&](auto OP_, auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 3) * 4
+    constexpr int op = decltype(OP_)::value, set = decltype(SET_)::value, off = decltype(OFF_)::value;
+    if constexpr (op < MT) sa[set][op] = lds_read_u8<off + op * 256>(adrSA);
+    else sb[set][op - MT] = lds_read_u8<off + (op - MT) * 256>(adrSB);
+  };
+  auto pin_scales = [&](auto SET_) {
+    constexpr int set = decltype(SET_)::value;
+    static_for<MT>([&](auto T_) { lds_use(sa[set][decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(sb[set][decltype(T_)::value]); });
+  };
+
+  // ---- fragment reads.  The 8-bit forms of the scaled MFMA split a lane's 32 bytes: registers 0-3 of the lane
+  // groups 2 b, 2 b + 1 together are scale block b, registers 4-7 block 2 + b, and block b takes its scale from
+  // lane group b.  So lane (l16, kg) reads chunk kg into its low and chunk 4 + kg into its high registers and
+  // supplies the scale of block kg.
+  LDS_PTR(const char) fragA[2];
+  LDS_PTR(const char) fragB[2];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int c = 0; c < 2; c++) {
+      const unsigned slot = ((MXFP8_CHUNK(kg, c)) ^ s) * 16;
+      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * 128 + l16) * ROWB + slot;
+      fragB[c] = (LDS_PTR(const char))lds_raw + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+  }
+  auto read_frag = [&](LDS_PTR(const char) (&base)[2], int off) {
+    i32x4 lo = *(LDS_PTR(const i32x4))(base[0] + off);
+    i32x4 hi = *(LDS_PTR(const i32x4))(base[1] + off);
+    return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  };
+  i32x8 a0[MH], a1[MH], b[2][NT];
+
+  f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
+
+  // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
+  issue_scales(0, std::true_type{});
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
+  wait_vmcnt<16>();
+  block_barrier();
+  static_for<MT + NT>([&](auto OP_) { read_scale(OP_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
+  lds_wait<0>();
+  pin_scales(std::integral_constant<int, 0>{});
+#pragma unroll
+  for (int t = 0; t < NT; t++) b[0][t] = read_frag(fragB, t * 16 * ROWB);
+#pragma unroll
+  for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
+
+  // K step U (0..7 within a group of eight: stage and register sets U & 1, scale slot U >> 2); its loads fetch
+  // K step `fk` of the fill tile.
+  auto step = [&](auto U_, int fk) {
+    constexpr int U = decltype(U_)::value, P = U & 1, cur = U & 1, nxt = cur ^ 1, UN = (U + 1) & 7;
+    constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp8(b[cur][j], a0[i], acc[i][j], sb[cur][j], sa[cur][i]);
+      if constexpr (n % 4 == 0 && n / 4 < MH) a1[n / 4] = read_frag(fragA, so + (MH + n / 4) * 16 * ROWB);
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    lds_wait<0>();
+    wait_vmcnt<0>();
+    block_barrier();
+    static_for<MH * NT>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp8(b[cur][j], a1[i], acc[MH + i][j], sb[cur][j], sa[cur][MH + i]);
+      if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
+      if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
+      if constexpr (n % 2 == 0)
+        read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, nxt>{}, std::integral_constant<int, (UN >> 2) * SC_SLOT + (UN & 3) * 4>{});
+      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE, std::false_type{});
+      // (the scales of the K steps fk .. fk + 3 are requested in the third step of every four, into the slot whose
+      // last reader was the read for the step before this one)
+      if constexpr ((U & 3) == 2 && n == 16) issue_scales(fk >> 2, std::false_type{});
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    lds_wait<0>();
+    pin_scales(std::integral_constant<int, nxt>{});
+  };
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 8) {
+      static_for<8>([&](auto U_) { step(U_, fk); advance(); });
+      if (kt + 8 >= nk_last) mfma_retire();
+    }
+    mfma_drain(acc);
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
+  }
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+#endif
+}
+
+bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
+  // whole tiles, K steps in groups of eight (K a multiple of 1024), scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 1024 == 0 && p.k_bytes >= 1024 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
+         p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
+         p.lds_a * 64 + p.k_bytes / 32 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 32 < (1ll << 31);
+}
+
+int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int tiles = (p.M / 256) * (p.N / 256);
+  const int grid = wave128_grid(tiles, p.num_programs);
+  gemm_wave128_mxfp8_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
+// MXFP4 (e2m1 codes, one e8m0 scale per 32 elements of K) on the same skeleton: scaled 16x16x128
+// f8f6f4 MFMAs, two per accumulator tile and K step (128 bytes of a row = 256 elements = 8 scale
+// blocks of 16 bytes).  Lane (r, kg) of sub-step ks multiplies block 4 ks + kg of its row.  (Which K positions
+// a lane takes is free as long as A, B and the scales agree; but with the lane group in the LOW bits of the
+// chunk number the fragment reads are free of LDS bank conflicts, with 2 kg + ks - the first version - every
+// ds_read_b128 took 8 instead of 4 cycles: measured, SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE.)  The
+// scales travel like the operands: 16 bytes per row (two K steps) per direct load into a two-slot LDS ring
+// (row r at 16 r); from there each fragment's scale byte of a sub-step is fetched with one `ds_read_u8`.
+// ---------------------------------------------------------------------------------------------
+// Scaled fp4 MFMA with the accumulator pinned to the accumulation registers (see mfma16): byte SEL of the two
+// scale dwords applies; fp4 operands are four registers.
+template <int SEL>
+__device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32x4& c, int sa, int sb) {
+#if MI355_DEVICE_PASS
+  if constexpr (SEL == 0)
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                 : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+  else
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel:[1,1,0] op_sel_hi:[0,0,0] cbsz:4 blgp:4"
+                 : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
+#endif
+}
+
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  constexpr int BM = 256, BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
+  constexpr int MT = 8, NT = 8, KS = 2, NM = MT * NT, NRD = MT + NT;
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int l16 = lane & 15, kg = lane >> 4;
+
+  const int num_m = p.M / BM, num_n = p.N / BN;
+  const int ntiles = num_m * num_n;
+  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
+  int pm, pn;
+  grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+  const int nk = p.k_bytes / ROWB;
+  int nk_last = nk;   // the same number, but opaque: see mfma_retire
+  asm volatile("" : "+s"(nk_last));
+
+  // ---- operand loads, as in the 16-bit kernel
+  const unsigned drow = lane >> 3, dslot = lane & 7;
+  unsigned voffA[2], voffB[2];
+#pragma unroll
+  for (int par = 0; par < 2; par++) {
+    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
+    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
+    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  }
+  // scalar bases (operands and scales) of the tile the loads are fetching, two K steps ahead of the MFMAs
+  const char* gA;
+  const char* gB;
+  const char* gSA;
+  const char* gSB;
+  auto set_fill_tile = [&](int fm, int fn) {
+    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
+  };
+  set_fill_tile(pm, pn);
+  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
+  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+    constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
+    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
+    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
+    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+  };
+  // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of rows 64 w .. 64 w + 63 of A and of B
+  const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
+  auto issue_scales = [&](int h, auto SETTLE_) {   // pair h of K steps of the fill tile -> slot h & 1 (K steps come in fours, so
+    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT + wave * 1024;   // the slots alternate across tiles too)
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)h * 16, slot);
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)h * 16, slot + BM * 16);
+  };
+
+  // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 2 kg + ks of row l16 (+ 16 t)
+  unsigned adrA[KS], adrB[KS];
+  {
+    const unsigned s = (l16 >> 1) & 7;
+#pragma unroll
+    for (int ks = 0; ks < KS; ks++) {
+      const unsigned slot = ((4 * ks + kg) ^ s) * 16;
+      adrA[ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      adrB[ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
+    }
+  }
+  struct Frags { i32x4 a[MT]; i32x4 b[NT]; };
+  Frags f[2];
+  auto read_one = [&](auto OP_, auto P_, auto KS_, Frags& dst) {
+    constexpr int op = decltype(OP_)::value, P = decltype(P_)::value, ks = decltype(KS_)::value;
+    constexpr unsigned so = P * STAGE;
+    if constexpr (op < MT) dst.a[op] = lds_read_b128<op * 16 * ROWB>(adrA[ks] + so);
+    else dst.b[op - MT] = lds_read_b128<(op - MT) * 16 * ROWB>(adrB[ks] + so);
+  };
+  auto pin = [&](Frags& x) {
+    static_for<MT>([&](auto T_) { lds_use(x.a[decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(x.b[decltype(T_)::value]); });
+  };
+  // scales: lane (r, kg) multiplies block kg of its row in sub-step 0 and block 4 + kg in sub-step 1; each is
+  // fetched as ONE BYTE (ds_read_u8: it arrives in byte 0, the position the MFMA's selector names, so no shift)
+  // into a register set of its own - sc[0] for sub-step 0, read during the sub-step 1 before, sc[1] for
+  // sub-step 1, read during the same step's sub-step 0 -, one read per two MFMAs.
+  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + kg;
+  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + kg;
+  int sa[2][MT], sb[2][NT];
+  auto read_scale = [&](auto OP_, auto KS_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 1) * 8
+    constexpr int op = decltype(OP_)::value, ks = decltype(KS_)::value, off = decltype(OFF_)::value + 4 * ks;
+    if constexpr (op < MT) sa[ks][op] = lds_read_u8<off + op * 256>(adrSA);
+    else sb[ks][op - MT] = lds_read_u8<off + (op - MT) * 256>(adrSB);
+  };
+  auto pin_scales = [&](auto KS_) {
+    constexpr int ks = decltype(KS_)::value;
+    static_for<MT>([&](auto T_) { lds_use(sa[ks][decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(sb[ks][decltype(T_)::value]); });
+  };
+
+  f32x4 acc[MT][NT];
+  auto zero_acc = [&]() {
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < NT; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  };
+  zero_acc();
+
+  // ---- prologue
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  using T = std::true_type; using F = std::false_type;
+  issue_scales(0, std::true_type{});
+  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
+  wait_vmcnt<16>();
+  block_barrier();
+  static_for<NRD>([&](auto OP_) { read_one(OP_, I0{}, I0{}, f[0]); });
+  static_for<NRD>([&](auto OP_) { read_scale(OP_, I0{}, I0{}); });
+  lds_wait<0>();
+  pin_scales(I0{});
+
+  // K step U (0..3 within a group of four: stage U & 1, scale slot U >> 1)
+  auto step = [&](auto U_, int fk) {   // fk: the K step (of the fill tile) that this step's loads fetch
+    constexpr int U = decltype(U_)::value, P = U & 1, UN = (U + 1) & 3;
+    using OffCur = std::integral_constant<int, (U >> 1) * SC_SLOT + (U & 1) * 8>;
+    using OffNext = std::integral_constant<int, (UN >> 1) * SC_SLOT + (UN & 1) * 8>;
+    // sub-step 0 (blocks kg); meanwhile the fragments and the scales of sub-step 1
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp4<0>(f[0].b[j], f[0].a[i], acc[i][j], sb[0][j], sa[0][i]);
+      if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P>{}, I1{}, f[1]);
+      if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, I1{}, OffCur{});
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    // sub-step 1 (blocks 4 + kg): meet, then read the next step's first fragments and scales and refill this stage
+    lds_wait<0>();
+    pin(f[1]);
+    pin_scales(I1{});
+    wait_vmcnt<0>();
+    block_barrier();
+    static_for<NM>([&](auto N_) {
+      constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+      mfma16_mxfp4<0>(f[1].b[j], f[1].a[i], acc[i][j], sb[1][j], sa[1][i]);
+      if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
+      // (sa[0] / sb[0] are free: sub-step 0 has issued all its MFMAs)
+      if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, I0{}, OffNext{});
+      if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fk, lds0 + P * STAGE, std::false_type{});   // one per 64 cycles
+      // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
+      // two steps back used: its last readers were the reads of that pair's second step, in its sub-step 0)
+      // (after the last operand load: the eight loads of an operand share the M0 value that the first one sets)
+      if constexpr (P == 0 && n == 62) issue_scales(fk >> 1, std::false_type{});
+      if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
+    });
+    // everything requested above has landed before the registers are touched again
+    lds_wait<0>();
+    pin(f[0]);
+    pin_scales(I0{});
+  };
+  using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
+  lds_wait<0>();
+  pin(f[0]);
+  // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
+  // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
+  // loop, the number of loads in flight and every wait uniform.
+  int fk = 2, ftile = tile;
+  auto advance = [&]() {
+    if (++fk == nk) {
+      fk = 0;
+      if (ftile + (int)gridDim.x < ntiles) {
+        ftile += gridDim.x;
+        int fm, fn;
+        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+        set_fill_tile(fm, fn);
+      }
+    }
+  };
+  while (true) {
+    for (int kt = 0; kt < nk; kt += 4) {
+      step(I0{}, fk); advance();
+      step(I1{}, fk); advance();
+      step(I2{}, fk); advance();
+      step(I3{}, fk); advance();
+      if (kt + 4 >= nk_last) mfma_retire();
+    }
+    mfma_drain(acc);
+    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
+    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    tile += gridDim.x;
+    if (tile >= ntiles) break;
+    grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
+    zero_acc();
+  }
+  wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
+#endif
+}
+
+bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
+  // whole tiles, K steps in groups of four (K a multiple of 1024 elements), scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 512 == 0 && p.k_bytes >= 512 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
+         p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
+         p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
+}
+
+int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int tiles = (p.M / 256) * (p.N / 256);
+  const int grid = wave128_grid(tiles, p.num_programs);
+  gemm_wave128_mxfp4_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  return (int)hipGetLastError();
+}
+
+}  // namespace mi355
