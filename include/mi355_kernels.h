@@ -175,9 +175,11 @@ int mi355_gemm_streamk_static(const void* A, const void* B, void* C,
  * (addend_dtype) and is added to the fp32 accumulator before the activation and the one
  * rounding to out_dtype.  The add-matrix form may alias C (the reference adds the previous
  * contents of Z); a broadcast D must not overlap C.
- * softmax = 1 then replaces every row of C by exp(c - max) / sum in a second launch on the
- * same stream (fp32 arithmetic; the reference does it inside its single tile).
- * CHAIN_DOT (:3142-3144) is two calls: the first with out_dtype = in_dtype, the second on its result.
+ * softmax = 1 then replaces every row of C by exp(c - max) / sum (fp32 arithmetic).  With fp16 / bf16
+ * operands and N <= 256 - a row fits one tile, the reference's case - product, addend, activation and
+ * softmax are ONE launch on the fp32 accumulator with one rounding at the store; wider rows are
+ * normalised by a second launch on the same stream, which re-reads the rounded C.
+ * CHAIN_DOT (:3142-3144) is mi355_gemm_chain below.
  */
 int mi355_gemm_epilogue(const void* A, const void* B, void* C,
                         int M, int N, int K,
@@ -188,6 +190,26 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C,
                         const float* a_scale, const float* b_scale,
                         const void* addend, int64_t stride_dm, int64_t stride_dn, int addend_dtype,
                         int activation, int softmax, void* stream);
+
+/*
+ * C[M,N2] = z^ @ W with z = softmax_rows?( act( (a_scale * b_scale) * A[M,K] @ B[K,N] + D ) ) and z^ = z rounded
+ * to the operand type: the CHAIN_DOT branch of the reference's dot test,
+ *   python/test/unit/language/test_core.py:3142-3144  `z = tl.dot(z.to(w.dtype), w)`
+ * (with the branches before it, :3128-3141, as in mi355_gemm_epilogue), in ONE launch: z stays in registers
+ * between the two products, as it stays inside the reference's single tile; fp32 accumulation in both, one
+ * rounding to out_dtype at the store (:3145).  A, B, W are fp16 or bf16 (in_dtype) with any element strides;
+ * the intermediate row must fit one tile: N <= 256 and N2 <= 256, else MI355_ESHAPE (chain two mi355_gemm calls).
+ */
+int mi355_gemm_chain(const void* A, const void* B, const void* W, void* C,
+                     int M, int N, int K, int N2,
+                     int64_t stride_am, int64_t stride_ak,
+                     int64_t stride_bk, int64_t stride_bn,
+                     int64_t stride_wn, int64_t stride_wn2,
+                     int64_t stride_cm, int64_t stride_cn,
+                     int in_dtype, int out_dtype,
+                     const float* a_scale, const float* b_scale,
+                     const void* addend, int64_t stride_dm, int64_t stride_dn, int addend_dtype,
+                     int activation, int softmax, void* stream);
 
 /*
  * Grouped GEMM: C_g[M_g,N_g] = A_g[M_g,K_g] @ B_g[K_g,N_g] for g = 0 .. group_size-1 in ONE launch.

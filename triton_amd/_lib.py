@@ -41,6 +41,10 @@ SIGNATURES = {
                                     c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                     c_int, c_int, c_void_p, c_void_p,
                                     c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
+    "mi355_gemm_chain": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                 c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                 c_int, c_int, c_void_p, c_void_p,
+                                 c_void_p, c_int64, c_int64, c_int, c_int, c_int, c_void_p]),
     "mi355_grouped_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "mi355_mx_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                               c_int, c_int, c_int, c_int, c_int,

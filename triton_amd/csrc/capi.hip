@@ -310,10 +310,39 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int
                         int activation, int softmax, void* stream_) {
   if (softmax != 0 && softmax != 1) return MI355_EINVAL;
   if (softmax && out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
+  // a row that fits one tile: product, addend, activation and softmax in ONE launch, on the fp32 accumulator,
+  // one rounding at the store - what the reference's single tile does
+  if (softmax && N <= 256 && (in_dtype == MI355_F16 || in_dtype == MI355_BF16)) {
+    if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
+    if (addend && addend_dtype != MI355_F16 && addend_dtype != MI355_BF16 && addend_dtype != MI355_F32) return MI355_EDTYPE;
+    if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
+    if (!device_info().gfx950) return MI355_EDEVICE;
+    RowFusedArgs r{A, B, C, nullptr, M, N, K, 0, sam, sak, sbk, sbn, 0, 0, scm, scn, a_scale, b_scale,
+                   activation, 1, out_dtype, addend, stride_dm, stride_dn, addend_dtype};
+    return gemm_rowfused_launch(r, in_dtype == MI355_BF16, (hipStream_t)stream_);
+  }
   int rc = gemm_impl(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale,
                      activation, addend, stride_dm, stride_dn, addend_dtype, -1, 0, stream_);
   if (rc || !softmax) return rc;
   return softmax_rows_launch(C, M, N, scm, scn, out_dtype, (hipStream_t)stream_);
+}
+
+int mi355_gemm_chain(const void* A, const void* B, const void* W, void* C, int M, int N, int K, int N2,
+                     int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t swn, int64_t swn2, int64_t scm, int64_t scn,
+                     int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                     const void* addend, int64_t stride_dm, int64_t stride_dn, int addend_dtype,
+                     int activation, int softmax, void* stream_) {
+  if (!A || !B || !W || !C || M <= 0 || N <= 0 || K <= 0 || N2 <= 0) return MI355_EINVAL;
+  if (softmax != 0 && softmax != 1) return MI355_EINVAL;
+  if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
+  if (in_dtype != MI355_F16 && in_dtype != MI355_BF16) return MI355_EDTYPE;
+  if (out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
+  if (addend && addend_dtype != MI355_F16 && addend_dtype != MI355_BF16 && addend_dtype != MI355_F32) return MI355_EDTYPE;
+  if (N > 256 || N2 > 256) return MI355_ESHAPE;   // the intermediate row must fit one tile (callers chain two products otherwise)
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  RowFusedArgs r{A, B, C, W, M, N, K, N2, sam, sak, sbk, sbn, swn, swn2, scm, scn, a_scale, b_scale,
+                 activation, softmax, out_dtype, addend, stride_dm, stride_dn, addend_dtype};
+  return gemm_rowfused_launch(r, in_dtype == MI355_BF16, (hipStream_t)stream_);
 }
 
 int mi355_grouped_gemm(const void* d_a_ptrs, const void* d_b_ptrs, const void* d_c_ptrs,

@@ -59,6 +59,17 @@ struct SkinnyArgs {
   int out_dtype;
 };
 
+// one-launch GEMM with row-wise epilogues (row softmax, chained product), N <= 256 and N2 <= 256
+struct RowFusedArgs {
+  const void* A; const void* B; void* C;
+  const void* W;                       // [N, N2] of the chained product, NULL = none
+  int M, N, K, N2;
+  int64_t sam, sak, sbk, sbn, swn, swn2, scm, scn;   // element strides
+  const float* a_scale; const float* b_scale;
+  int activation, softmax, out_dtype;
+  const void* aux; int64_t aux_sm, aux_sn; int aux_dtype;   // addend as in GemmArgs
+};
+
 struct AttnArgs {
   const char* q; const char* k; const char* v; char* o; float* lse;
   const char* d_o; const float* delta; char* dq; char* dk; char* dv;
@@ -106,6 +117,7 @@ int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_fwd8_launch(const AttnArgs& p, bool e5m2, hipStream_t stream);  // fp8 inputs, V with N contiguous
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+int gemm_rowfused_launch(const RowFusedArgs& p, bool bf16, hipStream_t stream);
 int softmax_rows_launch(void* C, int M, int N, int64_t scm, int64_t scn, int dtype, hipStream_t stream);
 int clock_probe_launch(unsigned long long* out, unsigned long long real_ticks, hipStream_t stream);
 int dequant_launch(const uint8_t* codes, float* out, int64_t n, int fmt, hipStream_t stream);

@@ -187,11 +187,37 @@ def matmul_streamk(a, b, *, out_dtype=None):
     return c
 
 
-def chain_dot(a, b, w, *, out_dtype=None):
-    """(A @ B) rounded to the input type, then @ W: the CHAIN_DOT branch of the reference's dot test
-    (python/test/unit/language/test_core.py:3142-3144, `tl.dot(z.to(w.dtype), w)`), as two launches."""
+def chain_dot(a, b, w, *, out_dtype=None, add=None, activation="", softmax=False):
+    """(A @ B [+ add, activation, row softmax]) rounded to the input type, then @ W: the CHAIN_DOT branch of
+    the reference's dot test (python/test/unit/language/test_core.py:3142-3144, `tl.dot(z.to(w.dtype), w)`).
+    When the intermediate row fits one tile (N <= 256 and W's N2 <= 256) this is ONE launch and z never
+    leaves the registers (`mi355_gemm_chain`); wider intermediates are two products with the rounding in
+    between."""
     assert a.dtype == b.dtype == w.dtype, "Incompatible dtypes"
-    z = matmul(a, b, out_dtype=a.dtype)
+    assert a.shape[1] == b.shape[0] and b.shape[1] == w.shape[0], "Incompatible dimensions"
+    in_dt = _abi_dtype(a)
+    M, K = a.shape
+    N, N2 = w.shape
+    if in_dt in (_lib.F16, _lib.BF16) and N <= 256 and N2 <= 256 and M > 0 and K > 0:
+        for i, t in enumerate((a, b, w)):
+            _check_device(i, t)
+        if out_dtype is None:
+            out_dtype = a.dtype
+        if activation not in ("", "leaky_relu"):
+            raise KeyError(f"unknown ACTIVATION {activation!r}")
+        c = torch.empty((M, N2), device=a.device, dtype=out_dtype)
+        d_ptr, d_sm, d_sn, d_dt = 0, 0, 0, 0
+        if add is not None:
+            d = torch.broadcast_to(add, (M, N))
+            d_ptr, d_sm, d_sn, d_dt = d.data_ptr(), d.stride(0), d.stride(1), _TORCH_TO_ABI[add.dtype]
+        rc = _lib.load().mi355_gemm_chain(
+            a.data_ptr(), b.data_ptr(), w.data_ptr(), c.data_ptr(), M, N, K, N2,
+            a.stride(0), a.stride(1), b.stride(0), b.stride(1), w.stride(0), w.stride(1), c.stride(0), c.stride(1),
+            in_dt, _TORCH_TO_ABI[out_dtype], None, None, d_ptr, d_sm, d_sn, d_dt,
+            _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE, int(bool(softmax)), _stream())
+        _lib.check(rc, "mi355_gemm_chain")
+        return c
+    z = matmul(a, b, activation, out_dtype=a.dtype, add=add, softmax=softmax)
     return matmul(z, w, out_dtype=out_dtype)
 
 
