@@ -253,6 +253,25 @@ def test_fp8_row_major_b_uses_the_strided_kernel_and_fp8_output(gpu):
     assert triton_amd.matmul_like_input(a16, b16).dtype == torch.float16
 
 
+def test_large_row_major_fp8_b_is_put_k_major_by_the_host_wrapper(gpu):
+    # 03:378-380 pre-transposes b on the host for fp8; `matmul` does the same for a large row-major fp8 B, so the
+    # product runs on the fp8 MFMAs (told apart from the strided kernel by time) and equals the K-major call
+    n = 4096
+    g = torch.Generator(device="cpu").manual_seed(12)
+    a = (torch.randn(n, n, generator=g) * 0.5).to(torch.float8_e4m3fn).to(gpu)
+    b = (torch.randn(n, n, generator=g) * 0.5).to(torch.float8_e4m3fn).to(gpu)     # [K, N] row-major
+    want = triton_amd.matmul(a, b.t().contiguous().t(), out_dtype=torch.bfloat16)
+    got = triton_amd.matmul(a, b, out_dtype=torch.bfloat16)
+    torch.cuda.synchronize()
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    got = triton_amd.matmul(a, b, out_dtype=torch.bfloat16)
+    ev1.record()
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert ev0.elapsed_time(ev1) < 5.0, ev0.elapsed_time(ev1)
+
+
 @pytest.mark.parametrize("tile", [None, 6])
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
 def test_fp8_output_of_the_mfma_epilogues_rounds_like_the_oracle(gpu, monkeypatch, fmt, tdt, tile):
@@ -561,11 +580,13 @@ def test_fused_addends_in_the_four_wave_fp8_kernel(gpu, monkeypatch, fmt, tdt):
 
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
-@pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512)])
+@pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512),
+                                   (1024, 32, 256)])
 def test_fused_epilogues_of_the_reference_dot_test(gpu, dtype, shape):
     # add-matrix / add-rows / add-cols / softmax / chain-dot (python/test/unit/language/test_core.py:3128-3145)
-    # through mi355_gemm_epilogue: MFMA tile kernels, the strided kernel (100, 70, 50) and a skinny
-    # shape (which takes the tile kernels when there is an addend).  Integer data: bit-exact.
+    # through mi355_gemm_epilogue: MFMA tile kernels, the strided kernel (100, 70, 50) and two skinny
+    # shapes (the streaming kernels add the addend in their own epilogue; the second one runs with the
+    # operands swapped).  Integer data: bit-exact.
     M, N, K = shape
     rng = np.random.default_rng(M + N + K)
     a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)

@@ -112,3 +112,56 @@ def test_host_time_per_launch(gpu):
         torch.cuda.synchronize()
     print(f"host time per matmul() call: {best * 1e6:.1f} us")
     assert best < 46e-6
+
+
+def test_torch_extension_is_the_default_binding_and_agrees_with_ctypes(gpu, monkeypatch):
+    # The PyTorch-ROCm extension (tensor objects in, c10::hip::getCurrentHIPStream(), one C-ABI call) is what the
+    # operators use when it is built; ctypes is the same C ABI reached from Python.  Same kernels, same bits;
+    # and the host time per call of both bindings, for the record.
+    from triton_amd import _lib
+
+    assert _lib.ext() is not None, "the torch extension was not built (python -m triton_amd.build)"
+    a = torch.randn(256, 512, device=gpu, dtype=torch.bfloat16)
+    b = torch.randn(512, 384, device=gpu, dtype=torch.bfloat16)
+    bias = torch.randn(1, 384, device=gpu, dtype=torch.float32)
+    q, k, v = (torch.randn(1, 2, 256, 64, device=gpu, dtype=torch.float16).requires_grad_() for _ in range(3))
+    do = torch.randn(1, 2, 256, 64, device=gpu, dtype=torch.float16)
+
+    def run():
+        c = triton_amd.matmul(a, b, activation="leaky_relu", add=bias)
+        o = triton_amd.attention(q, k, v, True, 0.125)
+        grads = torch.autograd.grad(o, (q, k, v), do)
+        return (c, o.detach(), *grads)
+
+    def host_us():
+        x = torch.randn(16, 64, device=gpu, dtype=torch.float16)
+        y = torch.randn(64, 64, device=gpu, dtype=torch.float16)
+        for _ in range(50):
+            triton_amd.matmul(x, y)
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(5):
+            t0 = time.perf_counter()
+            for _ in range(200):
+                triton_amd.matmul(x, y)
+            best = min(best, (time.perf_counter() - t0) / 200)
+            torch.cuda.synchronize()
+        return best * 1e6
+
+    with_ext = run()
+    us_ext = host_us()
+    monkeypatch.setattr(_lib, "_ext", None)          # ctypes from here on
+    with_ctypes = run()
+    us_ctypes = host_us()
+    for x, y in zip(with_ext, with_ctypes):
+        assert torch.equal(x, y)
+    print(f"host time per matmul() call: torch extension {us_ext:.1f} us, ctypes {us_ctypes:.1f} us")
+    with torch.cuda.stream(torch.cuda.Stream(device=gpu)):
+        monkeypatch.setattr(_lib, "_ext", False)     # (re-resolved: the extension again) on a side stream
+        e = torch.eye(512, device=gpu, dtype=torch.bfloat16)
+        acc = torch.zeros(512, 512, device=gpu, dtype=torch.bfloat16)
+        for _ in range(10):
+            acc.add_(1.0)
+        out = triton_amd.matmul(acc, e)
+    torch.cuda.synchronize()
+    assert torch.equal(out, torch.full_like(out, 10.0))   # launched on, and ordered by, the current (side) stream

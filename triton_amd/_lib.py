@@ -85,6 +85,26 @@ def load() -> ctypes.CDLL:
     return _lib
 
 
+_ext = False
+
+
+def ext():
+    """The PyTorch-ROCm extension `_mi355_torch` (tensor objects in, torch's current stream, one C-ABI call
+    per operator), or None when it has not been built or when MI355_KERNELS_LIB selects another build of the
+    kernel library (the extension is linked to the in-tree one).  The operators then go through ctypes."""
+    global _ext
+    if _ext is False:
+        _ext = None
+        if not os.environ.get("MI355_KERNELS_LIB") and not os.environ.get("MI355_NO_TORCH_EXT"):
+            load()  # the C library first: same build, and a clear error if it is missing
+            try:
+                from . import _mi355_torch  # noqa: PLC0415
+                _ext = _mi355_torch
+            except ImportError:
+                _ext = None
+    return _ext
+
+
 def strerror(code: int) -> str:
     return load().mi355_strerror(code).decode()
 

@@ -83,6 +83,40 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     os.replace(tmp, out)
+    build_torch_extension(verbose)
+    return out
+
+
+EXT_SRC = Path(__file__).resolve().parent / "csrc_ext" / "torch_ext.cpp"
+EXT_NAME = "_mi355_torch"
+
+
+def ext_path() -> Path:
+    return Path(__file__).resolve().parent / (EXT_NAME + ".so")
+
+
+def build_torch_extension(verbose: bool = False) -> Path:
+    """Compile the PyTorch-ROCm extension (host C++ only: tensor checks, current stream, one C-ABI call per
+    operator) with g++ against the installed torch and link it to the kernel library next to it."""
+    import sysconfig
+
+    from torch.utils import cpp_extension as ce
+
+    out = ext_path()
+    tmp = out.with_suffix(".so.tmp")
+    inc = [sysconfig.get_paths()["include"], *ce.include_paths("cuda"), "/opt/rocm/include"]
+    libdirs = ce.library_paths("cuda")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-DTORCH_EXTENSION_NAME={EXT_NAME}", "-DTORCH_API_INCLUDE_EXTENSION_H", "-Wno-deprecated-declarations",
+           *[f"-I{i}" for i in inc], str(EXT_SRC), "-o", str(tmp),
+           *[f"-L{d}" for d in libdirs], f"-L{CSRC}", "-lc10", "-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10_hip", "-ltorch_hip",
+           "-l:" + LIB_NAME, "-Wl,-rpath,$ORIGIN/csrc", *[f"-Wl,-rpath,{d}" for d in libdirs]]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"torch extension build failed:\n{res.stderr[-4000:]}")
+    os.replace(tmp, out)
     return out
 
 

@@ -198,9 +198,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;
-  // (the streaming kernels have no addend in their epilogue: with one, the tile kernels run)
   const bool skinny_allowed = tile_arg < 0 && knob(knobs().skinny, 1);  // an explicit tile means a tile kernel
-  if (!aux && skinny_allowed) {
+  if (skinny_allowed) {
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
@@ -209,10 +208,12 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     if (M <= 64) {
       sk.X = (const char*)A; sk.Y = (const char*)B; sk.S = M; sk.L = N;
       sk.x_pitch = p.lda; sk.y_pitch = p.ldb; sk.cs = scm; sk.cl = scn;
+      sk.aux = aux; sk.aux_ss = aux_sm; sk.aux_sl = aux_sn; sk.aux_dtype = aux_dtype;
       y_kmajor = b_kmajor; use = true;
     } else if (N <= 64) {
       sk.X = (const char*)B; sk.Y = (const char*)A; sk.S = N; sk.L = M;
       sk.x_pitch = p.ldb; sk.y_pitch = p.lda; sk.cs = scn; sk.cl = scm;
+      sk.aux = aux; sk.aux_ss = aux_sn; sk.aux_sl = aux_sm; sk.aux_dtype = aux_dtype;
       y_kmajor = true; x_kmajor = b_kmajor; use = true;
     }
     if (use && gemm_skinny_ok(sk, y_kmajor, x_kmajor, es))

@@ -246,10 +246,11 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
     for (int w = 0; w < NW; w++) v += red[(w * ST * 16 + rr) * 64 + lane];
     v *= alpha;
-    if (p.activation == 1) v = v >= 0.f ? v : 0.01f * v;
     // register r of lane: row l = 8 (r / 4) + 4 g + r % 4 of the tile, column s = l32
     const int s = 32 * t + l32, l = l0 + (r >> 2) * 8 + g * 4 + (r & 3);
     if (s < p.S && l < p.L) {
+      if (p.aux) v += load_aux(p.aux, (int64_t)s * p.aux_ss + (int64_t)l * p.aux_sl, p.aux_dtype);
+      if (p.activation == 1) v = v >= 0.f ? v : 0.01f * v;
       const int64_t off = (int64_t)s * p.cs + (int64_t)l * p.cl;
       if (p.out_dtype == 4) ((float*)p.C)[off] = v;
       else if (p.out_dtype == 2) ((uint8_t*)p.C)[off] = f32_to_e4m3(v);

@@ -57,6 +57,11 @@ struct SkinnyArgs {
   const float* b_scale;
   int activation;
   int out_dtype;
+  // optional addend of the epilogue, indexed like the output: aux[s * aux_ss + l * aux_sl] (a zero stride
+  // broadcasts), added in fp32 before the activation; NULL = none
+  const void* aux;
+  int64_t aux_ss, aux_sl;
+  int aux_dtype;
 };
 
 // one-launch GEMM with row-wise epilogues (row softmax, chained product), N <= 256 and N2 <= 256

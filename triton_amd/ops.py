@@ -118,11 +118,28 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         return c
     if K == 0:
         return c.zero_()
+    if (in_dt in (_lib.F8E4M3, _lib.F8E5M2) and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
+            and K % 16 == 0 and M * N * K >= 1 << 24):
+        # fp8 MFMAs want both operands K-contiguous: a row-major fp8 B is put into that layout first, as the
+        # reference does on the host for its fp8 case ("pre-transpose b for efficiency", 03:378-380) - one
+        # pass over B instead of the strided kernel (the C ABI itself runs whatever layout it is given)
+        b = b.t().contiguous().t()
     pa, keep_a = _scale_ptr(a_scale, device)
     pb, keep_b = _scale_ptr(b_scale, device)
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
     stream = _stream()
     md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K, _ELEM_BYTES[in_dt]))
+    ext = _lib.ext()
+    if ext is not None and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
+        # the PyTorch-ROCm extension: tensors in, torch's current stream taken in C++, one C-ABI call
+        d = None
+        if add is not None:
+            if add.dtype not in (torch.float16, torch.bfloat16, torch.float32):
+                raise TypeError(f"add must be fp16, bf16 or fp32, got {add.dtype}")
+            d = torch.broadcast_to(add, (M, N))
+        ext.gemm(a, b, c, act, keep_a, keep_b, d, bool(softmax))
+        hooks.exit(md)
+        return c
     if add is None and not softmax:
         rc = _lib.load().mi355_gemm(
             a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
@@ -312,6 +329,10 @@ def mx_matmul(a_packed, a_scale, b_packed, b_scale, fmt="mxfp4", out_dtype=torch
     assert K % 32 == 0, "K must be a multiple of the 32-element scale block"
     assert tuple(a_scale.shape) == (M, K // 32) and tuple(b_scale.shape) == (N, K // 32), "scale shape must be [rows, K/32]"
     c = torch.empty((M, N), device=a_packed.device, dtype=out_dtype)
+    ext = _lib.ext()
+    if ext is not None:
+        ext.mx_gemm(a_packed, a_scale, b_packed, b_scale, c, f, K)
+        return c
     rc = _lib.load().mi355_mx_gemm(
         a_packed.data_ptr(), a_scale.data_ptr(), b_packed.data_ptr(), b_scale.data_ptr(), c.data_ptr(),
         M, N, K, f, _TORCH_TO_ABI[out_dtype],
@@ -360,12 +381,16 @@ class _attention(torch.autograd.Function):
         stream = _stream()
         md = hooks.enter("mi355_attn_fwd", stream, hooks.attention_launch_metadata,
                          ("mi355_attn_fwd", Z, H, N_CTX, HEAD_DIM_K, causal, _ELEM_BYTES[dt]))
-        rc = _lib.load().mi355_attn_fwd(
-            q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr(),
-            Z, H, N_CTX, HEAD_DIM_K,
-            I4(*q.stride()), I4(*k.stride()), I4(*v.stride()), I4(*o.stride()),
-            float(sm_scale), int(bool(causal)), dt, stream)
-        _lib.check(rc, "mi355_attn_fwd")
+        ext = _lib.ext()
+        if ext is not None:
+            ext.attn_fwd(q, k, v, o, M, float(sm_scale), bool(causal))
+        else:
+            rc = _lib.load().mi355_attn_fwd(
+                q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr(),
+                Z, H, N_CTX, HEAD_DIM_K,
+                I4(*q.stride()), I4(*k.stride()), I4(*v.stride()), I4(*o.stride()),
+                float(sm_scale), int(bool(causal)), dt, stream)
+            _lib.check(rc, "mi355_attn_fwd")
         hooks.exit(md)
         ctx.save_for_backward(q, k, v, o, M)
         ctx.sm_scale = sm_scale
@@ -386,6 +411,10 @@ class _attention(torch.autograd.Function):
         assert N_CTX % PRE_BLOCK == 0
         delta = torch.empty_like(M)
         dt = _abi_dtype(q)
+        ext = _lib.ext()
+        if ext is not None:
+            ext.attn_bwd(q, k, v, o, do, M, delta, dq, dk, dv, float(ctx.sm_scale), bool(ctx.causal))
+            return dq, dk, dv, None, None
         I4 = _lib.I64x4
         lib = _lib.load()
         rc = lib.mi355_attn_bwd_preprocess(
