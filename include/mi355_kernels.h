@@ -105,7 +105,7 @@ int mi355_gemm(const void* A, const void* B, void* C,
  * 5 = the eight-wave pipelined kernel as persistent programs (one per CU, MI355_GEMM_PROGRAMS
  * overrides) that walk their tiles as one stream of K steps, the schedule of
  * python/tutorials/09-persistent-matmul.py:141-190, 6 = four waves of 128x128 from 16x16x32
- * (fp8: 16x16x128) MFMAs on 256x256 tiles (whole tiles, K bytes a multiple of 256, a row-major B with a
+ * (fp8: 16x16x128) MFMAs on 256x256 tiles (whole tiles, K at least 128 elements - fp8: K bytes a multiple of 256 -, a row-major B with a
  * pitch that is a multiple of 512 bytes, fp8 with a K-major B; the heuristic's choice for such products from
  * 128 tiles on, fp8 from 192; with more tiles than MI355_GEMM_PROGRAMS, default the CU count, its programs
  * take ceil(tiles / programs) tiles each as one stream of K steps)

@@ -427,6 +427,28 @@ def test_full_size_8192_fp16_sampled_rows(gpu):
     _sampled_rows_check(gpu, 8192, 8192, 8192, "fp16", seed=5)
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("layout", ["row_major_b", "k_major_b"])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_four_wave_kernel_k_tails_are_bit_exact(gpu, monkeypatch, dtype, layout, programs):
+    # K not a multiple of 128 elements in the four-wave kernel: the rest (8 .. 120 elements) is multiplied after the
+    # pipelined K loop through a buffer of its own, 32 elements at a time.  Every tail length class (one to four
+    # half-steps, full and partial last one), one and several tiles per program (the tail runs while the stages
+    # already hold the next tile's first K steps), integer data: the bits of the closed form.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(layout))
+    for K in (136, 264, 312, 376, 440, 504, 1016, 2056):
+        M, N = 768, 512
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ta, tb = from_np(a, dtype, gpu), from_np(b, dtype, gpu)
+        if layout == "k_major_b":
+            tb = tb.t().contiguous().t()
+        got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+        assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32")), (K, dtype, layout, programs)
+
+
 @pytest.mark.parametrize("layout", ["row_major_b", "k_major_b"])
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 def test_uneven_k_8192x8192x8176(gpu, dtype, layout):

@@ -193,7 +193,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // (an epilogue addend: instantiations of their own)
   // (fp8 from three quarters of a round: at 144 tiles the eight-wave kernel is 4-7 % ahead - 3072^3 1520 vs
   // 1450, 3072x3072x8192 2040 vs 1890 TFLOP/s -, at 196 tiles the four-wave one by 2 %, at 225 by 13 %)
-  if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && gemm_wave128_ok(p, b_kmajor)) tile = 6;
+  const bool w128_ok = gemm_wave128_ok(p, b_kmajor) && (!is8 || p.k_bytes % 256 == 0);   // (a K tail: the 16-bit forms only)
+  if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && w128_ok) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : knob(knobs().tile, tile);
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
@@ -220,7 +221,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && gemm_wave128_ok(p, true)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   if (tile == 6 && gemm_wave128_ok(p, b_kmajor)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);

@@ -43,7 +43,12 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 // The tiles `tile`, `tile + tile_step`, ... (< `tile_stop`, by default M/256 * N/256) of one problem, computed by the calling workgroup
 // with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  EPI: 0 = scales,
 // activation, any output type; 1 = C has the type of the operands, no scales, no activation; 2 = 0 plus the addend.
-template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0>
+// TAIL: K bytes need not be a multiple of 256; what is left behind the last pair of K steps (16 .. 240 bytes of
+// every operand row) is multiplied after the K loop, 64 bytes at a time, through a 32 KiB LDS buffer of its own
+// behind the two stages (which by then hold the next tile's first steps): plain loads with a zero fill, one
+// un-pipelined sub-step each - a per-tile cost of a few microseconds that only products with such a K pay
+// (the reference's own uneven-K shape 8192 x 8192 x 8176, python/test/regression/test_performance.py:46).
+template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0, bool TAIL = false>
 __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0, const int tile_stop = -1) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -65,7 +70,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   auto tile_at = [&](int t, int& tm, int& tn) { grouped_tile(XCD ? xcd_remap(t, ntiles) : t, num_m, num_n, p.group_m, tm, tn); };
   int pm, pn;
   tile_at(tile, pm, pn);
-  const int nk = p.k_bytes / ROWB;
+  const int nk = TAIL ? (p.k_bytes / (2 * ROWB)) * 2 : p.k_bytes / ROWB;   // K steps of the pipelined loop (an even number)
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
   asm volatile("" : "+s"(nk_last));
 
@@ -240,6 +245,67 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
       stage(I1{}, fk); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
+    if constexpr (TAIL) {
+      const int k_main = nk * ROWB, tail = p.k_bytes - k_main;   // bytes per row: done, and left (a multiple of 16)
+      const unsigned tailA = lds0 + 2 * STAGE, tailB = tailA + BM * 64;
+      const char* const tA = p.A + (int64_t)pm * BM * p.lda + k_main;
+      for (int h = 0; h * 64 < tail; h++) {
+        // this half-step's 64 bytes of the 256 A rows and of the 256 B rows (K-major B) or its 32 k rows of 512
+        // bytes (row-major B, in the column-group order of the stages): 1024 + 1024 chunks of 16 bytes, four
+        // each per thread, zeros beyond K
+        i32x4 va[4], vb[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int id = tid + 256 * i;
+          {
+            const int row = id >> 2, kb = h * 64 + (id & 3) * 16;
+            va[i] = i32x4{0, 0, 0, 0};
+            if (kb < tail) va[i] = *(const i32x4*)(tA + (int64_t)row * p.lda + kb);
+          }
+          vb[i] = i32x4{0, 0, 0, 0};
+          if constexpr (B_KMAJOR) {
+            const int row = id >> 2, kb = h * 64 + (id & 3) * 16;
+            if (kb < tail) vb[i] = *(const i32x4*)(p.B + ((int64_t)pn * BN + row) * p.ldb + k_main + kb);
+          } else {
+            const int kr = id >> 5, pc = id & 31;
+            const int k = k_main / 2 + h * 32 + kr;
+            const int lg = (pc >> 1) ^ (2 * (kr & 3)) ^ ((kr >> 3) & 1);
+            if (k < p.K) vb[i] = *(const i32x4*)(p.B + (int64_t)k * p.ldb + (int64_t)pn * BN * 2 + lg * 32 + (pc & 1) * 16);
+          }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int id = tid + 256 * i;
+          *(LDS_PTR(i32x4))(uintptr_t)(tailA + id * 16) = va[i];     // A: row id / 4 at 64 (id / 4), chunk id % 4
+          *(LDS_PTR(i32x4))(uintptr_t)(tailB + id * 16) = vb[i];     // B: the same, or k row id / 32, chunk id % 32
+        }
+        lds_wait<0>();
+        block_barrier();
+        static_for<MT>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          f[1].a[t] = __builtin_bit_cast(V8, lds_read_b128<t * 16 * 64>(tailA + (wm * 128 + l16) * 64 + kg * 16));
+        });
+        static_for<NT>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          if constexpr (B_KMAJOR) {
+            f[1].b[t] = __builtin_bit_cast(V8, lds_read_b128<t * 16 * 64>(tailB + (wn * 128 + l16) * 64 + kg * 16));
+          } else {
+            const unsigned ad = adrB[t] - (lds0 + A_BYTES) + tailB;
+            s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(uintptr_t)ad);
+            s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((LDS_PTR(s16x4))(uintptr_t)(ad + 4 * BN * 2));
+            f[1].b[t] = __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+          }
+        });
+        lds_wait<0>();
+        pin(f[1]);
+        block_barrier();   // every wave holds its fragments: the buffer may be overwritten
+        static_for<NM>([&](auto N_) {
+          constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+          mfma16(f[1].b[j], f[1].a[i], acc[i][j]);
+        });
+      }
+      mfma_retire();
+    }
     // The next tile's first fragments were requested by reads the compiler cannot see: have them landed
     // before the epilogue's register traffic could move their registers.  Nor does it know that the assembly
     // above are MFMAs: let the last ones retire before their results are read.
@@ -263,11 +329,11 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 }
 
 // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
-template <typename V8, bool B_KMAJOR, bool AUX>
+template <typename V8, bool B_KMAJOR, bool AUX, bool TAIL = false>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-  gemm_wave128_tiles<V8, B_KMAJOR, true, AUX ? 2 : 0>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
+  gemm_wave128_tiles<V8, B_KMAJOR, true, AUX ? 2 : 0, TAIL>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
 #endif
 }
 
@@ -517,26 +583,28 @@ int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
 }
 
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
-  // whole tiles, an even number (>= 2) of 128-byte K steps, 32-bit lane offsets
-  if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  // whole tiles, at least one pair of 128-byte K steps (what is left behind the last pair: the TAIL form, which
+  // has no addend instantiation), 32-bit lane offsets
+  if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 16 == 0 && p.k_bytes >= 256)) return false;
+  if (p.k_bytes % 256 != 0 && p.aux) return false;
   if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
   // (row-major B: the per-load XOR of the column group acts on the whole lane offset, so the row term
   // in it - a multiple of the pitch - must leave the bits of the 512-byte tile row alone)
   return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
-template <typename V8, bool B_KMAJOR, bool AUX>
+template <typename V8, bool B_KMAJOR, bool AUX, bool TAIL = false>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128;
+  constexpr int smem = 2 * 2 * 256 * 128 + (TAIL ? 2 * 256 * 64 : 0);   // (with the tail buffer: all 160 KiB of the CU)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, AUX>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, AUX, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_kernel<V8, B_KMAJOR, AUX><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_kernel<V8, B_KMAJOR, AUX, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -558,6 +626,10 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 }
 
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream) {
+  if (p.k_bytes % 256 != 0) {   // (gemm_wave128_ok: no addend then)
+    if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, false, true>(p, stream) : launch_wave128<f16x8, true, false, true>(p, stream);
+    return bf16 ? launch_wave128<bf16x8, false, false, true>(p, stream) : launch_wave128<f16x8, false, false, true>(p, stream);
+  }
   if (p.aux) {
     if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, true>(p, stream) : launch_wave128<f16x8, true, true>(p, stream);
     return bf16 ? launch_wave128<bf16x8, false, true>(p, stream) : launch_wave128<f16x8, false, true>(p, stream);
