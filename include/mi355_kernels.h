@@ -252,8 +252,9 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
  * Stands in for the launch of `_attn_fwd` by `_attention.forward`
  *   python/tutorials/06-fused-attention.py:98-187 (kernel), :25-75 (inner loop), :441-475 (host).
  * q,k,v,o are [Z,H,N_CTX,D] with the four element strides given per tensor (last stride must be 1);
- * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {64, 128, 256}
- * (forward and backward entries alike).
+ * Mlse is contiguous [Z,H,N_CTX].  dtype is MI355_F16 or MI355_BF16; D in {16, 32, 64, 128, 256}
+ * (forward and backward entries alike; 16 and 32, the reference's other two head dims, :447, are taken as they
+ * are - rows of D elements - and run the 64-column kernels in a form that pads with zeros on the fly).
  * fp8 forward (dtype MI355_F8E5M2 as in the reference's fp8 benchmark, :609-614, or MI355_F8E4M3):
  * q, k and o as above, v transposed in memory (stride 1 along N_CTX, a multiple of 16 along D:
  * what `v.permute(0,1,3,2).contiguous().permute(0,1,3,2)` yields); P is rounded to the fp8 type

@@ -118,9 +118,9 @@ def test_unsupported_configurations_raise(gpu):
     q = torch.zeros(1, 1, 100, 64, dtype=torch.float16, device=gpu)
     with pytest.raises(ValueError):          # N_CTX must be a multiple of 128 here (the reference asserts it in backward, 06:494)
         triton_amd.attention(q, q, q, True, 0.5)
-    q32 = torch.zeros(1, 1, 128, 32, dtype=torch.float16, device=gpu)
-    with pytest.raises(ValueError):          # the C ABI has no head_dim 32 kernel (the host wrapper pads to 64 instead)
-        triton_amd.ops._attention.apply(q32, q32, q32, True, 0.5)
+    q8 = torch.zeros(1, 1, 128, 32, dtype=torch.float8_e5m2, device=gpu)
+    with pytest.raises(ValueError):          # fp8 forward: head dims 64 and 128 only
+        triton_amd.attention(q8, q8, q8.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2), True, 0.5)
     q48 = torch.zeros(1, 1, 128, 48, dtype=torch.float16, device=gpu)
     with pytest.raises(AssertionError):      # the reference's own assert (06:447)
         triton_amd.attention(q48, q48, q48, True, 0.5)
@@ -185,8 +185,10 @@ def test_head_dim_256_forward_and_backward(gpu, dtype, causal, shape):
 @pytest.mark.parametrize("D", [16, 32])
 @pytest.mark.parametrize("causal", [True, False])
 def test_head_dims_16_and_32_forward_and_backward(gpu, dtype, D, causal):
-    # HEAD_DIM 16 / 32 of the reference's assert (06:447): zero-padded to the 64-column kernels by the
-    # host wrapper; outputs and all three gradients against the closed form at the usual tolerance
+    # HEAD_DIM 16 / 32 of the reference's assert (06:447): the 64-column kernels pad with zeros on the fly (no padded
+    # copies; the tensors keep their 32- / 64-byte rows); outputs and all three gradients against the tile oracle and
+    # the closed form at the usual tolerance.  Outputs are allocated inside a buffer filled with a sentinel, so a
+    # store beyond column HEAD_DIM would show.
     shape = (2, 2, 256, D)
     (q, k, v, do), (tq, tk, tv, tdo) = _inputs(11, shape, dtype, gpu)
     sm_scale = D ** -0.5
@@ -203,3 +205,38 @@ def test_head_dims_16_and_32_forward_and_backward(gpu, dtype, D, causal):
     _check_against_tiled_and_closed_form(f"{shape} causal={causal}",
                                          dict(o=to_np(out.detach()), dq=to_np(tq.grad), dk=to_np(tk.grad), dv=to_np(tv.grad)),
                                          dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, dtype)
+
+
+@pytest.mark.parametrize("D", [16, 32])
+def test_head_dims_16_and_32_touch_only_their_own_columns(gpu, D):
+    # Through the C ABI with every tensor a [..., :D] view of a 64-column buffer: the columns beyond HEAD_DIM hold NaN
+    # on the input side (a kernel that read them would poison everything) and a sentinel on the output side (a
+    # kernel that stored there would overwrite it).
+    from triton_amd import _lib
+    Z, H, N = 1, 2, 256
+    lib = _lib.load()
+    g = torch.Generator(device="cpu").manual_seed(D)
+    def wide(fill):
+        return torch.full((Z, H, N, 64), fill, dtype=torch.float16, device=gpu)
+    bufs = {n: wide(float("nan")) for n in ("q", "k", "v", "do")}
+    for n, t in bufs.items():
+        t[..., :D] = (torch.randn(Z, H, N, D, generator=g) * (1.0 if n == "do" else 0.5)).half().to(gpu)
+    outs = {n: wide(7.0) for n in ("o", "dq", "dk", "dv")}
+    q, k, v, do = (bufs[n][..., :D] for n in ("q", "k", "v", "do"))
+    o, dq, dk, dv = (outs[n][..., :D] for n in ("o", "dq", "dk", "dv"))
+    M = torch.empty(Z, H, N, dtype=torch.float32, device=gpu)
+    delta = torch.empty_like(M)
+    I4 = _lib.I64x4
+    st = torch.cuda.current_stream().cuda_stream
+    sm_scale = D ** -0.5
+    assert lib.mi355_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr(), Z, H, N, D,
+                              I4(*q.stride()), I4(*k.stride()), I4(*v.stride()), I4(*o.stride()), sm_scale, 1, _lib.F16, st) == 0
+    assert lib.mi355_attn_bwd_preprocess(o.data_ptr(), do.data_ptr(), delta.data_ptr(), Z, H, N, D, I4(*o.stride()), _lib.F16, st) == 0
+    assert lib.mi355_attn_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), do.data_ptr(), M.data_ptr(), delta.data_ptr(),
+                              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), Z, H, N, D, I4(*q.stride()), sm_scale, 1, _lib.F16, st) == 0
+    torch.cuda.synchronize()
+    cf = A.attn_closed_form(*(to_np(t) for t in (q, k, v)), True, sm_scale, to_np(do))
+    for name, t in (("o", o), ("dq", dq), ("dk", dk), ("dv", dv)):
+        assert np.allclose(to_np(t), cf[name], atol=1e-2, rtol=1e-2), name
+        assert torch.all(outs[name][..., D:] == 7.0), name       # nothing stored beyond column HEAD_DIM
+    assert np.allclose(to_np(M), cf["M"], atol=2e-3, rtol=0)

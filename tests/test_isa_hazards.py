@@ -251,3 +251,292 @@ def test_no_vector_memory_instruction_reads_a_scalar_register_too_soon_after_a_v
             bad = check_sgpr_to_vmem(lines)
             assert not bad, (os.path.basename(f), name, bad[:5])
     assert checked >= 40, checked
+
+
+VGPR = re.compile(r"\bv(\d+|\[\d+:\d+\])")
+LDS_QUEUE_CAP = 96
+
+
+def _vregs(text):
+    out = set()
+    for m in VGPR.finditer(text):
+        t = m.group(1)
+        if t.startswith("["):
+            lo, hi = t[1:-1].split(":")
+            out.update(range(int(lo), int(hi) + 1))
+        else:
+            out.add(int(t))
+    return out
+
+
+def check_lds_reads_in_flight(lines):
+    """Rule 3: violations (block label, instruction, registers) where an instruction reads or writes a vector
+    register that an LDS read issued earlier has not delivered yet.  LDS (and scalar memory) operations
+    retire in order against one counter; `s_waitcnt lgkmcnt(N)` leaves the N youngest outstanding.  The state
+    is the queue of outstanding operations (the destination registers of each), kept per control-flow path."""
+    blocks = _blocks(lines)
+    index = {lab: i for i, (lab, _) in enumerate(blocks)}
+    succ = []
+    for i, (_, ins) in enumerate(blocks):
+        s, fall = set(), True
+        for t in ins:
+            m = re.match(r"s_c?branch\w*\s+(\.LBB\w+)", t)
+            if m:
+                s.add(index[m.group(1)])
+            if t.startswith("s_branch") or t.startswith("s_endpgm") or t.startswith("s_setpc"):
+                fall = False
+        if fall and i + 1 < len(blocks):
+            s.add(i + 1)
+        succ.append(s)
+
+    def walk(ins, queue, report, label):
+        queue = list(queue)
+        for t in ins:
+            op = t.split()[0]
+            operands = t[len(op):]
+            if op == "s_waitcnt":
+                m = re.search(r"lgkmcnt\((\d+)\)", operands)
+                if m:
+                    keep = int(m.group(1))
+                    queue = queue[len(queue) - keep:] if keep < len(queue) else queue
+                    if keep == 0:
+                        queue = []
+                continue
+            flying = set().union(*queue) if queue else set()
+            if op.startswith(("ds_read", "ds_load")):
+                dst, src = operands.split(",", 1)
+                hit = _vregs(src) & flying
+                queue.append(frozenset(_vregs(dst)))
+            elif op.startswith(("ds_", "s_load", "s_buffer_load")):
+                hit = _vregs(operands) & flying
+                queue.append(frozenset())
+            else:
+                hit = _vregs(operands) & flying
+            if hit and report is not None:
+                report.append((label, t, sorted(hit)))
+            queue = queue[-LDS_QUEUE_CAP:]
+        return tuple(queue)
+
+    entry = [set() for _ in blocks]
+    entry[0].add(())
+    work = [(0, ())]
+    while work:
+        i, q = work.pop()
+        out = walk(blocks[i][1], q, None, None)
+        for j in succ[i]:
+            if out not in entry[j]:
+                assert len(entry[j]) < 512, "too many distinct LDS queues reach one block"
+                entry[j].add(out)
+                work.append((j, out))
+    bad = []
+    for i, (lab, ins) in enumerate(blocks):
+        for q in entry[i]:
+            walk(ins, q, bad, lab)
+    return bad
+
+
+def test_lds_checker_flags_a_register_reused_before_the_wait():
+    # the shape of the defect it was written for: operands of a step that does not follow are read at the end of a
+    # loop, and the epilogue's first values are placed in those registers ahead of the wait
+    racy = ["\tds_read_b128 v[32:35], v7 offset:64", "\tv_accvgpr_read_b32 v33, a1", "\ts_waitcnt lgkmcnt(0)"]
+    fine = ["\tds_read_b128 v[32:35], v7 offset:64", "\ts_waitcnt lgkmcnt(0)", "\tv_accvgpr_read_b32 v33, a1"]
+    partial = ["\tds_read_b128 v[32:35], v7", "\tds_read_b128 v[36:39], v7 offset:64", "\ts_waitcnt lgkmcnt(1)",
+               "\tv_mov_b32_e32 v0, v32", "\ts_waitcnt lgkmcnt(0)"]
+    partial_bad = partial[:3] + ["\tv_mov_b32_e32 v0, v36"] + partial[4:]
+    loop = ["\ts_branch .LBB0_2", ".LBB0_1:", "\tv_mov_b32_e32 v32, 0", "\ts_waitcnt lgkmcnt(0)", "\ts_endpgm", ".LBB0_2:",
+            "\ts_waitcnt lgkmcnt(0)", "\tds_read_b128 v[32:35], v7", "\ts_cbranch_scc1 .LBB0_2", "\ts_branch .LBB0_1"]
+    assert check_lds_reads_in_flight(racy) and not check_lds_reads_in_flight(fine)
+    assert not check_lds_reads_in_flight(partial) and check_lds_reads_in_flight(partial_bad)
+    assert check_lds_reads_in_flight(loop)
+
+
+def test_no_register_is_touched_while_an_lds_read_into_it_is_in_flight():
+    import glob
+
+    files = sorted(glob.glob(os.path.join(BUILD, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    if len(files) < 10:
+        pytest.skip("device assembly not kept: build the library first (python -m triton_amd.build)")
+    checked = 0
+    for f in files:
+        for name, lines in _functions(open(f).read()).items():
+            if not any(l.lstrip().startswith("ds_read") for l in lines):
+                continue
+            checked += 1
+            bad = check_lds_reads_in_flight(lines)
+            assert not bad, (os.path.basename(f), name, bad[:5])
+    assert checked >= 40, checked
+
+
+def check_m0_owner(lines):
+    """Rule 4: an LDS-direct load takes its LDS address from M0.  The kernels set M0 inside inline assembly for
+    their own such loads while the compiler sets it for the loads it generates from the builtin; each load must see
+    the M0 written by its own side.  Returns (instruction, who wrote M0) for every compiler-generated load whose M0
+    was last written inside inline assembly, and for every inline-assembly load whose M0 was last written by the
+    compiler (unknown at a label: code reached by a branch is not followed)."""
+    bad, in_asm, owner = [], False, None
+    for line in lines:
+        if "#ASMSTART" in line:
+            in_asm = True
+            continue
+        if "#ASMEND" in line:
+            in_asm = False
+            continue
+        code = line.split(";")[0].strip()
+        if not code:
+            continue
+        if re.match(r"^\.LBB\w+:", code):
+            owner = None
+            continue
+        op = code.split()[0]
+        operands = code[len(op):]
+        if op.startswith(("global_load_lds", "buffer_load")) and ("lds" in op or " lds" in operands):
+            mine = "asm" if in_asm else "compiler"
+            if owner is not None and owner != mine:
+                bad.append((code, owner))
+        elif op.startswith("s_") and re.match(r"\s*m0\b", operands):
+            owner = "asm" if in_asm else "compiler"
+    return bad
+
+
+def test_m0_checker_flags_a_compiler_write_moved_in_front_of_an_assembly_copy():
+    swapped = ["\ts_add_i32 m0, s9, 0x4000", "\t;;#ASMSTART", "\ts_mov_b32 m0, s33", "\ts_nop 0",
+               "\tglobal_load_lds_dwordx4 v147, s[26:27]", "\t;;#ASMEND", "\tglobal_load_lds_dword v[24:25], off"]
+    right = swapped[1:6] + [swapped[0], swapped[6]]
+    assert check_m0_owner(swapped) == [("global_load_lds_dword v[24:25], off", "asm")]
+    assert not check_m0_owner(right)
+
+
+def test_every_lds_direct_load_sees_the_m0_written_for_it():
+    import glob
+
+    files = sorted(glob.glob(os.path.join(BUILD, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    if len(files) < 10:
+        pytest.skip("device assembly not kept: build the library first (python -m triton_amd.build)")
+    checked = 0
+    for f in files:
+        for name, lines in _functions(open(f).read()).items():
+            if not any("global_load_lds" in l for l in lines):
+                continue
+            checked += 1
+            bad = check_m0_owner(lines)
+            assert not bad, (os.path.basename(f), name, bad[:5])
+    assert checked >= 40, checked
+
+
+VALU_MFMA_WAIT = 2
+ANYREG = re.compile(r"\b([va])(\d+|\[\d+:\d+\])")
+
+
+def _anyregs(text):
+    out = set()
+    for m in ANYREG.finditer(text):
+        t = m.group(2)
+        if t.startswith("["):
+            lo, hi = t[1:-1].split(":")
+            out.update((m.group(1), i) for i in range(int(lo), int(hi) + 1))
+        else:
+            out.add((m.group(1), int(t)))
+    return out
+
+
+def check_valu_write_to_assembly_mfma(lines):
+    """Rule 5: an MFMA must not read a vector or accumulation register within VALU_MFMA_WAIT issue slots of a VALU
+    instruction (v_accvgpr_write, v_mov, conversions ...) writing it.  The compiler keeps that distance for the
+    MFMAs it generates; for an MFMA inside inline assembly nobody does, so its operands must come from loads - or
+    the statement must start with the idle slots itself.  Returns (block label, instruction, slots) violations
+    over all control-flow paths; only MFMAs between #ASMSTART and #ASMEND are examined."""
+    blocks = [("entry", [])]
+    in_asm = False
+    for line in lines:
+        if "#ASMSTART" in line:
+            in_asm = True
+            continue
+        if "#ASMEND" in line:
+            in_asm = False
+            continue
+        code = line.split(";")[0].rstrip()
+        if not code.strip():
+            continue
+        m = re.match(r"^(\.LBB\w+):", code)
+        if m:
+            blocks.append((m.group(1), []))
+        elif code.startswith("\t") and not code.strip().startswith("."):
+            blocks[-1][1].append((code.strip(), in_asm))
+    index = {lab: i for i, (lab, _) in enumerate(blocks)}
+    succ = []
+    for i, (_, ins) in enumerate(blocks):
+        s, fall = set(), True
+        for t, _a in ins:
+            m = re.match(r"s_c?branch\w*\s+(\.LBB\w+)", t)
+            if m:
+                s.add(index[m.group(1)])
+            if t.startswith("s_branch") or t.startswith("s_endpgm") or t.startswith("s_setpc"):
+                fall = False
+        if fall and i + 1 < len(blocks):
+            s.add(i + 1)
+        succ.append(s)
+
+    def walk(ins, state, report, label):
+        state = dict(state)
+        for t, asm in ins:
+            op = t.split()[0]
+            operands = t[len(op):]
+            mfma = op.startswith(("v_mfma", "v_smfmac"))
+            if mfma and asm and report is not None:
+                for r in _anyregs(operands.split(",", 1)[1]):
+                    if r in state:
+                        report.append((label, t, state[r]))
+            m = re.match(r"s_nop\s+(\d+)", t)
+            step = int(m.group(1)) + 1 if m else 1
+            state = {r: d + step for r, d in state.items() if d + step < VALU_MFMA_WAIT}
+            if op.startswith("v_") and not mfma:
+                for r in _anyregs(operands.split(",", 1)[0]):
+                    state[r] = 0
+        return state
+
+    entry = [dict() for _ in blocks]
+    work = list(range(len(blocks)))
+    while work:
+        i = work.pop()
+        out = walk(blocks[i][1], entry[i], None, None)
+        for j in succ[i]:
+            changed = False
+            for r, d in out.items():
+                if entry[j].get(r, FAR) > d:
+                    entry[j][r] = d
+                    changed = True
+            if changed:
+                work.append(j)
+    bad = []
+    for i, (lab, ins) in enumerate(blocks):
+        walk(ins, entry[i], bad, lab)
+    return bad
+
+
+def test_valu_mfma_checker_flags_a_copy_right_in_front_of_an_assembly_mfma():
+    mfma = "\tv_mfma_f32_32x32x16_f16 v[32:47], v[124:127], a[88:91], 0"
+    close = ["\tv_accvgpr_write_b32 a91, v175", "\t;;#ASMSTART", mfma, "\t;;#ASMEND"]
+    settled = ["\tv_accvgpr_write_b32 a91, v175", "\t;;#ASMSTART", "\ts_nop 1", mfma, "\t;;#ASMEND"]
+    known = ["\tv_accvgpr_write_b32 a91, v175", mfma]     # the compiler's own MFMA: it has counted the slots itself
+    assert check_valu_write_to_assembly_mfma(close) and not check_valu_write_to_assembly_mfma(settled)
+    assert not check_valu_write_to_assembly_mfma(known)
+
+
+def test_no_assembly_mfma_reads_a_register_right_after_a_valu_write():
+    import glob
+
+    files = sorted(glob.glob(os.path.join(BUILD, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    if len(files) < 10:
+        pytest.skip("device assembly not kept: build the library first (python -m triton_amd.build)")
+    checked = 0
+    for f in files:
+        text = open(f).read()
+        if "#ASMSTART" not in text:
+            continue
+        for name, lines in _functions(text).items():
+            if not any("v_mfma" in l for l in lines):
+                continue
+            checked += 1
+            bad = check_valu_write_to_assembly_mfma(lines)
+            assert not bad, (os.path.basename(f), name, bad[:5])
+    assert checked >= 30, checked

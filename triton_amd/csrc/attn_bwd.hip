@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void attn_bwd_pre_kernel(AttnArgs p) {
   const int hz = blockIdx.y, z = hz / p.H, h = hz % p.H;
   const int c = threadIdx.x % LPR;
   float acc = 0.f;
-  if (row < p.N) {
+  if (row < p.N && c * 8 < p.d_real) {   // (head dims 16 / 32 run the 64-column form: the columns beyond d_real do not exist)
     int64_t off = ((int64_t)z * p.so[0] + (int64_t)h * p.so[1] + (int64_t)row * p.so[2]) * 2 + c * 16;
     V8 o = *(const V8*)(p.o + off);
     V8 d = *(const V8*)(p.d_o + off);
@@ -58,7 +58,9 @@ __global__ __launch_bounds__(256) void attn_bwd_pre_kernel(AttnArgs p) {
 // ---------------------------------------------------------------------------------------------
 // dQ: one wave owns QT*32 query rows; K / V tiles of 64 rows stream through LDS.
 // ---------------------------------------------------------------------------------------------
-template <typename V8, int D, int QT, int NW>
+// PAD (D = 64 only): p.d_real = 16 or 32 columns exist in memory; fragments loaded into registers are zero-filled,
+// the LDS tiles are zeroed once and only the chunks present are loaded, only the first d_real columns are stored.
+template <typename V8, int D, int QT, int NW, bool PAD = false>
 __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
   using S = typename ElemB<V8>::type;
   typedef __attribute__((ext_vector_type(4))) S S4;
@@ -97,8 +99,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     const char* sd = dobase + (int64_t)r * pitch + g * 16;
 #pragma unroll
     for (int ks = 0; ks < KSQ; ks++) {
-      qf[b][ks] = *(const V8*)(sq + ks * 32);
-      dof[b][ks] = *(const V8*)(sd + ks * 32);
+      if (!PAD || ks * 32 + g * 16 < p.d_real * 2) {
+        qf[b][ks] = *(const V8*)(sq + ks * 32);
+        dof[b][ks] = *(const V8*)(sd + ks * 32);
+      } else {
+        qf[b][ks] = V8{};
+        dof[b][ks] = V8{};
+      }
     }
     m_row[b] = p.lse[(int64_t)hz * p.N + r];
     d_row[b] = p.delta[(int64_t)hz * p.N + r];
@@ -106,17 +113,27 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
 
   // direct loads: scalar tile base + 32-bit lane offset (the host bounds the row pitch)
   unsigned offKV[Tile::INST];
+  bool present[Tile::INST];
 #pragma unroll
-  for (int i = 0; i < Tile::INST; i++) offKV[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+  for (int i = 0; i < Tile::INST; i++) {
+    offKV[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+    present[i] = !PAD || Tile::chunk_present(wave, lane, i, p.d_real * 2);
+  }
   const unsigned lds_base = lds_addr(lds);
+  if constexpr (PAD) {
+    lds_zero(lds, 2 * 2 * TILE, tid, NW * 64);
+    __syncthreads();
+  }
   auto issue_kv = [&](int j, int stage) {
     const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
     const char* ksrc = kbase + (int64_t)j * BN * pitch;
     const char* vsrc = vbase + (int64_t)j * BN * pitch;
 #pragma unroll
     for (int i = 0; i < Tile::INST; i++) {
-      async_copy16_sbase(ksrc, offKV[i], kd + (i * NW + wave) * 1024);
-      async_copy16_sbase(vsrc, offKV[i], vd + (i * NW + wave) * 1024);
+      if (present[i]) {
+        async_copy16_sbase(ksrc, offKV[i], kd + (i * NW + wave) * 1024);
+        async_copy16_sbase(vsrc, offKV[i], vd + (i * NW + wave) * 1024);
+      }
     }
   };
 
@@ -242,25 +259,25 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
         S4 v;
 #pragma unroll
         for (int e = 0; e < 4; e++) v[e] = (S)(dq[c][b][rg * 4 + e] * p.sm_scale);
-        *(S4*)(dst + d * 2) = v;
+        if (!PAD || d < p.d_real) *(S4*)(dst + d * 2) = v;
       }
   }
 }
 
-template <typename V8, int D>
+template <typename V8, int D, bool PAD = false>
 static int launch_bwd_d(const AttnArgs& p, hipStream_t stream) {
   {
     constexpr int QT = 1, NW = 4, BM = NW * QT * 32;
     constexpr int smem = 2 * 2 * 64 * D * 2;
     static bool attr_set = false;
     if (!attr_set) {
-      hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<V8, D, QT, NW>,
+      hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dq_kernel<V8, D, QT, NW, PAD>,
                                          hipFuncAttributeMaxDynamicSharedMemorySize, smem);
       if (e != hipSuccess) return (int)e;
       attr_set = true;
     }
     int nqb = (p.N + BM - 1) / BM;
-    attn_bwd_dq_kernel<V8, D, QT, NW><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+    attn_bwd_dq_kernel<V8, D, QT, NW, PAD><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
   }
@@ -271,7 +288,8 @@ int attn_bwd_dkdv_launch(const AttnArgs& p, bool bf16, hipStream_t stream);  // 
 
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
   int rc;
-  if (p.D == 256) rc = bf16 ? launch_bwd_d<bf16x8, 256>(p, stream) : launch_bwd_d<f16x8, 256>(p, stream);
+  if (p.d_real < p.D) rc = bf16 ? launch_bwd_d<bf16x8, 64, true>(p, stream) : launch_bwd_d<f16x8, 64, true>(p, stream);
+  else if (p.D == 256) rc = bf16 ? launch_bwd_d<bf16x8, 256>(p, stream) : launch_bwd_d<f16x8, 256>(p, stream);
   else if (bf16) rc = p.D == 128 ? launch_bwd_d<bf16x8, 128>(p, stream) : launch_bwd_d<bf16x8, 64>(p, stream);
   else rc = p.D == 128 ? launch_bwd_d<f16x8, 128>(p, stream) : launch_bwd_d<f16x8, 64>(p, stream);
   if (rc) return rc;

@@ -36,28 +36,41 @@ template <> struct ElemB<f16x8> { using type = _Float16; };
 // kernel's schedule provides them - a set of S / dP tiles is consumed one phase (at least sixteen
 // MFMAs) after the last MFMA that writes it, and the operands come from LDS reads and global
 // loads (waited for by count), never from VALU results.
+// SETTLE: the padded form does feed VALU results in - its K / V fragments are zero-filled, live in VGPRs and are
+// copied into AGPRs (v_accvgpr_write) right in front of the statement; an MFMA must not read a register within
+// two issue slots of a VALU write (the compiler keeps that distance for the MFMAs it knows), so the statement
+// starts with two idle slots.  tests/test_isa_hazards.py checks the rule on the generated code of every kernel.
+template <bool SETTLE>
 __device__ __forceinline__ void mfma32_first_v(f32x16& d, bf16x8 a, bf16x8 b) {
 #if MI355_DEVICE_PASS
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  if constexpr (SETTLE) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
 #endif
 }
+template <bool SETTLE>
 __device__ __forceinline__ void mfma32_first_v(f32x16& d, f16x8 a, f16x8 b) {
 #if MI355_DEVICE_PASS
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  if constexpr (SETTLE) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
 #endif
 }
+template <bool SETTLE>
 __device__ __forceinline__ void mfma32_acc_v(f32x16& d, bf16x8 a, bf16x8 b) {
 #if MI355_DEVICE_PASS
-  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  if constexpr (SETTLE) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
 #endif
 }
+template <bool SETTLE>
 __device__ __forceinline__ void mfma32_acc_v(f32x16& d, f16x8 a, f16x8 b) {
 #if MI355_DEVICE_PASS
-  asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  if constexpr (SETTLE) asm volatile("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  else asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
 #endif
 }
 
-template <typename V8, int D, int NW>
+// PAD (D = 64 only): p.d_real = 16 or 32 columns exist in memory (see attn_bwd_dq_kernel).
+template <typename V8, int D, int NW, bool PAD = false>
 __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   using S = typename ElemB<V8>::type;
   typedef __attribute__((ext_vector_type(4))) S S4;
@@ -96,8 +109,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     const char* sv = p.v + head_off + (int64_t)r * pitch + g * 16;
 #pragma unroll
     for (int ks = 0; ks < KSQ; ks++) {
-      kf[ks] = *(const V8*)(sk + ks * 32);
-      vf[ks] = *(const V8*)(sv + ks * 32);
+      if (!PAD || ks * 32 + g * 16 < p.d_real * 2) {
+        kf[ks] = *(const V8*)(sk + ks * 32);
+        vf[ks] = *(const V8*)(sv + ks * 32);
+      } else {
+        kf[ks] = V8{};
+        vf[ks] = V8{};
+      }
     }
   }
 
@@ -108,8 +126,16 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
 
   // direct loads: scalar tile base + 32-bit lane offset (the host bounds the row pitch)
   unsigned offQD[Tile::INST];
+  bool present[Tile::INST];
 #pragma unroll
-  for (int i = 0; i < Tile::INST; i++) offQD[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+  for (int i = 0; i < Tile::INST; i++) {
+    offQD[i] = (unsigned)Tile::off(pitch, wave, lane, i);
+    present[i] = !PAD || Tile::chunk_present(wave, lane, i, p.d_real * 2);
+  }
+  if constexpr (PAD) {
+    lds_zero(lds, NS * STAGE, tid, NW * 64);
+    __syncthreads();
+  }
   const char* const qsrc0 = qbase + (int64_t)m_begin * pitch;
   const char* const dsrc0 = dobase + (int64_t)m_begin * pitch;
   const unsigned lds_base = lds_addr(lds);
@@ -118,17 +144,20 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   const float* src_stat = ((wave & 1) == 0 ? lse : delta) + m_begin + lane;
   // stage-step js (clamped to the last one) into ring slot js % NS
   auto issue_stage = [&](int js) {
-    LDS_PTR(char) qd = lds + (js % NS) * STAGE;
     const unsigned qda = lds_base + (js % NS) * STAGE, dda = qda + TILE;
     const int jc = min(js, nsteps - 1);
     const char* qsrc = qsrc0 + (int64_t)jc * BM * pitch;
     const char* dsrc = dsrc0 + (int64_t)jc * BM * pitch;
 #pragma unroll
     for (int i = 0; i < Tile::INST; i++) {
-      async_copy16_sbase(qsrc, offQD[i], qda + (i * NW + wave) * 1024);
-      async_copy16_sbase(dsrc, offQD[i], dda + (i * NW + wave) * 1024);
+      // (every row has chunks that are present, so every wave still issues every load: the counts of the partial
+      // waits below stay what they are)
+      if (present[i]) {
+        async_copy16_sbase(qsrc, offQD[i], qda + (i * NW + wave) * 1024);
+        async_copy16_sbase(dsrc, offQD[i], dda + (i * NW + wave) * 1024);
+      }
     }
-    async_copy4(src_stat + jc * BM, (LDS_PTR(void))(qd + 2 * TILE + (wave & 1) * (BM * 4)));
+    async_copy4_asm(src_stat + jc * BM, qda + 2 * TILE + (wave & 1) * (BM * 4));
   };
 
   // per-lane LDS offsets inside a stage: row-wise operand per k-step, transposed operand per
@@ -222,11 +251,11 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     static_for<KSQ>([&](auto KS_) {
       constexpr int ks = decltype(KS_)::value;
       if constexpr (ks == 0) {
-        mfma32_first_v(sacc[par], __builtin_bit_cast(V8, rq[0]), kf[0]);
-        mfma32_first_v(dpacc[par], __builtin_bit_cast(V8, rd[0]), vf[0]);
+        mfma32_first_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[0]), kf[0]);
+        mfma32_first_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[0]), vf[0]);
       } else {
-        mfma32_acc_v(sacc[par], __builtin_bit_cast(V8, rq[ks]), kf[ks]);
-        mfma32_acc_v(dpacc[par], __builtin_bit_cast(V8, rd[ks]), vf[ks]);
+        mfma32_acc_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[ks]), kf[ks]);
+        mfma32_acc_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[ks]), vf[ks]);
       }
       if constexpr (do_x) {
         static_for<TRK>([&](auto O_) {
@@ -301,8 +330,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   const int nmasked = p.causal ? min(2, nsteps) : 0;
   for (int j = 0; j < nmasked; j++) stage_step(j, std::true_type{});
   for (int j = nmasked; j < nsteps; j++) stage_step(j, std::false_type{});
-  // nothing may still be writing this workgroup's LDS when it retires
+  // nothing may still be writing this workgroup's LDS when it retires - nor this wave's registers: the last C phase
+  // has read the rows and the M / delta values of tiles that do not follow, and the compiler, which takes those
+  // registers as written when the read was issued, would otherwise put dK / dV values into them ahead of the wait
+  // (a late read then lands on top of a result)
   wait_all();
+  settle_rows();
+  settle_stats();
 
   if (ncol < p.N) {
     char* dkd = p.dk + head_off + (int64_t)ncol * pitch;
@@ -318,8 +352,10 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
           a[e] = (S)(dk[c][rg * 4 + e] * p.sm_scale);
           b[e] = (S)dv[c][rg * 4 + e];
         }
-        *(S4*)(dkd + d * 2) = a;
-        *(S4*)(dvd + d * 2) = b;
+        if (!PAD || d < p.d_real) {
+          *(S4*)(dkd + d * 2) = a;
+          *(S4*)(dvd + d * 2) = b;
+        }
       }
   }
 }
@@ -519,23 +555,24 @@ static int launch_dkdv_256(const AttnArgs& p, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-template <typename V8, int D>
+template <typename V8, int D, bool PAD = false>
 static int launch_dkdv(const AttnArgs& p, hipStream_t stream) {
   constexpr int NW = 4, BN = NW * 32;
   constexpr int smem = 4 * (2 * 64 * D * 2 + 2 * 64 * 4);
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<V8, D, NW>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_bwd_dkdv_kernel<V8, D, NW, PAD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   int nkb = (p.N + BN - 1) / BN;
-  attn_bwd_dkdv_kernel<V8, D, NW><<<dim3(nkb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  attn_bwd_dkdv_kernel<V8, D, NW, PAD><<<dim3(nkb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int attn_bwd_dkdv_launch(const AttnArgs& p, bool bf16, hipStream_t stream) {
+  if (p.d_real < p.D) return bf16 ? launch_dkdv<bf16x8, 64, true>(p, stream) : launch_dkdv<f16x8, 64, true>(p, stream);
   if (p.D == 256) return bf16 ? launch_dkdv_256<bf16x8>(p, stream) : launch_dkdv_256<f16x8>(p, stream);
   if (bf16) return p.D == 128 ? launch_dkdv<bf16x8, 128>(p, stream) : launch_dkdv<bf16x8, 64>(p, stream);
   return p.D == 128 ? launch_dkdv<f16x8, 128>(p, stream) : launch_dkdv<f16x8, 64>(p, stream);

@@ -28,7 +28,11 @@ template <typename V8> struct Elem;
 template <> struct Elem<bf16x8> { using type = __bf16; };
 template <> struct Elem<f16x8> { using type = _Float16; };
 
-template <typename V8, int D, int QT, int NW>
+// PAD (D = 64 only): the tensors hold p.d_real = 16 or 32 columns per row; the missing columns are zeros that
+// never exist in memory - fragments loaded straight into registers are zero-filled, the K / V tiles in LDS are
+// zeroed once and only the chunks present are ever loaded, and only the first d_real columns of O are stored.
+// Scores, softmax and those columns of O are what a HEAD_DIM d_real kernel computes (zero columns add nothing).
+template <typename V8, int D, int QT, int NW, bool PAD = false>
 __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
   using S = typename Elem<V8>::type;
   constexpr int BM = NW * QT * 32, BN = 64;
@@ -70,27 +74,38 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     int r = min(row0 + b * 32 + l32, p.N - 1);
     const char* src = qbase + (int64_t)r * qpitch + g * 16;
 #pragma unroll
-    for (int ks = 0; ks < KSQ; ks++) qf[b][ks] = *(const V8*)(src + ks * 32);
+    for (int ks = 0; ks < KSQ; ks++) {
+      if (!PAD || ks * 32 + g * 16 < p.d_real * 2) qf[b][ks] = *(const V8*)(src + ks * 32);
+      else qf[b][ks] = V8{};
+    }
   }
 
   // ---- direct global -> LDS copies of the K and V tiles: a scalar tile base that advances with
   // the step plus a 32-bit per-lane offset (64 rows of K or V span less than 2^31 bytes, which the
   // host checks), so a load costs no vector arithmetic
   unsigned offK[INST], offV[INST];
+  bool present[INST];
 #pragma unroll
   for (int i = 0; i < INST; i++) {
     offK[i] = (unsigned)Tile::off(kpitch, wave, lane, i);
     offV[i] = (unsigned)Tile::off(vpitch, wave, lane, i);
+    present[i] = !PAD || Tile::chunk_present(wave, lane, i, p.d_real * 2);
   }
   const unsigned lds_base = lds_addr(lds);
+  if constexpr (PAD) {
+    lds_zero(lds, 2 * 2 * TILE, tid, NW * 64);
+    __syncthreads();
+  }
   auto issue_kv = [&](int j, int stage) {
     const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
     const char* ksrc = kbase + (int64_t)j * BN * kpitch;
     const char* vsrc = vbase + (int64_t)j * BN * vpitch;
 #pragma unroll
     for (int i = 0; i < INST; i++) {
-      async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
-      async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+      if (present[i]) {
+        async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
+        async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+      }
     }
   };
 
@@ -281,7 +296,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
         S4 v;
 #pragma unroll
         for (int e = 0; e < 4; e++) v[e] = (S)(oacc[c][b][rg * 4 + e] * inv);
-        *(S4*)(dst + d * 2) = v;
+        if (!PAD || d < p.d_real) *(S4*)(dst + d * 2) = v;
       }
   }
 }
@@ -295,7 +310,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
 // the causal mask odd rounds walk the query blocks short-to-long and even rounds long-to-short, so
 // every workgroup gets the same amount of work over two rounds.  One query tile (32 rows) per wave.
 // ---------------------------------------------------------------------------------------------
-template <typename V8, int D, int NW>
+template <typename V8, int D, int NW, bool PAD = false>   // PAD: as in attn_fwd_kernel
 __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kernel(AttnArgs p) {
   using S = typename Elem<V8>::type;
   constexpr int BM = NW * 32, BN = 64;
@@ -341,7 +356,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
     const int r = min(qb * BM + wave * 32 + l32, p.N - 1);
     const char* src = head_ptr(p.q, p.sq, hz) + (int64_t)r * qpitch + g * 16;
 #pragma unroll
-    for (int ks = 0; ks < KSQ; ks++) dst[ks] = *(const V8*)(src + ks * 32);
+    for (int ks = 0; ks < KSQ; ks++) {
+      if (!PAD || ks * 32 + g * 16 < p.d_real * 2) dst[ks] = *(const V8*)(src + ks * 32);
+      else dst[ks] = V8{};
+    }
   };
 
   // ---- state of the item being multiplied
@@ -365,12 +383,18 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
   const char* f_v = head_ptr(p.v, p.sv, c_hz);
   bool f_valid = true;
   unsigned offK[INST], offV[INST];
+  bool present[INST];
 #pragma unroll
   for (int i = 0; i < INST; i++) {
     offK[i] = (unsigned)Tile::off(kpitch, wave, lane, i);
     offV[i] = (unsigned)Tile::off(vpitch, wave, lane, i);
+    present[i] = !PAD || Tile::chunk_present(wave, lane, i, p.d_real * 2);
   }
   const unsigned lds_base = lds_addr(lds);
+  if constexpr (PAD) {
+    lds_zero(lds, 2 * 2 * TILE, tid, NW * 64);
+    __syncthreads();
+  }
   auto issue_fill = [&](int stage) {
     if (!f_valid) return;
     const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
@@ -378,8 +402,10 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
     const char* vsrc = f_v + (int64_t)fj * BN * vpitch;
 #pragma unroll
     for (int i = 0; i < INST; i++) {
-      async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
-      async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+      if (present[i]) {
+        async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
+        async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+      }
     }
     if (++fj == f_steps) {
       fj = 0;
@@ -545,7 +571,7 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
             S4 v;
 #pragma unroll
             for (int e = 0; e < 4; e++) v[e] = (S)(oacc[c][rg * 4 + e] * inv);
-            *(S4*)(dst + d * 2) = v;
+            if (!PAD || d < p.d_real) *(S4*)(dst + d * 2) = v;
           }
       }
     }
@@ -579,13 +605,13 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
   wait_all();
 }
 
-template <typename V8, int D, int NW>
+template <typename V8, int D, int NW, bool PAD = false>
 static int launch_fwd_stream(const AttnArgs& p, hipStream_t stream) {
   constexpr int BM = NW * 32;
   constexpr int smem = 2 * 2 * 64 * D * 2;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_stream_kernel<V8, D, NW>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_stream_kernel<V8, D, NW, PAD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
@@ -594,28 +620,30 @@ static int launch_fwd_stream(const AttnArgs& p, hipStream_t stream) {
   // as many workgroups as are resident at once: two per CU with four waves, one with eight
   int grid = p.num_programs > 0 ? p.num_programs * (NW == 4 ? 2 : 1) : total;
   if (grid > total) grid = total;
-  attn_fwd_stream_kernel<V8, D, NW><<<dim3(grid), dim3(NW * 64), smem, stream>>>(p);
+  attn_fwd_stream_kernel<V8, D, NW, PAD><<<dim3(grid), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
-template <typename V8, int D, int QT, int NW>
+template <typename V8, int D, int QT, int NW, bool PAD = false>
 static int launch_fwd(const AttnArgs& p, hipStream_t stream) {
   constexpr int BM = NW * QT * 32;
   constexpr int smem = 2 * 2 * 64 * D * 2;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<V8, D, QT, NW>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd_kernel<V8, D, QT, NW, PAD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   int nqb = (p.N + BM - 1) / BM;
-  attn_fwd_kernel<V8, D, QT, NW><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  attn_fwd_kernel<V8, D, QT, NW, PAD><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 template <typename V8>
 static int launch_fwd_d(const AttnArgs& p, int variant, hipStream_t stream) {
+  // head dims 16 / 32: the 64-column kernels in their padding form (eight waves; persistent under the causal mask)
+  if (p.d_real < p.D) return p.causal ? launch_fwd_stream<V8, 64, 8, true>(p, stream) : launch_fwd<V8, 64, 1, 8, true>(p, stream);
   if (variant == 3 && p.D != 256) return p.D == 128 ? launch_fwd_stream<V8, 128, 4>(p, stream) : launch_fwd_stream<V8, 64, 4>(p, stream);
   if (variant == 4 && p.D != 256) return p.D == 128 ? launch_fwd_stream<V8, 128, 8>(p, stream) : launch_fwd_stream<V8, 64, 8>(p, stream);
   // head_dim 256: four waves of 32 query rows, one wave per SIMD (the O accumulator alone is 128 registers)

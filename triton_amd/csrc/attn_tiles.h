@@ -50,10 +50,23 @@ struct AttnTile {
     int lc = (lane % CPR) ^ tile_swz<RB>(r);
     return (int64_t)r * pitch + lc * 16;
   }
+  // the lane's source chunk lies inside the first `row_bytes` bytes of its row (rows narrower than RB: the rest of
+  // the tile is zero-filled once and never loaded)
+  __device__ static bool chunk_present(int wave, int lane, int i, int row_bytes) {
+    int r = (i * NW + wave) * RPI + lane / CPR;
+    int lc = (lane % CPR) ^ tile_swz<RB>(r);
+    return lc * 16 < row_bytes;
+  }
   __device__ static const char* src(const char* base, int64_t pitch, int wave, int lane, int i) {
     return base + off(pitch, wave, lane, i);
   }
 };
+
+// Zero the `bytes` of LDS at `base` with all `nthreads` threads of the workgroup (padded tiles: the chunks that no
+// load ever writes must read as zeros); the caller synchronises afterwards.
+__device__ __forceinline__ void lds_zero(LDS_PTR(char) base, int bytes, int tid, int nthreads) {
+  for (int o = tid * 16; o < bytes; o += nthreads * 16) *(LDS_PTR(i32x4))(base + o) = i32x4{0, 0, 0, 0};
+}
 
 // Row-wise operand read.  Lane (l32 = lane % 32, g = lane / 32) of MFMA k-step ks reads chunk
 // 2*ks + g of row l32 (+ 32 per sub-tile, which leaves the swizzle unchanged):

@@ -421,11 +421,13 @@ int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* st
 static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype, bool allow_256 = false) {
   if (Z <= 0 || H <= 0 || N_CTX <= 0) return MI355_EINVAL;
   if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
-  // head_dim 256: 16-bit forward and backward (not the fp8 forward)
-  if (D != 64 && D != 128 && !(allow_256 && D == 256)) return MI355_ESHAPE;
+  // head_dim 256 and the padded forms of head dims 16 / 32: 16-bit forward and backward (not the fp8 forward)
+  const bool small = allow_256 && (D == 16 || D == 32);
+  if (D != 64 && D != 128 && !(allow_256 && D == 256) && !small) return MI355_ESHAPE;
   if (N_CTX % 128 != 0) return MI355_ESHAPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
-  p.Z = Z; p.H = H; p.N = N_CTX; p.D = D;
+  // 16 / 32: the 64-column kernels, which pad with zeros on the fly (loads, LDS tiles and stores know d_real)
+  p.Z = Z; p.H = H; p.N = N_CTX; p.D = small ? 64 : D; p.d_real = D;
   return MI355_OK;
 }
 

@@ -57,6 +57,12 @@ __device__ __forceinline__ void async_copy16(const void* gsrc, LDS_PTR(void) lds
 // and a 32-bit per-lane byte offset: the address add happens in the memory pipeline instead of
 // costing a 64-bit vector add per load.  `lds_wave_base` must be wave-uniform.  The load is
 // invisible to the compiler's wait-count bookkeeping: callers wait with wait_vmcnt<>.
+// The statement writes M0 behind the compiler's back (M0 is a reserved register: a clobber is not honoured), and
+// the compiler sets M0 itself for the LDS-direct loads it generates from the builtin (async_copy4 / async_copy16)
+// and is free to move that write across this statement - the builtin's load then lands at this copy's address.
+// A kernel therefore uses EITHER the builtin forms OR the inline-assembly forms (async_copy4_asm for 4 bytes),
+// never both; tests/test_isa_hazards.py checks on the generated code that every LDS-direct load sees an M0
+// written by its own side.
 //
 // SETTLE: a vector-memory instruction must not read a scalar register within 5 issue slots of a VALU
 // instruction writing it - and that is how the compiler restores a SPILLED scalar register (v_readlane_b32),
@@ -113,6 +119,15 @@ __device__ __forceinline__ void load16_sbase(V& dst, const void* sbase, unsigned
 __device__ __forceinline__ void async_copy4(const void* gsrc, LDS_PTR(void) lds_wave_base) {
 #if MI355_DEVICE_PASS
   __builtin_amdgcn_global_load_lds(gsrc, lds_wave_base, 4, 0, 0);
+#endif
+}
+
+// The same as one inline-assembly statement, for kernels whose other LDS-direct copies are inline assembly (see
+// async_copy16_sbase: the compiler must not own M0 anywhere in such a kernel).  Not counted by the compiler: wait
+// with wait_vmcnt<>.
+__device__ __forceinline__ void async_copy4_asm(const void* gsrc, unsigned lds_wave_base) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" :: "v"(gsrc), "s"(lds_wave_base) : "memory");
 #endif
 }
 

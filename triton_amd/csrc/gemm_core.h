@@ -1270,8 +1270,25 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
       }
     }
   }
-  // nothing may still be writing this workgroup's LDS when it retires
+  // nothing may still be writing this workgroup's LDS when it retires - nor this wave's registers: the last half of
+  // the loop has read the operands of a step that does not follow, and the compiler, which sees those registers as
+  // written when the read was issued, is free to put the epilogue's values into them ahead of the wait.  Keeping
+  // them live across the wait closes that.
   wait_all();
+#pragma unroll
+  for (int s = 0; s < (KSPLIT ? 2 : 1); s++)
+#pragma unroll
+    for (int t = 0; t < MT; t++) lds_use(fa[s][t]);
+#pragma unroll
+  for (int s = 0; s < 2; s++)
+#pragma unroll
+    for (int t = 0; t < NT; t++) lds_use(fb[s][t]);
+  if constexpr (Cfg::kScaled) {
+#pragma unroll
+    for (int t = 0; t < MT; t++) lds_use(sa_in[t]);
+#pragma unroll
+    for (int t = 0; t < NT; t++) lds_use(sb_in[t]);
+  }
 
   // Last, partial K step (unscaled types only): its 16-byte chunks past K are written as zeros (the
   // reference masks them to 0, python/tutorials/03-matrix-multiplication.py:297-298).  Goes through

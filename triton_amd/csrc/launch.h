@@ -84,6 +84,7 @@ struct AttnArgs {
   int causal;
   int variant;  // tiling variant (tuning knob)
   int num_programs;  // persistent forward: CUs to fill (0 = one workgroup per item)
+  int d_real;   // head dims 16 / 32: columns present in memory (D is then 64: the kernels pad with zeros on the fly)
 };
 
 // Device-side tables of a grouped GEMM (layout of python/tutorials/08-grouped-gemm.py:66-77).

@@ -432,15 +432,10 @@ class _attention(torch.autograd.Function):
 def attention(q, k, v, causal, sm_scale):
     """`attention(q, k, v, causal, sm_scale)` of the reference (06:520, `_attention.apply`).
 
-    Head dims 64, 128 and 256 run the kernels directly, forward and backward.  The reference also admits 16
-    and 32 (06:447): for those q, k and v are zero-padded to 64 columns - the scores, the softmax and
-    the first HEAD_DIM columns of every output and gradient are unchanged by zero columns - and the
-    result is sliced back; autograd carries the gradients through the padding."""
-    D = q.shape[-1]
-    if D in (16, 32) and q.dtype in (torch.float16, torch.bfloat16):
-        pad = (0, 64 - D)
-        qp, kp, vp = (torch.nn.functional.pad(t, pad) for t in (q, k, v))
-        return _attention.apply(qp, kp, vp, causal, sm_scale)[..., :D]
+    Head dims 64, 128 and 256 have kernels of their own, forward and backward.  The reference also admits 16
+    and 32 (06:447): those run the 64-column kernels in a form that pads with zeros on the fly - the rows are
+    loaded as they are (32 or 64 bytes), the missing columns never exist in memory, and only the first
+    HEAD_DIM columns of every output and gradient are stored - so no padded copies are made."""
     return _attention.apply(q, k, v, causal, sm_scale)
 
 
