@@ -540,3 +540,110 @@ def test_no_assembly_mfma_reads_a_register_right_after_a_valu_write():
             bad = check_valu_write_to_assembly_mfma(lines)
             assert not bad, (os.path.basename(f), name, bad[:5])
     assert checked >= 30, checked
+
+
+def check_assembly_mfma_results(lines):
+    """Rule 1 for every kernel and both register files: the destination of an MFMA issued inside inline assembly
+    (the compiler does not know it is one) must not be read or overwritten by a non-MFMA instruction, nor read as
+    the A / B operand of another MFMA, within MIN_WAIT issue slots - on any control-flow path.  (An MFMA taking it
+    as its addend is interlocked by the hardware.)"""
+    blocks = [("entry", [])]
+    in_asm = False
+    for line in lines:
+        if "#ASMSTART" in line:
+            in_asm = True
+            continue
+        if "#ASMEND" in line:
+            in_asm = False
+            continue
+        code = line.split(";")[0].rstrip()
+        if not code.strip():
+            continue
+        m = re.match(r"^(\.LBB\w+):", code)
+        if m:
+            blocks.append((m.group(1), []))
+        elif code.startswith("\t") and not code.strip().startswith("."):
+            blocks[-1][1].append((code.strip(), in_asm))
+    index = {lab: i for i, (lab, _) in enumerate(blocks)}
+    succ = []
+    for i, (_, ins) in enumerate(blocks):
+        s, fall = set(), True
+        for t, _a in ins:
+            m = re.match(r"s_c?branch\w*\s+(\.LBB\w+)", t)
+            if m:
+                s.add(index[m.group(1)])
+            if t.startswith("s_branch") or t.startswith("s_endpgm") or t.startswith("s_setpc"):
+                fall = False
+        if fall and i + 1 < len(blocks):
+            s.add(i + 1)
+        succ.append(s)
+
+    def walk(ins, state, report, label):
+        state = dict(state)
+        for t, asm in ins:
+            op = t.split()[0]
+            operands = t[len(op):]
+            mfma = op.startswith(("v_mfma", "v_smfmac"))
+            if mfma:
+                parts = [x.strip() for x in operands.split(",")]
+                touched = _anyregs(",".join(parts[1:3]))        # A and B operands (the addend is interlocked)
+            else:
+                touched = _anyregs(operands)
+            if report is not None:
+                for r in touched:
+                    if r in state:
+                        report.append((label, t, state[r]))
+            m = re.match(r"s_nop\s+(\d+)", t)
+            step = int(m.group(1)) + 1 if m else 1
+            state = {r: d + step for r, d in state.items() if d + step < MIN_WAIT}
+            if mfma and asm:
+                for r in _anyregs(operands.split(",", 1)[0]):
+                    state[r] = 0
+        return state
+
+    entry = [dict() for _ in blocks]
+    work = list(range(len(blocks)))
+    while work:
+        i = work.pop()
+        out = walk(blocks[i][1], entry[i], None, None)
+        for j in succ[i]:
+            changed = False
+            for r, d in out.items():
+                if entry[j].get(r, FAR) > d:
+                    entry[j][r] = d
+                    changed = True
+            if changed:
+                work.append(j)
+    bad = []
+    for i, (lab, ins) in enumerate(blocks):
+        walk(ins, entry[i], bad, lab)
+    return bad
+
+
+def test_assembly_mfma_result_checker_covers_vector_register_destinations():
+    mfma = ["\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_f16 v[32:47], v[124:127], a[88:91], 0", "\t;;#ASMEND"]
+    assert check_assembly_mfma_results(mfma + ["\tv_fma_f32 v0, v33, v161, -v92"])
+    assert not check_assembly_mfma_results(mfma + ["\ts_nop 11", "\tv_fma_f32 v0, v33, v161, -v92"])
+    # accumulating into the same tile right away is fine; feeding it to another MFMA as an operand is not
+    assert not check_assembly_mfma_results(mfma + ["\tv_mfma_f32_32x32x16_f16 v[32:47], v[0:3], a[0:3], v[32:47]"])
+    assert check_assembly_mfma_results(mfma + ["\tv_mfma_f32_32x32x16_f16 v[48:63], v[32:35], a[0:3], 0"])
+
+
+def test_no_result_of_an_assembly_mfma_is_touched_before_it_retires_in_any_kernel():
+    import glob
+
+    files = sorted(glob.glob(os.path.join(BUILD, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+    if len(files) < 10:
+        pytest.skip("device assembly not kept: build the library first (python -m triton_amd.build)")
+    checked = 0
+    for f in files:
+        text = open(f).read()
+        if "#ASMSTART" not in text:
+            continue
+        for name, lines in _functions(text).items():
+            if not any("v_mfma" in l for l in lines):
+                continue
+            checked += 1
+            bad = check_assembly_mfma_results(lines)
+            assert not bad, (os.path.basename(f), name, bad[:5])
+    assert checked >= 30, checked
