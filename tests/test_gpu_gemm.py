@@ -710,3 +710,39 @@ def test_stream_k_schedule_is_bit_exact_on_integers(gpu, monkeypatch, dtype, npr
         a2, b2 = randn_rounded(rng, (768, 1024), dtype), randn_rounded(rng, (1024, 512), dtype)
         c = to_np(triton_amd.matmul_streamk(from_np(a2, dtype, gpu), from_np(b2, dtype, gpu)))
         assert np.allclose(c, gemm.matmul_closed_form(a2, b2, out_dtype=dtype), rtol=1e-2, atol=1e-2)
+
+
+def test_lean_and_general_epilogue_of_the_four_wave_kernels_agree_bit_for_bit(gpu, monkeypatch):
+    # the four-wave kernels have a lean epilogue (16-bit C with unit column stride, per-tensor scales, nothing else)
+    # as instantiations of their own; MI355_GEMM_LEAN_EPILOGUE=0 sends the same products through the general one
+    rng = np.random.default_rng(77)
+    M = N = 2560
+    K = 1024
+    a16, b16 = (randn_rounded(rng, s, "bf16", 1.0) for s in ((M, K), (K, N)))
+    ta, tb = from_np(a16, "bf16", gpu), from_np(b16, "bf16", gpu)
+    q = lambda shape: torch.from_numpy(rng.integers(0, 0x78, size=shape).astype(np.uint8)).to(gpu).view(torch.float8_e4m3fn)
+    qa, qb = q((M, K)), q((N, K))
+    pa, pb = (torch.from_numpy(rng.integers(0, 256, size=(M, K // 2)).astype(np.uint8)).to(gpu) for _ in range(2))
+    sa, sb = (torch.from_numpy(rng.integers(123, 132, size=(M, K // 32)).astype(np.uint8)).to(gpu) for _ in range(2))
+    cases = {
+        "bf16": lambda: triton_amd.matmul(ta, tb),
+        "bf16 K-major B, K tail": lambda: triton_amd.matmul(ta[:, :K - 8].contiguous(), tb.t().contiguous().t()[:K - 8]),
+        "fp8 scaled -> bf16": lambda: triton_amd.matmul(qa, qb.t(), a_scale=0.37, b_scale=1.9, out_dtype=torch.bfloat16),
+        "fp8 scaled -> fp16": lambda: triton_amd.matmul(qa, qb.t(), a_scale=0.01, b_scale=0.02, out_dtype=torch.float16),
+        "mxfp4 -> bf16": lambda: triton_amd.mx_matmul(pa, sa, pb, sb, "mxfp4", out_dtype=torch.bfloat16),
+        "mxfp8 -> fp16": lambda: triton_amd.mx_matmul(pa.repeat(1, 2) & 0x77, sa, pb.repeat(1, 2) & 0x77, sb, "mxfp8", out_dtype=torch.float16),
+    }
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    results = {}
+    for lean in ("1", "0"):
+        set_knob(monkeypatch, "MI355_GEMM_LEAN_EPILOGUE", lean)
+        for name, fn in cases.items():
+            if lean == "0" and "K tail" in name:
+                continue        # (the tail form exists with the lean epilogue only; without it another kernel runs)
+            results[name, lean] = to_np(fn())
+    for name in cases:
+        if "K tail" in name:
+            ref = a16[:, :K - 8].astype(np.float64) @ b16[:K - 8].astype(np.float64)
+            assert np.allclose(results[name, "1"], ref, atol=1e-2 * np.abs(ref).max(), rtol=1e-2), name
+        else:
+            assert bits_equal(results[name, "1"], results[name, "0"]), name

@@ -593,12 +593,13 @@ def check_assembly_mfma_results(lines):
                 for r in touched:
                     if r in state:
                         report.append((label, t, state[r]))
-            m = re.match(r"s_nop\s+(\d+)", t)
-            step = int(m.group(1)) + 1 if m else 1
-            state = {r: d + step for r, d in state.items() if d + step < MIN_WAIT}
             if mfma and asm:
                 for r in _anyregs(operands.split(",", 1)[0]):
                     state[r] = 0
+            # (the MFMA's own slot counts, as in check_function: MIN_WAIT = required wait states + 1)
+            m = re.match(r"s_nop\s+(\d+)", t)
+            step = int(m.group(1)) + 1 if m else 1
+            state = {r: d + step for r, d in state.items() if d + step < MIN_WAIT}
         return state
 
     entry = [dict() for _ in blocks]
@@ -623,7 +624,8 @@ def check_assembly_mfma_results(lines):
 def test_assembly_mfma_result_checker_covers_vector_register_destinations():
     mfma = ["\t;;#ASMSTART", "\tv_mfma_f32_32x32x16_f16 v[32:47], v[124:127], a[88:91], 0", "\t;;#ASMEND"]
     assert check_assembly_mfma_results(mfma + ["\tv_fma_f32 v0, v33, v161, -v92"])
-    assert not check_assembly_mfma_results(mfma + ["\ts_nop 11", "\tv_fma_f32 v0, v33, v161, -v92"])
+    assert not check_assembly_mfma_results(mfma + ["\ts_nop 10", "\tv_fma_f32 v0, v33, v161, -v92"])   # 11 wait states
+    assert check_assembly_mfma_results(mfma + ["\ts_nop 9", "\tv_fma_f32 v0, v33, v161, -v92"])
     # accumulating into the same tile right away is fine; feeding it to another MFMA as an operand is not
     assert not check_assembly_mfma_results(mfma + ["\tv_mfma_f32_32x32x16_f16 v[32:47], v[0:3], a[0:3], v[32:47]"])
     assert check_assembly_mfma_results(mfma + ["\tv_mfma_f32_32x32x16_f16 v[48:63], v[32:35], a[0:3], 0"])

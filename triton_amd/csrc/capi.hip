@@ -44,7 +44,7 @@ const DeviceInfo& device_info() {
 constexpr int UNSET = INT_MIN;
 struct Knobs {
   int force_strided, group_m, tile, programs, skinny, grouped_big_min, grouped_wave128_min_k, grouped_chunk,
-      attn_fwd_variant, attn_programs;
+      attn_fwd_variant, attn_programs, lean_epilogue;
 };
 Knobs g_knobs;
 std::atomic<int> g_knobs_ready{0};
@@ -70,6 +70,7 @@ void load_knobs() {
   k.grouped_chunk = read_env("MI355_GROUPED_CHUNK", 1);
   k.attn_fwd_variant = read_env("MI355_ATTN_FWD_VARIANT", 0);
   k.attn_programs = read_env("MI355_ATTN_PROGRAMS", 1);
+  k.lean_epilogue = read_env("MI355_GEMM_LEAN_EPILOGUE", 0);
   g_knobs = k;
   g_knobs_ready.store(1, std::memory_order_release);
 }
@@ -175,6 +176,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // four consecutive C elements as one store: rows of 16-bit / fp32 elements 16-byte aligned (for fp8 that
   // makes every group of four 4-byte aligned)
   p.c_vec_ok = scn == 1 && scm % 4 == 0 && aligned(C, 16);
+  p.lean_ok = knob(knobs().lean_epilogue, 1);
   p.aux = aux; p.aux_sm = aux_sm; p.aux_sn = aux_sn; p.aux_dtype = aux_dtype;
 
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
@@ -193,7 +195,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // (an epilogue addend: instantiations of their own)
   // (fp8 from three quarters of a round: at 144 tiles the eight-wave kernel is 4-7 % ahead - 3072^3 1520 vs
   // 1450, 3072x3072x8192 2040 vs 1890 TFLOP/s -, at 196 tiles the four-wave one by 2 %, at 225 by 13 %)
-  const bool w128_ok = gemm_wave128_ok(p, b_kmajor) && (!is8 || p.k_bytes % 256 == 0);   // (a K tail: the 16-bit forms only)
+  const bool w128_ok = gemm_wave128_ok(p, b_kmajor, in_dtype) && (!is8 || p.k_bytes % 256 == 0);   // (a K tail: the 16-bit forms only)
   if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && w128_ok) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : knob(knobs().tile, tile);
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
@@ -221,10 +223,10 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true, in_dtype)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
-  if (tile == 6 && gemm_wave128_ok(p, b_kmajor)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
+  if (tile == 6 && gemm_wave128_ok(p, b_kmajor, in_dtype)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 
@@ -389,6 +391,7 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   p.out_dtype = out_dtype;
   p.group_m = knob(knobs().group_m, 8);
   p.c_vec_ok = ldc % 4 == 0 && aligned(C, 16);
+  p.lean_ok = knob(knobs().lean_epilogue, 1);
   p.sA = sA; p.sB = sB; p.lds_a = lds_a; p.lds_b = lds_b;
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);

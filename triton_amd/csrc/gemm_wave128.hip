@@ -42,7 +42,8 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 
 // The tiles `tile`, `tile + tile_step`, ... (< `tile_stop`, by default M/256 * N/256) of one problem, computed by the calling workgroup
 // with the 128 KiB of LDS at `lds0`.  XCD: pass the tile numbers through the per-XCD remap first.  EPI: 0 = scales,
-// activation, any output type; 1 = C has the type of the operands, no scales, no activation; 2 = 0 plus the addend.
+// activation, any output type; 1 = C has the type of the operands, no scales, no activation; 2 = 0 plus the addend;
+// 3 = the lean epilogue (gemm_epilogue16_lean) with C in the operands' type.
 // TAIL: K bytes need not be a multiple of 256; what is left behind the last pair of K steps (16 .. 240 bytes of
 // every operand row) is multiplied after the K loop, 64 bytes at a time, through a 32 KiB LDS buffer of its own
 // behind the two stages (which by then hold the next tile's first steps): plain loads with a zero fill, one
@@ -317,7 +318,9 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     // registers throughout the K loop)
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
-    if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>>(acc, p, em, en, el, ek);
+    using OwnT = std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>;
+    if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, OwnT>(acc, p, em, en, el, ek);
+    else if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, OwnT>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
     tile += tile_step;
     if (tile >= tend) break;
@@ -329,11 +332,11 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 }
 
 // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
-template <typename V8, bool B_KMAJOR, bool AUX, bool TAIL = false>
+template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-  gemm_wave128_tiles<V8, B_KMAJOR, true, AUX ? 2 : 0, TAIL>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
+  gemm_wave128_tiles<V8, B_KMAJOR, true, EPI, TAIL>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
 #endif
 }
 
@@ -414,7 +417,8 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 #endif
 }
 
-template <int FMT, bool AUX>
+// EPI: 0 = general epilogue, 2 = with the addend, 3 / 4 = lean epilogue writing fp16 / bf16
+template <int FMT, int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -552,7 +556,9 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
-    gemm_epilogue16<MT, NT, AUX>(acc, p, em, en, el, ek);
+    if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
+    else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
+    else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
     tile += gridDim.x;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
@@ -562,49 +568,52 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #endif
 }
 
-template <int FMT, bool AUX>
+template <int FMT, int EPI>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, AUX>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_f8_kernel<FMT, AUX><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_f8_kernel<FMT, EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
-  if (p.aux) return e5m2 ? launch_wave128_f8<1, true>(p, stream) : launch_wave128_f8<0, true>(p, stream);
-  return e5m2 ? launch_wave128_f8<1, false>(p, stream) : launch_wave128_f8<0, false>(p, stream);
+  if (p.aux) return e5m2 ? launch_wave128_f8<1, 2>(p, stream) : launch_wave128_f8<0, 2>(p, stream);
+  const int lean = lean_epilogue_type(p);
+  if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3>(p, stream) : launch_wave128_f8<0, 3>(p, stream);
+  if (lean == 2) return e5m2 ? launch_wave128_f8<1, 4>(p, stream) : launch_wave128_f8<0, 4>(p, stream);
+  return e5m2 ? launch_wave128_f8<1, 0>(p, stream) : launch_wave128_f8<0, 0>(p, stream);
 }
 
-bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor) {
+bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
   // whole tiles, at least one pair of 128-byte K steps (what is left behind the last pair: the TAIL form, which
-  // has no addend instantiation), 32-bit lane offsets
+  // exists for 16-bit operands with the lean epilogue - C in the operands' type - only), 32-bit lane offsets
   if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 16 == 0 && p.k_bytes >= 256)) return false;
-  if (p.k_bytes % 256 != 0 && p.aux) return false;
+  if (p.k_bytes % 256 != 0 && !((in_dtype == 0 || in_dtype == 1) && lean_epilogue_type(p) == in_dtype + 1)) return false;
   if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
   // (row-major B: the per-load XOR of the column group acts on the whole lane offset, so the row term
   // in it - a multiple of the pitch - must leave the bits of the 512-byte tile row alone)
   return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
-template <typename V8, bool B_KMAJOR, bool AUX, bool TAIL = false>
+template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + (TAIL ? 2 * 256 * 64 : 0);   // (with the tail buffer: all 160 KiB of the CU)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, AUX, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_kernel<V8, B_KMAJOR, AUX, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -625,17 +634,19 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
   return bf16 ? launch_wave128_grouped<bf16x8>(ga, nprog, stream) : launch_wave128_grouped<f16x8>(ga, nprog, stream);
 }
 
+template <typename V8>
+static int gemm_wave128_launch_typed(const GemmArgs& p, bool b_kmajor, bool own_type_lean, hipStream_t stream) {
+  if (p.k_bytes % 256 != 0)   // (gemm_wave128_ok: the lean epilogue then)
+    return b_kmajor ? launch_wave128<V8, true, 3, true>(p, stream) : launch_wave128<V8, false, 3, true>(p, stream);
+  if (p.aux) return b_kmajor ? launch_wave128<V8, true, 2>(p, stream) : launch_wave128<V8, false, 2>(p, stream);
+  if (own_type_lean) return b_kmajor ? launch_wave128<V8, true, 3>(p, stream) : launch_wave128<V8, false, 3>(p, stream);
+  return b_kmajor ? launch_wave128<V8, true, 0>(p, stream) : launch_wave128<V8, false, 0>(p, stream);
+}
+
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream) {
-  if (p.k_bytes % 256 != 0) {   // (gemm_wave128_ok: no addend then)
-    if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, false, true>(p, stream) : launch_wave128<f16x8, true, false, true>(p, stream);
-    return bf16 ? launch_wave128<bf16x8, false, false, true>(p, stream) : launch_wave128<f16x8, false, false, true>(p, stream);
-  }
-  if (p.aux) {
-    if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, true>(p, stream) : launch_wave128<f16x8, true, true>(p, stream);
-    return bf16 ? launch_wave128<bf16x8, false, true>(p, stream) : launch_wave128<f16x8, false, true>(p, stream);
-  }
-  if (b_kmajor) return bf16 ? launch_wave128<bf16x8, true, false>(p, stream) : launch_wave128<f16x8, true, false>(p, stream);
-  return bf16 ? launch_wave128<bf16x8, false, false>(p, stream) : launch_wave128<f16x8, false, false>(p, stream);
+  const bool own_type_lean = lean_epilogue_type(p) == (bf16 ? 2 : 1);   // lean epilogue, C in the operands' type
+  return bf16 ? gemm_wave128_launch_typed<bf16x8>(p, b_kmajor, own_type_lean, stream)
+              : gemm_wave128_launch_typed<f16x8>(p, b_kmajor, own_type_lean, stream);
 }
 
 }  // namespace mi355

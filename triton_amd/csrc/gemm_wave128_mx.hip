@@ -20,6 +20,8 @@ __device__ __forceinline__ void mfma16_mxfp8(const i32x8& a, const i32x8& b, f32
 // MXFP8 (e4m3 codes, one e8m0 scale per 32 elements): the fp8 kernel above with scaled MFMAs; a K step is
 // 128 elements = four scale blocks, the scales travel 16 bytes per row (four K steps) per direct load into a
 // two-slot LDS ring like those of the MXFP4 kernel below.
+// EPI: 0 = general epilogue, 3 / 4 = lean epilogue (gemm_epilogue16_lean) writing fp16 / bf16
+template <int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -195,7 +197,9 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
-    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
+    else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
+    else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
     tile += gridDim.x;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
@@ -213,18 +217,24 @@ bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
          p.lds_a * 64 + p.k_bytes / 32 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 32 < (1ll << 31);
 }
 
-int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
+template <int EPI>
+static int launch_wave128_mxfp8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp8_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp8_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
+}
+
+int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
+  const int lean = lean_epilogue_type(p);
+  return lean == 1 ? launch_wave128_mxfp8<3>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4>(p, stream) : launch_wave128_mxfp8<0>(p, stream);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -251,6 +261,8 @@ __device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32
 #endif
 }
 
+// EPI: 0 = general epilogue, 3 / 4 = lean epilogue (gemm_epilogue16_lean) writing fp16 / bf16
+template <int EPI>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -440,7 +452,9 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
-    gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
+    if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
+    else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
+    else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
     tile += gridDim.x;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
@@ -458,18 +472,24 @@ bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
          p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
 }
 
-int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
+template <int EPI>
+static int launch_wave128_mxfp4(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp4_kernel<<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp4_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
+}
+
+int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
+  const int lean = lean_epilogue_type(p);
+  return lean == 1 ? launch_wave128_mxfp4<3>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4>(p, stream) : launch_wave128_mxfp4<0>(p, stream);
 }
 
 }  // namespace mi355
