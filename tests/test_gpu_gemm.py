@@ -746,3 +746,36 @@ def test_lean_and_general_epilogue_of_the_four_wave_kernels_agree_bit_for_bit(gp
             assert np.allclose(results[name, "1"], ref, atol=1e-2 * np.abs(ref).max(), rtol=1e-2), name
         else:
             assert bits_equal(results[name, "1"], results[name, "0"]), name
+
+
+@pytest.mark.parametrize("case", ["bf16 row-major B", "fp16 K-major B", "fp8"])
+def test_k_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_zero_padding(gpu, case):
+    # rows that are not 16-byte multiples cannot be loaded by the MFMA kernels; the wrapper appends the zeros that the
+    # reference's K-tail mask stands for (03:297-298) instead of leaving the product to the strided kernel
+    rng = np.random.default_rng(5)
+    M, N = 512, 768
+    if case == "fp8":
+        K = 4104      # a multiple of 8 but not of 16 bytes
+        a = rng.integers(0, 0x78, size=(M, K)).astype(np.uint8)
+        b = rng.integers(0, 0x78, size=(N, K)).astype(np.uint8)
+        ta = torch.from_numpy(a).to(gpu).view(torch.float8_e4m3fn)
+        tb = torch.from_numpy(b).to(gpu).view(torch.float8_e4m3fn).t()
+        got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+        ref = ta.float().cpu().numpy().astype(np.float64) @ tb.float().cpu().numpy().astype(np.float64)
+        assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max())
+        return
+    K = 4100
+    dtype = "bf16" if case.startswith("bf16") else "fp16"
+    a, b = randn_rounded(rng, (M, K), dtype, 1.0), randn_rounded(rng, (K, N), dtype, 1.0)
+    ta, tb = from_np(a, dtype, gpu), from_np(b, dtype, gpu)
+    if "K-major" in case:
+        tb = tb.t().contiguous().t()
+    got = to_np(triton_amd.matmul(ta, tb))
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert got.shape == (M, N)
+    assert np.allclose(got, ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+    # integer-valued operands: exact sums, so the padded product is the strided kernel's product bit for bit
+    ai = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    bi = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    exact = to_np(triton_amd.matmul(from_np(ai, dtype, gpu), from_np(bi, dtype, gpu), out_dtype=torch.float32))
+    assert bits_equal(exact, (ai.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))

@@ -108,6 +108,7 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     _check_device(1, b)
     M, K = a.shape
     K, N = b.shape
+    K_caller = K
     if out_dtype is None:
         out_dtype = torch.bfloat16 if in_dt == _lib.BF16 else torch.float16
     if activation not in ("", "leaky_relu"):
@@ -118,6 +119,20 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         return c
     if K == 0:
         return c.zero_()
+    if (in_dt != _lib.F32 and (K * _ELEM_BYTES[in_dt]) % 16 != 0 and M * N * K >= 1 << 24
+            and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)):
+        # Rows of A that are not a multiple of 16 bytes long do not start on 16-byte boundaries, which every MFMA
+        # kernel's loads need: the C ABI then runs its strided kernel (4096 x 4096 x 4100 bf16: 43 TFLOP/s).  The
+        # reference masks the K tail to zero (03:297-298); appending those zeros to K here - one copy of each
+        # operand - gives the same sums on the fast kernels (the same shape: 1000 TFLOP/s).
+        pad = -K % (16 // _ELEM_BYTES[in_dt])
+        as_bytes = (lambda t: t.view(torch.uint8)) if _ELEM_BYTES[in_dt] == 1 else (lambda t: t)
+        a = torch.nn.functional.pad(as_bytes(a), (0, pad)).view(a.dtype)
+        if b.stride(0) == 1 and b.stride(1) != 1:      # K-major B: its K axis is the contiguous one of b.t()
+            b = torch.nn.functional.pad(as_bytes(b.t()), (0, pad)).view(b.dtype).t()
+        else:
+            b = torch.nn.functional.pad(as_bytes(b), (0, 0, 0, pad)).view(b.dtype)
+        K += pad        # (the launch metadata below keeps the caller's K)
     if (in_dt in (_lib.F8E4M3, _lib.F8E5M2) and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
             and K % 16 == 0 and M * N * K >= 1 << 24):
         # fp8 MFMAs want both operands K-contiguous: a row-major fp8 B is put into that layout first, as the
@@ -128,7 +143,7 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     pb, keep_b = _scale_ptr(b_scale, device)
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
     stream = _stream()
-    md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K, _ELEM_BYTES[in_dt]))
+    md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K_caller, _ELEM_BYTES[in_dt]))
     ext = _lib.ext()
     if ext is not None and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
         # the PyTorch-ROCm extension: tensors in, torch's current stream taken in C++, one C-ABI call
