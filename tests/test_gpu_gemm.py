@@ -779,3 +779,35 @@ def test_k_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_zero_paddin
     bi = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
     exact = to_np(triton_amd.matmul(from_np(ai, dtype, gpu), from_np(bi, dtype, gpu), out_dtype=torch.float32))
     assert bits_equal(exact, (ai.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("kmajor", [False, True])
+@pytest.mark.parametrize("shape", [(192, 256, 256), (1536, 1024, 1280), (3072, 768, 512)])
+def test_four_wave_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, dtype, kmajor, shape):
+    # M a multiple of 192: the four-wave kernel also runs on tiles of 192 x 256 (chosen by itself where they fill
+    # the CUs better, forced here); small integers make every sum exact
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    ta, tb = from_np(a, dtype, gpu), from_np(b, dtype, gpu)
+    if kmajor:
+        tb = tb.t().contiguous().t()
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    set_knob(monkeypatch, "MI355_GEMM_TILE_M", "192")
+    got = to_np(triton_amd.matmul(ta, tb))
+    assert bits_equal(got, to_np(from_np(ref, dtype, gpu))), "tiles of 192 rows"
+    set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
+    assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got), "tiles of 256 rows"
+
+
+def test_3072_cubed_takes_the_192_row_tiles_and_matches_sampled_rows(gpu):
+    # 144 tiles of 256 x 256 for 256 CUs, 192 tiles of 192 x 256: the size heuristic picks the latter
+    rng = np.random.default_rng(11)
+    n = 3072
+    a, b = randn_rounded(rng, (n, n), "bf16", 1.0), randn_rounded(rng, (n, n), "bf16", 1.0)
+    got = to_np(triton_amd.matmul(from_np(a, "bf16", gpu), from_np(b, "bf16", gpu)))
+    rows = rng.choice(n, size=24, replace=False)
+    ref = a[rows].astype(np.float64) @ b.astype(np.float64)
+    assert np.allclose(got[rows], ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())

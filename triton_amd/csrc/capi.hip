@@ -44,7 +44,7 @@ const DeviceInfo& device_info() {
 constexpr int UNSET = INT_MIN;
 struct Knobs {
   int force_strided, group_m, tile, programs, skinny, grouped_big_min, grouped_wave128_min_k, grouped_chunk,
-      attn_fwd_variant, attn_programs, lean_epilogue;
+      attn_fwd_variant, attn_programs, lean_epilogue, tile_m;
 };
 Knobs g_knobs;
 std::atomic<int> g_knobs_ready{0};
@@ -71,6 +71,7 @@ void load_knobs() {
   k.attn_fwd_variant = read_env("MI355_ATTN_FWD_VARIANT", 0);
   k.attn_programs = read_env("MI355_ATTN_PROGRAMS", 1);
   k.lean_epilogue = read_env("MI355_GEMM_LEAN_EPILOGUE", 0);
+  k.tile_m = read_env("MI355_GEMM_TILE_M", 0);
   g_knobs = k;
   g_knobs_ready.store(1, std::memory_order_release);
 }
@@ -198,6 +199,17 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const bool w128_ok = gemm_wave128_ok(p, b_kmajor, in_dtype) && (!is8 || p.k_bytes % 256 == 0);   // (a K tail: the 16-bit forms only)
   if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && w128_ok) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : knob(knobs().tile, tile);
+  // 16-bit products whose 256 x 256 tiles fill the last round of CUs badly (or whose M is a multiple of 192 only): the
+  // same kernel on tiles of 192 x 256 where those use the CUs better (3072^3: 192 tiles instead of 144 for 256 CUs)
+  if (!is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 192) && gemm_wave128_192_ok(p, b_kmajor, in_dtype)) {
+    auto fill = [&](long t) { return t <= 0 ? 0.0 : (double)t / (double)(((t + cus - 1) / cus) * cus); };
+    const long tiles192 = (long)(M / 192) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    if (want == 192 || (want == 0 && tiles192 * 2 >= cus && (tile != 6 || fill(tiles192) > fill(tiles256) + 0.08))) {
+      tile = 6;
+      p.tile_m = 192;
+    }
+  }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;
@@ -226,7 +238,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true, in_dtype)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
-  if (tile == 6 && gemm_wave128_ok(p, b_kmajor, in_dtype)) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
+  if (tile == 6 && (p.tile_m == 192 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 

@@ -49,12 +49,16 @@ __device__ __forceinline__ void mfma16(f16x8 a, f16x8 b, f32x4& c) {
 // behind the two stages (which by then hold the next tile's first steps): plain loads with a zero fill, one
 // un-pipelined sub-step each - a per-tile cost of a few microseconds that only products with such a K pay
 // (the reference's own uneven-K shape 8192 x 8192 x 8176, python/test/regression/test_performance.py:46).
-template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0, bool TAIL = false>
+template <typename V8, bool B_KMAJOR, bool XCD, int EPI = 0, bool TAIL = false, int BM = 256>
 __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, const int tile_step, const unsigned lds0, const int tile_stop = -1) {
 #if MI355_DEVICE_PASS
-  constexpr int BM = 256, BN = 256, ROWB = 128;
-  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
-  constexpr int MT = 8, NT = 8, KS = 2;                             // 16x16 tiles per wave, 16x16x32 sub-steps per stage
+  // BM = 192: tiles of 192 x 256 (96 x 128 per wave) for problems whose 256 x 256 tiles would leave a quarter or more of
+  // the CUs idle - only the A side changes: six direct loads per wave and K step instead of eight, six fragments
+  static_assert((BM == 256 || BM == 192) && !(TAIL && BM != 256), "tile heights");
+  constexpr int BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
+  constexpr int MT = BM / 32, NT = 8, KS = 2;                       // 16x16 tiles per wave, 16x16x32 sub-steps per stage
+  constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
   constexpr int NM = MT * NT;                                       // MFMAs per sub-step
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -100,7 +104,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   const char* gA;
   const char* gB;
   auto set_fill_tile = [&](int fm, int fn) {
-    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    gA = p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda;
     gB = B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb
                   : p.B + (int64_t)fn * BN * 2 + (int64_t)(wave * 16) * p.ldb;
   };
@@ -109,10 +113,11 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   const unsigned kstepB = B_KMAJOR ? ROWB : 64 * (unsigned)p.ldb;   // bytes from one K step to the next
   // load j (0..7: A, 8..15: B) of tile kt into the stage at `stage_base`.  M0 = middle of the wave's
   // 8 KiB of that operand, instruction offsets -4096 .. 3072 (taken back out of the scalar base).
+  auto load_of = [](int slot) constexpr { return slot < LA ? slot : 8 + slot - LA; };   // load slot -> j (A: 0 .. LA-1, B: 8 .. 15)
   auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
     const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
-    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned dst = stage_base + (j < 8 ? wave * (LA * 1024) : A_BYTES + wave * 8192) + 4096;
     unsigned lane_off;
     if constexpr (j < 8) lane_off = voffA[j & 1] + (unsigned)kt * ROWB;
     else if constexpr (B_KMAJOR) lane_off = voffB[j & 1] + (unsigned)kt * ROWB;
@@ -127,7 +132,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       const unsigned slot = ((4 * ks + kg) ^ s) * 16;
-      adrA[ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      adrA[ks] = lds0 + (wm * (BM / 2) + l16) * ROWB + slot;
       if constexpr (B_KMAJOR) adrB[ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
     }
     // row-major B: lane i of the 16-lane group kg addresses k row 8 kg + i / 4 (+ 32 ks, + 4 for the second
@@ -139,7 +144,6 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
       for (int t = 0; t < NT; t++) adrB[t] = lds0 + A_BYTES + k * (BN * 2) + ((wn * 8 + (t ^ m)) * 32) + (l16 & 3) * 8;
     }
   }
-  static_assert(STAGE == 65536, "stage 1 = stage 0 + 64 KiB");
   struct Frags { V8 a[MT]; V8 b[NT]; };
   Frags f[2];
   constexpr int NRD = MT + NT;  // fragment reads per sub-step (a row-major B fragment takes two instructions)
@@ -176,9 +180,9 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   zero_acc();
 
   // ---- prologue: both stages requested, first fragments of stage 0 read
-  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
-  wait_vmcnt<16>();
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, 0, lds0, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, 1, lds0 + STAGE, std::true_type{}); });
+  wait_vmcnt<NLOADS>();
   block_barrier();
   using Z = std::integral_constant<int, 0>;
   static_for<NRD>([&](auto OP_) { read_one(OP_, Z{}, Z{}, f[0]); });
@@ -208,7 +212,9 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
       if constexpr (more && n % 2 == 0 && n / 2 < NRD)
         read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, last ? (P ^ 1) : P>{},
                  std::integral_constant<int, last ? 0 : ks + 1>{}, f[nxt]);
-      if constexpr (refill && n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, kt + 2, lds0 + P * STAGE, std::false_type{});
+      constexpr int every = NM / 16;   // MFMAs per load slot: 4 (64 MFMAs) or 3 (48)
+      if constexpr (refill && n % every == 1 && n / every < NLOADS)
+        issue(std::integral_constant<int, load_of(n / every)>{}, kt + 2, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -316,7 +322,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     // (the tile and lane coordinates pass through an empty assembly statement so that none of the
     // epilogue's address arithmetic is hoisted out of the tile loop, where it would occupy - and spill -
     // registers throughout the K loop)
-    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    int em = pm * BM + wm * (BM / 2), en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
     using OwnT = std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>;
     if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, OwnT>(acc, p, em, en, el, ek);
@@ -332,11 +338,11 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 }
 
 // Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
-template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false>
+template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
-  gemm_wave128_tiles<V8, B_KMAJOR, true, EPI, TAIL>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
+  gemm_wave128_tiles<V8, B_KMAJOR, true, EPI, TAIL, BM>(p, blockIdx.x, gridDim.x, lds_addr((LDS_PTR(const void))lds_raw));
 #endif
 }
 
@@ -602,18 +608,28 @@ bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
   return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
-template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false>
+// The 192 x 256 tiles: M a multiple of 192, whole pairs of K steps, C in the operands' type through the lean epilogue
+// (the one instantiation per type and B layout).  Worth it where the 256 x 256 tiles leave CUs idle in the last round:
+// 3072^3 has 144 of those for 256 CUs and 192 of these.
+bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
+  if (!(p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  if (!((in_dtype == 0 || in_dtype == 1) && lean_epilogue_type(p) == in_dtype + 1)) return false;
+  if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
+  return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
+}
+
+template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false, int BM = 256>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + (TAIL ? 2 * 256 * 64 : 0);   // (with the tail buffer: all 160 KiB of the CU)
+  constexpr int smem = 2 * (BM + 256) * 128 + (TAIL ? 2 * 256 * 64 : 0);   // (with the tail buffer: all 160 KiB of the CU)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int tiles = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / BM) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL, BM><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -636,6 +652,8 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 
 template <typename V8>
 static int gemm_wave128_launch_typed(const GemmArgs& p, bool b_kmajor, bool own_type_lean, hipStream_t stream) {
+  if (p.tile_m == 192)   // (gemm_wave128_192_ok: whole K steps, the lean epilogue)
+    return b_kmajor ? launch_wave128<V8, true, 3, false, 192>(p, stream) : launch_wave128<V8, false, 3, false, 192>(p, stream);
   if (p.k_bytes % 256 != 0)   // (gemm_wave128_ok: the lean epilogue then)
     return b_kmajor ? launch_wave128<V8, true, 3, true>(p, stream) : launch_wave128<V8, false, 3, true>(p, stream);
   if (p.aux) return b_kmajor ? launch_wave128<V8, true, 2>(p, stream) : launch_wave128<V8, false, 2>(p, stream);

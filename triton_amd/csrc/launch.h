@@ -23,6 +23,7 @@ struct GemmArgs {
   int num_programs;  // persistent kernels: workgroups to launch (0 = not persistent)
   float* workspace;  // stream-K: 2 * num_programs tiles of 256x256 fp32 (NULL = no stream-K)
   int c_vec_ok;   // scn == 1 and every C row start is 16-byte aligned
+  int tile_m;     // four-wave 16-bit kernel: 0 / 256 = tiles of 256 x 256, 192 = tiles of 192 x 256
   int lean_ok;    // the four-wave kernels may take their lean epilogue (tuning knob MI355_GEMM_LEAN_EPILOGUE, default 1)
   // optional addend of the epilogue: acc * alpha + aux[m * aux_sm + n * aux_sn] (a zero stride broadcasts
   // a row or a column vector), added in fp32 before the activation; NULL = none
@@ -107,6 +108,7 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream);
+bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype);   // the same for tiles of 192 x 256
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype);   // in_dtype: C ABI code of the operands' type
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream);
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
