@@ -798,6 +798,8 @@ def test_four_wave_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, dt
     set_knob(monkeypatch, "MI355_GEMM_TILE_M", "192")
     got = to_np(triton_amd.matmul(ta, tb))
     assert bits_equal(got, to_np(from_np(ref, dtype, gpu))), "tiles of 192 rows"
+    set_knob(monkeypatch, "MI355_GEMM_TILE_M", "128")
+    assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got), "tiles of 128 rows"
     set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
     assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got), "tiles of 256 rows"
 

@@ -210,6 +210,17 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 192;
     }
   }
+  // and on tiles of 128 x 256 where the 256 x 256 tiles are too few for their kernel (less than half a round) but these
+  // fill most of one round (2560^3: 100 and 200 tiles; 716 -> 825 TFLOP/s against the 128 x 128 tiles)
+  if (!is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 128) && p.tile_m == 0 &&
+      gemm_wave128_192_ok(p, b_kmajor, in_dtype, 128)) {
+    const long tiles128 = (long)(M / 128) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    if (want == 128 || (want == 0 && tile == 1 && tiles128 * 10 >= cus * 7 && tiles128 <= cus)) {
+      tile = 6;
+      p.tile_m = 128;
+    }
+  }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;

@@ -54,7 +54,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
 #if MI355_DEVICE_PASS
   // BM = 192: tiles of 192 x 256 (96 x 128 per wave) for problems whose 256 x 256 tiles would leave a quarter or more of
   // the CUs idle - only the A side changes: six direct loads per wave and K step instead of eight, six fragments
-  static_assert((BM == 256 || BM == 192) && !(TAIL && BM != 256), "tile heights");
+  static_assert((BM == 256 || BM == 192 || BM == 128) && !(TAIL && BM != 256), "tile heights");
   constexpr int BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
   constexpr int MT = BM / 32, NT = 8, KS = 2;                       // 16x16 tiles per wave, 16x16x32 sub-steps per stage
@@ -611,8 +611,8 @@ bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
 // The 192 x 256 tiles: M a multiple of 192, whole pairs of K steps, C in the operands' type through the lean epilogue
 // (the one instantiation per type and B layout).  Worth it where the 256 x 256 tiles leave CUs idle in the last round:
 // 3072^3 has 144 of those for 256 CUs and 192 of these.
-bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
-  if (!(p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int tile_m) {
+  if (!(p.M % tile_m == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
   if (!((in_dtype == 0 || in_dtype == 1) && lean_epilogue_type(p) == in_dtype + 1)) return false;
   if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
   return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
@@ -654,6 +654,8 @@ template <typename V8>
 static int gemm_wave128_launch_typed(const GemmArgs& p, bool b_kmajor, bool own_type_lean, hipStream_t stream) {
   if (p.tile_m == 192)   // (gemm_wave128_192_ok: whole K steps, the lean epilogue)
     return b_kmajor ? launch_wave128<V8, true, 3, false, 192>(p, stream) : launch_wave128<V8, false, 3, false, 192>(p, stream);
+  if (p.tile_m == 128)
+    return b_kmajor ? launch_wave128<V8, true, 3, false, 128>(p, stream) : launch_wave128<V8, false, 3, false, 128>(p, stream);
   if (p.k_bytes % 256 != 0)   // (gemm_wave128_ok: the lean epilogue then)
     return b_kmajor ? launch_wave128<V8, true, 3, true>(p, stream) : launch_wave128<V8, false, 3, true>(p, stream);
   if (p.aux) return b_kmajor ? launch_wave128<V8, true, 2>(p, stream) : launch_wave128<V8, false, 2>(p, stream);
