@@ -80,49 +80,61 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   asm volatile("" : "+s"(nk_last));
 
   // ---- direct loads: instruction q = 8 * wave + j moves rows 8 q .. 8 q + 7 of a tile; the swizzle of
-  // those rows is 4 (q & 1) + lane / 16, so the lane offset depends on the parity of j only
+  // those rows is 4 (q & 1) + lane / 16.  Each of a wave's loads has a lane offset of its own - row, chunk, and the
+  // instruction offset taken back out - and the loads of one operand share one scalar base, the K step being
+  // fetched: two scalar additions per K step are all the address arithmetic of the loop.  (Sixteen scalar
+  // bases instead - one per load, rebuilt from the tile base at every load once that base changes inside the
+  // loop - were 56 scalar instructions per K step.)
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[2], voffB[B_KMAJOR ? 2 : 1];
+  auto ioff_of = [](int q) constexpr { return (q - 4) * 1024; };
+  unsigned voffA[LA], voffB[8];
 #pragma unroll
-  for (int par = 0; par < 2; par++) {
-    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
-    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
-    if constexpr (B_KMAJOR) voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  for (int q = 0; q < LA; q++) {
+    const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)ioff_of(q);
   }
   // Row-major B[K, N]: the stage holds 64 k rows of 512 bytes; instruction q = 8 * wave + j moves the k rows
   // 2 q, 2 q + 1 (lane i: row i / 32, physical 16-byte chunk i % 32).  Element (k, n) lives in the 32-byte
   // column group (n / 16) ^ 2 (k & 3) ^ ((k >> 3) & 1) of its row: a transpose read is served two 16-lane
   // groups at a time - four consecutive k rows each, eight rows apart, the same 16 columns - and this
   // spreads those 8 x 32 bytes over all banks.  With k = 16 wave + 2 j + i / 32 the XOR terms are
-  // 4 (j & 1) + 2 (i / 32) and (j >> 2) & 1: the j terms are XORed into the lane offset at each load.
-  if constexpr (!B_KMAJOR) {
-    const unsigned pg = (lane & 31) >> 1, half = lane & 1;
-    // j = 0; other j: XOR below (which needs a pitch that is a multiple of 512 bytes)
-    voffB[0] = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;
+  // 4 (j & 1) + 2 (i / 32) and (j >> 2) & 1 (which needs a pitch that is a multiple of 512 bytes).
+#pragma unroll
+  for (int q = 0; q < 8; q++) {
+    if constexpr (B_KMAJOR) {
+      const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+      voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)ioff_of(q);
+    } else {
+      const unsigned pg = (lane & 31) >> 1, half = lane & 1;
+      const unsigned v0 = (lane >> 5) * (unsigned)p.ldb + ((pg ^ (2 * (lane >> 5))) * 32) + half * 16;
+      voffB[q] = (v0 ^ ((4 * (q & 1) + ((q >> 2) & 1)) * 32)) + 2 * q * (unsigned)p.ldb - (unsigned)ioff_of(q);
+    }
   }
-  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
-  const char* gA;
-  const char* gB;
+  // scalar bases of the K step the loads are fetching (two K steps ahead of the MFMAs)
+  const char* fA;
+  const char* fB;
+  // (wave-uniform values, but the grouped kernel reads its pointers from device tables with vector loads: the
+  // scalar operand of the load instructions needs them in scalar registers)
+  auto scalar_ptr = [](const char* x) {
+    const uint64_t v = (uint64_t)x;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const char*)(((uint64_t)hi << 32) | lo);
+  };
   auto set_fill_tile = [&](int fm, int fn) {
-    gA = p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda;
-    gB = B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb
-                  : p.B + (int64_t)fn * BN * 2 + (int64_t)(wave * 16) * p.ldb;
+    fA = scalar_ptr(p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda);
+    fB = scalar_ptr(B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb
+                             : p.B + (int64_t)fn * BN * 2 + (int64_t)(wave * 16) * p.ldb);
   };
   set_fill_tile(pm, pn);
-  const int64_t stepA = 8 * p.lda, stepB = (B_KMAJOR ? 8 : 2) * p.ldb;
   const unsigned kstepB = B_KMAJOR ? ROWB : 64 * (unsigned)p.ldb;   // bytes from one K step to the next
-  // load j (0..7: A, 8..15: B) of tile kt into the stage at `stage_base`.  M0 = middle of the wave's
-  // 8 KiB of that operand, instruction offsets -4096 .. 3072 (taken back out of the scalar base).
+  // load j (0..7: A, 8..15: B) of the K step at (srcA, srcB) into the stage at `stage_base`.  M0 = middle of the
+  // wave's 8 KiB of that operand, instruction offsets -4096 .. 3072.
   auto load_of = [](int slot) constexpr { return slot < LA ? slot : 8 + slot - LA; };   // load slot -> j (A: 0 .. LA-1, B: 8 .. 15)
-  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+  auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
     const unsigned dst = stage_base + (j < 8 ? wave * (LA * 1024) : A_BYTES + wave * 8192) + 4096;
-    unsigned lane_off;
-    if constexpr (j < 8) lane_off = voffA[j & 1] + (unsigned)kt * ROWB;
-    else if constexpr (B_KMAJOR) lane_off = voffB[j & 1] + (unsigned)kt * ROWB;
-    else lane_off = (voffB[0] ^ ((4 * (q & 1) + ((q >> 2) & 1)) * 32)) + (unsigned)kt * kstepB;
-    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+    if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
+    else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
 
   // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 4 ks + kg of row l16 (+ 16 t)
@@ -180,8 +192,10 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   zero_acc();
 
   // ---- prologue: both stages requested, first fragments of stage 0 read
-  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, 0, lds0, std::true_type{}); });
-  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, 1, lds0 + STAGE, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA, fB, lds0, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA + ROWB, fB + kstepB, lds0 + STAGE, std::true_type{}); });
+  fA += 2 * ROWB;
+  fB += 2 * (int64_t)kstepB;
   wait_vmcnt<NLOADS>();
   block_barrier();
   using Z = std::integral_constant<int, 0>;
@@ -192,7 +206,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   // (every wave has then read all it needs of this stage, and the other stage has landed), reads the
   // first fragments of the other stage and refills this one with the tile two steps ahead (one load
   // per four MFMAs).
-  auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_, int kt) {
+  auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_) {
     constexpr int P = decltype(P_)::value, ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
     constexpr bool last = ks == KS - 1;
     constexpr bool more = decltype(MORE_)::value;              // there is a next sub-step to read for
@@ -214,16 +228,16 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
                  std::integral_constant<int, last ? 0 : ks + 1>{}, f[nxt]);
       constexpr int every = NM / 16;   // MFMAs per load slot: 4 (64 MFMAs) or 3 (48)
       if constexpr (refill && n % every == 1 && n / every < NLOADS)
-        issue(std::integral_constant<int, load_of(n / every)>{}, kt + 2, lds0 + P * STAGE, std::false_type{});
+        issue(std::integral_constant<int, load_of(n / every)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   using T = std::true_type; using F = std::false_type;
-  // A K step: `fk` is the K step (of the tile the scalar bases point at) that its loads fetch.
-  auto stage = [&](auto P_, int fk) {
-    substep(P_, I0{}, T{}, F{}, fk - 2);
-    substep(P_, I1{}, T{}, T{}, fk - 2);
+  // A K step; its loads fetch the K step that the scalar bases point at.
+  auto stage = [&](auto P_) {
+    substep(P_, I0{}, T{}, F{});
+    substep(P_, I1{}, T{}, T{});
     // The fragment reads above are invisible to the compiler: have them landed before control reaches a loop
     // edge, where the register allocator may copy the registers they write.  (They were issued over the first
     // half of the sub-step, so this does not wait.)
@@ -235,21 +249,21 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;   // next K step to fetch, and the tile it belongs to
   auto advance = [&]() {
+    fA += ROWB;
+    fB += kstepB;
     if (++fk == nk) {
       fk = 0;
-      if (ftile + tile_step < tend) {
-        ftile += tile_step;
-        int fm, fn;
-        tile_at(ftile, fm, fn);
-        set_fill_tile(fm, fn);
-      }
+      if (ftile + tile_step < tend) ftile += tile_step;
+      int fm, fn;
+      tile_at(ftile, fm, fn);
+      set_fill_tile(fm, fn);
     }
   };
   if (nk == 2) { fk = 1; advance(); }   // (two steps per tile: the prologue fetched both, the cursor is on the next tile)
   while (true) {
     for (int kt = 0; kt < nk; kt += 2) {
-      stage(I0{}, fk); advance();
-      stage(I1{}, fk); advance();
+      stage(I0{}); advance();
+      stage(I1{}); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
     if constexpr (TAIL) {
@@ -447,30 +461,29 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
   asm volatile("" : "+s"(nk_last));
 
-  // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
+  // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes): a lane offset per load,
+  // one scalar base per operand that moves with the K step being fetched
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[2], voffB[2];
+  unsigned voffA[8], voffB[8];
 #pragma unroll
-  for (int par = 0; par < 2; par++) {
-    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
-    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
-    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  for (int q = 0; q < 8; q++) {
+    const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
-  // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
-  const char* gA;
-  const char* gB;
+  // scalar bases of the K step the loads are fetching (two K steps ahead of the MFMAs)
+  const char* fA;
+  const char* fB;
   auto set_fill_tile = [&](int fm, int fn) {
-    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
-    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
   };
   set_fill_tile(pm, pn);
-  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
-  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+  auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
     const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
-    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
-    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+    if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
+    else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
 
   // ---- fragment reads: lane (l16, kg) wants the chunks kg, 4 + kg of row l16 (+ 16 t)
@@ -502,8 +515,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   zero_acc();
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
-  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  fA += 2 * ROWB;
+  fB += 2 * ROWB;
   wait_vmcnt<16>();
   block_barrier();
 #pragma unroll
@@ -511,8 +526,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #pragma unroll
   for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
 
-  // One K step on stage P with the B fragments of set `cur`; its loads fetch K step `fk` of the fill tile.
-  auto step = [&](auto P_, auto CUR_, int fk) {
+  // One K step on stage P with the B fragments of set `cur`; its loads fetch the K step the scalar bases point at.
+  auto step = [&](auto P_, auto CUR_) {
     constexpr int P = decltype(P_)::value, cur = decltype(CUR_)::value, nxt = cur ^ 1;
     constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
     // first half: rows 0..3 of A; the A fragments 4..7 of this stage are read meanwhile
@@ -532,7 +547,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
       if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
-      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE, std::false_type{});
+      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -542,21 +557,21 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;
   auto advance = [&]() {
+    fA += ROWB;
+    fB += ROWB;
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) {
-        ftile += gridDim.x;
-        int fm, fn;
-        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
-        set_fill_tile(fm, fn);
-      }
+      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      int fm, fn;
+      grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+      set_fill_tile(fm, fn);
     }
   };
   if (nk == 2) { fk = 1; advance(); }
   while (true) {
     for (int kt = 0; kt < nk; kt += 2) {
-      step(I0{}, I0{}, fk); advance();
-      step(I1{}, I1{}, fk); advance();
+      step(I0{}, I0{}); advance();
+      step(I1{}, I1{}); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
     mfma_drain(acc);

@@ -46,33 +46,33 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   asm volatile("" : "+s"(nk_last));
 
   // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes)
+  // (a lane offset per load - row, chunk, and the instruction offset taken back out - and one scalar base per
+  // operand that moves with the K step being fetched)
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[2], voffB[2];
+  unsigned voffA[8], voffB[8];
 #pragma unroll
-  for (int par = 0; par < 2; par++) {
-    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
-    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
-    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  for (int q = 0; q < 8; q++) {
+    const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
   // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
-  const char* gA;
-  const char* gB;
+  const char* fA;   // operands: the K step being fetched
+  const char* fB;
   const char* gSA;
   const char* gSB;
   auto set_fill_tile = [&](int fm, int fn) {
-    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
-    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
     gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
   set_fill_tile(pm, pn);
-  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
-  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+  auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
     const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
-    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
-    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+    if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
+    else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
 
   // ---- scale loads: wave w fetches the 16 scale bytes (four K steps) of rows 64 w .. 64 w + 63 of A and of B
@@ -131,8 +131,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
   issue_scales(0, std::true_type{});
-  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  fA += 2 * ROWB;
+  fB += 2 * ROWB;
   wait_vmcnt<16>();
   block_barrier();
   static_for<MT + NT>([&](auto OP_) { read_scale(OP_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
       if constexpr (n % 2 == 0)
         read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, nxt>{}, std::integral_constant<int, (UN >> 2) * SC_SLOT + (UN & 3) * 4>{});
-      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fk, lds0 + P * STAGE, std::false_type{});
+      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       // (the scales of the K steps fk .. fk + 3 are requested in the third step of every four, into the slot whose
       // last reader was the read for the step before this one)
       if constexpr ((U & 3) == 2 && n == 16) issue_scales(fk >> 2, std::false_type{});
@@ -179,14 +181,14 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;
   auto advance = [&]() {
+    fA += ROWB;
+    fB += ROWB;
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) {
-        ftile += gridDim.x;
-        int fm, fn;
-        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
-        set_fill_tile(fm, fn);
-      }
+      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      int fm, fn;
+      grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+      set_fill_tile(fm, fn);
     }
   };
   while (true) {
@@ -287,33 +289,33 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   asm volatile("" : "+s"(nk_last));
 
   // ---- operand loads, as in the 16-bit kernel
+  // (a lane offset per load - row, chunk, and the instruction offset taken back out - and one scalar base per
+  // operand that moves with the K step being fetched)
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[2], voffB[2];
+  unsigned voffA[8], voffB[8];
 #pragma unroll
-  for (int par = 0; par < 2; par++) {
-    const unsigned chunk = dslot ^ ((par * 4 + (lane >> 4)) & 7);
-    voffA[par] = drow * (unsigned)p.lda + chunk * 16;
-    voffB[par] = drow * (unsigned)p.ldb + chunk * 16;
+  for (int q = 0; q < 8; q++) {
+    const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
   // scalar bases (operands and scales) of the tile the loads are fetching, two K steps ahead of the MFMAs
-  const char* gA;
-  const char* gB;
+  const char* fA;   // operands: the K step being fetched
+  const char* fB;
   const char* gSA;
   const char* gSB;
   auto set_fill_tile = [&](int fm, int fn) {
-    gA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
-    gB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
     gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
   set_fill_tile(pm, pn);
-  const int64_t stepA = 8 * p.lda, stepB = 8 * p.ldb;
-  auto issue = [&](auto J_, int kt, unsigned stage_base, auto SETTLE_) {
+  auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const char* src = (j < 8 ? gA + q * stepA : gB + q * stepB) - ioff;
     const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
-    const unsigned lane_off = (j < 8 ? voffA[j & 1] : voffB[j & 1]) + (unsigned)kt * ROWB;
-    async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(src, lane_off, dst);
+    if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
+    else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
   // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of rows 64 w .. 64 w + 63 of A and of B
   const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
@@ -377,8 +379,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   using T = std::true_type; using F = std::false_type;
   issue_scales(0, std::true_type{});
-  static_for<16>([&](auto J_) { issue(J_, 0, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, 1, lds0 + STAGE, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  fA += 2 * ROWB;
+  fB += 2 * ROWB;
   wait_vmcnt<16>();
   block_barrier();
   static_for<NRD>([&](auto OP_) { read_one(OP_, I0{}, I0{}, f[0]); });
@@ -411,7 +415,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
       // (sa[0] / sb[0] are free: sub-step 0 has issued all its MFMAs)
       if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, I0{}, OffNext{});
-      if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fk, lds0 + P * STAGE, std::false_type{});   // one per 64 cycles
+      if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fA, fB, lds0 + P * STAGE, std::false_type{});   // one per 64 cycles
       // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
       // two steps back used: its last readers were the reads of that pair's second step, in its sub-step 0)
       // (after the last operand load: the eight loads of an operand share the M0 value that the first one sets)
@@ -431,14 +435,14 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;
   auto advance = [&]() {
+    fA += ROWB;
+    fB += ROWB;
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) {
-        ftile += gridDim.x;
-        int fm, fn;
-        grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
-        set_fill_tile(fm, fn);
-      }
+      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      int fm, fn;
+      grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
+      set_fill_tile(fm, fn);
     }
   };
   while (true) {
