@@ -137,8 +137,23 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     }
   };
 
+  // per-lane LDS addresses of the fragment reads, one register per k-step (row-wise) and per (column block, half)
+  // (transposed); stage, tile and sub-row offsets ride in the instructions' immediates, so the loop has no address
+  // arithmetic at all (computed per read they were 150 of the loop's 355 vector instructions per step).  With
+  // 512-byte rows (head_dim 256) the registers are not there and a stage no longer fits the 16-bit immediate: that
+  // width computes its addresses per read.
   const RowRead<RB> rr(l32, g);
   const TrRead<RB> tt(i16, q4);
+  constexpr bool kPre = D <= 128;
+  unsigned ra[kPre ? KSQ : 1], ta[kPre ? DT : 1][2];
+  if constexpr (kPre) {
+#pragma unroll
+    for (int ks = 0; ks < KSQ; ks++) ra[ks] = lds_base + rr.rowb + (rr.xk ^ (ks * 32));
+#pragma unroll
+    for (int c = 0; c < DT; c++)
+#pragma unroll
+      for (int h2 = 0; h2 < 2; h2++) ta[c][h2] = lds_base + (tt.tl ^ ((c << 6) | (h2 << 5)));
+  }
 
   f32x16 dq[DT][QT];
 #pragma unroll
@@ -158,92 +173,117 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
   wait_all();
   __syncthreads();
 
-  for (int j = 0; j < nsteps; j++) {
-    const int stage = j & 1;
-    if (j + 1 < nsteps) issue_kv(j + 1, stage ^ 1);
-    if (j <= wave_last && row0 < p.N) {
-      const unsigned kb = lds_addr(lds + stage * (2 * TILE));
-      const unsigned vb = kb + TILE;
-      V8 dsf[QT][4];
-#pragma unroll
-      for (int a = 0; a < 2; a++) {
-        // S^T and dP^T for key tile a: [QT q tiles]
-        f32x16 s[QT], dp[QT];
-#pragma unroll
-        for (int b = 0; b < QT; b++)
-#pragma unroll
-          for (int r = 0; r < 16; r++) { s[b][r] = 0.f; dp[b][r] = 0.f; }
-        i32x4 kf[2], vf[2];
-        kf[0] = a == 0 ? lds_read_b128<0>(rr.template addr<0>(kb)) : lds_read_b128<32 * RB>(rr.template addr<0>(kb));
-        vf[0] = a == 0 ? lds_read_b128<0>(rr.template addr<0>(vb)) : lds_read_b128<32 * RB>(rr.template addr<0>(vb));
-        static_for<KSQ>([&](auto KS_) {
-          constexpr int ks = decltype(KS_)::value;
-          constexpr int cur = ks & 1, nxt = cur ^ 1;
-          if constexpr (ks + 1 < KSQ) {
-            kf[nxt] = a == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(kb)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(kb));
-            vf[nxt] = a == 0 ? lds_read_b128<0>(rr.template addr<ks + 1>(vb)) : lds_read_b128<32 * RB>(rr.template addr<ks + 1>(vb));
-            lds_wait<2>();
-          } else {
-            lds_wait<0>();
-          }
-          lds_use(kf[cur]);
-          lds_use(vf[cur]);
-#pragma unroll
-          for (int b = 0; b < QT; b++) {
-            s[b] = mfma32(__builtin_bit_cast(V8, kf[cur]), qf[b][ks], s[b]);
-            dp[b] = mfma32(__builtin_bit_cast(V8, vf[cur]), dof[b][ks], dp[b]);
-          }
-        });
+  // one K/V step on LDS stage STAGE; MASKED: the step meets the causal diagonal of this wave's rows
+  auto step = [&](const int j, auto STAGE_, auto MASKED_) {
+    constexpr int stage = decltype(STAGE_)::value;
+    constexpr bool masked = decltype(MASKED_)::value;
+    constexpr int KOFF = kPre ? stage * 2 * TILE : 0, VOFF = KOFF + TILE;
+    const unsigned sbase = kPre ? 0u : lds_base + (unsigned)(stage * 2 * TILE);
+    auto row_addr = [&](auto KS_) {
+      constexpr int ks = decltype(KS_)::value;
+      if constexpr (kPre) return ra[ks];
+      else return rr.template addr<ks>(sbase);
+    };
+    auto tr_addr = [&](auto C_, auto H_) {
+      constexpr int c = decltype(C_)::value, h2 = decltype(H_)::value;
+      if constexpr (kPre) return ta[c][h2];
+      else return tt.template addr<c, h2>(sbase);
+    };
+    using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+    V8 dsf[QT][4];
+    static_for<2>([&](auto A_) {
+      constexpr int a = decltype(A_)::value;
+      // S^T and dP^T for key tile a: [QT q tiles]
+      f32x16 s[QT], dp[QT];
+      i32x4 kf[2], vf[2];
+      kf[0] = lds_read_b128<KOFF + a * 32 * RB>(row_addr(I0{}));
+      vf[0] = lds_read_b128<VOFF + a * 32 * RB>(row_addr(I0{}));
+      static_for<KSQ>([&](auto KS_) {
+        constexpr int ks = decltype(KS_)::value;
+        constexpr int cur = ks & 1, nxt = cur ^ 1;
+        if constexpr (ks + 1 < KSQ) {
+          kf[nxt] = lds_read_b128<KOFF + a * 32 * RB>(row_addr(std::integral_constant<int, ks + 1 < KSQ ? ks + 1 : 0>{}));
+          vf[nxt] = lds_read_b128<VOFF + a * 32 * RB>(row_addr(std::integral_constant<int, ks + 1 < KSQ ? ks + 1 : 0>{}));
+          lds_wait<2>();
+        } else {
+          lds_wait<0>();
+        }
+        lds_use(kf[cur]);
+        lds_use(vf[cur]);
 #pragma unroll
         for (int b = 0; b < QT; b++) {
-          const int qrow = row0 + b * 32 + l32;
-          const bool masked = j >= wave_first_masked;
+          // (the first k-step takes a constant zero as its addend: no registers to clear)
+          s[b] = mfma32(__builtin_bit_cast(V8, kf[cur]), qf[b][ks], ks == 0 ? f32x16{} : s[b]);
+          dp[b] = mfma32(__builtin_bit_cast(V8, vf[cur]), dof[b][ks], ks == 0 ? f32x16{} : dp[b]);
+        }
+      });
 #pragma unroll
-          for (int r = 0; r < 16; r++) {
-            float pv = fast_exp2(fmaf(s[b][r], qk_scale, -m_row[b]));
-            if (masked) {
-              int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-              if (kv > qrow) pv = 0.f;
-            }
-            float dsv = pv * (dp[b][r] - d_row[b]);
-            dsf[b][a * 2 + (r >> 3)][r & 7] = (S)dsv;
+      for (int b = 0; b < QT; b++) {
+        const int qrow = row0 + b * 32 + l32;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+          float pv = fast_exp2(fmaf(s[b][r], qk_scale, -m_row[b]));
+          if constexpr (masked) {
+            int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+            if (kv > qrow) pv = 0.f;
           }
+          float dsv = pv * (dp[b][r] - d_row[b]);
+          dsf[b][a * 2 + (r >> 3)][r & 7] = (S)dsv;
         }
       }
-      // dQ^T += K^T ds^T : [DT d tiles][QT q tiles], 4 k-steps of 16 key rows
-      {
-        i32x2 tf[2][DT][2];
-        auto read_t = [&](auto T_, i32x2 (&dst)[DT][2]) {
-          constexpr int t = decltype(T_)::value;
-          static_for<DT>([&](auto C_) {
-            constexpr int c = decltype(C_)::value;
-            dst[c][0] = lds_read_tr16_b64<16 * t * RB>(tt.template addr<c, 0>(kb));
-            dst[c][1] = lds_read_tr16_b64<(16 * t + 8) * RB>(tt.template addr<c, 1>(kb));
-          });
-        };
-        read_t(std::integral_constant<int, 0>{}, tf[0]);
-        static_for<4>([&](auto T_) {
-          constexpr int t = decltype(T_)::value;
-          constexpr int cur = t & 1, nxt = cur ^ 1;
-          if constexpr (t + 1 < 4) {
-            read_t(std::integral_constant<int, t + 1>{}, tf[nxt]);
-            lds_wait<2 * DT>();
-          } else {
-            lds_wait<0>();
-          }
-#pragma unroll
-          for (int c = 0; c < DT; c++) {
-            lds_use(tf[cur][c][0]);
-            lds_use(tf[cur][c][1]);
-            i32x4 both = __builtin_shufflevector(tf[cur][c][0], tf[cur][c][1], 0, 1, 2, 3);
-#pragma unroll
-            for (int b = 0; b < QT; b++) dq[c][b] = mfma32(__builtin_bit_cast(V8, both), dsf[b][t], dq[c][b]);
-          }
+    });
+    // dQ^T += K^T ds^T : [DT d tiles][QT q tiles], 4 k-steps of 16 key rows
+    {
+      i32x2 tf[2][DT][2];
+      auto read_t = [&](auto T_, i32x2 (&dst)[DT][2]) {
+        constexpr int t = decltype(T_)::value;
+        static_for<DT>([&](auto C_) {
+          dst[decltype(C_)::value][0] = lds_read_tr16_b64<KOFF + 16 * t * RB>(tr_addr(C_, I0{}));
+          dst[decltype(C_)::value][1] = lds_read_tr16_b64<KOFF + (16 * t + 8) * RB>(tr_addr(C_, I1{}));
         });
-      }
+      };
+      read_t(I0{}, tf[0]);
+      static_for<4>([&](auto T_) {
+        constexpr int t = decltype(T_)::value;
+        constexpr int cur = t & 1, nxt = cur ^ 1;
+        if constexpr (t + 1 < 4) {
+          read_t(std::integral_constant<int, t + 1>{}, tf[nxt]);
+          lds_wait<2 * DT>();
+        } else {
+          lds_wait<0>();
+        }
+#pragma unroll
+        for (int c = 0; c < DT; c++) {
+          lds_use(tf[cur][c][0]);
+          lds_use(tf[cur][c][1]);
+          i32x4 both = __builtin_shufflevector(tf[cur][c][0], tf[cur][c][1], 0, 1, 2, 3);
+#pragma unroll
+          for (int b = 0; b < QT; b++) dq[c][b] = mfma32(__builtin_bit_cast(V8, both), dsf[b][t], dq[c][b]);
+        }
+      });
     }
+  };
+  auto run = [&](const int j, auto STAGE_, auto MASKED_) {
+    if (j + 1 < nsteps) issue_kv(j + 1, decltype(STAGE_)::value ^ 1);
+    if (j <= wave_last && row0 < p.N) step(j, STAGE_, MASKED_);
     wait_all();
     __syncthreads();
+  };
+  // The steps below the diagonal run in a loop of their own, the few that meet it in a second one: with both
+  // forms behind a branch inside one loop the register allocator gave the two bodies different registers for the
+  // accumulators and copied all 64 of them back and forth at the join of every step.  (Every wave runs every
+  // step's loads and barrier in either loop, so the waves of a workgroup may split at different steps.)
+  using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+  const int nplain = min(wave_first_masked, nsteps);
+  int j = 0;
+  for (; j + 1 < nplain; j += 2) {
+    run(j, I0{}, std::false_type{});
+    run(j + 1, I1{}, std::false_type{});
+  }
+  if (j < nplain) { run(j, I0{}, std::false_type{}); j++; }
+  for (; j < nsteps; j++) {
+    if (j & 1) run(j, I1{}, std::true_type{});
+    else run(j, I0{}, std::true_type{});
   }
 
 #pragma unroll
