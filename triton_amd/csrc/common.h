@@ -103,6 +103,25 @@ __device__ __forceinline__ void async_copy16_sbase_off(const void* sbase, unsign
 #endif
 }
 
+// A touch of one dword per lane, lanes 0 .. NLANES-1 only, at (wave-uniform 64-bit base + 32-bit lane offset),
+// landing in 256 bytes of LDS that nobody reads: brings those lanes' cache lines into the L2 ahead of the loads that
+// want them.  Counts in vmcnt like any load; sets M0 like the copies above (SETM0) or uses the value a preceding
+// touch has set.  Only for code in which all 64 lanes are active: the execution mask is narrowed for the one
+// instruction (every lane is a request to the cache, wanted or not) and set back to all lanes.
+template <bool SETM0, int NLANES>
+__device__ __forceinline__ void touch_line_sbase(const void* sbase, unsigned lane_off, unsigned lds_junk) {
+#if MI355_DEVICE_PASS
+  static_assert(NLANES >= 1 && NLANES <= 32, "lane mask as a 32-bit literal");
+  constexpr unsigned MASK = NLANES == 32 ? 0xffffffffu : ((1u << NLANES) - 1u);
+  if constexpr (SETM0)
+    asm volatile("s_mov_b32 m0, %2\n\ts_mov_b64 exec, %3\n\tglobal_load_lds_dword %0, %1\n\ts_mov_b64 exec, -1"
+                 :: "v"(lane_off), "s"(sbase), "s"(lds_junk), "i"(MASK) : "memory");
+  else
+    asm volatile("s_mov_b64 exec, %2\n\tglobal_load_lds_dword %0, %1\n\ts_mov_b64 exec, -1"
+                 :: "v"(lane_off), "s"(sbase), "i"(MASK) : "memory");
+#endif
+}
+
 // 16 bytes per lane from (wave-uniform 64-bit base + 32-bit lane offset + immediate) into
 // registers, issued as inline assembly so that the compiler neither counts it nor waits for it:
 // for loops that keep many loads in flight and wait with wait_vmcnt<> by hand.  The result may be

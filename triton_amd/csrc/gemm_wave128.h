@@ -1,6 +1,15 @@
 // Pieces shared by the four-wave GEMM kernels (gemm_wave128.hip: 16-bit and fp8; gemm_wave128_mx.hip: the
 // block-scaled forms): the wait for the last MFMAs, the grid size, and the epilogue of 16x16 accumulator tiles.
 #pragma once
+
+// L2 touches ahead of the direct loads in the four-wave kernels (see gemm_wave128_tiles): on / off and the number of
+// K steps they run ahead of the loads, as build-time switches for A/B measurements.
+#ifndef MI355_W128_PREFETCH
+#define MI355_W128_PREFETCH 1
+#endif
+#ifndef MI355_W128_PREFETCH_DISTANCE
+#define MI355_W128_PREFETCH_DISTANCE 2
+#endif
 #include "gemm_core.h"
 
 namespace mi355 {

@@ -120,10 +120,32 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
     return (const char*)(((uint64_t)hi << 32) | lo);
   };
+  // L2 prefetch (dense kernels without a K tail, whose buffer has the LDS this needs): the two LDS stages let a load
+  // run at most one K step ahead of its use, about a microsecond - enough for operands that the last-level cache
+  // holds, not for a first touch in HBM (after the reference's cache flush between timed calls every line is one).
+  // So PFD K steps ahead of the loads each wave touches a few lines of the step to come: the 32 tiles that run on
+  // one XCD at a time form a patch of 8 x 4, every A panel is shared by four of its programs and every B panel by
+  // eight, and the programs split a panel's lines among themselves by their tile coordinates (tile column & 3 picks
+  // the quarter of the A rows, tile row & 7 the eighth of the B rows), the four waves split that share again.  One
+  // lane per 128-byte line, 16 + 8 lines per wave and K step.
+  constexpr bool PF = XCD && !TAIL && MI355_W128_PREFETCH;
+  constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
+  const char* pA = nullptr;
+  const char* pB = nullptr;
+  unsigned voffPA = 0, voffPB = 0;
+  if constexpr (PF) {
+    voffPA = (lane % (BM / 16)) * (unsigned)p.lda;
+    voffPB = B_KMAJOR ? (lane & 7) * (unsigned)p.ldb : ((lane & 7) >> 2) * (unsigned)p.ldb + (lane & 3) * 128;
+  }
   auto set_fill_tile = [&](int fm, int fn) {
     fA = scalar_ptr(p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda);
     fB = scalar_ptr(B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb
                              : p.B + (int64_t)fn * BN * 2 + (int64_t)(wave * 16) * p.ldb);
+    if constexpr (PF) {
+      pA = scalar_ptr(p.A + ((int64_t)fm * BM + (fn & 3) * (BM / 4) + wave * (BM / 16)) * p.lda);
+      pB = scalar_ptr(B_KMAJOR ? p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb
+                               : p.B + (int64_t)fn * BN * 2 + (int64_t)((fm & 7) * 8 + wave * 2) * p.ldb);
+    }
   };
   set_fill_tile(pm, pn);
   const unsigned kstepB = B_KMAJOR ? ROWB : 64 * (unsigned)p.ldb;   // bytes from one K step to the next
@@ -196,7 +218,18 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA + ROWB, fB + kstepB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * (int64_t)kstepB;
-  wait_vmcnt<NLOADS>();
+  if constexpr (PF) {
+    // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
+    // the loop's waits leave outstanding from the first step on
+    const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
+    touch_line_sbase<true, BM / 16>(pA + k2 * ROWB, voffPA, lds0 + 2 * STAGE + wave * 256);
+    touch_line_sbase<false, 8>(pB + (int64_t)k2 * kstepB, voffPB, 0u);
+    touch_line_sbase<false, BM / 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, 8>(pB + (int64_t)k3 * kstepB, voffPB, 0u);
+    pA += 2 * ROWB;
+    pB += 2 * (int64_t)kstepB;
+  }
+  wait_vmcnt<NLOADS + (PF ? 4 : 0)>();
   block_barrier();
   using Z = std::integral_constant<int, 0>;
   static_for<NRD>([&](auto OP_) { read_one(OP_, Z{}, Z{}, f[0]); });
@@ -206,7 +239,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   // (every wave has then read all it needs of this stage, and the other stage has landed), reads the
   // first fragments of the other stage and refills this one with the tile two steps ahead (one load
   // per four MFMAs).
-  auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_) {
+  auto substep = [&](auto P_, auto KS_, auto MORE_, auto REFILL_, const char* tA, const char* tB) {
     constexpr int P = decltype(P_)::value, ks = decltype(KS_)::value, cur = ks & 1, nxt = cur ^ 1;
     constexpr bool last = ks == KS - 1;
     constexpr bool more = decltype(MORE_)::value;              // there is a next sub-step to read for
@@ -214,7 +247,7 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     lds_wait<0>();
     pin(f[cur]);
     if constexpr (last) {
-      wait_vmcnt<0>();
+      wait_vmcnt<PF ? 2 : 0>();   // (all but the two touches of the previous step, which are the youngest loads)
       block_barrier();
     }
     static_for<NM>([&](auto N_) {
@@ -229,15 +262,17 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
       constexpr int every = NM / 16;   // MFMAs per load slot: 4 (64 MFMAs) or 3 (48)
       if constexpr (refill && n % every == 1 && n / every < NLOADS)
         issue(std::integral_constant<int, load_of(n / every)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      if constexpr (refill && PF && n == NM - 2) touch_line_sbase<true, BM / 16>(tA, voffPA, lds0 + 2 * STAGE + wave * 256);
+      if constexpr (refill && PF && n == NM - 1) touch_line_sbase<false, 8>(tB, voffPB, 0u);
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   using T = std::true_type; using F = std::false_type;
   // A K step; its loads fetch the K step that the scalar bases point at.
-  auto stage = [&](auto P_) {
-    substep(P_, I0{}, T{}, F{});
-    substep(P_, I1{}, T{}, T{});
+  auto stage = [&](auto P_, const char* tA, const char* tB) {
+    substep(P_, I0{}, T{}, F{}, tA, tB);
+    substep(P_, I1{}, T{}, T{}, tA, tB);
     // The fragment reads above are invisible to the compiler: have them landed before control reaches a loop
     // edge, where the register allocator may copy the registers they write.  (They were issued over the first
     // half of the sub-step, so this does not wait.)
@@ -248,9 +283,14 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;   // next K step to fetch, and the tile it belongs to
+  // the lines to touch: K step fk + PFD of the fill tile, or (past its end) the step being fetched anyway
+  const int64_t pfdB = (int64_t)PFD * kstepB;
+  auto touch_a = [&]() { return PF ? pA + (fk + PFD < nk ? PFD * ROWB : 0) : nullptr; };
+  auto touch_b = [&]() { return PF ? pB + (fk + PFD < nk ? pfdB : (int64_t)0) : nullptr; };
   auto advance = [&]() {
     fA += ROWB;
     fB += kstepB;
+    if constexpr (PF) { pA += ROWB; pB += kstepB; }
     if (++fk == nk) {
       fk = 0;
       if (ftile + tile_step < tend) ftile += tile_step;
@@ -261,9 +301,15 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
   };
   if (nk == 2) { fk = 1; advance(); }   // (two steps per tile: the prologue fetched both, the cursor is on the next tile)
   while (true) {
+    // With the touches in flight the loop's waits leave two loads outstanding, and the compiler, which counts only
+    // the loads IT knows, must then assume that the last two registers it reloaded behind the epilogue (lane offsets
+    // of the loads, spilled there) are still on their way: it guarded their first use - inside the K loop - with a
+    // wait for ALL outstanding loads, a full drain in every step (-6 to -12 %).  One full wait per tile in front of
+    // the loop tells it that its reloads have landed; the stores of the epilogue are all that this waits for.
+    if constexpr (PF) wait_all();
     for (int kt = 0; kt < nk; kt += 2) {
-      stage(I0{}); advance();
-      stage(I1{}); advance();
+      stage(I0{}, touch_a(), touch_b()); advance();
+      stage(I1{}, touch_a(), touch_b()); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
     if constexpr (TAIL) {
@@ -474,9 +520,20 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   // scalar bases of the K step the loads are fetching (two K steps ahead of the MFMAs)
   const char* fA;
   const char* fB;
+  // L2 touches two K steps ahead of the loads, as in the 16-bit kernel: the programs of an XCD's 8 x 4 patch of
+  // tiles share out the lines of the panels they have in common
+  constexpr bool PF = MI355_W128_PREFETCH;
+  constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
+  const char* pA = nullptr;
+  const char* pB = nullptr;
+  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
   auto set_fill_tile = [&](int fm, int fn) {
     fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
     fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    if constexpr (PF) {
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
+    }
   };
   set_fill_tile(pm, pn);
   auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
@@ -519,7 +576,18 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * ROWB;
-  wait_vmcnt<16>();
+  if constexpr (PF) {
+    // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
+    // the loop's waits leave outstanding from the first step on
+    const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
+    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, lds0 + 2 * STAGE + wave * 256);
+    touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
+    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
+    pA += 2 * ROWB;
+    pB += 2 * ROWB;
+  }
+  wait_vmcnt<16 + (PF ? 4 : 0)>();
   block_barrier();
 #pragma unroll
   for (int t = 0; t < NT; t++) b[0][t] = read_frag(fragB, t * 16 * ROWB);
@@ -527,7 +595,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
 
   // One K step on stage P with the B fragments of set `cur`; its loads fetch the K step the scalar bases point at.
-  auto step = [&](auto P_, auto CUR_) {
+  auto step = [&](auto P_, auto CUR_, const char* tA, const char* tB) {
     constexpr int P = decltype(P_)::value, cur = decltype(CUR_)::value, nxt = cur ^ 1;
     constexpr int so = P * STAGE, sn = (P ^ 1) * STAGE;
     // first half: rows 0..3 of A; the A fragments 4..7 of this stage are read meanwhile
@@ -540,7 +608,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     // every wave has now requested all it needs of stage P: once those reads are back and the other
     // stage has landed, meet, then read the next fragments from the other stage and refill this one
     lds_wait<0>();
-    wait_vmcnt<0>();
+    wait_vmcnt<PF ? 2 : 0>();   // (all but the two touches of the previous step, which are the youngest loads)
     block_barrier();
     static_for<MH * NT>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
@@ -550,15 +618,23 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (PF) {
+      touch_line_sbase<true, 16>(tA, voffPA, lds0 + 2 * STAGE + wave * 256);
+      touch_line_sbase<false, 8>(tB, voffPB, 0u);
+    }
   };
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   // The fill cursor runs two K steps ahead of the MFMAs, across tile boundaries; behind the last tile it
   // wraps to that tile's first steps again (fetched into stages nobody reads any more), which keeps the
   // loop, the number of loads in flight and every wait uniform.
   int fk = 2, ftile = tile;
+  // the lines to touch: K step fk + PFD of the fill tile, or (past its end) the step being fetched anyway
+  auto touch_a = [&]() { return PF ? pA + (fk + PFD < nk ? PFD * ROWB : 0) : nullptr; };
+  auto touch_b = [&]() { return PF ? pB + (fk + PFD < nk ? PFD * ROWB : 0) : nullptr; };
   auto advance = [&]() {
     fA += ROWB;
     fB += ROWB;
+    if constexpr (PF) { pA += ROWB; pB += ROWB; }
     if (++fk == nk) {
       fk = 0;
       if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
@@ -569,9 +645,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   };
   if (nk == 2) { fk = 1; advance(); }
   while (true) {
+    if constexpr (PF) wait_all();   // (once per tile: tells the compiler that its own loads have landed, see the 16-bit kernel)
     for (int kt = 0; kt < nk; kt += 2) {
-      step(I0{}, I0{}); advance();
-      step(I1{}, I1{}); advance();
+      step(I0{}, I0{}, touch_a(), touch_b()); advance();
+      step(I1{}, I1{}, touch_a(), touch_b()); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
     mfma_drain(acc);
@@ -591,7 +668,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 
 template <int FMT, int EPI>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128;
+  constexpr int smem = 2 * 2 * 256 * 128 + 1024;   // (two stages and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -635,7 +712,7 @@ bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int til
 
 template <typename V8, bool B_KMAJOR, int EPI, bool TAIL = false, int BM = 256>
 static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * (BM + 256) * 128 + (TAIL ? 2 * 256 * 64 : 0);   // (with the tail buffer: all 160 KiB of the CU)
+  constexpr int smem = 2 * (BM + 256) * 128 + (TAIL ? 2 * 256 * 64 : 1024);   // (with the tail buffer: all 160 KiB of the CU; without: 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);

@@ -61,9 +61,21 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   const char* fB;
   const char* gSA;
   const char* gSB;
+  // L2 touches two K steps ahead of the loads, as in the 16-bit kernel: the programs of an XCD's 8 x 4 patch of
+  // tiles share out the lines of the panels they have in common
+  constexpr bool PF = MI355_W128_PREFETCH;
+  constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
+  const char* pA = nullptr;
+  const char* pB = nullptr;
+  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
+  const unsigned touch_lds = lds0 + SC_BASE + 2 * SC_SLOT + wave * 256;
   auto set_fill_tile = [&](int fm, int fn) {
     fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
     fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    if constexpr (PF) {
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
+    }
     gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
@@ -135,7 +147,18 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * ROWB;
-  wait_vmcnt<16>();
+  if constexpr (PF) {
+    // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
+    // the loop's waits leave outstanding from the first step on
+    const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
+    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, touch_lds);
+    touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
+    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
+    pA += 2 * ROWB;
+    pB += 2 * ROWB;
+  }
+  wait_vmcnt<16 + (PF ? 4 : 0)>();
   block_barrier();
   static_for<MT + NT>([&](auto OP_) { read_scale(OP_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
   lds_wait<0>();
@@ -157,7 +180,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     lds_wait<0>();
-    wait_vmcnt<0>();
+    wait_vmcnt<PF ? 2 : 0>();   // (all but the two touches of the previous step, which are the youngest loads)
     block_barrier();
     static_for<MH * NT>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
@@ -172,6 +195,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       if constexpr ((U & 3) == 2 && n == 16) issue_scales(fk >> 2, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (PF) {
+      touch_line_sbase<true, 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
+      touch_line_sbase<false, 8>(pB + (fk + PFD < nk ? PFD * ROWB : 0), voffPB, 0u);
+    }
     lds_wait<0>();
     pin_scales(std::integral_constant<int, nxt>{});
   };
@@ -183,6 +210,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   auto advance = [&]() {
     fA += ROWB;
     fB += ROWB;
+    if constexpr (PF) { pA += ROWB; pB += ROWB; }
     if (++fk == nk) {
       fk = 0;
       if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
@@ -192,6 +220,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
     }
   };
   while (true) {
+    if constexpr (PF) wait_all();   // (once per tile: tells the compiler that its own loads have landed, see the 16-bit kernel)
     for (int kt = 0; kt < nk; kt += 8) {
       static_for<8>([&](auto U_) { step(U_, fk); advance(); });
       if (kt + 8 >= nk_last) mfma_retire();
@@ -221,7 +250,7 @@ bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
 
 template <int EPI>
 static int launch_wave128_mxfp8(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -304,9 +333,21 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   const char* fB;
   const char* gSA;
   const char* gSB;
+  // L2 touches two K steps ahead of the loads, as in the 16-bit kernel: the programs of an XCD's 8 x 4 patch of
+  // tiles share out the lines of the panels they have in common
+  constexpr bool PF = MI355_W128_PREFETCH;
+  constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
+  const char* pA = nullptr;
+  const char* pB = nullptr;
+  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
+  const unsigned touch_lds = lds0 + SC_BASE + 2 * SC_SLOT + wave * 256;
   auto set_fill_tile = [&](int fm, int fn) {
     fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
     fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    if constexpr (PF) {
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
+    }
     gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
@@ -383,7 +424,18 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * ROWB;
-  wait_vmcnt<16>();
+  if constexpr (PF) {
+    // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
+    // the loop's waits leave outstanding from the first step on
+    const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
+    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, touch_lds);
+    touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
+    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
+    pA += 2 * ROWB;
+    pB += 2 * ROWB;
+  }
+  wait_vmcnt<16 + (PF ? 4 : 0)>();
   block_barrier();
   static_for<NRD>([&](auto OP_) { read_one(OP_, I0{}, I0{}, f[0]); });
   static_for<NRD>([&](auto OP_) { read_scale(OP_, I0{}, I0{}); });
@@ -407,7 +459,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     lds_wait<0>();
     pin(f[1]);
     pin_scales(I1{});
-    wait_vmcnt<0>();
+    wait_vmcnt<PF ? 2 : 0>();   // (all but the two touches of the previous step, which are the youngest loads)
     block_barrier();
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
@@ -422,6 +474,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       if constexpr (P == 0 && n == 62) issue_scales(fk >> 1, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
+    if constexpr (PF) {
+      touch_line_sbase<true, 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
+      touch_line_sbase<false, 8>(pB + (fk + PFD < nk ? PFD * ROWB : 0), voffPB, 0u);
+    }
     // everything requested above has landed before the registers are touched again
     lds_wait<0>();
     pin(f[0]);
@@ -437,6 +493,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   auto advance = [&]() {
     fA += ROWB;
     fB += ROWB;
+    if constexpr (PF) { pA += ROWB; pB += ROWB; }
     if (++fk == nk) {
       fk = 0;
       if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
@@ -446,6 +503,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     }
   };
   while (true) {
+    if constexpr (PF) wait_all();   // (once per tile: tells the compiler that its own loads have landed, see the 16-bit kernel)
     for (int kt = 0; kt < nk; kt += 4) {
       step(I0{}, fk); advance();
       step(I1{}, fk); advance();
@@ -478,7 +536,7 @@ bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
 
 template <int EPI>
 static int launch_wave128_mxfp4(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16;
+  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
