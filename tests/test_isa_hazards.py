@@ -649,3 +649,48 @@ def test_no_result_of_an_assembly_mfma_is_touched_before_it_retires_in_any_kerne
             bad = check_assembly_mfma_results(lines)
             assert not bad, (os.path.basename(f), name, bad[:5])
     assert checked >= 30, checked
+
+
+# ---------------------------------------------------------------------------------------------
+# A performance property of the same family.  The K loops of the four-wave GEMM kernels keep their direct loads in
+# flight across iterations and wait for them by hand, once per K step.  The compiler counts only the loads it knows
+# (spill reloads, the epilogue's own loads); when one of those is still outstanding by ITS count at the first use of
+# the loaded register and that use sits inside the K loop, it guards the use with a wait that in reality drains
+# every load of the loop, in every step (seen: -6 to -12 % after the loop's own wait changed from vmcnt(0) to
+# vmcnt(2), with correct results).  So: no basic block of a K loop may wait for vector memory more than once.
+# ---------------------------------------------------------------------------------------------
+def k_loop_blocks_with_extra_waits(lines, min_mfma=64):
+    bad = []
+    for label, ins in _blocks(lines):
+        if sum("v_mfma" in i for i in ins) < min_mfma:
+            continue
+        waits = [i for i in ins if i.startswith("s_waitcnt") and "vmcnt" in i]
+        if len(waits) > 1:
+            bad.append((label, waits))
+    return bad
+
+
+def test_extra_wait_checker_flags_a_guarded_reload_inside_a_k_loop():
+    mf = ["\tv_mfma_f32_16x16x32_bf16 a[0:3], v[0:3], v[4:7], a[0:3]"] * 64
+    good = [".LBB0_1:", "\ts_waitcnt vmcnt(2)"] + mf
+    guarded = [".LBB0_1:", "\ts_waitcnt vmcnt(2)"] + mf[:60] + ["\ts_waitcnt vmcnt(0)", "\tglobal_load_lds_dwordx4 v147, s[34:35] offset:0xc00"] + mf[60:]
+    assert k_loop_blocks_with_extra_waits(good) == []
+    assert [b[0] for b in k_loop_blocks_with_extra_waits(guarded)] == [".LBB0_1"]
+
+
+def test_k_loops_of_the_four_wave_kernels_wait_for_loads_once_per_step():
+    if not all(os.path.exists(f) for f in ASM):
+        pytest.skip("device assembly not kept: build the library first (python -m triton_amd.build)")
+    checked = 0
+    for f in ASM:
+        for name, lines in _functions(open(f).read()).items():
+            if "gemm_wave128" not in name:
+                continue
+            # (the K-tail instantiations - template arguments <..., EPI, true, 256> - multiply their tail from plain
+            # loads that the compiler waits for itself, in blocks of 64 MFMAs of their own)
+            if re.search(r"Li\dELb1ELi256EEE", name):
+                continue
+            checked += 1
+            bad = k_loop_blocks_with_extra_waits(lines)
+            assert not bad, (name, bad[:3])
+    assert checked >= 30, checked
