@@ -211,6 +211,14 @@ __device__ __forceinline__ int lds_read_b32(unsigned addr) {
   return v;
 }
 template <int OFF>
+__device__ __forceinline__ int lds_read_u16(unsigned addr) {   // two bytes, zero-extended
+  int v = 0;
+#if MI355_DEVICE_PASS
+  asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "i"(OFF));
+#endif
+  return v;
+}
+template <int OFF>
 __device__ __forceinline__ int lds_read_u8(unsigned addr) {   // one byte, zero-extended
   int v = 0;
 #if MI355_DEVICE_PASS

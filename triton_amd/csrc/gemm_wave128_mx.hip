@@ -271,12 +271,12 @@ int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
 // ---------------------------------------------------------------------------------------------
 // MXFP4 (e2m1 codes, one e8m0 scale per 32 elements of K) on the same skeleton: scaled 16x16x128
 // f8f6f4 MFMAs, two per accumulator tile and K step (128 bytes of a row = 256 elements = 8 scale
-// blocks of 16 bytes).  Lane (r, kg) of sub-step ks multiplies block 4 ks + kg of its row.  (Which K positions
+// blocks of 16 bytes).  Lane (r, kg) of sub-step ks multiplies block 2 kg + ks of its row, which the loads have put into LDS slot 4 ks + kg.  (Which K positions
 // a lane takes is free as long as A, B and the scales agree; but with the lane group in the LOW bits of the
 // chunk number the fragment reads are free of LDS bank conflicts, with 2 kg + ks - the first version - every
 // ds_read_b128 took 8 instead of 4 cycles: measured, SQ_LDS_BANK_CONFLICT = half of SQ_LDS_IDX_ACTIVE.)  The
 // scales travel like the operands: 16 bytes per row (two K steps) per direct load into a two-slot LDS ring
-// (row r at 16 r); from there each fragment's scale byte of a sub-step is fetched with one `ds_read_u8`.
+// (row r at 16 r); from there the two scale bytes of a fragment and K step are fetched with one `ds_read_u16`.
 // ---------------------------------------------------------------------------------------------
 // Scaled fp4 MFMA with the accumulator pinned to the accumulation registers (see mfma16): byte SEL of the two
 // scale dwords applies; fp4 operands are four registers.
@@ -324,7 +324,10 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   unsigned voffA[8], voffB[8];
 #pragma unroll
   for (int q = 0; q < 8; q++) {
-    const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    // (LDS slot s of a row takes the row's chunk 2 (s & 3) + (s >> 2): the fragment reads keep their conflict-free
+    // slots 4 ks + kg and find the chunks 2 kg + ks there - the two scale blocks of a lane are then neighbours)
+    const unsigned slot = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
+    const unsigned chunk = 2 * (slot & 3) + (slot >> 2);
     voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
     voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
@@ -389,22 +392,21 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     static_for<MT>([&](auto T_) { lds_use(x.a[decltype(T_)::value]); });
     static_for<NT>([&](auto T_) { lds_use(x.b[decltype(T_)::value]); });
   };
-  // scales: lane (r, kg) multiplies block kg of its row in sub-step 0 and block 4 + kg in sub-step 1; each is
-  // fetched as ONE BYTE (ds_read_u8: it arrives in byte 0, the position the MFMA's selector names, so no shift)
-  // into a register set of its own - sc[0] for sub-step 0, read during the sub-step 1 before, sc[1] for
-  // sub-step 1, read during the same step's sub-step 0 -, one read per two MFMAs.
-  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + kg;
-  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + kg;
+  // scales: lane (r, kg) multiplies block 2 kg of its row in sub-step 0 and block 2 kg + 1 in sub-step 1: ONE 16-bit
+  // read per fragment and K step fetches both (bytes 0 and 1 of the register, which the MFMA's compile-time selector
+  // names: no shift), into the register set of the step's parity, read during the second half of the step before.
+  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + 2 * kg;
+  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + 2 * kg;
   int sa[2][MT], sb[2][NT];
-  auto read_scale = [&](auto OP_, auto KS_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 1) * 8
-    constexpr int op = decltype(OP_)::value, ks = decltype(KS_)::value, off = decltype(OFF_)::value + 4 * ks;
-    if constexpr (op < MT) sa[ks][op] = lds_read_u8<off + op * 256>(adrSA);
-    else sb[ks][op - MT] = lds_read_u8<off + (op - MT) * 256>(adrSB);
+  auto read_scale = [&](auto OP_, auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 1) * 8
+    constexpr int op = decltype(OP_)::value, set = decltype(SET_)::value, off = decltype(OFF_)::value;
+    if constexpr (op < MT) sa[set][op] = lds_read_u16<off + op * 256>(adrSA);
+    else sb[set][op - MT] = lds_read_u16<off + (op - MT) * 256>(adrSB);
   };
-  auto pin_scales = [&](auto KS_) {
-    constexpr int ks = decltype(KS_)::value;
-    static_for<MT>([&](auto T_) { lds_use(sa[ks][decltype(T_)::value]); });
-    static_for<NT>([&](auto T_) { lds_use(sb[ks][decltype(T_)::value]); });
+  auto pin_scales = [&](auto SET_) {
+    constexpr int set = decltype(SET_)::value;
+    static_for<MT>([&](auto T_) { lds_use(sa[set][decltype(T_)::value]); });
+    static_for<NT>([&](auto T_) { lds_use(sb[set][decltype(T_)::value]); });
   };
 
   f32x4 acc[MT][NT];
@@ -445,28 +447,24 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   // K step U (0..3 within a group of four: stage U & 1, scale slot U >> 1)
   auto step = [&](auto U_, int fk) {   // fk: the K step (of the fill tile) that this step's loads fetch
     constexpr int U = decltype(U_)::value, P = U & 1, UN = (U + 1) & 3;
-    using OffCur = std::integral_constant<int, (U >> 1) * SC_SLOT + (U & 1) * 8>;
     using OffNext = std::integral_constant<int, (UN >> 1) * SC_SLOT + (UN & 1) * 8>;
-    // sub-step 0 (blocks kg); meanwhile the fragments and the scales of sub-step 1
+    // sub-step 0 (blocks 2 kg); meanwhile the fragments of sub-step 1
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
-      mfma16_mxfp4<0>(f[0].b[j], f[0].a[i], acc[i][j], sb[0][j], sa[0][i]);
+      mfma16_mxfp4<0>(f[0].b[j], f[0].a[i], acc[i][j], sb[P][j], sa[P][i]);
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P>{}, I1{}, f[1]);
-      if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, I1{}, OffCur{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
-    // sub-step 1 (blocks 4 + kg): meet, then read the next step's first fragments and scales and refill this stage
+    // sub-step 1 (blocks 2 kg + 1): meet, then read the next step's first fragments and scales and refill this stage
     lds_wait<0>();
     pin(f[1]);
-    pin_scales(I1{});
     wait_vmcnt<PF ? 2 : 0>();   // (all but the two touches of the previous step, which are the youngest loads)
     block_barrier();
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
-      mfma16_mxfp4<0>(f[1].b[j], f[1].a[i], acc[i][j], sb[1][j], sa[1][i]);
+      mfma16_mxfp4<1>(f[1].b[j], f[1].a[i], acc[i][j], sb[P][j], sa[P][i]);
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
-      // (sa[0] / sb[0] are free: sub-step 0 has issued all its MFMAs)
-      if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, I0{}, OffNext{});
+      if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, OffNext{});
       if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fA, fB, lds0 + P * STAGE, std::false_type{});   // one per 64 cycles
       // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
       // two steps back used: its last readers were the reads of that pair's second step, in its sub-step 0)
@@ -481,7 +479,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     // everything requested above has landed before the registers are touched again
     lds_wait<0>();
     pin(f[0]);
-    pin_scales(I0{});
+    pin_scales(std::integral_constant<int, P ^ 1>{});
   };
   using I2 = std::integral_constant<int, 2>; using I3 = std::integral_constant<int, 3>;
   lds_wait<0>();
