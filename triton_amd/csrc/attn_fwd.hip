@@ -22,6 +22,13 @@
 #include "attn_tiles.h"
 #include "launch.h"
 
+#ifndef MI355_ATTN_K_AHEAD
+#define MI355_ATTN_K_AHEAD 1
+#endif
+#ifndef MI355_ATTN_V_EARLY
+#define MI355_ATTN_V_EARLY 1
+#endif
+
 namespace mi355 {
 
 template <typename V8> struct Elem;
@@ -167,19 +174,27 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
 #pragma unroll
           for (int r = 0; r < 16; r++) s[a][b][r] = 0.f;
       {
-        i32x4 kf[2][2];
-        kf[0][0] = lds_read_b128<KOFF>(ka[0] + sreg);
-        kf[0][1] = lds_read_b128<KOFF + 32 * RB>(ka[0] + sreg);
+        // K fragments KAHEAD k-steps ahead of their MFMAs (KAHEAD + 1 register sets).  Measured: one, two or three
+        // k-steps ahead run the same - what the K reads cost (15 % of the kernel in a knock-out) is not their latency
+        constexpr int KAHEAD = MI355_ATTN_K_AHEAD;
+        i32x4 kf[KAHEAD + 1][2];
+        static_for<KAHEAD>([&](auto I_) {
+          constexpr int i = decltype(I_)::value;
+          if constexpr (i < KSQ) {
+            kf[i][0] = lds_read_b128<KOFF>(ka[i] + sreg);
+            kf[i][1] = lds_read_b128<KOFF + 32 * RB>(ka[i] + sreg);
+          }
+        });
         static_for<KSQ>([&](auto KS_) {
           constexpr int ks = decltype(KS_)::value;
-          constexpr int cur = ks & 1, nxt = cur ^ 1;
-          if constexpr (ks + 1 < KSQ) {
-            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + 1] + sreg);
-            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + 1] + sreg);
-            lds_wait<2>();
-          } else {
-            lds_wait<0>();
+          constexpr int cur = ks % (KAHEAD + 1), nxt = (ks + KAHEAD) % (KAHEAD + 1);
+          if constexpr (ks + KAHEAD < KSQ) {
+            kf[nxt][0] = lds_read_b128<KOFF>(ka[ks + KAHEAD < KSQ ? ks + KAHEAD : 0] + sreg);
+            kf[nxt][1] = lds_read_b128<KOFF + 32 * RB>(ka[ks + KAHEAD < KSQ ? ks + KAHEAD : 0] + sreg);
           }
+          // reads issued behind those of k-step ks: two per k-step still to come, at most KAHEAD of them
+          constexpr int behind = (KSQ - 1 - ks) < KAHEAD ? (KSQ - 1 - ks) : KAHEAD;
+          lds_wait<2 * behind>();
           lds_use(kf[cur][0]);
           lds_use(kf[cur][1]);
 #pragma unroll
@@ -189,6 +204,17 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
               s[a][b] = mfma32(__builtin_bit_cast(V8, kf[cur][a]), qf[b][ks], s[a][b]);
         });
       }
+      // (the first V fragments are requested here already: their latency passes behind the softmax arithmetic)
+      i32x2 vf[2][DT][2];
+      auto read_v = [&](auto T_, i32x2 (&dst)[DT][2]) {
+        constexpr int t = decltype(T_)::value;
+        static_for<DT>([&](auto C_) {
+          constexpr int c = decltype(C_)::value;
+          dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0] + sreg);
+          dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1] + sreg);
+        });
+      };
+      if constexpr (MI355_ATTN_V_EARLY) read_v(std::integral_constant<int, 0>{}, vf[0]);
       // ---- online softmax, one query row per lane (pair of lanes l, l+32 shares a row)
       V8 pf[QT][4];  // P^T as B operand of the second product, per 16-column k-step
 #pragma unroll
@@ -238,16 +264,7 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
       }
       // ---- O^T += V^T P^T : [DT d tiles][QT q tiles], 4 k-steps of 16 columns
       {
-        i32x2 vf[2][DT][2];
-        auto read_v = [&](auto T_, i32x2 (&dst)[DT][2]) {
-          constexpr int t = decltype(T_)::value;
-          static_for<DT>([&](auto C_) {
-            constexpr int c = decltype(C_)::value;
-            dst[c][0] = lds_read_tr16_b64<VOFF + 16 * t * RB>(va[c][0] + sreg);
-            dst[c][1] = lds_read_tr16_b64<VOFF + (16 * t + 8) * RB>(va[c][1] + sreg);
-          });
-        };
-        read_v(std::integral_constant<int, 0>{}, vf[0]);
+        if constexpr (!MI355_ATTN_V_EARLY) read_v(std::integral_constant<int, 0>{}, vf[0]);
         static_for<4>([&](auto T_) {
           constexpr int t = decltype(T_)::value;
           constexpr int cur = t & 1, nxt = cur ^ 1;
