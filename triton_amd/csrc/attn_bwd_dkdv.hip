@@ -142,22 +142,32 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   // even waves copy the stage's 64 M values, odd waves its 64 deltas (4 bytes per lane; the
   // duplicates keep the number of loads per wave uniform for the partial waits)
   const float* src_stat = ((wave & 1) == 0 ? lse : delta) + m_begin + lane;
-  // stage-step js (clamped to the last one) into ring slot js % NS
-  auto issue_stage = [&](int js) {
-    const unsigned qda = lds_base + (js % NS) * STAGE, dda = qda + TILE;
+  // stage-step js (clamped to the last one) into ring slot js % NS: nine loads per wave (kShare), issued as a burst
+  // in the prologue and one at a time between the MFMAs of the loop (a burst there held the wave up for about 380
+  // cycles per stage: with one wave per SIMD nothing else issues while the memory pipeline takes the loads)
+  struct StageSrc { const char* q; const char* d; const float* stat; unsigned lds; };
+  auto stage_src = [&](int js) {
     const int jc = min(js, nsteps - 1);
-    const char* qsrc = qsrc0 + (int64_t)jc * BM * pitch;
-    const char* dsrc = dsrc0 + (int64_t)jc * BM * pitch;
-#pragma unroll
-    for (int i = 0; i < Tile::INST; i++) {
+    const int64_t off = (int64_t)jc * BM * pitch;
+    return StageSrc{qsrc0 + off, dsrc0 + off, src_stat + jc * BM, lds_base + (js % NS) * STAGE};
+  };
+  auto stage_load = [&](auto I_, const StageSrc& ss) {   // load number I of kShare
+    constexpr int I = decltype(I_)::value;
+    if constexpr (I < 2 * Tile::INST) {
+      constexpr int i = I >> 1;
       // (every row has chunks that are present, so every wave still issues every load: the counts of the partial
       // waits below stay what they are)
       if (present[i]) {
-        async_copy16_sbase(qsrc, offQD[i], qda + (i * NW + wave) * 1024);
-        async_copy16_sbase(dsrc, offQD[i], dda + (i * NW + wave) * 1024);
+        if constexpr ((I & 1) == 0) async_copy16_sbase(ss.q, offQD[i], ss.lds + (i * NW + wave) * 1024);
+        else async_copy16_sbase(ss.d, offQD[i], ss.lds + TILE + (i * NW + wave) * 1024);
       }
+    } else {
+      async_copy4_asm(ss.stat, ss.lds + 2 * TILE + (wave & 1) * (BM * 4));
     }
-    async_copy4_asm(src_stat + jc * BM, qda + 2 * TILE + (wave & 1) * (BM * 4));
+  };
+  auto issue_stage = [&](int js) {
+    const StageSrc ss = stage_src(js);
+    static_for<kShare>([&](auto I_) { stage_load(I_, ss); });
   };
 
   // per-lane LDS offsets inside a stage: row-wise operand per k-step, transposed operand per
@@ -241,29 +251,39 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     }
   };
   // A(next tile) into set PAR with X(previous tile, set PAR^1) and its transposed reads in between
+  // (Every MFMA is followed by its share of the other work.  Two MFMAs back to back leave the first one's 32 cycles
+  // empty: the second cannot issue before the pipe is free, and nothing behind it can issue before it - measured on
+  // the kernel's own cycle counter, phase A took 977 cycles per tile = 532 of MFMAs + 285 of softmax + 204 of
+  // transposed reads, every part in full.)
   auto phase_a_impl = [&](auto PAR_, auto MTX_, auto DOX_, auto MASKED_, int mrow0_x, unsigned sbase_x) {
     constexpr int par = decltype(PAR_)::value;
     constexpr bool do_x = decltype(DOX_)::value;
-    constexpr int EPK = 16 / KSQ;             // X elements per k-step
-    constexpr int TRK = 2 * (8 * DT) / KSQ;   // transposed reads per k-step, all within the first half
+    constexpr int EPK = 16 / KSQ, EH = EPK / 2;                   // X elements per k-step, per MFMA
+    constexpr int TRK = (8 * DT + KSQ - 2) / (KSQ - 1), TH = (TRK + 1) / 2;   // transposed reads per k-step (none in the last), first share
     settle_rows();
     settle_stats();
     static_for<KSQ>([&](auto KS_) {
       constexpr int ks = decltype(KS_)::value;
-      if constexpr (ks == 0) {
-        mfma32_first_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[0]), kf[0]);
-        mfma32_first_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[0]), vf[0]);
-      } else {
-        mfma32_acc_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[ks]), kf[ks]);
-        mfma32_acc_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[ks]), vf[ks]);
-      }
+      if constexpr (ks == 0) mfma32_first_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[0]), kf[0]);
+      else mfma32_acc_v<PAD>(sacc[par], __builtin_bit_cast(V8, rq[ks]), kf[ks]);
       if constexpr (do_x) {
-        static_for<TRK>([&](auto O_) {
+        static_for<TH>([&](auto O_) {
           constexpr int i = ks * TRK + decltype(O_)::value;
           if constexpr (i < 8 * DT) read_tr(std::integral_constant<int, i>{}, MTX_, sbase_x);
         });
         softmax_part(std::integral_constant<int, par ^ 1>{}, std::integral_constant<int, ks * EPK>{},
-                     std::integral_constant<int, EPK>{}, mrow0_x, MASKED_);
+                     std::integral_constant<int, EH>{}, mrow0_x, MASKED_);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (ks == 0) mfma32_first_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[0]), vf[0]);
+      else mfma32_acc_v<PAD>(dpacc[par], __builtin_bit_cast(V8, rd[ks]), vf[ks]);
+      if constexpr (do_x) {
+        static_for<TRK - TH>([&](auto O_) {
+          constexpr int i = ks * TRK + TH + decltype(O_)::value;
+          if constexpr (i < 8 * DT) read_tr(std::integral_constant<int, i>{}, MTX_, sbase_x);
+        });
+        softmax_part(std::integral_constant<int, par ^ 1>{}, std::integral_constant<int, ks * EPK + EH>{},
+                     std::integral_constant<int, EPK - EH>{}, mrow0_x, MASKED_);
       }
       __builtin_amdgcn_sched_barrier(0);
     });
@@ -271,22 +291,36 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
 
   // C(tile) with the row-wise reads of the tile after next (stage sbase_r, half MTR) and the
   // M / delta reads of the next tile (stage sbase_s, half MTS) in between
-  auto phase_c = [&](auto MTR_, unsigned sbase_r, auto MTS_, unsigned sbase_s) {
+  // LOADS: this phase also requests the next stage of the ring, one load behind each MFMA pair's first MFMA
+  auto phase_c = [&](auto MTR_, unsigned sbase_r, auto MTS_, unsigned sbase_s, auto LOADS_, const StageSrc& ss) {
     constexpr int NM = 2 * DT;               // MFMA pairs
     constexpr int NRD = 2 * KSQ + 8;         // reads to place
-    constexpr int PER = (2 * NRD + NM - 1) / NM;  // all within the first half of the MFMAs
+    constexpr int PER = (NRD + NM - 3) / (NM - 2), PH = (PER + 1) / 2;   // per pair (none in the last two), first share
+    constexpr bool loads = decltype(LOADS_)::value;
+    constexpr int LPP = (kShare + NM - 1) / NM;   // loads per pair
+    auto reads = [&](auto FROM_, auto N_) {
+      static_for<decltype(N_)::value>([&](auto O_) {
+        constexpr int i = decltype(FROM_)::value + decltype(O_)::value;
+        if constexpr (i < 2 * KSQ) read_rows(std::integral_constant<int, i>{}, MTR_, sbase_r);
+        else if constexpr (i < NRD) read_stats(std::integral_constant<int, i - 2 * KSQ>{}, MTS_, sbase_s);
+      });
+    };
     settle_tr();
     static_for<NM>([&](auto N_) {
       constexpr int n = decltype(N_)::value, t = n / DT, c = n % DT;
       i32x4 qt = __builtin_shufflevector(tq[t][c][0], tq[t][c][1], 0, 1, 2, 3);
       i32x4 dt = __builtin_shufflevector(td[t][c][0], td[t][c][1], 0, 1, 2, 3);
       dv[c] = mfma32(__builtin_bit_cast(V8, dt), pf[t], dv[c]);
+      reads(std::integral_constant<int, n * PER>{}, std::integral_constant<int, PH>{});
+      if constexpr (loads) {
+        static_for<LPP>([&](auto L_) {
+          constexpr int l = n * LPP + decltype(L_)::value;
+          if constexpr (l < kShare) stage_load(std::integral_constant<int, l>{}, ss);
+        });
+      }
+      __builtin_amdgcn_sched_barrier(0);
       dk[c] = mfma32(__builtin_bit_cast(V8, qt), dsf[t], dk[c]);
-      static_for<PER>([&](auto O_) {
-        constexpr int i = n * PER + decltype(O_)::value;
-        if constexpr (i < 2 * KSQ) read_rows(std::integral_constant<int, i>{}, MTR_, sbase_r);
-        else if constexpr (i < NRD) read_stats(std::integral_constant<int, i - 2 * KSQ>{}, MTS_, sbase_s);
-      });
+      reads(std::integral_constant<int, n * PER + PH>{}, std::integral_constant<int, PER - PH>{});
       __builtin_amdgcn_sched_barrier(0);
     });
   };
@@ -317,13 +351,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
     __builtin_amdgcn_sched_barrier(0);
     block_barrier();
     __builtin_amdgcn_sched_barrier(0);
-    issue_stage(j + NS - 1);
-    // C(2j) | row-wise reads of tile 2j+2 (next stage), M/delta of tile 2j+1
-    phase_c(I0{}, sb_nxt, I1{}, sb_cur);
+    const StageSrc ss = stage_src(j + NS - 1);
+    // C(2j) | row-wise reads of tile 2j+2 (next stage), M/delta of tile 2j+1, the loads of stage j + NS - 1
+    phase_c(I0{}, sb_nxt, I1{}, sb_cur, std::true_type{}, ss);
     // A(2j+2) | X(2j+1), transposed reads of tile 2j+1
     phase_a_impl(I0{}, I1{}, std::true_type{}, MASKED_, ms + 32, sb_cur);
     // C(2j+1) | row-wise reads of tile 2j+3, M/delta of tile 2j+2
-    phase_c(I1{}, sb_nxt, I0{}, sb_nxt);
+    phase_c(I1{}, sb_nxt, I0{}, sb_nxt, std::false_type{}, ss);
   };
   // causal: the workgroup's 128 key rows meet the diagonal in its first two stages (query rows
   // n0 .. n0+127); only those pay for the mask
