@@ -124,17 +124,23 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     lds_zero(lds, 2 * 2 * TILE, tid, NW * 64);
     __syncthreads();
   }
-  auto issue_kv = [&](int j, int stage) {
-    const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
-    const char* ksrc = kbase + (int64_t)j * BN * pitch;
-    const char* vsrc = vbase + (int64_t)j * BN * pitch;
-#pragma unroll
-    for (int i = 0; i < Tile::INST; i++) {
-      if (present[i]) {
-        async_copy16_sbase(ksrc, offKV[i], kd + (i * NW + wave) * 1024);
-        async_copy16_sbase(vsrc, offKV[i], vd + (i * NW + wave) * 1024);
-      }
+  // the K and V tiles of step j into LDS stage `stage`: 2 * INST loads per wave, as a burst (prologue, waves without
+  // work in a step) or one at a time between the MFMAs of the step before
+  struct KvSrc { const char* k; const char* v; unsigned lds; };
+  auto kv_src = [&](int j, int stage) {
+    const int64_t off = (int64_t)j * BN * pitch;
+    return KvSrc{kbase + off, vbase + off, lds_base + stage * (2 * TILE)};
+  };
+  auto kv_load = [&](auto I_, const KvSrc& src) {
+    constexpr int I = decltype(I_)::value, i = I >> 1;
+    if (present[i]) {
+      if constexpr ((I & 1) == 0) async_copy16_sbase(src.k, offKV[i], src.lds + (i * NW + wave) * 1024);
+      else async_copy16_sbase(src.v, offKV[i], src.lds + TILE + (i * NW + wave) * 1024);
     }
+  };
+  auto issue_kv = [&](int j, int stage) {
+    const KvSrc src = kv_src(j, stage);
+    static_for<2 * Tile::INST>([&](auto I_) { kv_load(I_, src); });
   };
 
   // per-lane LDS addresses of the fragment reads, one register per k-step (row-wise) and per (column block, half)
@@ -173,7 +179,18 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
   wait_all();
   __syncthreads();
 
-  // one K/V step on LDS stage STAGE; MASKED: the step meets the causal diagonal of this wave's rows
+  // One K/V step on LDS stage STAGE; MASKED: the step meets the causal diagonal of this wave's rows.
+  // One wave per SIMD (the kernel's registers allow no second), so whatever
+  // is to overlap the MFMAs stands between them in this wave's own instruction stream:
+  //   phase 1   S^T, dP^T of key tile 0         | the loads of the next step's tiles, one behind each k-step's first MFMA
+  //   phase 2   S^T, dP^T of key tile 1         | the softmax / dS arithmetic of key tile 0; the first K^T fragments
+  //   phase 3   dQ^T += K^T dS^T, key tile 0    | the softmax / dS arithmetic of key tile 1
+  //   phase 4   dQ^T += K^T dS^T, key tile 1
+  // (Measured on the kernel's cycle counter before: 16 MFMAs 500 cycles, the arithmetic of a key tile 527 cycles with
+  // no MFMA in flight, the eight loads as a burst 323, the step 3283 for 1536 cycles of MFMAs.)
+  // The arithmetic of a key tile is a list of independent operations, stage after stage over its 16 elements per
+  // lane - u = dP - delta, t = S * scale - M, p = 2^t, (mask,) dS = p * u, conversions in pairs -, of which each
+  // MFMA slot takes a slice: an operation and the one that needs its result are then 16 operations apart.
   auto step = [&](const int j, auto STAGE_, auto MASKED_) {
     constexpr int stage = decltype(STAGE_)::value;
     constexpr bool masked = decltype(MASKED_)::value;
@@ -190,82 +207,119 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
       else return tt.template addr<c, h2>(sbase);
     };
     using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
+    // (behind the last step its own tiles once more, into the stage nobody reads: no branch around the loads, whose
+    // join the register allocator could use to copy fragment registers with reads still in flight)
+    const KvSrc nsrc = kv_src(min(j + 1, nsteps - 1), stage ^ 1);
     V8 dsf[QT][4];
+    f32x16 s[2][QT], dp[2][QT];
+    i32x4 kf[2], vf[2];
+    i32x2 tf[2][DT][2];
+    constexpr int NOPS = 16 * (masked ? 5 : 4) + 8;   // operations of a key tile's arithmetic
+    auto softmax_ops = [&](auto A_, auto FROM_, auto N_) {
+      constexpr int a = decltype(A_)::value;
+      static_for<decltype(N_)::value>([&](auto O_) {
+        constexpr int i = decltype(FROM_)::value + decltype(O_)::value;
+        if constexpr (i < NOPS) {
+          constexpr int st = i / 16, r = i % 16;
+          constexpr int kind = (!masked && st >= 3) ? st + 1 : st;   // 0 u, 1 t, 2 p, 3 mask, 4 dS, 5 conversions
+#pragma unroll
+          for (int b = 0; b < QT; b++) {
+            if constexpr (kind == 0) dp[a][b][r] -= d_row[b];
+            else if constexpr (kind == 1) s[a][b][r] = fmaf(s[a][b][r], qk_scale, -m_row[b]);
+            else if constexpr (kind == 2) s[a][b][r] = fast_exp2(s[a][b][r]);
+            else if constexpr (kind == 3) {
+              const int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
+              if (kv > row0 + b * 32 + l32) s[a][b][r] = 0.f;
+            } else if constexpr (kind == 4) dp[a][b][r] *= s[a][b][r];
+            else if constexpr (r < 8) {   // elements 2 r, 2 r + 1
+              dsf[b][a * 2 + (r >> 2)][(2 * r) & 7] = (S)dp[a][b][2 * r];
+              dsf[b][a * 2 + (r >> 2)][(2 * r + 1) & 7] = (S)dp[a][b][2 * r + 1];
+            }
+          }
+        }
+      });
+    };
+    auto read_t = [&](auto T_, auto C_, i32x2 (&dst)[DT][2]) {   // the two halves of K^T fragment (t, c)
+      constexpr int t = decltype(T_)::value, c = decltype(C_)::value;
+      dst[c][0] = lds_read_tr16_b64<KOFF + 16 * t * RB>(tr_addr(C_, I0{}));
+      dst[c][1] = lds_read_tr16_b64<KOFF + (16 * t + 8) * RB>(tr_addr(C_, I1{}));
+    };
+    // (the padded forms guard every load with a per-lane test - control flow, at whose joins the register allocator
+    // may copy registers: their loads go first, while no fragment read is in flight)
+    if constexpr (PAD) static_for<2 * Tile::INST>([&](auto I_) { kv_load(I_, nsrc); });
+    // ---- phases 1 and 2: S^T and dP^T of key tile a
+    kf[0] = lds_read_b128<KOFF>(row_addr(I0{}));
+    vf[0] = lds_read_b128<VOFF>(row_addr(I0{}));
     static_for<2>([&](auto A_) {
       constexpr int a = decltype(A_)::value;
-      // S^T and dP^T for key tile a: [QT q tiles]
-      f32x16 s[QT], dp[QT];
-      i32x4 kf[2], vf[2];
-      kf[0] = lds_read_b128<KOFF + a * 32 * RB>(row_addr(I0{}));
-      vf[0] = lds_read_b128<VOFF + a * 32 * RB>(row_addr(I0{}));
+      constexpr int XPS = (NOPS + 2 * KSQ - 1) / (2 * KSQ);   // operations per MFMA slot of phase 2
       static_for<KSQ>([&](auto KS_) {
         constexpr int ks = decltype(KS_)::value;
         constexpr int cur = ks & 1, nxt = cur ^ 1;
+        // the reads of the k-step to come; in phase 2's last two k-steps the first K^T fragments instead / as well
+        constexpr int late = (a == 1 && ks >= KSQ - 2) ? DT * (ks - (KSQ - 2) + 0) : 0;   // K^T reads issued before this k-step
         if constexpr (ks + 1 < KSQ) {
           kf[nxt] = lds_read_b128<KOFF + a * 32 * RB>(row_addr(std::integral_constant<int, ks + 1 < KSQ ? ks + 1 : 0>{}));
           vf[nxt] = lds_read_b128<VOFF + a * 32 * RB>(row_addr(std::integral_constant<int, ks + 1 < KSQ ? ks + 1 : 0>{}));
+          lds_wait<2 + late>();
+        } else if constexpr (a == 0) {
+          // (the first fragments of key tile 1, so that phase 2 starts with its operands on the way)
+          kf[nxt] = lds_read_b128<KOFF + 32 * RB>(row_addr(I0{}));
+          vf[nxt] = lds_read_b128<VOFF + 32 * RB>(row_addr(I0{}));
           lds_wait<2>();
         } else {
-          lds_wait<0>();
+          lds_wait<late>();
         }
         lds_use(kf[cur]);
         lds_use(vf[cur]);
 #pragma unroll
-        for (int b = 0; b < QT; b++) {
-          // (the first k-step takes a constant zero as its addend: no registers to clear)
-          s[b] = mfma32(__builtin_bit_cast(V8, kf[cur]), qf[b][ks], ks == 0 ? f32x16{} : s[b]);
-          dp[b] = mfma32(__builtin_bit_cast(V8, vf[cur]), dof[b][ks], ks == 0 ? f32x16{} : dp[b]);
-        }
-      });
-#pragma unroll
-      for (int b = 0; b < QT; b++) {
-        const int qrow = row0 + b * 32 + l32;
-#pragma unroll
-        for (int r = 0; r < 16; r++) {
-          float pv = fast_exp2(fmaf(s[b][r], qk_scale, -m_row[b]));
-          if constexpr (masked) {
-            int kv = j * BN + a * 32 + (r >> 2) * 8 + g * 4 + (r & 3);
-            if (kv > qrow) pv = 0.f;
-          }
-          float dsv = pv * (dp[b][r] - d_row[b]);
-          dsf[b][a * 2 + (r >> 3)][r & 7] = (S)dsv;
-        }
-      }
-    });
-    // dQ^T += K^T ds^T : [DT d tiles][QT q tiles], 4 k-steps of 16 key rows
-    {
-      i32x2 tf[2][DT][2];
-      auto read_t = [&](auto T_, i32x2 (&dst)[DT][2]) {
-        constexpr int t = decltype(T_)::value;
-        static_for<DT>([&](auto C_) {
-          dst[decltype(C_)::value][0] = lds_read_tr16_b64<KOFF + 16 * t * RB>(tr_addr(C_, I0{}));
-          dst[decltype(C_)::value][1] = lds_read_tr16_b64<KOFF + (16 * t + 8) * RB>(tr_addr(C_, I1{}));
-        });
-      };
-      read_t(I0{}, tf[0]);
-      static_for<4>([&](auto T_) {
-        constexpr int t = decltype(T_)::value;
-        constexpr int cur = t & 1, nxt = cur ^ 1;
-        if constexpr (t + 1 < 4) {
-          read_t(std::integral_constant<int, t + 1>{}, tf[nxt]);
-          lds_wait<2 * DT>();
+        for (int b = 0; b < QT; b++)
+          s[a][b] = mfma32(__builtin_bit_cast(V8, kf[cur]), qf[b][ks], ks == 0 ? f32x16{} : s[a][b]);
+        if constexpr (a == 0) {
+          if constexpr (!PAD && 2 * ks < 2 * Tile::INST) kv_load(std::integral_constant<int, 2 * ks < 2 * Tile::INST ? 2 * ks : 0>{}, nsrc);
         } else {
-          lds_wait<0>();
+          softmax_ops(I0{}, std::integral_constant<int, 2 * ks * XPS>{}, std::integral_constant<int, XPS>{});
         }
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int c = 0; c < DT; c++) {
-          lds_use(tf[cur][c][0]);
-          lds_use(tf[cur][c][1]);
-          i32x4 both = __builtin_shufflevector(tf[cur][c][0], tf[cur][c][1], 0, 1, 2, 3);
-#pragma unroll
-          for (int b = 0; b < QT; b++) dq[c][b] = mfma32(__builtin_bit_cast(V8, both), dsf[b][t], dq[c][b]);
+        for (int b = 0; b < QT; b++)
+          dp[a][b] = mfma32(__builtin_bit_cast(V8, vf[cur]), dof[b][ks], ks == 0 ? f32x16{} : dp[a][b]);
+        if constexpr (a == 0) {
+          if constexpr (!PAD && 2 * ks + 1 < 2 * Tile::INST) kv_load(std::integral_constant<int, 2 * ks + 1 < 2 * Tile::INST ? 2 * ks + 1 : 0>{}, nsrc);
+        } else {
+          softmax_ops(I0{}, std::integral_constant<int, (2 * ks + 1) * XPS>{}, std::integral_constant<int, XPS>{});
+          if constexpr (ks >= KSQ - 2) {
+            // half of the first K^T fragments behind each of the last two k-steps
+            static_for<DT / 2>([&](auto C_) { read_t(I0{}, std::integral_constant<int, (ks - (KSQ - 2)) * (DT / 2) + decltype(C_)::value>{}, tf[0]); });
+          }
         }
+        __builtin_amdgcn_sched_barrier(0);
       });
-    }
+    });
+    // ---- phases 3 and 4: dQ^T += K^T dS^T, [DT d tiles][QT q tiles], 4 k-steps of 16 key rows.  The fragments of
+    // k-step t + 1 are requested one behind each MFMA of k-step t, so a fragment is DT MFMAs old when it is used
+    // and DT - 1 younger requests may still be outstanding.
+    constexpr int XPD = (NOPS + 2 * DT - 1) / (2 * DT);   // operations per MFMA slot of phase 3
+    static_for<4>([&](auto T_) {
+      constexpr int t = decltype(T_)::value;
+      constexpr int cur = t & 1, nxt = cur ^ 1;
+      static_for<DT>([&](auto C_) {
+        constexpr int c = decltype(C_)::value;
+        lds_wait<(t + 1 < 4) ? 2 * (DT - 1) : 2 * (DT - 1 - c)>();
+        lds_use(tf[cur][c][0]);
+        lds_use(tf[cur][c][1]);
+        i32x4 both = __builtin_shufflevector(tf[cur][c][0], tf[cur][c][1], 0, 1, 2, 3);
+#pragma unroll
+        for (int b = 0; b < QT; b++) dq[c][b] = mfma32(__builtin_bit_cast(V8, both), dsf[b][t], dq[c][b]);
+        if constexpr (t + 1 < 4) read_t(std::integral_constant<int, t + 1 < 4 ? t + 1 : 0>{}, C_, tf[nxt]);
+        if constexpr (t < 2) softmax_ops(I1{}, std::integral_constant<int, (t * DT + c) * XPD>{}, std::integral_constant<int, XPD>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
   };
   auto run = [&](const int j, auto STAGE_, auto MASKED_) {
-    if (j + 1 < nsteps) issue_kv(j + 1, decltype(STAGE_)::value ^ 1);
     if (j <= wave_last && row0 < p.N) step(j, STAGE_, MASKED_);
+    else issue_kv(min(j + 1, nsteps - 1), decltype(STAGE_)::value ^ 1);
     wait_all();
     __syncthreads();
   };
