@@ -374,8 +374,11 @@ def main():
             sys.exit(2)
         fn, work, kind, info, _ = table[args.only]()
         wall_ms, ev_ms, _ = time_launches(fn, args.steps, args.warmup)
-        print(json.dumps({"workload": args.only, "steps": args.steps, "ms_per_launch": round(ev_ms, 5),
-                          ("tflops" if kind == "flops" else "gbps"): round(work / ev_ms / (1e9 if kind == "flops" else 1e6), 1)}))
+        rec = {"workload": args.only, "steps": args.steps, "ms_per_launch": round(ev_ms, 5),
+               ("tflops" if kind == "flops" else "gbps"): round(work / ev_ms / (1e9 if kind == "flops" else 1e6), 1)}
+        if info.get("clock"):
+            rec["sclk_mhz"] = observed_clock_mhz(fn, 0.5)
+        print(json.dumps(rec))
         return
     a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
     b = torch.randn(n, n, device=dev, dtype=torch.bfloat16)

@@ -340,21 +340,16 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dq_kernel(AttnArgs p) {
     else run(j, I0{}, std::true_type{});
   }
 
+  // dQ rows through this wave's share of the K/V stages (free: every step ends with a full wait and a barrier)
 #pragma unroll
   for (int b = 0; b < QT; b++) {
-    const int row = row0 + b * 32 + l32;
-    if (row >= p.N) continue;
-    char* dst = p.dq + head_off + (int64_t)row * pitch;
+    const int r0 = row0 + b * 32;
+    if (r0 >= p.N) continue;   // (wave-uniform)
+    f32x16 t[DT];
 #pragma unroll
-    for (int c = 0; c < DT; c++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        int d = c * 32 + rg * 8 + g * 4;
-        S4 v;
-#pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = (S)(dq[c][b][rg * 4 + e] * p.sm_scale);
-        if (!PAD || d < p.d_real) *(S4*)(dst + d * 2) = v;
-      }
+    for (int c = 0; c < DT; c++) t[c] = dq[c][b];
+    store_rows_transposed<S, D, PAD>(t, p.sm_scale, lds_base + (wave * QT + b) * 32 * (D * 2), p.dq + head_off + (int64_t)r0 * pitch,
+                                     pitch, p.N - r0, p.d_real, lane);
   }
 }
 

@@ -372,25 +372,13 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_kernel(AttnArgs p) {
   settle_rows();
   settle_stats();
 
-  if (ncol < p.N) {
-    char* dkd = p.dk + head_off + (int64_t)ncol * pitch;
-    char* dvd = p.dv + head_off + (int64_t)ncol * pitch;
-#pragma unroll
-    for (int c = 0; c < DT; c++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        int d = c * 32 + rg * 8 + g * 4;
-        S4 a, b;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          a[e] = (S)(dk[c][rg * 4 + e] * p.sm_scale);
-          b[e] = (S)dv[c][rg * 4 + e];
-        }
-        if (!PAD || d < p.d_real) {
-          *(S4*)(dkd + d * 2) = a;
-          *(S4*)(dvd + d * 2) = b;
-        }
-      }
+  // dK and dV rows through LDS (store_rows_transposed), one after the other through the same 32 x D elements per
+  // wave at the start of the ring - once every wave has left the loop
+  __syncthreads();
+  if (nrow0 < p.N) {
+    const unsigned mine = lds0 + wave * 32 * RB;
+    store_rows_transposed<S, D, PAD>(dk, p.sm_scale, mine, p.dk + head_off + (int64_t)nrow0 * pitch, pitch, p.N - nrow0, p.d_real, lane);
+    store_rows_transposed<S, D, PAD>(dv, 1.f, mine, p.dv + head_off + (int64_t)nrow0 * pitch, pitch, p.N - nrow0, p.d_real, lane);
   }
 }
 
@@ -553,23 +541,12 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_bwd_dkdv_split_kernel(AttnArg
     __syncthreads();
   }
 
-  if (ncol < p.N) {
-    char* dkd = p.dk + head_off + (int64_t)ncol * pitch;
-    char* dvd = p.dv + head_off + (int64_t)ncol * pitch;
-#pragma unroll
-    for (int c = 0; c < DT; c++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        const int d = dhalf * DH + c * 32 + rg * 8 + g * 4;
-        S4 a, b;
-#pragma unroll
-        for (int e = 0; e < 4; e++) {
-          a[e] = (S)(dk[c][rg * 4 + e] * p.sm_scale);
-          b[e] = (S)dv[c][rg * 4 + e];
-        }
-        *(S4*)(dkd + d * 2) = a;
-        *(S4*)(dvd + d * 2) = b;
-      }
+  // this program's DH columns of the dK and dV rows, through LDS (the loop ended with a full wait and a barrier)
+  if (nrow0 < p.N) {
+    const unsigned mine = lds_addr(lds) + wave * 32 * (DH * 2);
+    const int64_t at = head_off + (int64_t)nrow0 * pitch + dhalf * DH * 2;
+    store_rows_transposed<S, DH, false>(dk, p.sm_scale, mine, p.dk + at, pitch, p.N - nrow0, DH, lane);
+    store_rows_transposed<S, DH, false>(dv, 1.f, mine, p.dv + at, pitch, p.N - nrow0, DH, lane);
   }
 }
 

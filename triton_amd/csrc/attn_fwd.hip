@@ -300,21 +300,15 @@ __global__ __launch_bounds__(NW * 64, 1) void attn_fwd_kernel(AttnArgs p) {
     float l = l_i[b];
     l = pair_sum(l);
     const int row = row0 + b * 32 + l32;
-    if (row >= p.N) continue;
+    if (row0 + b * 32 >= p.N) continue;   // (wave-uniform: N is a multiple of 32)
     const float inv = 1.f / l;
-    if (g == 0) p.lse[(int64_t)hz * p.N + row] = m_i[b] + log2f(l);
-    char* dst = obase + (int64_t)row * opitch;
+    if (g == 0 && row < p.N) p.lse[(int64_t)hz * p.N + row] = m_i[b] + log2f(l);
+    // (the K/V stages are free: the last step requested nothing and ended with a barrier)
+    f32x16 ob[DT];
 #pragma unroll
-    for (int c = 0; c < DT; c++)
-#pragma unroll
-      for (int rg = 0; rg < 4; rg++) {
-        int d = c * 32 + rg * 8 + g * 4;
-        typedef __attribute__((ext_vector_type(4))) S S4;
-        S4 v;
-#pragma unroll
-        for (int e = 0; e < 4; e++) v[e] = (S)(oacc[c][b][rg * 4 + e] * inv);
-        if (!PAD || d < p.d_real) *(S4*)(dst + d * 2) = v;
-      }
+    for (int c = 0; c < DT; c++) ob[c] = oacc[c][b];
+    store_rows_transposed<S, D, PAD>(ob, inv, lds0 + (wave * QT + b) * 32 * RB, obase + (int64_t)(row0 + b * 32) * opitch, opitch,
+                            p.N - (row0 + b * 32), p.d_real, lane);
   }
 }
 
@@ -575,6 +569,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
     {
       float l = pair_sum(l_i);
       const int row = row0 + l32;
+      // (stored straight from the registers: the stores of an item overlap the next item's steps here, and the
+      // detour through LDS of attn_fwd_kernel's epilogue measured 0-2 % slower in this kernel)
       if (row < p.N) {
         const float inv = 1.f / l;
         if (g == 0) p.lse[(int64_t)c_hz * p.N + row] = m_i + log2f(l);

@@ -96,4 +96,40 @@ struct TrRead {
   __device__ __forceinline__ unsigned addr(unsigned base) const { return base + xor_imm<(C << 6) | (H << 5)>(tl); }
 };
 
+// A wave's result tile of 32 rows x W columns (each element times `scale`) to global memory through 32 * W
+// elements of LDS that belong to this wave alone (`lds_w`), for accumulators that hold the tile TRANSPOSED: the
+// 32x32 MFMA tile c has the tile's columns 32 c .. 32 c + 31 as its rows, so lane (l32, g) owns row l32 and, in
+// register quad rg, the columns 32 c + 8 rg + 4 g .. + 3.  Stores straight from those registers are 64 pieces of 8
+// bytes in 32 different rows per instruction, and at one request per piece the memory pipeline of the CU is busy for
+// about 8000 cycles per 256 x 128 tile (a twentieth of the forward's 4096-key item, a tenth of a 1024-key one).
+// Written to LDS row-wise (16-byte chunks XOR-ed with the row, so that the 8-byte writes of 32 rows spread over the
+// banks) and read back 16 bytes per lane, a store instruction covers whole rows.  No barrier inside: only this wave
+// touches the buffer and a wave's LDS accesses execute in order - but the CALLER makes sure that nobody else still
+// reads or loads into that part of LDS.  PAD: only the first `cols_valid` columns (a multiple of 8) exist in memory.
+template <typename S, int W, bool PAD>
+__device__ __forceinline__ void store_rows_transposed(const f32x16 (&acc)[W / 32], float scale, unsigned lds_w, char* grow0,
+                                                      int64_t gpitch, int rows_valid, int cols_valid, int lane) {
+  constexpr int RB = W * 2, CPR = RB / 16, WT = W / 32;
+  constexpr int SWEEP = RB >= 256 ? 1 : 256 / RB;   // rows per 256 bytes (one pass over the 64 banks)
+  typedef __attribute__((ext_vector_type(4))) S S4;
+  const int l32 = lane & 31, g = lane >> 5;
+  const unsigned wbase = lds_w + l32 * RB + g * 8, wswz = (l32 / SWEEP) & (CPR - 1);
+#pragma unroll
+  for (int c = 0; c < WT; c++)
+#pragma unroll
+    for (int rg = 0; rg < 4; rg++) {
+      S4 v;
+#pragma unroll
+      for (int e = 0; e < 4; e++) v[e] = (S)(acc[c][rg * 4 + e] * scale);
+      *(LDS_PTR(S4))(uintptr_t)(wbase + (((4 * c + rg) ^ wswz) * 16)) = v;
+    }
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int k = 0; k < CPR / 2; k++) {
+    const int f = k * 64 + lane, row = f / CPR, chunk = f % CPR;
+    const i32x4 v = *(LDS_PTR(i32x4))(uintptr_t)(lds_w + row * RB + ((chunk ^ ((row / SWEEP) & (CPR - 1))) * 16));
+    if (row < rows_valid && (!PAD || chunk * 8 < cols_valid)) *(i32x4*)(grow0 + (int64_t)row * gpitch + chunk * 16) = v;
+  }
+}
+
 }  // namespace mi355
