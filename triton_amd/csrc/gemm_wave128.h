@@ -163,25 +163,45 @@ __device__ __forceinline__ void gemm_epilogue16_plain(f32x4 (&acc)[MT][NT], cons
 // more than the instruction cache holds, fetched anew at the end of every tile (and from memory when the kernel
 // starts on cold caches): same call, 8192^3 bf16 1425 -> 1457 TFLOP/s back to back and 1352 -> 1397 with flushed
 // caches, 4096^3 1201 -> 1301 and 1011 -> 1205.  Kernels take it as a separate instantiation, chosen on the host.
+// A lane holds 4 consecutive columns of a 16-column tile (8 bytes of C), so stores straight from the registers are 64
+// pieces of 8 bytes per instruction and the memory pipeline takes a request per piece: 16384 of them per 256 x 256
+// tile.  Two neighbouring tiles are therefore exchanged between the lane pairs (kg, kg ^ 1) first
+// (v_permlane16_swap: the odd 16-lane rows of its first register with the even rows of its second): the even lane
+// then holds 8 consecutive columns of the first tile and the odd lane 8 of the second - 16 bytes per lane, half the
+// requests and half the store instructions (rows need 16-byte alignment: lean_epilogue_type).
+__device__ __forceinline__ void swap16(int& a, int& b) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 1\n\tv_permlane16_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+#endif
+}
 template <int MT, int NT, typename OutT>
 __device__ __forceinline__ void gemm_epilogue16_lean(f32x4 (&acc)[MT][NT], const GemmArgs& p, int mrow0, int ncol0, int l16, int kg) {
-  typedef OutT Out4 __attribute__((ext_vector_type(4)));
+  static_assert(NT % 2 == 0 && sizeof(OutT) == 2, "pairs of 16-column tiles of a 16-bit type");
+  typedef OutT Out2 __attribute__((ext_vector_type(2)));
   float alpha = 1.f;
   if (p.a_scale) alpha *= *p.a_scale;
   if (p.b_scale) alpha *= *p.b_scale;
+  // even kg: columns 4 kg .. 4 kg + 7 of the pair's first tile; odd kg: 4 (kg - 1) .. 4 (kg - 1) + 7 of its second
+  const int col = ncol0 + 4 * (kg & 2) + 16 * (kg & 1);
   static_for<MT>([&](auto I_) {
     constexpr int i = decltype(I_)::value;
-    OutT* row = (OutT*)p.C + (int64_t)(mrow0 + i * 16 + l16) * p.ldc + ncol0 + kg * 4;
-    static_for<NT>([&](auto J_) {
-      constexpr int j = decltype(J_)::value;
-      const f32x4 v = acc[i][j];
-      *(Out4*)(row + j * 16) = Out4{(OutT)(v[0] * alpha), (OutT)(v[1] * alpha), (OutT)(v[2] * alpha), (OutT)(v[3] * alpha)};
+    OutT* row = (OutT*)p.C + (int64_t)(mrow0 + i * 16 + l16) * p.ldc + col;
+    static_for<NT / 2>([&](auto J_) {
+      constexpr int j = 2 * decltype(J_)::value;
+      const f32x4 u = acc[i][j], v = acc[i][j + 1];
+      int a0 = __builtin_bit_cast(int, Out2{(OutT)(u[0] * alpha), (OutT)(u[1] * alpha)});
+      int a1 = __builtin_bit_cast(int, Out2{(OutT)(u[2] * alpha), (OutT)(u[3] * alpha)});
+      int b0 = __builtin_bit_cast(int, Out2{(OutT)(v[0] * alpha), (OutT)(v[1] * alpha)});
+      int b1 = __builtin_bit_cast(int, Out2{(OutT)(v[2] * alpha), (OutT)(v[3] * alpha)});
+      swap16(a0, b0);
+      swap16(a1, b1);
+      *(i32x4*)(row + j * 16) = i32x4{a0, a1, b0, b1};
     });
   });
 }
 // 0 = the problem needs the general epilogue; else the C ABI code + 1 of the 16-bit output type the lean one writes
 static inline int lean_epilogue_type(const GemmArgs& p) {
-  if (!p.lean_ok || p.aux || p.activation != 0 || p.scn != 1 || !p.c_vec_ok) return 0;
+  if (!p.lean_ok || p.aux || p.activation != 0 || p.scn != 1 || !p.c_vec_ok || p.ldc % 8 != 0) return 0;
   return p.out_dtype == 0 ? 1 : p.out_dtype == 1 ? 2 : 0;
 }
 

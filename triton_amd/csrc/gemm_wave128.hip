@@ -385,8 +385,12 @@ __device__ __forceinline__ void gemm_wave128_tiles(const GemmArgs& p, int tile, 
     int em = pm * BM + wm * (BM / 2), en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));
     using OwnT = std::conditional_t<std::is_same<V8, bf16x8>::value, __bf16, _Float16>;
-    if constexpr (EPI == 1) gemm_epilogue16_plain<MT, NT, OwnT>(acc, p, em, en, el, ek);
-    else if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, OwnT>(acc, p, em, en, el, ek);
+    if constexpr (EPI == 1) {
+      // (the grouped GEMM: C rows of 16-byte alignment, as the reference's own groups have them, take the stores of
+      // the lean epilogue - the scales are null pointers here)
+      if (p.c_vec_ok && p.ldc % 8 == 0) gemm_epilogue16_lean<MT, NT, OwnT>(acc, p, em, en, el, ek);
+      else gemm_epilogue16_plain<MT, NT, OwnT>(acc, p, em, en, el, ek);
+    } else if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, OwnT>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
     tile += tile_step;
     if (tile >= tend) break;
