@@ -173,6 +173,12 @@ __device__ __forceinline__ void swap32(float x, float& r0, float& r1) {
   r0 = a;
   r1 = b;
 }
+// The same exchange on two registers of the caller: the upper half (lanes 32 .. 63) of `a` with the lower half of `b`.
+__device__ __forceinline__ void swap32_regs(int& a, int& b) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+#endif
+}
 __device__ __forceinline__ float pair_max(float x) { float a, b; swap32(x, a, b); return fmaxf(a, b); }
 __device__ __forceinline__ float pair_sum(float x) { float a, b; swap32(x, a, b); return a + b; }
 

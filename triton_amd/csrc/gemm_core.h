@@ -91,24 +91,34 @@ __device__ __forceinline__ void gemm_epilogue(f32x16 (&acc)[MT][NT], const GemmA
   // group of four values inside the unrolled tiles - tens of KiB of code that the instruction cache has to
   // fetch at the end of every tile (the four-wave kernels, whose epilogue is the same in larger, gained 4-15 %
   // from a lean instantiation; here the choice is a branch, uniform over the workgroup).
-  if (p.lean_ok && !p.aux && p.activation == 0 && p.scn == 1 && p.c_vec_ok && (p.out_dtype == 0 || p.out_dtype == 1) &&
+  if (p.lean_ok && !p.aux && p.activation == 0 && p.scn == 1 && p.c_vec_ok && p.ldc % 8 == 0 && (p.out_dtype == 0 || p.out_dtype == 1) &&
       mrow0 + MT * 32 <= p.M && ncol0 + NT * 32 <= p.N) {
-    auto lean = [&](auto* c0) {
+    // (Rows of 16-byte alignment.)  Register groups 2 a and 2 a + 1 are exchanged between the two lanes of a row
+    // (v_permlane32_swap) - lane l32 then holds the 8 consecutive columns 16 a .. 16 a + 7 of the tile, lane
+    // l32 + 32 the next 8 - and a lane stores 16 bytes instead of two pieces of 8: half the requests to the memory
+    // pipeline, which takes one per piece (see gemm_epilogue16_lean of the four-wave kernels).
+    auto lean16 = [&](auto* c0) {
       using OutT = std::remove_pointer_t<decltype(c0)>;
-      typedef OutT Out4 __attribute__((ext_vector_type(4)));
+      typedef OutT Out2 __attribute__((ext_vector_type(2)));
       static_for<MT>([&](auto I_) {
         constexpr int i = decltype(I_)::value;
-        OutT* row = c0 + (int64_t)(mrow0 + i * 32 + l32) * p.ldc + ncol0 + g * 4;
+        OutT* row = c0 + (int64_t)(mrow0 + i * 32 + l32) * p.ldc + ncol0 + g * 8;
         static_for<NT>([&](auto J_) {
           constexpr int j = decltype(J_)::value;
 #pragma unroll
-          for (int rg = 0; rg < 4; rg++)
-            *(Out4*)(row + j * 32 + rg * 8) = Out4{(OutT)(acc[i][j][rg * 4] * alpha), (OutT)(acc[i][j][rg * 4 + 1] * alpha),
-                                                   (OutT)(acc[i][j][rg * 4 + 2] * alpha), (OutT)(acc[i][j][rg * 4 + 3] * alpha)};
+          for (int a = 0; a < 2; a++) {
+            int x0 = __builtin_bit_cast(int, Out2{(OutT)(acc[i][j][a * 8] * alpha), (OutT)(acc[i][j][a * 8 + 1] * alpha)});
+            int x1 = __builtin_bit_cast(int, Out2{(OutT)(acc[i][j][a * 8 + 2] * alpha), (OutT)(acc[i][j][a * 8 + 3] * alpha)});
+            int y0 = __builtin_bit_cast(int, Out2{(OutT)(acc[i][j][a * 8 + 4] * alpha), (OutT)(acc[i][j][a * 8 + 5] * alpha)});
+            int y1 = __builtin_bit_cast(int, Out2{(OutT)(acc[i][j][a * 8 + 6] * alpha), (OutT)(acc[i][j][a * 8 + 7] * alpha)});
+            swap32_regs(x0, y0);
+            swap32_regs(x1, y1);
+            *(i32x4*)(row + j * 32 + a * 16) = i32x4{x0, x1, y0, y1};
+          }
         });
       });
     };
-    if (p.out_dtype == 1) lean((__bf16*)p.C); else lean((_Float16*)p.C);
+    if (p.out_dtype == 1) lean16((__bf16*)p.C); else lean16((_Float16*)p.C);
     return;
   }
   const bool leaky = p.activation == 1;
