@@ -27,7 +27,7 @@ HBM_GBPS = 8000.0
 # rocprofv3 around the process): taken from the two rocprofv3 --pmc runs of this same command that
 # profiles/gemm_bf16_8192.md records - FETCH_SIZE and WRITE_SIZE in KiB per dispatch, each scaled by what
 # the same counter reads for a plain device copy of known size (--copy-calibration).
-MEASURED_TRAFFIC_KIB = {"FETCH_SIZE": 847261, "FETCH_scale": 2.000, "WRITE_SIZE": 137311, "WRITE_scale": 1.000}   # medians over > 1100 dispatches
+MEASURED_TRAFFIC_KIB = {"FETCH_SIZE": 844913, "FETCH_scale": 2.000, "WRITE_SIZE": 136400, "WRITE_scale": 1.000}   # medians over > 1100 dispatches
 MEASURED_TRAFFIC_BYTES = int((MEASURED_TRAFFIC_KIB["FETCH_SIZE"] * MEASURED_TRAFFIC_KIB["FETCH_scale"]
                               + MEASURED_TRAFFIC_KIB["WRITE_SIZE"] * MEASURED_TRAFFIC_KIB["WRITE_scale"]) * 1024)
 TRAFFIC_SOURCE = "profiles/gemm_bf16_8192.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, separate runs of this command; not measured in this run)"
