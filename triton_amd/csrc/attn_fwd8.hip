@@ -245,18 +245,25 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd8_kernel(Att
   {
     const float l = pair_sum(l_i);
     const int row = row0 + l32;
-    if (row < p.N) {
+    if (row0 < p.N) {   // (wave-uniform: N is a multiple of 32)
       const float inv = 1.f / l;
       if (g == 0) p.lse[(int64_t)hz * p.N + row] = m_i + log2f(l);
-      char* dst = obase + (int64_t)row * opitch;
+      // A lane owns one dword (4 codes) per register group: dwords 0, 2, 4, 6 of a tile's 32-byte row segment in lane
+      // l32, dwords 1, 3, 5, 7 in lane l32 + 32.  Two exchanges between the lanes of a row (v_permlane32_swap: the
+      // upper half of the first register with the lower half of the second) give lane l32 the dwords 0 .. 3 and lane
+      // l32 + 32 the dwords 4 .. 7: one store of 16 bytes per tile instead of four of 4 bytes - the memory pipeline
+      // takes a request per piece.
+      char* dst = obase + (int64_t)row * opitch + g * 16;
 #pragma unroll
-      for (int c = 0; c < DT; c++)
+      for (int c = 0; c < DT; c++) {
+        int w[4];
 #pragma unroll
-        for (int rg = 0; rg < 4; rg++) {
-          const int d = c * 32 + rg * 8 + g * 4;
-          *(int*)(dst + d) = pack4_fp8<FMT>(oacc[c][rg * 4] * inv, oacc[c][rg * 4 + 1] * inv,
-                                            oacc[c][rg * 4 + 2] * inv, oacc[c][rg * 4 + 3] * inv);
-        }
+        for (int rg = 0; rg < 4; rg++)
+          w[rg] = pack4_fp8<FMT>(oacc[c][rg * 4] * inv, oacc[c][rg * 4 + 1] * inv, oacc[c][rg * 4 + 2] * inv, oacc[c][rg * 4 + 3] * inv);
+        swap32_regs(w[0], w[2]);
+        swap32_regs(w[1], w[3]);
+        *(i32x4*)(dst + c * 32) = i32x4{w[0], w[2], w[1], w[3]};
+      }
     }
   }
 }
