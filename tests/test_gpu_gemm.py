@@ -447,6 +447,10 @@ def test_four_wave_kernel_k_tails_are_bit_exact(gpu, monkeypatch, dtype, layout,
             tb = tb.t().contiguous().t()
         got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
         assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32")), (K, dtype, layout, programs)
+        # C in the operands' own type: the form of the four-wave kernel that has the tail (the fp32 output above is
+        # another kernel's); the exact integer sums, rounded once
+        own = to_np(triton_amd.matmul(ta, tb))
+        assert bits_equal(own, gemm.matmul_closed_form(a, b, out_dtype=dtype)), (K, dtype, layout, programs, "own type")
 
 
 @pytest.mark.parametrize("layout", ["row_major_b", "k_major_b"])
