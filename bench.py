@@ -53,9 +53,24 @@ def time_launches(fn, steps, warmup):
     return wall_ms, sum(per) / len(per), per
 
 
+def settle(fn, seconds=0.06, limit=4000):
+    """Untimed launches for `seconds` of wall time (at most `limit` of them): after a change of kernel, and more so
+    after an idle phase, the board takes tens of milliseconds to settle its clocks - the first 10 launches of the
+    8192^3 GEMM read 3 % below what follows, 40 launches of the 0.25 ms grouped GEMM 14 % (975 against 1110-1130
+    TFLOP/s), and the 15-30 us skinny kernels never got there within their warm-up launches."""
+    import torch
+
+    t0 = time.perf_counter()
+    done = 0
+    while done < limit and time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        done += 20
+        torch.cuda.synchronize()
+
+
 def quick(fn, iters=60, warmup=20):
-    # (long enough for the clock to settle after the change of kernel: at 10 + 30 launches of ~0.4 ms the
-    # block-scaled and fp8 GEMMs read 8-10 % below what they sustain)
+    settle(fn)
     _, ev_ms, _ = time_launches(fn, iters, warmup)
     return ev_ms
 
@@ -342,8 +357,9 @@ def secondary_workloads(lib, dev, n):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    # (100 launches = 75 ms: the clocks have settled by then; with 10 the timed region starts 3 % low)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--size", type=int, default=8192)
@@ -373,6 +389,7 @@ def main():
             print("bench.py: --only takes one of " + ", ".join(table), file=sys.stderr)
             sys.exit(2)
         fn, work, kind, info, _ = table[args.only]()
+        settle(fn)
         wall_ms, ev_ms, _ = time_launches(fn, args.steps, args.warmup)
         rec = {"workload": args.only, "steps": args.steps, "ms_per_launch": round(ev_ms, 5),
                ("tflops" if kind == "flops" else "gbps"): round(work / ev_ms / (1e9 if kind == "flops" else 1e6), 1)}
