@@ -817,3 +817,30 @@ def test_3072_cubed_takes_the_192_row_tiles_and_matches_sampled_rows(gpu):
     rows = rng.choice(n, size=24, replace=False)
     ref = a[rows].astype(np.float64) @ b.astype(np.float64)
     assert np.allclose(got[rows], ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(512, 512, 512), (4096, 4096, 512)])
+@pytest.mark.parametrize("pad", [4, 8])
+def test_c_rows_of_8_and_16_byte_alignment_through_the_c_abi(gpu, shape, pad):
+    # The short epilogues store 16 bytes per lane (neighbouring accumulator groups exchanged between lanes first),
+    # which needs C rows of 16-byte alignment; a row pitch that is a multiple of 4 but not of 8 elements takes the
+    # general epilogue with its 8-byte stores.  Both through mi355_gemm directly with C a view into a wider buffer
+    # (the Python surface always allocates a dense C): small tiles and the four-wave kernel, integer data, the bits
+    # of the closed form, and the columns beyond N untouched.
+    from triton_amd import _lib
+
+    M, N, K = shape
+    rng = np.random.default_rng(M + pad)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    ta, tb = from_np(a, "bf16", gpu), from_np(b, "bf16", gpu)
+    buf = torch.full((M, N + pad), 7.0, dtype=torch.bfloat16, device=gpu)
+    c = buf[:, :N]
+    rc = _lib.load().mi355_gemm(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), M, N, K,
+                                ta.stride(0), ta.stride(1), tb.stride(0), tb.stride(1), c.stride(0), c.stride(1),
+                                _lib.BF16, _lib.BF16, None, None, 0, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert bits_equal(to_np(c), gemm.matmul_closed_form(a, b, out_dtype="bf16")), (shape, pad)
+    assert bool((buf[:, N:] == 7.0).all())
