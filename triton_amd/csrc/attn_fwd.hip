@@ -406,11 +406,14 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
     lds_zero(lds, 2 * 2 * TILE, tid, NW * 64);
     __syncthreads();
   }
+  // (f_k / f_v point at the tile to fetch and move on by one tile per step: two scalar additions instead of the
+  // 64-bit products of a step number - the bookkeeping of this function stands in front of every step's MFMAs)
+  const int64_t kstep = (int64_t)BN * kpitch, vstep = (int64_t)BN * vpitch;
   auto issue_fill = [&](int stage) {
     if (!f_valid) return;
     const unsigned kd = lds_base + stage * (2 * TILE), vd = kd + TILE;
-    const char* ksrc = f_k + (int64_t)fj * BN * kpitch;
-    const char* vsrc = f_v + (int64_t)fj * BN * vpitch;
+    const char* ksrc = f_k;
+    const char* vsrc = f_v;
 #pragma unroll
     for (int i = 0; i < INST; i++) {
       if (present[i]) {
@@ -418,6 +421,8 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd_stream_kern
         async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
       }
     }
+    f_k += kstep;
+    f_v += vstep;
     if (++fj == f_steps) {
       fj = 0;
       if (++f_item < nitems) {
