@@ -26,10 +26,15 @@ namespace mi355 {
 template <typename V8_> struct Skinny16 { using V = V8_; static constexpr bool kF8 = false; static constexpr int kFmt = 0; };
 template <int FMT> struct Skinny8 { using V = i32x4; static constexpr bool kF8 = true; static constexpr int kFmt = FMT; };  // 0 e4m3fn, 1 e5m2
 
-template <typename E, bool Y_LDS, int XM, int ST, int NW, int NS>
+// YM: 0 = K-contiguous Y, every lane streams its own row straight into registers (32-byte pieces of 32 rows per
+//         instruction; kept for comparison);
+//     1 = L-contiguous Y through LDS with a transposed read;
+//     2 = K-contiguous Y through LDS (64-byte pieces of 16 rows per instruction, as for X)
+template <typename E, int YM, int XM, int ST, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   using V8 = typename E::V;  // one 16-byte register group of an operand
   constexpr bool F8 = E::kF8;
+  constexpr bool Y_LDS = YM == 1;
   static_assert(!F8 || (!Y_LDS && XM == 2), "fp8: both operands K-contiguous, X through LDS");
   constexpr int PD = NS - 1;          // stages in flight
   constexpr int LPS = 2 + 2 * ST;     // vector-memory operations per stage: 2 of Y, 2 per 32 rows of X
@@ -39,7 +44,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr bool X_LDS = XM != 0;
   static_assert(!(Y_LDS && XM == 1), "one operand at most is transposed through LDS");
   constexpr int XROW = 64 * ST;       // bytes of one k row of an S-contiguous X tile: S = 32 ST
-  constexpr int YSLOT = Y_LDS ? 2048 : 0;        // [32 k][32 l] 16-bit
+  constexpr int YSLOT = YM != 0 ? 2048 : 0;      // [32 k][32 l] 16-bit, or [32 l][64 bytes of k]
   constexpr int XSLOT = X_LDS ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
   constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
   static_assert(PD * LPS < 64, "vmcnt has 6 bits");
@@ -92,6 +97,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) xrd[ks] = ring + YSLOT + l32 * 64 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 2) & 3)) << 4);
 
+  // K-contiguous Y through LDS: direct load i moves rows 16 i .. 16 i + 15, 64 bytes of k each, chunk c of row r at
+  // position c ^ ((r >> 2) & 3); read back row-wise like X
+  unsigned ydma2[2], yrd[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int r = 16 * i + (lane >> 2);
+    ydma2[i] = (unsigned)r * (unsigned)p.y_pitch + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
+  }
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) yrd[ks] = ring + l32 * 64 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 2) & 3)) << 4);
   V8 xr[NS][2][ST], yr[NS][2];
   auto issue = [&](int j, auto SLOT_) {
     constexpr int sl = decltype(SLOT_)::value;
@@ -99,6 +114,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       const char* src = ybase + (int64_t)j * 32 * p.y_pitch;
       async_copy16_sbase(src, yoff, ring + sl * SLOT);
       async_copy16_sbase(src + 16 * p.y_pitch, yoff, ring + sl * SLOT + 1024);
+    } else if constexpr (YM == 2) {
+      const char* src = ybase + (int64_t)j * 64;
+      async_copy16_sbase(src, ydma2[0], ring + sl * SLOT);
+      async_copy16_sbase(src, ydma2[1], ring + sl * SLOT + 1024);
     } else {
       const char* src = ybase + (int64_t)j * 64;
       load16_sbase<0>(yr[sl][0], src, yoff);
@@ -108,7 +127,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       const char* xsrc = p.X + (int64_t)j * 32 * p.x_pitch;
 #pragma unroll
       for (int i = 0; i < 2 * ST; i++)
-        async_copy16_sbase(xsrc + (int64_t)i * (16 / ST) * p.x_pitch, xdma, ring + sl * SLOT + i * 1024);
+        async_copy16_sbase(xsrc + (int64_t)i * (16 / ST) * p.x_pitch, xdma, ring + sl * SLOT + YSLOT + i * 1024);
     } else if constexpr (XM == 2) {
       const char* xsrc = p.X + (int64_t)j * 64;
 #pragma unroll
@@ -138,6 +157,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
         lds_use(hi[ks]);
         yf[ks] = __builtin_bit_cast(V8, (i32x4)__builtin_shufflevector(lo[ks], hi[ks], 0, 1, 2, 3));
       }
+    } else if constexpr (YM == 2) {
+      i32x4 yv[2];
+      yv[0] = lds_read_b128<sl * SLOT>(yrd[0]);
+      yv[1] = lds_read_b128<sl * SLOT>(yrd[1]);
+      lds_wait<0>();
+      lds_use(yv[0]);
+      lds_use(yv[1]);
+      yf[0] = __builtin_bit_cast(V8, yv[0]);
+      yf[1] = __builtin_bit_cast(V8, yv[1]);
     } else {
       lds_use(yr[sl][0]);
       lds_use(yr[sl][1]);
@@ -168,8 +196,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
         constexpr int ks = decltype(KS_)::value;
         static_for<ST>([&](auto T_) {
           constexpr int t = decltype(T_)::value;
-          lo[ks][t] = lds_read_tr16_b64<sl * SLOT + 16 * ks * XROW + t * 64>(tl);
-          hi[ks][t] = lds_read_tr16_b64<sl * SLOT + (16 * ks + 4) * XROW + t * 64>(tl);
+          lo[ks][t] = lds_read_tr16_b64<sl * SLOT + YSLOT + 16 * ks * XROW + t * 64>(tl);
+          hi[ks][t] = lds_read_tr16_b64<sl * SLOT + YSLOT + (16 * ks + 4) * XROW + t * 64>(tl);
         });
       });
       lds_wait<0>();
@@ -261,21 +289,21 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   }
 }
 
-template <typename E, bool Y_LDS, int XM, int ST>
+template <typename E, int YM, int XM, int ST>
 static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   // four waves with three stages in flight each already saturate what this access pattern gets
   // from HBM; the small LDS footprint lets several workgroups share a CU
   constexpr int NW = 4, NS = 4;
-  constexpr int ring = NW * NS * ((Y_LDS ? 2048 : 0) + (XM ? 2048 * ST : 0)), red = NW * ST * 16 * 64 * 4;
+  constexpr int ring = NW * NS * ((YM ? 2048 : 0) + (XM ? 2048 * ST : 0)), red = NW * ST * 16 * 64 * 4;
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<E, Y_LDS, XM, ST, NW, NS>,
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_skinny_kernel<E, YM, XM, ST, NW, NS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  gemm_skinny_kernel<E, Y_LDS, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
+  gemm_skinny_kernel<E, YM, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -291,20 +319,26 @@ bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_
          p.x_pitch % 16 == 0 && p.y_pitch % 16 == 0 && p.x_pitch < (1 << 25) && p.y_pitch < (1 << 26);
 }
 
+// how a K-contiguous Y travels (see YM above)
+#ifndef MI355_SKINNY_Y_KMAJOR_MODE
+#define MI355_SKINNY_Y_KMAJOR_MODE 2
+#endif
+constexpr int YK = MI355_SKINNY_Y_KMAJOR_MODE;
+
 template <typename V8>
 static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
   using E = Skinny16<V8>;
   const bool two = p.S > 32;
-  if (!x_kmajor) return two ? launch_skinny<E, false, 1, 2>(p, stream) : launch_skinny<E, false, 1, 1>(p, stream);
-  if (y_kmajor) return two ? launch_skinny<E, false, 2, 2>(p, stream) : launch_skinny<E, false, 2, 1>(p, stream);
-  return two ? launch_skinny<E, true, 2, 2>(p, stream) : launch_skinny<E, true, 2, 1>(p, stream);
+  if (!x_kmajor) return two ? launch_skinny<E, YK, 1, 2>(p, stream) : launch_skinny<E, YK, 1, 1>(p, stream);
+  if (y_kmajor) return two ? launch_skinny<E, YK, 2, 2>(p, stream) : launch_skinny<E, YK, 2, 1>(p, stream);
+  return two ? launch_skinny<E, 1, 2, 2>(p, stream) : launch_skinny<E, 1, 2, 1>(p, stream);
 }
 
 // kind: 0 fp16, 1 bf16, 2 fp8 e4m3fn, 3 fp8 e5m2 (the dtype codes of the C ABI)
 int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
   const bool two = p.S > 32;
-  if (kind == 2) return two ? launch_skinny<Skinny8<0>, false, 2, 2>(p, stream) : launch_skinny<Skinny8<0>, false, 2, 1>(p, stream);
-  if (kind == 3) return two ? launch_skinny<Skinny8<1>, false, 2, 2>(p, stream) : launch_skinny<Skinny8<1>, false, 2, 1>(p, stream);
+  if (kind == 2) return two ? launch_skinny<Skinny8<0>, YK, 2, 2>(p, stream) : launch_skinny<Skinny8<0>, YK, 2, 1>(p, stream);
+  if (kind == 3) return two ? launch_skinny<Skinny8<1>, YK, 2, 2>(p, stream) : launch_skinny<Skinny8<1>, YK, 2, 1>(p, stream);
   return kind == 1 ? launch_skinny_v<bf16x8>(p, y_kmajor, x_kmajor, stream) : launch_skinny_v<f16x8>(p, y_kmajor, x_kmajor, stream);
 }
 
