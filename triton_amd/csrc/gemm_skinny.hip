@@ -29,7 +29,11 @@ template <int FMT> struct Skinny8 { using V = i32x4; static constexpr bool kF8 =
 // YM: 0 = K-contiguous Y, every lane streams its own row straight into registers (32-byte pieces of 32 rows per
 //         instruction; kept for comparison);
 //     1 = L-contiguous Y through LDS with a transposed read;
-//     2 = K-contiguous Y through LDS (64-byte pieces of 16 rows per instruction, as for X)
+//     2 = K-contiguous Y through LDS (64-byte pieces of 16 rows per instruction, as for X);
+//     3 = K-contiguous Y through LDS in whole 128-byte lines (8 rows per instruction): two stages share a tile of
+//         [32 l][128 bytes of k] in a ring of its own; the loads of rows 0-15 ride with the odd stage before the
+//         pair, those of rows 16-31 with its even stage, so every stage still issues two Y loads (needs K bytes a
+//         multiple of 128)
 template <typename E, int YM, int XM, int ST, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   using V8 = typename E::V;  // one 16-byte register group of an operand
@@ -44,7 +48,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr bool X_LDS = XM != 0;
   static_assert(!(Y_LDS && XM == 1), "one operand at most is transposed through LDS");
   constexpr int XROW = 64 * ST;       // bytes of one k row of an S-contiguous X tile: S = 32 ST
-  constexpr int YSLOT = YM != 0 ? 2048 : 0;      // [32 k][32 l] 16-bit, or [32 l][64 bytes of k]
+  constexpr int YSLOT = (YM == 1 || YM == 2) ? 2048 : 0;   // [32 k][32 l] 16-bit, or [32 l][64 bytes of k]
+  constexpr int ND = 4, YPAIR = 4096;            // YM == 3: ring of ND tiles [32 l][128 bytes of k] behind the stage ring
   constexpr int XSLOT = X_LDS ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
   constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
   static_assert(PD * LPS < 64, "vmcnt has 6 bits");
@@ -58,7 +63,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   const int l0 = xcd_remap(blockIdx.x, gridDim.x) * 32;
 
   const int nstages = p.K / (F8 ? 64 : 32);
-  const int per = (nstages + NW - 1) / NW;
+  const int per = YM == 3 ? (((nstages + NW - 1) / NW + 1) & ~1) : (nstages + NW - 1) / NW;   // (YM 3: whole pairs of stages)
   const int j_lo = wave * per, j_hi = min(nstages, j_lo + per);
 
   f32x16 acc[ST];
@@ -107,6 +112,17 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   }
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) yrd[ks] = ring + l32 * 64 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 2) & 3)) << 4);
+  // YM == 3: load instruction i of a pair moves rows 8 i .. 8 i + 7, all 128 bytes; chunk c of row r at position
+  // c ^ ((r >> 1) & 7) (rows are 128 bytes apart: two rows per sweep of the banks)
+  const unsigned yring = lds_addr(lds) + NW * (NS * SLOT) + wave * (ND * YPAIR);
+  // (row r = 8 i + lane / 8: (r >> 1) & 7 = 4 (i & 1) + lane / 16; the lane's slot is lane % 8, so it fetches chunk
+  // (lane % 8) ^ that term)
+  unsigned ydma3[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++) ydma3[i] = (unsigned)(lane >> 3) * (unsigned)p.y_pitch + (((lane & 7) ^ (4 * i + (lane >> 4))) << 4);
+  unsigned yrd3[2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ks++) yrd3[ks] = yring + l32 * 128 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 1) & 7)) << 4);
   V8 xr[NS][2][ST], yr[NS][2];
   auto issue = [&](int j, auto SLOT_) {
     constexpr int sl = decltype(SLOT_)::value;
@@ -118,6 +134,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       const char* src = ybase + (int64_t)j * 64;
       async_copy16_sbase(src, ydma2[0], ring + sl * SLOT);
       async_copy16_sbase(src, ydma2[1], ring + sl * SLOT + 1024);
+    } else if constexpr (YM == 3) {
+      // odd stage: rows 0-15 of the NEXT pair (the last pair again where there is none); even stage: rows 16-31 of its own
+      const int d = min((j + 1) >> 1, (j_hi >> 1) - 1), half = (j & 1) ^ 1;
+      const char* src = ybase + (int64_t)d * 128 + (int64_t)(16 * half) * p.y_pitch;
+      const unsigned dst = yring + (d & (ND - 1)) * YPAIR + half * 2048;
+      // (the XOR term of rows 8 .. 15 of a half is 4 more than that of rows 0 .. 7)
+      async_copy16_sbase(src, ydma3[0], dst);
+      async_copy16_sbase(src + 8 * p.y_pitch, ydma3[1], dst + 1024);
     } else {
       const char* src = ybase + (int64_t)j * 64;
       load16_sbase<0>(yr[sl][0], src, yoff);
@@ -141,7 +165,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       }
     }
   };
-  auto compute = [&](auto SLOT_) {
+  auto compute = [&](const int j, auto SLOT_) {
     constexpr int sl = decltype(SLOT_)::value;
     V8 yf[2];
     if constexpr (Y_LDS) {
@@ -157,6 +181,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
         lds_use(hi[ks]);
         yf[ks] = __builtin_bit_cast(V8, (i32x4)__builtin_shufflevector(lo[ks], hi[ks], 0, 1, 2, 3));
       }
+    } else if constexpr (YM == 3) {
+      // (the stage's parity is the slot's: ranges start on even stages and the ring has an even number of slots;
+      // the odd stage's chunks are 4 further, which flips bit 2 of the swizzled position)
+      const unsigned yb = (unsigned)((j >> 1) & (ND - 1)) * YPAIR;
+      i32x4 yv[2];
+      yv[0] = lds_read_b128<0>((yrd3[0] ^ ((sl & 1) * 64u)) + yb);
+      yv[1] = lds_read_b128<0>((yrd3[1] ^ ((sl & 1) * 64u)) + yb);
+      lds_wait<0>();
+      lds_use(yv[0]);
+      lds_use(yv[1]);
+      yf[0] = __builtin_bit_cast(V8, yv[0]);
+      yf[1] = __builtin_bit_cast(V8, yv[1]);
     } else if constexpr (YM == 2) {
       i32x4 yv[2];
       yv[0] = lds_read_b128<sl * SLOT>(yrd[0]);
@@ -238,6 +274,14 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   if (j_lo < j_hi) {
     // past the end of the range the last stage is fetched again: the number of outstanding
     // operations, and with it the partial wait, stays uniform
+    if constexpr (YM == 3) {
+      // rows 0-15 of the first pair (in the stream they ride with the odd stage before a pair)
+      const int d = j_lo >> 1;
+      const char* src = ybase + (int64_t)d * 128;
+      const unsigned dst = yring + (d & (ND - 1)) * YPAIR;
+      async_copy16_sbase(src, ydma3[0], dst);
+      async_copy16_sbase(src + 8 * p.y_pitch, ydma3[1], dst + 1024);
+    }
     static_for<PD>([&](auto S_) { issue(min(j_lo + decltype(S_)::value, j_hi - 1), S_); });
     for (int j = j_lo; j < j_hi; j += NS) {
       static_for<NS>([&](auto U_) {
@@ -246,7 +290,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
           issue(min(j + u + PD, j_hi - 1), std::integral_constant<int, (u + PD) % NS>{});
           wait_vmcnt<PD * LPS>();
           __builtin_amdgcn_sched_barrier(0);
-          compute(U_);
+          compute(j + u, U_);
           __builtin_amdgcn_sched_barrier(0);
         }
       });
@@ -294,7 +338,7 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   // four waves with three stages in flight each already saturate what this access pattern gets
   // from HBM; the small LDS footprint lets several workgroups share a CU
   constexpr int NW = 4, NS = 4;
-  constexpr int ring = NW * NS * ((YM ? 2048 : 0) + (XM ? 2048 * ST : 0)), red = NW * ST * 16 * 64 * 4;
+  constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : 0) + (XM ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0), red = NW * ST * 16 * 64 * 4;
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
@@ -321,24 +365,34 @@ bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_
 
 // how a K-contiguous Y travels (see YM above)
 #ifndef MI355_SKINNY_Y_KMAJOR_MODE
-#define MI355_SKINNY_Y_KMAJOR_MODE 2
+#define MI355_SKINNY_Y_KMAJOR_MODE 3
 #endif
 constexpr int YK = MI355_SKINNY_Y_KMAJOR_MODE;
+// a K-contiguous Y: whole lines (mode 3) where K bytes are a multiple of 128, else 64-byte pieces
+template <typename E, int XM, int ST>
+static int launch_skinny_yk(const SkinnyArgs& p, int elem_bytes, hipStream_t stream) {
+  if constexpr (YK == 3) {
+    if (((int64_t)p.K * elem_bytes) % 128 == 0) return launch_skinny<E, 3, XM, ST>(p, stream);
+    return launch_skinny<E, 2, XM, ST>(p, stream);
+  } else {
+    return launch_skinny<E, YK, XM, ST>(p, stream);
+  }
+}
 
 template <typename V8>
 static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
   using E = Skinny16<V8>;
   const bool two = p.S > 32;
-  if (!x_kmajor) return two ? launch_skinny<E, YK, 1, 2>(p, stream) : launch_skinny<E, YK, 1, 1>(p, stream);
-  if (y_kmajor) return two ? launch_skinny<E, YK, 2, 2>(p, stream) : launch_skinny<E, YK, 2, 1>(p, stream);
+  if (!x_kmajor) return two ? launch_skinny_yk<E, 1, 2>(p, 2, stream) : launch_skinny_yk<E, 1, 1>(p, 2, stream);
+  if (y_kmajor) return two ? launch_skinny_yk<E, 2, 2>(p, 2, stream) : launch_skinny_yk<E, 2, 1>(p, 2, stream);
   return two ? launch_skinny<E, 1, 2, 2>(p, stream) : launch_skinny<E, 1, 2, 1>(p, stream);
 }
 
 // kind: 0 fp16, 1 bf16, 2 fp8 e4m3fn, 3 fp8 e5m2 (the dtype codes of the C ABI)
 int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmajor, hipStream_t stream) {
   const bool two = p.S > 32;
-  if (kind == 2) return two ? launch_skinny<Skinny8<0>, YK, 2, 2>(p, stream) : launch_skinny<Skinny8<0>, YK, 2, 1>(p, stream);
-  if (kind == 3) return two ? launch_skinny<Skinny8<1>, YK, 2, 2>(p, stream) : launch_skinny<Skinny8<1>, YK, 2, 1>(p, stream);
+  if (kind == 2) return two ? launch_skinny_yk<Skinny8<0>, 2, 2>(p, 1, stream) : launch_skinny_yk<Skinny8<0>, 2, 1>(p, 1, stream);
+  if (kind == 3) return two ? launch_skinny_yk<Skinny8<1>, 2, 2>(p, 1, stream) : launch_skinny_yk<Skinny8<1>, 2, 1>(p, 1, stream);
   return kind == 1 ? launch_skinny_v<bf16x8>(p, y_kmajor, x_kmajor, stream) : launch_skinny_v<f16x8>(p, y_kmajor, x_kmajor, stream);
 }
 
