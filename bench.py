@@ -270,6 +270,20 @@ def secondary_workloads(lib, dev, n):
     for (sm, sn, sk) in ((16, n, n), (64, n, n), (n, 64, n)):
         W[f"fp16_skinny_{sm}x{sn}x{sk}"] = skinny(sm, sn, sk)
 
+    # the decode shape with the weight as a linear layer stores it: B[N, K], K contiguous (x @ W^T)
+    def decode_kmajor():
+        xa = torch.randn(16, n, device=dev, dtype=torch.float16)
+        xw = torch.randn(n, n, device=dev, dtype=torch.float16)   # [N, K]
+        xc = torch.empty(16, n, device=dev, dtype=torch.float16)
+
+        def fn():
+            rc = lib.mi355_gemm(xa.data_ptr(), xw.data_ptr(), xc.data_ptr(), 16, n, n, n, 1, 1, n, n, 1,
+                                _lib.F16, _lib.F16, None, None, 0, stream)
+            assert rc == 0, rc
+
+        return fn, 2 * (16 * n + n * n + 16 * n), "bytes", {}, 50
+    W["fp16_decode_m16_kmajor_weight"] = decode_kmajor
+
     # grouped GEMM (tutorial 08): 16 fp16 problems of 2048^3 in one launch; launch only, device tables prepared
     # once (like `triton_perf_fn`, 08:217-228)
     def grouped():
