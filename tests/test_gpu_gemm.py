@@ -844,3 +844,23 @@ def test_c_rows_of_8_and_16_byte_alignment_through_the_c_abi(gpu, shape, pad):
     torch.cuda.synchronize()
     assert bits_equal(to_np(c), gemm.matmul_closed_form(a, b, out_dtype="bf16")), (shape, pad)
     assert bool((buf[:, N:] == 7.0).all())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("shape", [(16, 16384, 512), (7, 32768, 192), (32, 16448, 96), (1, 16384, 2048)])
+def test_skinny_kernel_with_64_columns_per_workgroup_is_bit_exact(gpu, dtype, shape):
+    # a row-major B wide enough that 64 columns per workgroup still cover the compute units (N / 64 >= 256): the
+    # form of the streaming kernel that fetches whole 128-byte lines of B - two column tiles per wave, eight waves
+    # splitting K, k rows with bit 1 set stored with their halves swapped.  Exact integer sums (K from 3 to 64
+    # stages, so some waves get none), every M class, an epilogue with the addend; N = 16448 has 257 workgroups.
+    M, N, K = shape
+    rng = np.random.default_rng(M + N + K)
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    d = rng.integers(-3, 4, size=(M, N)).astype(np.float32)
+    ta, tb, td = from_np(a, dtype, gpu), from_np(b, dtype, gpu), torch.from_numpy(d).to(gpu)
+    got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+    assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32")), (dtype, shape)
+    got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=td))
+    assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32") + d), (dtype, shape, "addend")

@@ -229,7 +229,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
-    sk.activation = activation; sk.out_dtype = out_dtype;
+    sk.activation = activation; sk.out_dtype = out_dtype; sk.cus = device_info().cus;
     bool use = false, y_kmajor = false, x_kmajor = true;
     if (M <= 64) {
       sk.X = (const char*)A; sk.Y = (const char*)B; sk.S = M; sk.L = N;

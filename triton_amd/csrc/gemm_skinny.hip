@@ -33,22 +33,27 @@ template <int FMT> struct Skinny8 { using V = i32x4; static constexpr bool kF8 =
 //     3 = K-contiguous Y through LDS in whole 128-byte lines (8 rows per instruction): two stages share a tile of
 //         [32 l][128 bytes of k] in a ring of its own; the loads of rows 0-15 ride with the odd stage before the
 //         pair, those of rows 16-31 with its even stage, so every stage still issues two Y loads (needs K bytes a
-//         multiple of 128)
+//         multiple of 128);
+//     4 = L-contiguous Y in whole 128-byte lines: the workgroup owns 64 columns (two 32-column tiles per wave, eight
+//         waves that split K eight ways), a stage is a [32 k][64 l] tile fetched 8 k rows per instruction and read back
+//         transposed (needs L a multiple of 64; chosen where L / 64 workgroups still cover the compute units)
 template <typename E, int YM, int XM, int ST, int NW, int NS>
 __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   using V8 = typename E::V;  // one 16-byte register group of an operand
   constexpr bool F8 = E::kF8;
   constexpr bool Y_LDS = YM == 1;
-  static_assert(!F8 || (!Y_LDS && XM == 2), "fp8: both operands K-contiguous, X through LDS");
+  constexpr int LT = YM == 4 ? 2 : 1;   // 32-column tiles of the output per wave
+  constexpr int TT = LT * ST;           // accumulator tiles per wave: [LT][ST]
+  static_assert(!F8 || (!Y_LDS && YM != 4 && XM == 2), "fp8: both operands K-contiguous, X through LDS");
   constexpr int PD = NS - 1;          // stages in flight
-  constexpr int LPS = 2 + 2 * ST;     // vector-memory operations per stage: 2 of Y, 2 per 32 rows of X
+  constexpr int LPS = (YM == 4 ? 4 : 2) + 2 * ST;   // vector-memory operations per stage: 2 (4) of Y, 2 per 32 rows of X
   // X: 0 = K contiguous, straight into registers (32-byte pieces of 32 rows per instruction: slower,
   //        kept for comparison); 1 = S contiguous, through LDS with a transposed read;
   //    2 = K contiguous, through LDS (64-byte pieces of 16 rows per instruction)
   constexpr bool X_LDS = XM != 0;
-  static_assert(!(Y_LDS && XM == 1), "one operand at most is transposed through LDS");
+  static_assert(!((Y_LDS || YM == 4) && XM == 1), "one operand at most is transposed through LDS");
   constexpr int XROW = 64 * ST;       // bytes of one k row of an S-contiguous X tile: S = 32 ST
-  constexpr int YSLOT = (YM == 1 || YM == 2) ? 2048 : 0;   // [32 k][32 l] 16-bit, or [32 l][64 bytes of k]
+  constexpr int YSLOT = (YM == 1 || YM == 2) ? 2048 : YM == 4 ? 4096 : 0;   // [32 k][32 l] 16-bit, [32 l][64 bytes of k], or [32 k][64 l]
   constexpr int ND = 4, YPAIR = 4096;            // YM == 3: ring of ND tiles [32 l][128 bytes of k] behind the stage ring
   constexpr int XSLOT = X_LDS ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
   constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
@@ -60,15 +65,15 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l32 = lane & 31, g = lane >> 5, i16 = lane & 15, q = lane >> 4;
   // neighbouring 32-column blocks (the two halves of a 128-byte line of an L-contiguous Y) on one XCD
-  const int l0 = xcd_remap(blockIdx.x, gridDim.x) * 32;
+  const int l0 = xcd_remap(blockIdx.x, gridDim.x) * (32 * LT);
 
   const int nstages = p.K / (F8 ? 64 : 32);
   const int per = YM == 3 ? (((nstages + NW - 1) / NW + 1) & ~1) : (nstages + NW - 1) / NW;   // (YM 3: whole pairs of stages)
   const int j_lo = wave * per, j_hi = min(nstages, j_lo + per);
 
-  f32x16 acc[ST];
+  f32x16 acc[TT];
 #pragma unroll
-  for (int t = 0; t < ST; t++)
+  for (int t = 0; t < TT; t++)
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[t][r] = 0.f;
 
@@ -88,7 +93,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
     xdma2[i] = (unsigned)min(r, p.S - 1) * (unsigned)p.x_pitch + (((lane & 3) ^ ((r >> 2) & 3)) << 4);
   }
   // K-contiguous Y: the lane's own row
-  const char* const ybase = Y_LDS ? p.Y + (int64_t)l0 * 2 : p.Y + (int64_t)l0 * p.y_pitch;
+  const char* const ybase = (Y_LDS || YM == 4) ? p.Y + (int64_t)l0 * 2 : p.Y + (int64_t)l0 * p.y_pitch;
   // L-contiguous Y: direct load i of a stage moves k rows 16 i .. 16 i + 15, 64 bytes (32 l) each
   const unsigned yoff = Y_LDS ? (unsigned)(lane >> 2) * (unsigned)p.y_pitch + (lane & 3) * 16
                               : (unsigned)l32 * (unsigned)p.y_pitch + g * (F8 ? 32 : 16);
@@ -123,6 +128,12 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   unsigned yrd3[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) yrd3[ks] = yring + l32 * 128 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 1) & 7)) << 4);
+  // YM == 4: load instruction i of a stage moves k rows 8 i .. 8 i + 7 of 128 bytes (64 l); in the rows with bit 1 of
+  // k set the two 64-byte halves change places (chunk c at position c ^ 4), so that the four k rows of a transposed
+  // read - 128 bytes apart - lie in four different quarters of the banks.  Lane of a read: k row 8 g + i16 / 4 (+ 4,
+  // 16, 20 by the instruction offset: bit 1 of k stays), columns 16 (q & 1) + 4 (i16 & 3) .. of tile lt.
+  const unsigned yoff4 = (unsigned)(lane >> 3) * (unsigned)p.y_pitch + (((lane & 7) ^ (((lane >> 4) & 1) << 2)) << 4);
+  const unsigned tl4 = ring + (8 * (q >> 1) + (i16 >> 2)) * 128 + (((2 * (q & 1) + ((i16 & 3) >> 1)) ^ (((i16 >> 3) & 1) << 2)) << 4) + (i16 & 1) * 8;
   V8 xr[NS][2][ST], yr[NS][2];
   auto issue = [&](int j, auto SLOT_) {
     constexpr int sl = decltype(SLOT_)::value;
@@ -130,6 +141,10 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       const char* src = ybase + (int64_t)j * 32 * p.y_pitch;
       async_copy16_sbase(src, yoff, ring + sl * SLOT);
       async_copy16_sbase(src + 16 * p.y_pitch, yoff, ring + sl * SLOT + 1024);
+    } else if constexpr (YM == 4) {
+      const char* src = ybase + (int64_t)j * 32 * p.y_pitch;
+#pragma unroll
+      for (int i = 0; i < 4; i++) async_copy16_sbase(src + (int64_t)(8 * i) * p.y_pitch, yoff4, ring + sl * SLOT + i * 1024);
     } else if constexpr (YM == 2) {
       const char* src = ybase + (int64_t)j * 64;
       async_copy16_sbase(src, ydma2[0], ring + sl * SLOT);
@@ -167,8 +182,28 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   };
   auto compute = [&](const int j, auto SLOT_) {
     constexpr int sl = decltype(SLOT_)::value;
-    V8 yf[2];
-    if constexpr (Y_LDS) {
+    V8 yfl[LT][2];
+    V8 (&yf)[2] = yfl[0];
+    if constexpr (YM == 4) {
+      i32x2 lo[2][2], hi[2][2];
+      static_for<2>([&](auto LT_) {
+        constexpr int lt = decltype(LT_)::value;
+        const unsigned ad = tl4 ^ (lt * 64u);   // (the second tile's chunks are 4 further: bit 2 of the position)
+        lo[lt][0] = lds_read_tr16_b64<sl * SLOT>(ad);
+        hi[lt][0] = lds_read_tr16_b64<sl * SLOT + 4 * 128>(ad);
+        lo[lt][1] = lds_read_tr16_b64<sl * SLOT + 16 * 128>(ad);
+        hi[lt][1] = lds_read_tr16_b64<sl * SLOT + 20 * 128>(ad);
+      });
+      lds_wait<0>();
+#pragma unroll
+      for (int lt = 0; lt < 2; lt++)
+#pragma unroll
+        for (int ks = 0; ks < 2; ks++) {
+          lds_use(lo[lt][ks]);
+          lds_use(hi[lt][ks]);
+          yfl[lt][ks] = __builtin_bit_cast(V8, (i32x4)__builtin_shufflevector(lo[lt][ks], hi[lt][ks], 0, 1, 2, 3));
+        }
+    } else if constexpr (Y_LDS) {
       i32x2 lo[2], hi[2];
       lo[0] = lds_read_tr16_b64<sl * SLOT>(tl);
       hi[0] = lds_read_tr16_b64<sl * SLOT + 4 * 64>(tl);
@@ -267,7 +302,9 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
       for (int ks = 0; ks < 2; ks++)
 #pragma unroll
-        for (int t = 0; t < ST; t++) acc[t] = mfma32(yf[ks], xf[ks][t], acc[t]);
+        for (int lt = 0; lt < LT; lt++)
+#pragma unroll
+          for (int t = 0; t < ST; t++) acc[lt * ST + t] = mfma32(yfl[lt][ks], xf[ks][t], acc[lt * ST + t]);
     }
   };
 
@@ -300,26 +337,26 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
 
   // ---- sum the waves' partial tiles through LDS (the rings are dead after the barrier)
   __syncthreads();
-  LDS_PTR(float) const red = (LDS_PTR(float))lds;  // [NW][ST * 16][64]
+  LDS_PTR(float) const red = (LDS_PTR(float))lds;  // [NW][TT * 16][64]
 #pragma unroll
-  for (int t = 0; t < ST; t++)
+  for (int t = 0; t < TT; t++)
 #pragma unroll
-    for (int r = 0; r < 16; r++) red[(wave * ST * 16 + t * 16 + r) * 64 + lane] = acc[t][r];
+    for (int r = 0; r < 16; r++) red[(wave * TT * 16 + t * 16 + r) * 64 + lane] = acc[t][r];
   __syncthreads();
   float alpha = 1.f;
   if (p.a_scale) alpha *= *p.a_scale;
   if (p.b_scale) alpha *= *p.b_scale;
-  constexpr int RPW = ST * 16 / NW;  // accumulator registers finished by each wave
+  constexpr int RPW = TT * 16 / NW;  // accumulator registers finished by each wave
   static_assert(RPW >= 1, "more waves than accumulator registers");
 #pragma unroll
   for (int e = 0; e < RPW; e++) {
-    const int rr = wave * RPW + e, t = rr >> 4, r = rr & 15;
+    const int rr = wave * RPW + e, tt = rr >> 4, r = rr & 15, lt = tt / ST, t = tt % ST;
     float v = 0.f;
 #pragma unroll
-    for (int w = 0; w < NW; w++) v += red[(w * ST * 16 + rr) * 64 + lane];
+    for (int w = 0; w < NW; w++) v += red[(w * TT * 16 + rr) * 64 + lane];
     v *= alpha;
     // register r of lane: row l = 8 (r / 4) + 4 g + r % 4 of the tile, column s = l32
-    const int s = 32 * t + l32, l = l0 + (r >> 2) * 8 + g * 4 + (r & 3);
+    const int s = 32 * t + l32, l = l0 + 32 * lt + (r >> 2) * 8 + g * 4 + (r & 3);
     if (s < p.S && l < p.L) {
       if (p.aux) v += load_aux(p.aux, (int64_t)s * p.aux_ss + (int64_t)l * p.aux_sl, p.aux_dtype);
       if (p.activation == 1) v = v >= 0.f ? v : 0.01f * v;
@@ -337,8 +374,10 @@ template <typename E, int YM, int XM, int ST>
 static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   // four waves with three stages in flight each already saturate what this access pattern gets
   // from HBM; the small LDS footprint lets several workgroups share a CU
-  constexpr int NW = 4, NS = 4;
-  constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : 0) + (XM ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0), red = NW * ST * 16 * 64 * 4;
+  // (YM 4, 64 columns per workgroup: half as many workgroups, so eight waves each split K eight ways)
+  constexpr int NW = YM == 4 ? 8 : 4, NS = YM == 4 ? 3 : 4;
+  constexpr int LT = YM == 4 ? 2 : 1;
+  constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : YM == 4 ? 4096 : 0) + (XM ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0), red = NW * LT * ST * 16 * 64 * 4;
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
@@ -347,7 +386,7 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  gemm_skinny_kernel<E, YM, XM, ST, NW, NS><<<dim3(p.L / 32), dim3(NW * 64), smem, stream>>>(p);
+  gemm_skinny_kernel<E, YM, XM, ST, NW, NS><<<dim3(p.L / (32 * LT)), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
@@ -368,6 +407,9 @@ bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_
 #define MI355_SKINNY_Y_KMAJOR_MODE 3
 #endif
 constexpr int YK = MI355_SKINNY_Y_KMAJOR_MODE;
+#ifndef MI355_SKINNY_Y_LMAJOR_MODE
+#define MI355_SKINNY_Y_LMAJOR_MODE 4
+#endif
 // a K-contiguous Y: whole lines (mode 3) where K bytes are a multiple of 128, else 64-byte pieces
 template <typename E, int XM, int ST>
 static int launch_skinny_yk(const SkinnyArgs& p, int elem_bytes, hipStream_t stream) {
@@ -385,6 +427,10 @@ static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hi
   const bool two = p.S > 32;
   if (!x_kmajor) return two ? launch_skinny_yk<E, 1, 2>(p, 2, stream) : launch_skinny_yk<E, 1, 1>(p, 2, stream);
   if (y_kmajor) return two ? launch_skinny_yk<E, 2, 2>(p, 2, stream) : launch_skinny_yk<E, 2, 1>(p, 2, stream);
+  // an L-contiguous Y: whole lines (64 columns per workgroup) where L is a multiple of 64
+  // (at most 32 rows of X: eight waves of two column tiles each fit LDS; and enough columns that 64 per workgroup still
+  // give every compute unit one - 16 x 16384 x 8192 5250 -> 6050 GB/s, but 16 x 8192 x 8192, 128 workgroups, 4685 -> 4580)
+  if (MI355_SKINNY_Y_LMAJOR_MODE == 4 && p.L % 64 == 0 && !two && p.cus > 0 && p.L / 64 >= p.cus) return launch_skinny<E, 4, 2, 1>(p, stream);
   return two ? launch_skinny<E, 1, 2, 2>(p, stream) : launch_skinny<E, 1, 2, 1>(p, stream);
 }
 

@@ -64,6 +64,7 @@ struct SkinnyArgs {
   const void* aux;
   int64_t aux_ss, aux_sl;
   int aux_dtype;
+  int cus;          // compute units of the device (0 = unknown): picks the workgroup width for an L-contiguous Y
 };
 
 // one-launch GEMM with row-wise epilogues (row softmax, chained product), N <= 256 and N2 <= 256
