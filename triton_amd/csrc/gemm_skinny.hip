@@ -45,17 +45,22 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr int LT = YM == 4 ? 2 : 1;   // 32-column tiles of the output per wave
   constexpr int TT = LT * ST;           // accumulator tiles per wave: [LT][ST]
   static_assert(!F8 || (!Y_LDS && YM != 4 && XM == 2), "fp8: both operands K-contiguous, X through LDS");
+  static_assert(XM != 3 || (NS % 2 == 0 && YM != 4), "pair tiles: a stage's parity is its slot's");
   constexpr int PD = NS - 1;          // stages in flight
   constexpr int LPS = (YM == 4 ? 4 : 2) + 2 * ST;   // vector-memory operations per stage: 2 (4) of Y, 2 per 32 rows of X
   // X: 0 = K contiguous, straight into registers (32-byte pieces of 32 rows per instruction: slower,
   //        kept for comparison); 1 = S contiguous, through LDS with a transposed read;
-  //    2 = K contiguous, through LDS (64-byte pieces of 16 rows per instruction)
+  //    2 = K contiguous, through LDS (64-byte pieces of 16 rows per instruction);
+  //    3 = K contiguous, through LDS in whole 128-byte lines (8 rows per instruction): pair tiles of [32 ST s][128
+  //        bytes of k] in a ring of their own, loaded like the pair tiles of YM 3 - first half of the rows with the odd
+  //        stage before the pair, second half with its even stage (needs K bytes a multiple of 128; not for fp8)
   constexpr bool X_LDS = XM != 0;
   static_assert(!((Y_LDS || YM == 4) && XM == 1), "one operand at most is transposed through LDS");
   constexpr int XROW = 64 * ST;       // bytes of one k row of an S-contiguous X tile: S = 32 ST
   constexpr int YSLOT = (YM == 1 || YM == 2) ? 2048 : YM == 4 ? 4096 : 0;   // [32 k][32 l] 16-bit, [32 l][64 bytes of k], or [32 k][64 l]
   constexpr int ND = 4, YPAIR = 4096;            // YM == 3: ring of ND tiles [32 l][128 bytes of k] behind the stage ring
-  constexpr int XSLOT = X_LDS ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
+  constexpr int XSLOT = (XM == 1 || XM == 2) ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
+  constexpr int XPAIR = 4096 * ST;               // XM == 3: [32 ST s][128 bytes of k]
   constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
   static_assert(PD * LPS < 64, "vmcnt has 6 bits");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   const int l0 = xcd_remap(blockIdx.x, gridDim.x) * (32 * LT);
 
   const int nstages = p.K / (F8 ? 64 : 32);
-  const int per = YM == 3 ? (((nstages + NW - 1) / NW + 1) & ~1) : (nstages + NW - 1) / NW;   // (YM 3: whole pairs of stages)
+  const int per = (YM == 3 || XM == 3) ? (((nstages + NW - 1) / NW + 1) & ~1) : (nstages + NW - 1) / NW;   // (pair tiles: whole pairs of stages)
   const int j_lo = wave * per, j_hi = min(nstages, j_lo + per);
 
   f32x16 acc[TT];
@@ -128,6 +133,18 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   unsigned yrd3[2];
 #pragma unroll
   for (int ks = 0; ks < 2; ks++) yrd3[ks] = yring + l32 * 128 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 1) & 7)) << 4);
+  // XM == 3: the same for X; instruction i of a pair (0 .. 4 ST - 1) moves rows 8 i .. 8 i + 7 (rows beyond S fetch
+  // row S - 1 into their place)
+  const unsigned xring = lds_addr(lds) + NW * (NS * SLOT) + (YM == 3 ? NW * (ND * YPAIR) : 0) + wave * (ND * XPAIR);
+  unsigned xdma3[XM == 3 ? 4 * ST : 1];
+  unsigned xrd3[2];
+  if constexpr (XM == 3) {
+#pragma unroll
+    for (int i = 0; i < 4 * ST; i++)
+      xdma3[i] = (unsigned)min(8 * i + (lane >> 3), p.S - 1) * (unsigned)p.x_pitch + (((lane & 7) ^ (4 * (i & 1) + (lane >> 4))) << 4);
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++) xrd3[ks] = xring + l32 * 128 + (((2 * ks + g) ^ ((l32 >> 1) & 7)) << 4);
+  }
   // YM == 4: load instruction i of a stage moves k rows 8 i .. 8 i + 7 of 128 bytes (64 l); in the rows with bit 1 of
   // k set the two 64-byte halves change places (chunk c at position c ^ 4), so that the four k rows of a transposed
   // read - 128 bytes apart - lie in four different quarters of the banks.  Lane of a read: k row 8 g + i16 / 4 (+ 4,
@@ -167,6 +184,16 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
       for (int i = 0; i < 2 * ST; i++)
         async_copy16_sbase(xsrc + (int64_t)i * (16 / ST) * p.x_pitch, xdma, ring + sl * SLOT + YSLOT + i * 1024);
+    } else if constexpr (XM == 3) {
+      // odd stage: first half of the rows of the NEXT pair (the last pair again where there is none); even: second half of its own
+      const int d = min((j + 1) >> 1, (j_hi >> 1) - 1), half = (j & 1) ^ 1;
+      const char* xsrc = p.X + (int64_t)d * 128;
+      const unsigned dst = xring + (d & (ND - 1)) * XPAIR + half * (2 * ST * 1024);
+      static_for<2 * ST>([&](auto I_) {
+        constexpr int i = decltype(I_)::value;
+        if (half) async_copy16_sbase(xsrc, xdma3[2 * ST + i], dst + i * 1024);
+        else async_copy16_sbase(xsrc, xdma3[i], dst + i * 1024);
+      });
     } else if constexpr (XM == 2) {
       const char* xsrc = p.X + (int64_t)j * 64;
 #pragma unroll
@@ -244,7 +271,25 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       yf[1] = yr[sl][1];
     }
     V8 xf[2][ST];
-    if constexpr (XM == 2) {
+    if constexpr (XM == 3) {
+      const unsigned xb = (unsigned)((j >> 1) & (ND - 1)) * XPAIR;
+      i32x4 xv[2][ST];
+      static_for<2>([&](auto KS_) {
+        constexpr int ks = decltype(KS_)::value;
+        static_for<ST>([&](auto T_) {
+          constexpr int t = decltype(T_)::value;
+          xv[ks][t] = lds_read_b128<t * 4096>((xrd3[ks] ^ ((sl & 1) * 64u)) + xb);
+        });
+      });
+      lds_wait<0>();
+#pragma unroll
+      for (int ks = 0; ks < 2; ks++)
+#pragma unroll
+        for (int t = 0; t < ST; t++) {
+          lds_use(xv[ks][t]);
+          xf[ks][t] = __builtin_bit_cast(V8, xv[ks][t]);
+        }
+    } else if constexpr (XM == 2) {
       i32x4 xv[2][ST];
       static_for<2>([&](auto KS_) {
         constexpr int ks = decltype(KS_)::value;
@@ -319,6 +364,13 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       async_copy16_sbase(src, ydma3[0], dst);
       async_copy16_sbase(src + 8 * p.y_pitch, ydma3[1], dst + 1024);
     }
+    if constexpr (XM == 3) {
+      // first half of the rows of the first pair
+      const int d = j_lo >> 1;
+      const char* xsrc = p.X + (int64_t)d * 128;
+      const unsigned dst = xring + (d & (ND - 1)) * XPAIR;
+      static_for<2 * ST>([&](auto I_) { async_copy16_sbase(xsrc, xdma3[decltype(I_)::value], dst + decltype(I_)::value * 1024); });
+    }
     static_for<PD>([&](auto S_) { issue(min(j_lo + decltype(S_)::value, j_hi - 1), S_); });
     for (int j = j_lo; j < j_hi; j += NS) {
       static_for<NS>([&](auto U_) {
@@ -377,7 +429,9 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   // (YM 4, 64 columns per workgroup: half as many workgroups, so eight waves each split K eight ways)
   constexpr int NW = YM == 4 ? 8 : 4, NS = YM == 4 ? 3 : 4;
   constexpr int LT = YM == 4 ? 2 : 1;
-  constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : YM == 4 ? 4096 : 0) + (XM ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0), red = NW * LT * ST * 16 * 64 * 4;
+  constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : YM == 4 ? 4096 : 0) + (XM == 1 || XM == 2 ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0) +
+                       (XM == 3 ? NW * 4 * 4096 * ST : 0), red = NW * LT * ST * 16 * 64 * 4;
+  static_assert(ring <= 160 * 1024, "LDS of one CU");
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
   if (!attr_set) {
@@ -411,6 +465,12 @@ constexpr int YK = MI355_SKINNY_Y_KMAJOR_MODE;
 #define MI355_SKINNY_Y_LMAJOR_MODE 4
 #endif
 // a K-contiguous Y: whole lines (mode 3) where K bytes are a multiple of 128, else 64-byte pieces
+// how the 33 .. 64 K-contiguous rows of X travel next to an L-contiguous Y where K bytes are a multiple of 128 (see XM in
+// the kernel): 3 = whole lines (64 x 8192 x 8192 3520 -> 3745 GB/s), 2 = 64-byte pieces.  With at most 32 rows, and
+// next to a K-contiguous Y in pair tiles of its own, whole lines for X measured +-0 and -1.2 %: 64-byte pieces there.
+#ifndef MI355_SKINNY_X_KMAJOR_MODE
+#define MI355_SKINNY_X_KMAJOR_MODE 3
+#endif
 template <typename E, int XM, int ST>
 static int launch_skinny_yk(const SkinnyArgs& p, int elem_bytes, hipStream_t stream) {
   if constexpr (YK == 3) {
@@ -431,6 +491,7 @@ static int launch_skinny_v(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, hi
   // (at most 32 rows of X: eight waves of two column tiles each fit LDS; and enough columns that 64 per workgroup still
   // give every compute unit one - 16 x 16384 x 8192 5250 -> 6050 GB/s, but 16 x 8192 x 8192, 128 workgroups, 4685 -> 4580)
   if (MI355_SKINNY_Y_LMAJOR_MODE == 4 && p.L % 64 == 0 && !two && p.cus > 0 && p.L / 64 >= p.cus) return launch_skinny<E, 4, 2, 1>(p, stream);
+  if (MI355_SKINNY_X_KMAJOR_MODE == 3 && two && ((int64_t)p.K * 2) % 128 == 0) return launch_skinny<E, 1, 3, 2>(p, stream);
   return two ? launch_skinny<E, 1, 2, 2>(p, stream) : launch_skinny<E, 1, 2, 1>(p, stream);
 }
 
