@@ -61,6 +61,8 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   constexpr int ND = 4, YPAIR = 4096;            // YM == 3: ring of ND tiles [32 l][128 bytes of k] behind the stage ring
   constexpr int XSLOT = (XM == 1 || XM == 2) ? 2048 * ST : 0;   // [32 k][32 ST s] or [32 ST s][32 k]
   constexpr int XPAIR = 4096 * ST;               // XM == 3: [32 ST s][128 bytes of k]
+  constexpr int XND = (YM == 3 && ST == 2) ? 3 : 4;   // pair tiles of X in its ring (three where four do not fit next to Y's; a tile is dead
+                                                     // before the loads that re-use its place are issued from three on)
   constexpr int SLOT = YSLOT + XSLOT;            // bytes of one stage in LDS
   static_assert(PD * LPS < 64, "vmcnt has 6 bits");
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
   for (int ks = 0; ks < 2; ks++) yrd3[ks] = yring + l32 * 128 + ((((F8 ? 2 * g + ks : 2 * ks + g)) ^ ((l32 >> 1) & 7)) << 4);
   // XM == 3: the same for X; instruction i of a pair (0 .. 4 ST - 1) moves rows 8 i .. 8 i + 7 (rows beyond S fetch
   // row S - 1 into their place)
-  const unsigned xring = lds_addr(lds) + NW * (NS * SLOT) + (YM == 3 ? NW * (ND * YPAIR) : 0) + wave * (ND * XPAIR);
+  const unsigned xring = lds_addr(lds) + NW * (NS * SLOT) + (YM == 3 ? NW * (ND * YPAIR) : 0) + wave * (XND * XPAIR);
   unsigned xdma3[XM == 3 ? 4 * ST : 1];
   unsigned xrd3[2];
   if constexpr (XM == 3) {
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       // odd stage: first half of the rows of the NEXT pair (the last pair again where there is none); even: second half of its own
       const int d = min((j + 1) >> 1, (j_hi >> 1) - 1), half = (j & 1) ^ 1;
       const char* xsrc = p.X + (int64_t)d * 128;
-      const unsigned dst = xring + (d & (ND - 1)) * XPAIR + half * (2 * ST * 1024);
+      const unsigned dst = xring + (d % XND) * XPAIR + half * (2 * ST * 1024);
       static_for<2 * ST>([&](auto I_) {
         constexpr int i = decltype(I_)::value;
         if (half) async_copy16_sbase(xsrc, xdma3[2 * ST + i], dst + i * 1024);
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
     }
     V8 xf[2][ST];
     if constexpr (XM == 3) {
-      const unsigned xb = (unsigned)((j >> 1) & (ND - 1)) * XPAIR;
+      const unsigned xb = (unsigned)((j >> 1) % XND) * XPAIR;
       i32x4 xv[2][ST];
       static_for<2>([&](auto KS_) {
         constexpr int ks = decltype(KS_)::value;
@@ -368,7 +370,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(SkinnyArgs p) {
       // first half of the rows of the first pair
       const int d = j_lo >> 1;
       const char* xsrc = p.X + (int64_t)d * 128;
-      const unsigned dst = xring + (d & (ND - 1)) * XPAIR;
+      const unsigned dst = xring + (d % XND) * XPAIR;
       static_for<2 * ST>([&](auto I_) { async_copy16_sbase(xsrc, xdma3[decltype(I_)::value], dst + decltype(I_)::value * 1024); });
     }
     static_for<PD>([&](auto S_) { issue(min(j_lo + decltype(S_)::value, j_hi - 1), S_); });
@@ -430,7 +432,7 @@ static int launch_skinny(const SkinnyArgs& p, hipStream_t stream) {
   constexpr int NW = YM == 4 ? 8 : 4, NS = YM == 4 ? 3 : 4;
   constexpr int LT = YM == 4 ? 2 : 1;
   constexpr int ring = NW * NS * ((YM == 1 || YM == 2 ? 2048 : YM == 4 ? 4096 : 0) + (XM == 1 || XM == 2 ? 2048 * ST : 0)) + (YM == 3 ? NW * 4 * 4096 : 0) +
-                       (XM == 3 ? NW * 4 * 4096 * ST : 0), red = NW * LT * ST * 16 * 64 * 4;
+                       (XM == 3 ? NW * ((YM == 3 && ST == 2) ? 3 : 4) * 4096 * ST : 0), red = NW * LT * ST * 16 * 64 * 4;
   static_assert(ring <= 160 * 1024, "LDS of one CU");
   constexpr int smem = ring > red ? ring : red;
   static bool attr_set = false;
@@ -474,7 +476,14 @@ constexpr int YK = MI355_SKINNY_Y_KMAJOR_MODE;
 template <typename E, int XM, int ST>
 static int launch_skinny_yk(const SkinnyArgs& p, int elem_bytes, hipStream_t stream) {
   if constexpr (YK == 3) {
-    if (((int64_t)p.K * elem_bytes) % 128 == 0) return launch_skinny<E, 3, XM, ST>(p, stream);
+    if (((int64_t)p.K * elem_bytes) % 128 == 0) {
+      // (49 .. 64 K-contiguous rows of X: whole lines for X too, in a ring of three pair tiles next to Y's four; 16-bit.
+      // 64 x 8192 x 8192 with a K-contiguous weight 32.0 -> 30.0 us, 8192 x 64 x 8192 30.1 -> 28.2; but 48 rows 26.0 -> 27.5)
+      if constexpr (MI355_SKINNY_X_KMAJOR_MODE == 3 && XM == 2 && ST == 2 && !E::kF8) {
+        if (p.S > 48) return launch_skinny<E, 3, 3, ST>(p, stream);
+      }
+      return launch_skinny<E, 3, XM, ST>(p, stream);
+    }
     return launch_skinny<E, 2, XM, ST>(p, stream);
   } else {
     return launch_skinny<E, YK, XM, ST>(p, stream);
