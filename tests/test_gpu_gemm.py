@@ -682,6 +682,18 @@ def test_skinny_16bit_full_decode_size(gpu):
     assert np.allclose(c, gemm.matmul_closed_form(a, b), rtol=1e-2, atol=1e-2)
     c2 = to_np(triton_amd.matmul(ta * 2, tb, out_dtype=torch.float32))
     assert bits_equal(c2, 2 * c)
+    # the same product with the weight stored K-contiguous (x @ W^T, the whole-line form of the streaming kernel) and
+    # with 64 rows of A (X in whole lines too): the same sums in another order, so equal to the tolerance - and exact
+    # on the integer operands of the second pair
+    tbk = tb.t().contiguous().t()
+    ck = to_np(triton_amd.matmul(ta, tbk, out_dtype=torch.float32))
+    assert np.allclose(ck, c, rtol=1e-3, atol=1e-3)
+    ai = rng.integers(-2, 3, size=(64, 8192)).astype(np.float32)
+    bi = rng.integers(-2, 3, size=(8192, 8192)).astype(np.float32)
+    tai, tbi = from_np(ai, "fp16", gpu), from_np(bi, "fp16", gpu)
+    want = gemm.matmul_closed_form(ai, bi, out_dtype="fp32")
+    assert bits_equal(to_np(triton_amd.matmul(tai, tbi, out_dtype=torch.float32)), want)
+    assert bits_equal(to_np(triton_amd.matmul(tai, tbi.t().contiguous().t(), out_dtype=torch.float32)), want)
 
 
 @pytest.mark.parametrize("nprog", [None, 7, 3])
