@@ -67,6 +67,7 @@ def settle(fn, seconds=0.06, limit=4000):
             fn()
         done += 20
         torch.cuda.synchronize()
+    return done
 
 
 def quick(fn, iters=60, warmup=20):
@@ -75,14 +76,15 @@ def quick(fn, iters=60, warmup=20):
     return ev_ms
 
 
-def observed_clock_mhz(fn, seconds=1.0):
-    """Shader clock while `fn` runs back to back (an untimed leg of its own): the driver's current-clock
-    reading (the starred line of /sys/class/drm/card*/device/pp_dpm_sclk, what rocm-smi --showclocks
-    prints) sampled every 10 ms by a host thread over `seconds` of sustained launches; the median of the
-    samples taken after the first quarter.  None where the file is not readable.  (The board holds its
-    power limit by lowering the clock of MFMA-heavy kernels, so the nominal clock says little.  The
-    library's own mi355_clock_probe reads the counters on the device, but a probe wave next to a kernel
-    that fills every SIMD costs that kernel a round of tiles, and the clock is back up within
+def observed_board_state(fn, seconds=1.0):
+    """Shader clock and board power while `fn` runs back to back (an untimed leg of its own), from the driver's
+    own files: the current-clock line of /sys/class/drm/card*/device/pp_dpm_sclk (what rocm-smi --showclocks
+    prints) and hwmon's power1_average / power1_input with power1_cap (microwatts; what rocm-smi --showpower /
+    --showmaxpower print), sampled every 10 ms by a host thread over `seconds` of sustained launches; medians of
+    the samples taken after the first quarter.  Fields that cannot be read are None.  (The board holds its power
+    limit by lowering the clock of MFMA-heavy kernels, so the nominal clock says little and the watts next to
+    the cap say why.  The library's own mi355_clock_probe reads the counters on the device, but a probe wave next
+    to a kernel that fills every SIMD costs that kernel a round of tiles, and the clock is back up within
     microseconds of a kernel's end - so it suits kernels that leave a wave slot free, not these.)"""
     import glob
     import re
@@ -90,23 +92,40 @@ def observed_clock_mhz(fn, seconds=1.0):
 
     import torch
 
-    paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
-    if not paths:
-        return None
-    samples, stop = [], [False]
+    clk_paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+    hw = sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*"))
+    pw_paths = [q for d in hw for q in (os.path.join(d, "power1_average"), os.path.join(d, "power1_input")) if os.path.exists(q)]
+    cap = None
+    for d in hw:
+        try:
+            cap = max(cap or 0.0, int(open(os.path.join(d, "power1_cap")).read()) / 1e6)
+        except (OSError, ValueError):
+            pass
+    clk, watts, stop = [], [], [False]
+
+    def read_max(paths, parse):
+        best = None
+        for path in paths:   # (one GPU per box; with several cards, the busiest one is the one under test)
+            try:
+                v = parse(open(path).read())
+            except (OSError, ValueError):
+                v = None
+            if v is not None:
+                best = max(best or 0, v)
+        return best
+
+    def sclk(text):
+        m = re.search(r"(\d+)\s*Mhz\s*\*", text, re.I)
+        return int(m.group(1)) if m else None
 
     def poll():
         while not stop[0]:
-            best = None
-            for path in paths:   # (one GPU per box; with several cards, the busiest one is the one under test)
-                try:
-                    m = re.search(r"(\d+)\s*Mhz\s*\*", open(path).read(), re.I)
-                except OSError:
-                    m = None
-                if m:
-                    best = max(best or 0, int(m.group(1)))
-            if best is not None:
-                samples.append(best)
+            c = read_max(clk_paths, sclk)
+            w = read_max(pw_paths, lambda t: int(t) / 1e6)
+            if c is not None:
+                clk.append(c)
+            if w is not None:
+                watts.append(w)
             time.sleep(0.01)
 
     for _ in range(5):
@@ -124,8 +143,12 @@ def observed_clock_mhz(fn, seconds=1.0):
     stop[0] = True
     th.join()
     torch.cuda.synchronize()
-    tail = sorted(samples[len(samples) // 4:])
-    return float(tail[len(tail) // 2]) if tail else None
+
+    def median_tail(xs):
+        tail = sorted(xs[len(xs) // 4:])
+        return round(float(tail[len(tail) // 2]), 1) if tail else None
+
+    return {"sclk_mhz": median_tail(clk), "power_w": median_tail(watts), "power_cap_w": cap}
 
 
 def _median_of_3(fn):
@@ -374,6 +397,9 @@ def main():
     ap.add_argument("--steps", type=int, default=100)
     # (100 launches = 75 ms: the clocks have settled by then; with 10 the timed region starts 3 % low)
     ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-ms", type=float, default=150.0,
+                    help="wall time of untimed launches of the headline GEMM in front of the warm-up (the board's clocks "
+                         "take tens of milliseconds to settle after an idle phase); reported as settle_launches")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--size", type=int, default=8192)
@@ -408,7 +434,7 @@ def main():
         rec = {"workload": args.only, "steps": args.steps, "ms_per_launch": round(ev_ms, 5),
                ("tflops" if kind == "flops" else "gbps"): round(work / ev_ms / (1e9 if kind == "flops" else 1e6), 1)}
         if info.get("clock"):
-            rec["sclk_mhz"] = observed_clock_mhz(fn, 0.5)
+            rec.update(observed_board_state(fn, 0.5))
         print(json.dumps(rec))
         return
     a = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
@@ -425,6 +451,9 @@ def main():
         for _ in range(5):
             c.copy_(a)   # reads n*n*2 bytes, writes n*n*2 bytes
         torch.cuda.synchronize()
+    # untimed launches until the clocks have settled (as for every secondary workload), then W warm-up launches,
+    # then exactly K timed ones
+    settle_launches = settle(step, args.settle_ms * 1e-3)
     wall_ms, ev_ms, per = time_launches(step, args.steps, args.warmup)
     flops = 2.0 * n ** 3
     tflops = flops / (wall_ms * 1e-3) / 1e12
@@ -432,6 +461,7 @@ def main():
     out = {
         "metric": "TFLOP/s & % MFMA peak: bf16/fp8 GEMM 8192^3; flash-attn fwd D=128 N=4096",
         "value": round(tflops, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "settle_launches": settle_launches,
         "ms_per_step": round(wall_ms, 5), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"bf16 GEMM M=N=K={n}, A row-major MxK, B row-major KxN, fp32 accumulate, bf16 out (BASELINE config 2)"},
@@ -442,7 +472,7 @@ def main():
                      "algorithmic_bytes": 3 * 2 * n * n},
         "device": {"name": torch.cuda.get_device_name(0), "cus": lib.mi355_query(_lib.Q_CU_COUNT),
                    "nominal_clock_khz": lib.mi355_query(_lib.Q_CLOCK_KHZ),
-                   "observed_sclk_mhz_during_headline_gemm": observed_clock_mhz(step)},
+                   "during_headline_gemm": observed_board_state(step)},
     }
     out["roofline"]["traffic_source"] = TRAFFIC_SOURCE
 
@@ -455,13 +485,30 @@ def main():
         extra["bf16_gemm_do_bench"] = {"ms_median": round(med, 4), "ms_p20": round(p20, 4), "ms_p80": round(p80, 4),
                                        "tflops_median": round(testing.matmul_tflops(n, n, n, med), 1)}
         del a, b, c
+        # config 2's sweep: square sizes 1024 .. 8192 in steps of 1024, bf16, row-major B, the reference's protocol
+        # (flushed do_bench medians, 03:424-438) through the same C-ABI call as the headline
+        sweep = {}
+        for m in range(1024, 8192 + 1, 1024):
+            sa_, sb_ = (torch.randn(m, m, device=dev, dtype=torch.bfloat16) for _ in range(2))
+            sc_ = torch.empty(m, m, device=dev, dtype=torch.bfloat16)
+
+            def sweep_step(m=m, sa_=sa_, sb_=sb_, sc_=sc_):
+                rc = lib.mi355_gemm(sa_.data_ptr(), sb_.data_ptr(), sc_.data_ptr(), m, m, m, m, 1, m, 1, m, 1,
+                                    _lib.BF16, _lib.BF16, None, None, 0, stream)
+                assert rc == 0, rc
+
+            settle(sweep_step, 0.03)
+            med = testing.do_bench(sweep_step, warmup=10, rep=40, quantiles=[0.5])
+            sweep[str(m)] = {"ms_median": round(med, 4), "tflops": round(testing.matmul_tflops(m, m, m, med), 1)}
+            del sa_, sb_, sc_
+        extra["bf16_gemm_sweep"] = sweep
         for name, build in secondary_workloads(lib, dev, n).items():
             fn, work, kind, info, iters = build()
             ms = quick(fn, iters=iters, warmup=max(5, iters // 3))
             if kind == "flops":
                 rec = {"ms": round(ms, 4), "tflops": round(work / ms / 1e9, 1), "frac_of_peak": round(work / ms / 1e9 / PEAK[info["peak"]], 4)}
                 if info.get("clock"):
-                    rec["sclk_mhz"] = observed_clock_mhz(fn)
+                    rec.update(observed_board_state(fn))
             else:
                 rec = {"us": round(ms * 1e3, 2), "gbps": round(work / ms / 1e6, 1), "frac_of_hbm": round(work / ms / 1e6 / HBM_GBPS, 4)}
             if info.get("data"):

@@ -21,6 +21,13 @@
 #include <stdint.h>
 #include <stddef.h>
 
+/* Version of this interface, returned by mi355_query(MI355_Q_ABI_VERSION).  It goes up whenever an entry point, an
+ * enum value or the meaning of an argument is added; a binding built for version V works with any library that
+ * reports at least V.  (1: GEMM, MX GEMM, attention, dequant; 2: stream-K with and without a workspace, chained
+ * product, clock probe, environment refresh, MI355_ESCRATCH, head dims 16 / 32 / 256 in the backward, fp8 output
+ * of the MFMA epilogues; 3: MFMA burn probe, per-device properties.) */
+#define MI355_ABI_VERSION 3
+
 #ifdef __cplusplus
 extern "C" {
 #endif
@@ -312,6 +319,26 @@ int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* st
  * clock argument) need the observed one.  Asynchronous like every other entry.
  */
 int mi355_clock_probe(uint64_t* ticks, int duration_us, void* stream);
+
+/*
+ * What the matrix pipes of this board sustain: every SIMD of every CU runs `waves_per_simd` (1 or 2) waves that issue
+ * `iters` rounds of one MFMA shape back to back from registers - no memory traffic -, on pseudo-random operand bits
+ * (`random_operands` != 0: finite values, the switching activity of real data) or on one constant.  One round is
+ * 8 x 32768 flop per wave for the 16-bit shapes, twice that for fp8, four times for fp4, so a launch is
+ * CUs x 4 x waves_per_simd x iters x 262144 x {1, 2, 4} flop; the caller times it with events and reads watts and
+ * clock next to it.  Under the board's power limit this, not the nominal peak, is what a GEMM built from that MFMA
+ * shape can approach.  `sink` is one float of device memory (practically never written).  The measurement analogue of
+ * the reference's peak helper (python/triton/testing.py:404-426), which takes its rate from a table.
+ */
+enum {
+  MI355_BURN_BF16_32X32X16 = 0,
+  MI355_BURN_BF16_16X16X32 = 1,
+  MI355_BURN_FP8_32X32X64 = 2,
+  MI355_BURN_FP8_16X16X128 = 3,
+  MI355_BURN_FP4_32X32X64 = 4,
+  MI355_BURN_FP4_16X16X128 = 5
+};
+int mi355_mfma_burn(float* sink, int shape, int random_operands, int iters, int waves_per_simd, void* stream);
 
 /* Device facts needed by callers (analogue of get_device_properties,
  * third_party/amd/backend/driver.c:125-141).  Returns -1 for an unknown selector. */

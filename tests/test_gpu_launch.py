@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import triton_amd
-from triton_amd import hooks
+from triton_amd import _lib, hooks
 
 pytestmark = pytest.mark.gpu
 
@@ -165,3 +165,39 @@ def test_torch_extension_is_the_default_binding_and_agrees_with_ctypes(gpu, monk
         out = triton_amd.matmul(acc, e)
     torch.cuda.synchronize()
     assert torch.equal(out, torch.full_like(out, 10.0))   # launched on, and ordered by, the current (side) stream
+
+
+@pytest.mark.gpu
+def test_clock_and_mfma_burn_probes(gpu):
+    """The two measurement entries: the clock probe reports a plausible shader clock next to a burn of every MFMA
+    shape, a burn launch finishes and leaves its sink alone, and bad arguments are rejected before any launch."""
+    lib = _lib.load()
+    sink = torch.zeros(4, device=gpu, dtype=torch.float32)
+    ticks = torch.zeros(2, device=gpu, dtype=torch.int64)
+    stream = torch.cuda.current_stream().cuda_stream
+    side = torch.cuda.Stream(device=gpu)
+    for shape in range(6):
+        for rnd in (0, 1):
+            assert lib.mi355_mfma_burn(sink.data_ptr(), shape, rnd, 200, 1, stream) == 0
+    assert lib.mi355_clock_probe(ticks.data_ptr(), 2000, side.cuda_stream) == 0   # 2 ms next to the queued burns
+    torch.cuda.synchronize()
+    assert torch.equal(sink.cpu(), torch.zeros(4))
+    cyc, real = ticks.tolist()
+    mhz = cyc / real * lib.mi355_query(_lib.Q_WALL_CLOCK_KHZ) / 1e3
+    assert 90 < mhz < 2600, mhz
+    for bad in ((0, 0, 0, 100, 1), (sink.data_ptr(), 6, 0, 100, 1), (sink.data_ptr(), 0, 0, 0, 1), (sink.data_ptr(), 0, 0, 100, 3)):
+        assert lib.mi355_mfma_burn(*bad, stream) == -1
+
+
+@pytest.mark.gpu
+def test_power_probe_module_reports_every_leg(gpu, capsys):
+    from triton_amd import power_probe
+
+    assert power_probe.main(["--seconds", "0.05", "--json"]) == 0
+    import json
+
+    rec = json.loads(capsys.readouterr().out)
+    assert len(rec["legs"]) == 12 and all(leg["tflops"] > 100 for leg in rec["legs"])
+    # the constant-operand legs are never slower than the random ones by more than noise (less switching, same work)
+    by = {(leg["shape"], leg["operands"]): leg["tflops"] for leg in rec["legs"]}
+    assert by[("bf16 16x16x32", "constant")] > 0.9 * by[("bf16 16x16x32", "random")]

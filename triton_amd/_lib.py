@@ -23,6 +23,9 @@ Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORK
 
 I64x4 = c_int64 * 4
 
+# MI355_ABI_VERSION of include/mi355_kernels.h that this binding was written for
+ABI_VERSION = 3
+
 # name -> (restype, argtypes); kept in one table so tests can check it against the header
 SIGNATURES = {
     "mi355_gemm": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
@@ -60,6 +63,7 @@ SIGNATURES = {
                                POINTER(c_int64), c_float, c_int, c_int, c_void_p]),
     "mi355_dequant": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "mi355_clock_probe": (c_int, [c_void_p, c_int, c_void_p]),
+    "mi355_mfma_burn": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mi355_query": (c_int, [c_int]),
     "mi355_refresh_env": (None, []),
     "mi355_strerror": (c_char_p, [c_int]),
@@ -77,6 +81,11 @@ def load() -> ctypes.CDLL:
                 f"{LIB_PATH} is missing: build the HIP kernels first with "
                 "`python -m triton_amd.build` (needs hipcc); there is no CPU fallback")
         lib = ctypes.CDLL(str(LIB_PATH))
+        lib.mi355_query.restype, lib.mi355_query.argtypes = c_int, [c_int]
+        have = lib.mi355_query(Q_ABI_VERSION)
+        if have < ABI_VERSION:
+            raise ImportError(f"{LIB_PATH} reports ABI version {have}, this binding needs {ABI_VERSION}: rebuild it with "
+                              "`python -m triton_amd.build` (or point MI355_KERNELS_LIB at a current build)")
         for name, (res, args) in SIGNATURES.items():
             fn = getattr(lib, name)
             fn.restype = res

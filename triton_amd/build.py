@@ -83,7 +83,13 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     os.replace(tmp, out)
-    build_torch_extension(verbose)
+    try:
+        build_torch_extension(verbose)
+    except Exception as e:   # the operators then bind the C ABI through ctypes (_lib.ext() returns None)
+        import warnings
+
+        ext_path().unlink(missing_ok=True)   # never leave an extension of an older build next to a new library
+        warnings.warn(f"PyTorch-ROCm extension not built, the operators will use the ctypes binding: {e}")
     return out
 
 

@@ -19,21 +19,28 @@ struct DeviceInfo {
   int ok = 0, cus = 0, gfx950 = 0, lds = 0, clock_khz = 0, wall_clock_khz = 0;
 };
 
+// properties of the CURRENT device, read once per device (a process may hold several)
 const DeviceInfo& device_info() {
-  static DeviceInfo info;
-  static std::once_flag once;
-  std::call_once(once, [] {
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return;
-    hipDeviceProp_t prop;
-    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return;
-    info.cus = prop.multiProcessorCount;
-    info.gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
-    info.lds = (int)prop.sharedMemPerBlock;
-    info.clock_khz = prop.clockRate;
-    if (hipDeviceGetAttribute(&info.wall_clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) info.wall_clock_khz = 0;
-    info.ok = 1;
-  });
+  constexpr int kMax = 64;
+  static DeviceInfo infos[kMax];
+  static std::atomic<int> ready[kMax];
+  static std::mutex mutex;
+  static const DeviceInfo none;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMax) return none;
+  if (ready[dev].load(std::memory_order_acquire)) return infos[dev];
+  std::lock_guard<std::mutex> lock(mutex);
+  if (ready[dev].load(std::memory_order_relaxed)) return infos[dev];
+  DeviceInfo& info = infos[dev];
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, dev) != hipSuccess) return none;
+  info.cus = prop.multiProcessorCount;
+  info.gfx950 = strncmp(prop.gcnArchName, "gfx950", 6) == 0;
+  info.lds = (int)prop.sharedMemPerBlock;
+  info.clock_khz = prop.clockRate;
+  if (hipDeviceGetAttribute(&info.wall_clock_khz, hipDeviceAttributeWallClockRate, dev) != hipSuccess) info.wall_clock_khz = 0;
+  info.ok = 1;
+  ready[dev].store(1, std::memory_order_release);
   return info;
 }
 
@@ -44,7 +51,7 @@ const DeviceInfo& device_info() {
 constexpr int UNSET = INT_MIN;
 struct Knobs {
   int force_strided, group_m, tile, programs, skinny, grouped_big_min, grouped_wave128_min_k, grouped_chunk,
-      attn_fwd_variant, attn_programs, lean_epilogue, tile_m;
+      attn_fwd_variant, attn_programs, lean_epilogue, tile_m, rowfused_max_mk;
 };
 Knobs g_knobs;
 std::atomic<int> g_knobs_ready{0};
@@ -72,6 +79,7 @@ void load_knobs() {
   k.attn_programs = read_env("MI355_ATTN_PROGRAMS", 1);
   k.lean_epilogue = read_env("MI355_GEMM_LEAN_EPILOGUE", 0);
   k.tile_m = read_env("MI355_GEMM_TILE_M", 0);
+  k.rowfused_max_mk = read_env("MI355_ROWFUSED_MAX_MK", 0);
   g_knobs = k;
   g_knobs_ready.store(1, std::memory_order_release);
 }
@@ -105,9 +113,10 @@ bool copy_strides(const int64_t* src, int64_t* dst) {
 extern "C" {
 
 int mi355_query(int what) {
+  if (what == MI355_Q_ABI_VERSION) return MI355_ABI_VERSION;   // (answered without touching the device)
   const DeviceInfo& d = device_info();
   switch (what) {
-    case MI355_Q_ABI_VERSION: return 1;
+    case MI355_Q_ABI_VERSION: return MI355_ABI_VERSION;
     case MI355_Q_CU_COUNT: return d.cus;
     case MI355_Q_IS_GFX950: return d.gfx950;
     case MI355_Q_LDS_BYTES: return d.lds;
@@ -249,7 +258,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true, in_dtype)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
-  if (tile == 6 && (p.tile_m == 192 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
+  // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)
+  if (tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }
 
@@ -339,7 +349,11 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int
   if (softmax && out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
   // a row that fits one tile: product, addend, activation and softmax in ONE launch, on the fp32 accumulator,
   // one rounding at the store - what the reference's single tile does
-  if (softmax && N <= 256 && (in_dtype == MI355_F16 || in_dtype == MI355_BF16)) {
+  // (that kernel is one workgroup per 128 rows with an unpipelined K loop, built for the small, latency-bound
+  // products of the reference's test: larger ones - more than 2^21 elements of A by default,
+  // MI355_ROWFUSED_MAX_MK - take the tiled GEMM and the softmax as a second launch)
+  const int64_t rowfused_max = (int64_t)knob(knobs().rowfused_max_mk, 1 << 21);
+  if (softmax && N <= 256 && (in_dtype == MI355_F16 || in_dtype == MI355_BF16) && (int64_t)M * K <= rowfused_max) {
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
     if (addend && addend_dtype != MI355_F16 && addend_dtype != MI355_BF16 && addend_dtype != MI355_F32) return MI355_EDTYPE;
     if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
@@ -434,6 +448,14 @@ int mi355_clock_probe(uint64_t* ticks, int duration_us, void* stream_) {
   if (!device_info().gfx950 || device_info().wall_clock_khz <= 0) return MI355_EDEVICE;
   const unsigned long long real_ticks = (unsigned long long)duration_us * (unsigned long long)device_info().wall_clock_khz / 1000ull;
   return clock_probe_launch((unsigned long long*)ticks, real_ticks, (hipStream_t)stream_);
+}
+
+int mi355_mfma_burn(float* sink, int shape, int random_operands, int iters, int waves_per_simd, void* stream_) {
+  if (!sink || !aligned(sink, 4) || shape < MI355_BURN_BF16_32X32X16 || shape > MI355_BURN_FP4_16X16X128) return MI355_EINVAL;
+  if (iters <= 0 || iters > (1 << 24) || waves_per_simd < 1 || waves_per_simd > 2) return MI355_EINVAL;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  return mfma_burn_launch(sink, shape, random_operands != 0, iters, waves_per_simd, device_info().cus > 0 ? device_info().cus : 256,
+                          (hipStream_t)stream_);
 }
 
 int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* stream_) {

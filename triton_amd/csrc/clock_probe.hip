@@ -34,3 +34,126 @@ int clock_probe_launch(unsigned long long* out, unsigned long long real_ticks, h
 }
 
 }  // namespace mi355
+
+// ---- MFMA burn: what the matrix pipes of this board sustain with nothing else in the way.  Every SIMD of every
+// CU runs `waves` waves that issue one MFMA shape back to back (eight independent accumulator chains, operands in
+// registers, no memory traffic); the operands are either pseudo-random bit patterns per lane - finite values of
+// every magnitude, the switching activity of real data - or one constant.  Timed by the caller with events and
+// sampled for watts and clock, this is the ceiling that a GEMM of that MFMA shape can approach under the board's
+// power limit: the denominator for "fraction of what the board sustains" next to the nominal peak.
+namespace mi355 {
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) int burn_i32x8;
+
+__device__ inline unsigned burn_rnd(unsigned x) { x ^= x << 13; x ^= x >> 17; x ^= x << 5; return x; }
+
+// two bf16 bit patterns: random sign and mantissa, exponent 0x78 .. 0x7f (magnitudes 2^-7 .. 2, where N(0, 1) data lives)
+__device__ inline unsigned burn_bf16_pair(unsigned& s) {
+  s = burn_rnd(s);
+  const unsigned lo = (s & 0x807f) | ((((s >> 7) & 7) + 0x78) << 7);
+  s = burn_rnd(s);
+  const unsigned hi = (s & 0x807f) | ((((s >> 7) & 7) + 0x78) << 7);
+  return lo | (hi << 16);
+}
+
+// four e4m3fn codes, uniform over the finite ones (0x7f / 0xff, the NaNs, lose their lowest bit)
+__device__ inline unsigned burn_e4m3_quad(unsigned& s) {
+  s = burn_rnd(s);
+  const unsigned m = s & 0x7f7f7f7fu;
+  const unsigned nan = m & (m >> 1) & (m >> 2) & (m >> 3) & (m >> 4) & (m >> 5) & (m >> 6) & 0x01010101u;
+  return s & ~nan;
+}
+
+template <int SHAPE>
+__global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, int random_operands) {
+#if MI355_DEVICE_PASS
+  unsigned s = threadIdx.x * 2654435761u + blockIdx.x * 97u + 1u;
+  burn_i32x8 a[2], b[2];
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+      if (SHAPE < 2) {                       // 16-bit operands: four registers used
+        a[i][e] = random_operands ? (int)burn_bf16_pair(s) : 0x3f803f80;
+        b[i][e] = random_operands ? (int)burn_bf16_pair(s) : 0x3f803f80;
+      } else if (SHAPE < 4) {                // e4m3 bytes: every finite code (0x7f / 0xff, the NaNs, mapped away)
+        a[i][e] = random_operands ? (int)burn_e4m3_quad(s) : 0x38383838;
+        b[i][e] = random_operands ? (int)burn_e4m3_quad(s) : 0x38383838;
+      } else {                               // e2m1 nibbles: every code is finite
+        s = burn_rnd(s); a[i][e] = random_operands ? (int)s : 0x22222222;
+        s = burn_rnd(s); b[i][e] = random_operands ? (int)s : 0x22222222;
+      }
+    }
+  float total = 0.f;
+  if constexpr (SHAPE == 0 || SHAPE == 2 || SHAPE == 4) {         // 32 x 32 tiles: four chains of 16 registers
+    f32x16 acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+      for (int u = 0; u < 8; u++) {
+        if constexpr (SHAPE == 0) {
+          const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a[u & 1], a[u & 1], 0, 1, 2, 3));
+          const bf16x8 bv = __builtin_bit_cast(bf16x8, __builtin_shufflevector(b[(u >> 1) & 1], b[(u >> 1) & 1], 0, 1, 2, 3));
+          acc[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[u & 3], 0, 0, 0);
+        } else if constexpr (SHAPE == 2) {
+          acc[u & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 3], 0, 0, 0, 0, 0, 0);
+        } else {
+          acc[u & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 3], 4, 4, 0, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+      for (int r = 0; r < 16; r++) total += acc[c][r];
+  } else {                                                         // 16 x 16 tiles: eight chains of 4 registers
+    f32x4 acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) acc[c][r] = 0.f;
+    for (int i = 0; i < iters; i++) {
+#pragma unroll
+      for (int u = 0; u < 16; u++) {
+        if constexpr (SHAPE == 1) {
+          const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a[u & 1], a[u & 1], 0, 1, 2, 3));
+          const bf16x8 bv = __builtin_bit_cast(bf16x8, __builtin_shufflevector(b[(u >> 1) & 1], b[(u >> 1) & 1], 0, 1, 2, 3));
+          acc[u & 7] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[u & 7], 0, 0, 0);
+        } else if constexpr (SHAPE == 3) {
+          acc[u & 7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 7], 0, 0, 0, 0, 0, 0);
+        } else {
+          acc[u & 7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 7], 4, 4, 0, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+#pragma unroll
+      for (int r = 0; r < 4; r++) total += acc[c][r];
+  }
+  if (total == 12345.678f) sink[0] = total;   // (keeps the chains alive; practically never true)
+#endif
+}
+
+}  // namespace
+
+// flop of one launch: every shape's inner loop is 8 x 32768 (16-bit), x2 (fp8), x4 (fp4) flop per wave and iteration
+int mfma_burn_launch(float* sink, int shape, int random_operands, int iters, int waves_per_simd, int cus, hipStream_t stream) {
+  const dim3 grid(cus * waves_per_simd), block(256);
+  switch (shape) {
+    case 0: hipLaunchKernelGGL(mfma_burn_kernel<0>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 1: hipLaunchKernelGGL(mfma_burn_kernel<1>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 2: hipLaunchKernelGGL(mfma_burn_kernel<2>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 3: hipLaunchKernelGGL(mfma_burn_kernel<3>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 4: hipLaunchKernelGGL(mfma_burn_kernel<4>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 5: hipLaunchKernelGGL(mfma_burn_kernel<5>, grid, block, 0, stream, sink, iters, random_operands); break;
+    default: return -1;
+  }
+  return (int)hipGetLastError();
+}
+
+}  // namespace mi355

@@ -130,6 +130,7 @@ int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int gemm_rowfused_launch(const RowFusedArgs& p, bool bf16, hipStream_t stream);
 int softmax_rows_launch(void* C, int M, int N, int64_t scm, int64_t scn, int dtype, hipStream_t stream);
 int clock_probe_launch(unsigned long long* out, unsigned long long real_ticks, hipStream_t stream);
+int mfma_burn_launch(float* sink, int shape, int random_operands, int iters, int waves_per_simd, int cus, hipStream_t stream);
 int dequant_launch(const uint8_t* codes, float* out, int64_t n, int fmt, hipStream_t stream);
 
 }  // namespace mi355

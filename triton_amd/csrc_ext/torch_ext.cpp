@@ -7,6 +7,7 @@
 // becomes the exception the reference raises for the same condition (RuntimeError "Triton Error [HIP]"
 // for launch failures, :258-269; ValueError for pointers the device cannot reach, :313-317).
 #include <torch/extension.h>
+#include <c10/core/DeviceGuard.h>
 #include <c10/hip/HIPStream.h>
 
 #include <stdexcept>
@@ -40,6 +41,11 @@ void check(int rc, const char* what) {
   throw std::invalid_argument(std::string(what) + ": " + msg + " (code " + std::to_string(rc) + ")");
 }
 
+// The C library launches on the CURRENT device: every operator makes its first tensor's device current for the call.
+// (the generic guard: it resolves the implementation registered for the tensor's device type, which on ROCm builds of
+// torch is the HIP one under the name "cuda")
+using DeviceGuard = c10::DeviceGuard;
+
 void* stream_of(const at::Tensor& t) { return (void*)c10::hip::getCurrentHIPStream(t.device().index()).stream(); }
 
 const float* scale_ptr(const c10::optional<at::Tensor>& s) {
@@ -55,6 +61,7 @@ void gemm(const at::Tensor& a, const at::Tensor& b, at::Tensor& c, int64_t activ
           const c10::optional<at::Tensor>& add, bool softmax) {
   TORCH_CHECK(a.dim() == 2 && b.dim() == 2 && c.dim() == 2 && a.size(1) == b.size(0), "Incompatible dimensions");
   on_device(a, 0); on_device(b, 1); on_device(c, 2);
+  const DeviceGuard guard(a.device());
   const int M = (int)a.size(0), K = (int)a.size(1), N = (int)b.size(1);
   int rc;
   if (!add.has_value() && !softmax) {
@@ -79,6 +86,8 @@ void gemm(const at::Tensor& a, const at::Tensor& b, at::Tensor& c, int64_t activ
 
 void mx_gemm(const at::Tensor& a, const at::Tensor& sa, const at::Tensor& b, const at::Tensor& sb, at::Tensor& c, int64_t fmt, int64_t K) {
   on_device(a, 0); on_device(sa, 1); on_device(b, 2); on_device(sb, 3); on_device(c, 4);
+  TORCH_CHECK(a.dim() == 2 && b.dim() == 2 && sa.dim() == 2 && sb.dim() == 2 && c.dim() == 2, "MX operands, scales and result are matrices");
+  const DeviceGuard guard(a.device());
   const int rc = mi355_mx_gemm((const uint8_t*)a.data_ptr(), (const uint8_t*)sa.data_ptr(), (const uint8_t*)b.data_ptr(),
                                (const uint8_t*)sb.data_ptr(), c.data_ptr(), (int)a.size(0), (int)b.size(0), (int)K, (int)fmt,
                                abi_dtype(c), a.stride(0), b.stride(0), sa.stride(0), sb.stride(0), c.stride(0), stream_of(a));
@@ -92,6 +101,7 @@ void strides4(const at::Tensor& t, int64_t (&s)[4]) {
 
 void attn_fwd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, at::Tensor& o, at::Tensor& M, double sm_scale, bool causal) {
   on_device(q, 0); on_device(k, 1); on_device(v, 2); on_device(o, 3); on_device(M, 4);
+  const DeviceGuard guard(q.device());
   int64_t sq[4], sk[4], sv[4], so[4];
   strides4(q, sq); strides4(k, sk); strides4(v, sv); strides4(o, so);
   const int rc = mi355_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), o.data_ptr(), M.data_ptr<float>(), (int)q.size(0),
@@ -102,7 +112,9 @@ void attn_fwd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, at:
 
 void attn_bwd(const at::Tensor& q, const at::Tensor& k, const at::Tensor& v, const at::Tensor& o, const at::Tensor& d_o,
               const at::Tensor& M, at::Tensor& delta, at::Tensor& dq, at::Tensor& dk, at::Tensor& dv, double sm_scale, bool causal) {
-  on_device(q, 0); on_device(d_o, 4);
+  on_device(q, 0); on_device(k, 1); on_device(v, 2); on_device(o, 3); on_device(d_o, 4); on_device(M, 5);
+  on_device(delta, 6); on_device(dq, 7); on_device(dk, 8); on_device(dv, 9);
+  const DeviceGuard guard(q.device());
   int64_t s[4], so[4];
   strides4(q, s); strides4(o, so);
   const int Z = (int)q.size(0), H = (int)q.size(1), N = (int)q.size(2), D = (int)q.size(3);

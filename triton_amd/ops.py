@@ -179,7 +179,21 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     return c
 
 
-_streamk_workspace = {}
+_streamk_workspace = {}   # device -> [workspace tensor, stream handle of its last user, event recorded behind that launch]
+
+
+def _streamk_workspace_for(device, stream, nbytes):
+    """ONE partial-tile workspace per device (128 MiB on an MI355X), however many streams call: a call on another
+    stream than the previous user's first waits (on the device) for the event recorded behind that launch, so
+    launches that share the slots never overlap."""
+    entry = _streamk_workspace.get(device)
+    if entry is None or entry[0].numel() < nbytes:
+        entry = _streamk_workspace[device] = [torch.empty(nbytes, device=device, dtype=torch.uint8), stream, None]
+    if entry[1] != stream and entry[2] is not None:
+        torch.cuda.current_stream(device).wait_event(entry[2])
+    entry[1] = stream
+    return entry
+
 
 
 def matmul_streamk(a, b, *, out_dtype=None):
@@ -187,9 +201,8 @@ def matmul_streamk(a, b, *, out_dtype=None):
     tiles dealt evenly, so tile counts that are not a multiple of the CU count - or smaller than it,
     where this becomes split-K - keep every CU busy.  The scheduling idea of the persistent
     tutorial (python/tutorials/09-persistent-matmul.py:141-190) taken one step further; the
-    result is the same `a @ b` (partial tiles are added in a fixed order).  An fp32 workspace per
-    (device, stream) is allocated on first use and kept: calls on different streams may overlap, so
-    they must not share partial-tile slots."""
+    result is the same `a @ b` (partial tiles are added in a fixed order).  One fp32 workspace per device is
+    allocated on first use and kept; calls on different streams are ordered behind one another by an event."""
     assert a.shape[1] == b.shape[0], "Incompatible dimensions"
     assert _is_contiguous(a), "Matrix A must be contiguous"
     in_dt = _abi_dtype(a)
@@ -207,15 +220,16 @@ def matmul_streamk(a, b, *, out_dtype=None):
         return c.zero_()
     lib = _lib.load()
     stream = _stream()
-    ws = _streamk_workspace.get((a.device, stream))
-    if ws is None:
-        ws = torch.empty(lib.mi355_query(_lib.Q_STREAMK_WORKSPACE_BYTES), device=a.device, dtype=torch.uint8)
-        _streamk_workspace[(a.device, stream)] = ws
+    entry = _streamk_workspace_for(a.device, stream, lib.mi355_query(_lib.Q_STREAMK_WORKSPACE_BYTES))
+    ws = entry[0]
     rc = lib.mi355_gemm_streamk(
         a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
         a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
         in_dt, _TORCH_TO_ABI[out_dtype], 0, 0, _lib.ACT_NONE, ws.data_ptr(), ws.numel(), stream)
     _lib.check(rc, "mi355_gemm_streamk")
+    if entry[2] is None:
+        entry[2] = torch.cuda.Event()
+    entry[2].record(torch.cuda.current_stream(a.device))
     return c
 
 
