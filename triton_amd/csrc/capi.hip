@@ -521,6 +521,8 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
   // query blocks per program; without a mask the one-item-per-workgroup form (2) is the faster one.
   p.variant = knob(knobs().attn_fwd_variant, causal ? 4 : 2);
   p.num_programs = knob(knobs().attn_programs, device_info().cus > 0 ? device_info().cus : 256);
+  // 5: four waves of 64 query rows, 16x16x32 MFMAs, software pipelined inside the wave (head_dim 128)
+  if (p.variant == 5 && attn_fwd_p16_ok(p)) return attn_fwd_p16_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 

@@ -66,6 +66,29 @@ __device__ inline unsigned burn_e4m3_quad(unsigned& s) {
 }
 
 template <int SHAPE>
+__device__ __forceinline__ void burn_mfma32(f32x16& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4) {
+#if MI355_DEVICE_PASS
+  if constexpr (SHAPE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
+  else if constexpr (SHAPE == 2) asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0 cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4));
+#endif
+}
+template <int SHAPE>
+__device__ __forceinline__ void burn_mfma16(f32x4& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4) {
+#if MI355_DEVICE_PASS
+  if constexpr (SHAPE == 1) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
+  else if constexpr (SHAPE == 3) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4));
+#endif
+}
+template <typename V>
+__device__ __forceinline__ void burn_pin(V& c) {
+#if MI355_DEVICE_PASS
+  asm volatile("" : "+a"(c));
+#endif
+}
+
+template <int SHAPE>
 __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, int random_operands) {
 #if MI355_DEVICE_PASS
   unsigned s = threadIdx.x * 2654435761u + blockIdx.x * 97u + 1u;
@@ -85,7 +108,12 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
         s = burn_rnd(s); b[i][e] = random_operands ? (int)s : 0x22222222;
       }
     }
+  // The MFMAs are issued as assembly with the accumulators pinned to accumulation registers, as the GEMM kernels
+  // issue theirs (left to the register allocator, the chains of four-register tiles were rotated through
+  // architectural registers in every round, at half the rate).  16-bit and fp4 operands are four registers, fp8 eight.
   float total = 0.f;
+  const i32x4 a4[2] = {__builtin_shufflevector(a[0], a[0], 0, 1, 2, 3), __builtin_shufflevector(a[1], a[1], 0, 1, 2, 3)};
+  const i32x4 b4[2] = {__builtin_shufflevector(b[0], b[0], 0, 1, 2, 3), __builtin_shufflevector(b[1], b[1], 0, 1, 2, 3)};
   if constexpr (SHAPE == 0 || SHAPE == 2 || SHAPE == 4) {         // 32 x 32 tiles: four chains of 16 registers
     f32x16 acc[4];
 #pragma unroll
@@ -94,22 +122,15 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
       for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
     for (int i = 0; i < iters; i++) {
 #pragma unroll
-      for (int u = 0; u < 8; u++) {
-        if constexpr (SHAPE == 0) {
-          const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a[u & 1], a[u & 1], 0, 1, 2, 3));
-          const bf16x8 bv = __builtin_bit_cast(bf16x8, __builtin_shufflevector(b[(u >> 1) & 1], b[(u >> 1) & 1], 0, 1, 2, 3));
-          acc[u & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av, bv, acc[u & 3], 0, 0, 0);
-        } else if constexpr (SHAPE == 2) {
-          acc[u & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 3], 0, 0, 0, 0, 0, 0);
-        } else {
-          acc[u & 3] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 3], 4, 4, 0, 0, 0, 0);
-        }
-      }
+      for (int u = 0; u < 8; u++) burn_mfma32<SHAPE>(acc[u & 3], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);
     }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");          // the last MFMAs retire before their results are read
 #pragma unroll
-    for (int c = 0; c < 4; c++)
+    for (int c = 0; c < 4; c++) {
+      burn_pin(acc[c]);
 #pragma unroll
       for (int r = 0; r < 16; r++) total += acc[c][r];
+    }
   } else {                                                         // 16 x 16 tiles: eight chains of 4 registers
     f32x4 acc[8];
 #pragma unroll
@@ -118,22 +139,15 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
       for (int r = 0; r < 4; r++) acc[c][r] = 0.f;
     for (int i = 0; i < iters; i++) {
 #pragma unroll
-      for (int u = 0; u < 16; u++) {
-        if constexpr (SHAPE == 1) {
-          const bf16x8 av = __builtin_bit_cast(bf16x8, __builtin_shufflevector(a[u & 1], a[u & 1], 0, 1, 2, 3));
-          const bf16x8 bv = __builtin_bit_cast(bf16x8, __builtin_shufflevector(b[(u >> 1) & 1], b[(u >> 1) & 1], 0, 1, 2, 3));
-          acc[u & 7] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bv, acc[u & 7], 0, 0, 0);
-        } else if constexpr (SHAPE == 3) {
-          acc[u & 7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 7], 0, 0, 0, 0, 0, 0);
-        } else {
-          acc[u & 7] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a[u & 1], b[(u >> 1) & 1], acc[u & 7], 4, 4, 0, 0, 0, 0);
-        }
-      }
+      for (int u = 0; u < 16; u++) burn_mfma16<SHAPE>(acc[u & 7], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);
     }
+    asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
-    for (int c = 0; c < 8; c++)
+    for (int c = 0; c < 8; c++) {
+      burn_pin(acc[c]);
 #pragma unroll
       for (int r = 0; r < 4; r++) total += acc[c][r];
+    }
   }
   if (total == 12345.678f) sink[0] = total;   // (keeps the chains alive; practically never true)
 #endif
