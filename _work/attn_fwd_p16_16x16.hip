@@ -28,6 +28,12 @@
 #include "attn_tiles.h"
 #include "launch.h"
 
+// Build-time knock-outs for timing experiments (results are wrong with any of them set): 1 = no softmax arithmetic,
+// 2 = no maximum check, 4 = no LDS fragment reads, 8 = no global loads, 16 = no MFMAs.
+#ifndef MI355_P16_KO
+#define MI355_P16_KO 0
+#endif
+
 namespace mi355 {
 
 namespace {
@@ -37,6 +43,7 @@ namespace {
 template <bool BF>
 __device__ __forceinline__ void mfma16_s_first(f32x4& d, const i32x4& k, const i32x4& q, const f32x4& bias) {
 #if MI355_DEVICE_PASS
+  if constexpr ((MI355_P16_KO & 16) != 0) { d = bias; return; }
   if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(bias));
   else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %3" : "=&v"(d) : "v"(k), "a"(q), "v"(bias));
 #endif
@@ -44,6 +51,7 @@ __device__ __forceinline__ void mfma16_s_first(f32x4& d, const i32x4& k, const i
 template <bool BF>
 __device__ __forceinline__ void mfma16_s_acc(f32x4& d, const i32x4& k, const i32x4& q) {
 #if MI355_DEVICE_PASS
+  if constexpr ((MI355_P16_KO & 16) != 0) return;
   if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(k), "a"(q));
   else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(d) : "v"(k), "a"(q));
 #endif
@@ -51,6 +59,7 @@ __device__ __forceinline__ void mfma16_s_acc(f32x4& d, const i32x4& k, const i32
 template <bool BF>
 __device__ __forceinline__ void mfma16_o(f32x4& d, const i32x4& v, const i32x4& pt) {
 #if MI355_DEVICE_PASS
+  if constexpr ((MI355_P16_KO & 16) != 0) return;
   if constexpr (BF) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(d) : "v"(v), "v"(pt));
   else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(d) : "v"(v), "v"(pt));
 #endif
@@ -223,10 +232,11 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_p16_kernel(AttnArgs p) {
   // fragment reads: K fragment n = 2 ks + a of the half HK of the current K slot; V fragment c of the half HV
   auto read_k = [&](auto N_, auto HK_, i32x4& dst) {
     constexpr int n = decltype(N_)::value, ks = n >> 1, a = n & 1, hk = decltype(HK_)::value;
-    dst = lds_read_b128<hk * 32 * RB + a * 16 * RB>(kad[ks]);
+    if constexpr ((MI355_P16_KO & 4) == 0) dst = lds_read_b128<hk * 32 * RB + a * 16 * RB>(kad[ks]);
   };
   auto read_v = [&](auto C_, auto HV_, i32x2 (&dst)[2]) {
     constexpr int c = decltype(C_)::value, hv = decltype(HV_)::value;
+    if constexpr ((MI355_P16_KO & 4) != 0) return;
     dst[0] = lds_read_tr16_b64<hv * 32 * RB>(vad[c]);
     dst[1] = lds_read_tr16_b64<hv * 32 * RB + 16 * RB>(vad[c]);
   };
@@ -235,6 +245,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_p16_kernel(AttnArgs p) {
   // into l_i[b] of neighbouring slices do not wait for one another
   auto x_elem = [&](auto PAR_, auto E_) {
     constexpr int par = decltype(PAR_)::value, e = decltype(E_)::value, b = e & 3, i = e >> 2, a = i >> 2, r = i & 3;
+    if constexpr ((MI355_P16_KO & 1) != 0) return;
     pin_v(s[par][a][b]);
     const float pv = fast_exp2(fmaf(s[par][a][b][r], qk_scale, -m_i[b]));
     s[par][a][b][r] = pv;
@@ -249,6 +260,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_p16_kernel(AttnArgs p) {
   // the lane's largest score of query tile b in buffer PAR
   auto check_b = [&](auto PAR_, auto B_) {
     constexpr int par = decltype(PAR_)::value, b = decltype(B_)::value;
+    if constexpr ((MI355_P16_KO & 2) != 0) return;
     float mx = fmaxf(fmaxf(s[par][0][b][0], s[par][0][b][1]), s[par][0][b][2]);
     mx = fmaxf(fmaxf(mx, s[par][0][b][3]), s[par][1][b][0]);
     mx = fmaxf(fmaxf(mx, s[par][1][b][1]), s[par][1][b][2]);
@@ -356,7 +368,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_p16_kernel(AttnArgs p) {
         if constexpr (do_x && (slot & 1) == 0) x_elem(PAR_, std::integral_constant<int, slot / 2>{});
         if constexpr (par == 1 && (slot & 3) == 3 && slot / 4 >= 4) {
           // second half of the load group issued behind barrier X_j of the phase before: K tile j + 3
-          load_k(std::integral_constant<int, slot / 4 - 4>{}, j + 3, F{});
+          if constexpr ((MI355_P16_KO & 8) == 0) load_k(std::integral_constant<int, slot / 4 - 4>{}, j + 3, F{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -393,7 +405,7 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_p16_kernel(AttnArgs p) {
         if constexpr (do_s && slot >= 44 && slot < 60 && (slot & 3) == 0) check_b(HK{}, std::integral_constant<int, (slot - 44) / 4>{});
         if constexpr (par == 0 && (slot & 3) == 3 && (slot - 32) / 4 < 4) {
           // first half of the load group behind X_j: V tile j + 2
-          load_v(std::integral_constant<int, (slot - 32) / 4>{}, j + 2, F{});
+          if constexpr ((MI355_P16_KO & 8) == 0) load_v(std::integral_constant<int, (slot - 32) / 4>{}, j + 2, F{});
         }
         __builtin_amdgcn_sched_barrier(0);
       });

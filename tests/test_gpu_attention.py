@@ -75,6 +75,35 @@ def test_forward_backward_against_oracle(gpu, dtype, causal, shape):
                                          dict(o=ro, dq=rdq, dk=rdk, dv=rdv), cf, dtype)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("causal", [True, False])
+@pytest.mark.parametrize("shape,std", [((1, 2, 256, 128), 0.5), ((2, 3, 1024, 128), 0.5), ((1, 2, 1024, 128), 4.0)])
+def test_in_wave_pipelined_forward_against_the_tiled_oracle(gpu, monkeypatch, dtype, causal, shape, std):
+    # variant 5 (attn_fwd_pipe.hip): the forward program of 06:25-75, :98-187 with a lazily raised running maximum -
+    # O at 1e-2 against the restated tile program in the kernel's own type, M at 2e-3 against the closed form.  The
+    # wide scores (std 4: exponents that differ by hundreds from key to key) exercise the raise of the maximum and the
+    # deferred rescale of the accumulators in nearly every sub-step.
+    from triton_amd import _lib
+    rng = np.random.default_rng(sum(shape) + int(std * 10))
+    q, k = (randn_rounded(rng, shape, dtype, std) for _ in range(2))
+    v = randn_rounded(rng, shape, dtype, 0.5)
+    tq, tk, tv = (from_np(x, dtype, gpu) for x in (q, k, v))
+    sm_scale = shape[-1] ** -0.5
+    set_knob(monkeypatch, "MI355_ATTN_FWD_VARIANT", "5")
+    Z, H, N, D = shape
+    o = torch.empty_like(tq)
+    M = torch.empty(Z, H, N, dtype=torch.float32, device=gpu)
+    I4 = _lib.I64x4
+    rc = _lib.load().mi355_attn_fwd(tq.data_ptr(), tk.data_ptr(), tv.data_ptr(), o.data_ptr(), M.data_ptr(), Z, H, N, D,
+                                    I4(*tq.stride()), I4(*tk.stride()), I4(*tv.stride()), I4(*o.stride()), sm_scale, int(causal),
+                                    _lib.BF16 if dtype == "bf16" else _lib.F16, torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    ro, _ = A.attn_fwd_tiled(q, k, v, causal, sm_scale, dtype)
+    cf = A.attn_closed_form(q, k, v, causal, sm_scale)
+    assert np.allclose(to_np(o), ro, atol=1e-2, rtol=1e-2), np.abs(to_np(o) - ro).max()
+    assert np.allclose(to_np(M), cf["M"], atol=2e-3, rtol=1e-6), np.abs(to_np(M) - cf["M"]).max()
+
+
 @pytest.mark.parametrize("n_ctx", [512, 384])
 @pytest.mark.parametrize("causal", [True, False])
 def test_forward_variants_and_lse(gpu, causal, n_ctx, monkeypatch):
@@ -84,8 +113,9 @@ def test_forward_variants_and_lse(gpu, causal, n_ctx, monkeypatch):
     cf = A.attn_closed_form(q, k, v, causal, 0.125)
     # 0: 64 query rows per wave, 1: four waves of 32 rows, 2: eight waves of 32 rows (n_ctx = 384 leaves
     # half of its second 256-row block empty), 3 and 4: 1 and 2 as persistent programs (two programs here, so
-    # that each walks several items)
-    for variant in ("0", "1", "2", "3", "4"):
+    # that each walks several items), 5: four waves of 64 rows, software pipelined inside the wave (N_CTX a multiple
+    # of 256 and head_dim 128, else it is variant 2's kernel that runs)
+    for variant in ("0", "1", "2", "3", "4", "5"):
         set_knob(monkeypatch, "MI355_ATTN_FWD_VARIANT", variant)
         set_knob(monkeypatch, "MI355_ATTN_PROGRAMS", "1")
         o = torch.empty_like(tq)

@@ -522,7 +522,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
   p.variant = knob(knobs().attn_fwd_variant, causal ? 4 : 2);
   p.num_programs = knob(knobs().attn_programs, device_info().cus > 0 ? device_info().cus : 256);
   // 5: four waves of 64 query rows, 16x16x32 MFMAs, software pipelined inside the wave (head_dim 128)
-  if (p.variant == 5 && attn_fwd_p16_ok(p)) return attn_fwd_p16_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
+  if (p.variant == 5 && attn_fwd_pipe_ok(p)) return attn_fwd_pipe_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
   return attn_fwd_launch(p, dtype == MI355_BF16, (hipStream_t)stream_);
 }
 

@@ -81,6 +81,20 @@ __device__ __forceinline__ void burn_mfma16(f32x4& c, const burn_i32x8& a, const
   else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4));
 #endif
 }
+// two idle slots behind the (vector) write of an accumulator, tied to it: an assembly MFMA must not read a register
+// within two slots of a vector write, and the compiler, which keeps that distance for MFMAs it knows, cannot here
+template <typename V>
+__device__ __forceinline__ void burn_settle(V& c) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 1" : "+a"(c));
+#endif
+}
+__device__ __forceinline__ void burn_settle_operands(burn_i32x8& a0, burn_i32x8& a1, burn_i32x8& b0, burn_i32x8& b1,
+                                                     i32x4& c0, i32x4& c1, i32x4& d0, i32x4& d1) {
+#if MI355_DEVICE_PASS
+  asm volatile("s_nop 1" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1), "+v"(c0), "+v"(c1), "+v"(d0), "+v"(d1));
+#endif
+}
 template <typename V>
 __device__ __forceinline__ void burn_pin(V& c) {
 #if MI355_DEVICE_PASS
@@ -112,14 +126,17 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
   // issue theirs (left to the register allocator, the chains of four-register tiles were rotated through
   // architectural registers in every round, at half the rate).  16-bit and fp4 operands are four registers, fp8 eight.
   float total = 0.f;
-  const i32x4 a4[2] = {__builtin_shufflevector(a[0], a[0], 0, 1, 2, 3), __builtin_shufflevector(a[1], a[1], 0, 1, 2, 3)};
-  const i32x4 b4[2] = {__builtin_shufflevector(b[0], b[0], 0, 1, 2, 3), __builtin_shufflevector(b[1], b[1], 0, 1, 2, 3)};
+  i32x4 a4[2] = {__builtin_shufflevector(a[0], a[0], 0, 1, 2, 3), __builtin_shufflevector(a[1], a[1], 0, 1, 2, 3)};
+  i32x4 b4[2] = {__builtin_shufflevector(b[0], b[0], 0, 1, 2, 3), __builtin_shufflevector(b[1], b[1], 0, 1, 2, 3)};
   if constexpr (SHAPE == 0 || SHAPE == 2 || SHAPE == 4) {         // 32 x 32 tiles: four chains of 16 registers
     f32x16 acc[4];
 #pragma unroll
     for (int c = 0; c < 4; c++)
 #pragma unroll
       for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; c++) burn_settle(acc[c]);
+    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1]);
     for (int i = 0; i < iters; i++) {
 #pragma unroll
       for (int u = 0; u < 8; u++) burn_mfma32<SHAPE>(acc[u & 3], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);
@@ -137,6 +154,9 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
     for (int c = 0; c < 8; c++)
 #pragma unroll
       for (int r = 0; r < 4; r++) acc[c][r] = 0.f;
+#pragma unroll
+    for (int c = 0; c < 8; c++) burn_settle(acc[c]);
+    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1]);
     for (int i = 0; i < iters; i++) {
 #pragma unroll
       for (int u = 0; u < 16; u++) burn_mfma16<SHAPE>(acc[u & 7], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);

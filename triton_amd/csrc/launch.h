@@ -124,8 +124,8 @@ int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmaj
 int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
-bool attn_fwd_p16_ok(const AttnArgs& p);
-int attn_fwd_p16_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
+bool attn_fwd_pipe_ok(const AttnArgs& p);
+int attn_fwd_pipe_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_fwd8_launch(const AttnArgs& p, bool e5m2, hipStream_t stream);  // fp8 inputs, V with N contiguous
 int attn_bwd_pre_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 int attn_bwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
