@@ -39,6 +39,10 @@
 #endif
 // Build-time switch for a timing experiment: the waves accumulate shader-clock cycles per part of the main loop's
 // phases and workgroup 0 writes its sums over M (which is wrong then).
+// 1: the main loop's phases with each pair of MFMA slots as one assembly statement; 0: as separate statements
+#ifndef MI355_ATTN_PIPE_FUSED_SLOTS
+#define MI355_ATTN_PIPE_FUSED_SLOTS 1
+#endif
 #ifndef MI355_ATTN_PIPE_TIMING
 #define MI355_ATTN_PIPE_TIMING 0
 #endif
@@ -121,6 +125,90 @@ template <typename S>
 __device__ __forceinline__ int pack2(float x, float y) {
   typedef __attribute__((ext_vector_type(2))) S S2;
   return __builtin_bit_cast(int, S2{(S)x, (S)y});
+}
+
+
+// ---- One pair of MFMA slots as ONE assembly statement (the full phases of the key loop): the wait for the pair's
+// fragment, the two MFMAs on it (query tiles 0 and 1), and behind each its slice of the softmax pipeline - finish
+// element i (sum, and with CVT the conversion of a pair of probabilities), exponentiate element i + 1, start element
+// i + 2 - plus, in the PV part, one step of the maximum of the next sub-step's scores.  Written out because what
+// bounds this kernel is instruction issue: measured on the device, a 32-cycle MFMA slot hides about 24 cycles of
+// other instructions (4 per vector instruction, 8 per exponential) and every cycle beyond that is paid in full,
+// and around statements of its own the compiler pads uses of assembly results with idle slots (79 per phase).
+// sA .. sD: scores [tile 0, r], [tile 1, r], [tile 0, r + 1], [tile 1, r + 1] of the sub-step being exponentiated;
+// sP0 / sP1: [tile 0 / 1, r - 1] (CVT: r odd).  Distances inside: an exponential is read two or more instructions
+// later, a multiply-add result three or more.
+#define MI355_X_SLOT0(CVS) "v_add_f32 %[l0], %[sA], %[l0]\n\t" CVS "v_exp_f32 %[sB], %[sB]\n\tv_fma_f32 %[sC], %[sC], %[sc], -%[m0]\n\t"
+#define MI355_X_SLOT1(CVS) "v_add_f32 %[l1], %[sB], %[l1]\n\t" CVS "v_exp_f32 %[sC], %[sC]\n\tv_fma_f32 %[sD], %[sD], %[sc], -%[m1]\n\t"
+#define MI355_WAITL "s_waitcnt lgkmcnt(%[n])\n\t"
+#define MI355_X_OUT "+v"(l0), "+v"(l1), "+v"(sB), "+v"(sC), "+v"(sD)
+#define MI355_X_IN [sA] "v"(sA), [sc] "s"(sc), [m0] "v"(m0), [m1] "v"(m1), [n] "i"(N)
+
+// S part: scores of the next sub-step, tiles 0 and 1, k-step of fragment `fr`; FIRST: from the bias tiles
+template <bool BF, bool FIRST, bool CVT, int N>
+__device__ __forceinline__ void pair_s(f32x16& a0, f32x16& a1, const i32x4& fr, const i32x4& q0, const i32x4& q1, const f32x16& bi0,
+                                       const f32x16& bi1, float& l0, float& l1, float sA, float& sB, float& sC, float& sD, float sP0, float sP1,
+                                       int& w0, int& w1, float sc, float m0, float m1) {
+#if MI355_DEVICE_PASS
+#define MI355_PAIR_S(T, CV)                                                                                                        \
+  if constexpr (FIRST)                                                                                                             \
+    asm volatile(MI355_WAITL "v_mfma_f32_32x32x16_" T " %[a0], %[fr], %[q0], %[bi0]\n\t" MI355_X_SLOT0("")                        \
+                 "v_mfma_f32_32x32x16_" T " %[a1], %[fr], %[q1], %[bi1]\n\t" MI355_X_SLOT1("")                                    \
+                 : [a0] "=&v"(a0), [a1] "=&v"(a1), [l0] "+v"(l0), [l1] "+v"(l1), [sB] "+v"(sB), [sC] "+v"(sC), [sD] "+v"(sD)      \
+                 : [fr] "v"(fr), [q0] "a"(q0), [q1] "a"(q1), [bi0] "v"(bi0), [bi1] "v"(bi1), MI355_X_IN);                         \
+  else if constexpr (CVT)                                                                                                          \
+    asm volatile(MI355_WAITL "v_mfma_f32_32x32x16_" T " %[a0], %[fr], %[q0], %[a0]\n\t" MI355_X_SLOT0(CV " %[w0], %[sP0], %[sA]\n\t") \
+                 "v_mfma_f32_32x32x16_" T " %[a1], %[fr], %[q1], %[a1]\n\t" MI355_X_SLOT1(CV " %[w1], %[sP1], %[sB]\n\t")         \
+                 : [a0] "+v"(a0), [a1] "+v"(a1), [l0] "+v"(l0), [l1] "+v"(l1), [sB] "+v"(sB), [sC] "+v"(sC), [sD] "+v"(sD),       \
+                   [w0] "=&v"(w0), [w1] "=&v"(w1)                                                                                 \
+                 : [fr] "v"(fr), [q0] "a"(q0), [q1] "a"(q1), [sP0] "v"(sP0), [sP1] "v"(sP1), MI355_X_IN);                         \
+  else                                                                                                                             \
+    asm volatile(MI355_WAITL "v_mfma_f32_32x32x16_" T " %[a0], %[fr], %[q0], %[a0]\n\t" MI355_X_SLOT0("")                         \
+                 "v_mfma_f32_32x32x16_" T " %[a1], %[fr], %[q1], %[a1]\n\t" MI355_X_SLOT1("")                                     \
+                 : [a0] "+v"(a0), [a1] "+v"(a1), [l0] "+v"(l0), [l1] "+v"(l1), [sB] "+v"(sB), [sC] "+v"(sC), [sD] "+v"(sD)        \
+                 : [fr] "v"(fr), [q0] "a"(q0), [q1] "a"(q1), MI355_X_IN)
+  if constexpr (BF) { MI355_PAIR_S("bf16", "v_cvt_pk_bf16_f32"); } else { MI355_PAIR_S("f16", "v_cvt_pk_f16_f32"); }
+#undef MI355_PAIR_S
+#endif
+}
+
+// PV part: O^T tiles 0 and 1 += V^T fragment `fr` times P^T operands p0 / p1, and step CHK of the lane's maximum of
+// the next sub-step's scores (ca*: two registers of its tile 0, cb*: of its tile 1; CHK == 1: the first step)
+template <bool BF, bool CVT, int CHK, int N>
+__device__ __forceinline__ void pair_pv(f32x16& a0, f32x16& a1, const i32x4& fr, const i32x4& p0, const i32x4& p1, float& l0, float& l1,
+                                        float sA, float& sB, float& sC, float& sD, float sP0, float sP1, int& w0, int& w1, float sc,
+                                        float m0, float m1, float& mx0, float& mx1, float ca0, float ca1, float cb0, float cb1) {
+#if MI355_DEVICE_PASS
+#define MI355_CHK0 "v_max3_f32 %[mx0], %[mx0], %[ca0], %[ca1]\n\t"
+#define MI355_CHK1 "v_max3_f32 %[mx1], %[mx1], %[cb0], %[cb1]\n\t"
+#define MI355_CHF0 "v_max_f32 %[mx0], %[ca0], %[ca1]\n\t"
+#define MI355_CHF1 "v_max_f32 %[mx1], %[cb0], %[cb1]\n\t"
+#define MI355_PAIR_PV(T, CV, K0, K1, MXC)                                                                                          \
+  if constexpr (CVT)                                                                                                               \
+    asm volatile(MI355_WAITL "v_mfma_f32_32x32x16_" T " %[a0], %[fr], %[p0], %[a0]\n\t" MI355_X_SLOT0(CV " %[w0], %[sP0], %[sA]\n\t") K0 \
+                 "v_mfma_f32_32x32x16_" T " %[a1], %[fr], %[p1], %[a1]\n\t" MI355_X_SLOT1(CV " %[w1], %[sP1], %[sB]\n\t") K1      \
+                 : [a0] "+a"(a0), [a1] "+a"(a1), [l0] "+v"(l0), [l1] "+v"(l1), [sB] "+v"(sB), [sC] "+v"(sC), [sD] "+v"(sD),       \
+                   [w0] "=&v"(w0), [w1] "=&v"(w1), [mx0] MXC(mx0), [mx1] MXC(mx1)                                                 \
+                 : [fr] "v"(fr), [p0] "v"(p0), [p1] "v"(p1), [sP0] "v"(sP0), [sP1] "v"(sP1), [ca0] "v"(ca0), [ca1] "v"(ca1),      \
+                   [cb0] "v"(cb0), [cb1] "v"(cb1), MI355_X_IN);                                                                   \
+  else                                                                                                                             \
+    asm volatile(MI355_WAITL "v_mfma_f32_32x32x16_" T " %[a0], %[fr], %[p0], %[a0]\n\t" MI355_X_SLOT0("") K0                      \
+                 "v_mfma_f32_32x32x16_" T " %[a1], %[fr], %[p1], %[a1]\n\t" MI355_X_SLOT1("") K1                                  \
+                 : [a0] "+a"(a0), [a1] "+a"(a1), [l0] "+v"(l0), [l1] "+v"(l1), [sB] "+v"(sB), [sC] "+v"(sC), [sD] "+v"(sD),       \
+                   [mx0] MXC(mx0), [mx1] MXC(mx1)                                                                                 \
+                 : [fr] "v"(fr), [p0] "v"(p0), [p1] "v"(p1), [ca0] "v"(ca0), [ca1] "v"(ca1), [cb0] "v"(cb0), [cb1] "v"(cb1),      \
+                   MI355_X_IN)
+#define MI355_RW "+v"
+#define MI355_WO "=&v"
+  if constexpr (BF) {
+    if constexpr (CHK == 1) { MI355_PAIR_PV("bf16", "v_cvt_pk_bf16_f32", MI355_CHF0, MI355_CHF1, MI355_WO); }
+    else { MI355_PAIR_PV("bf16", "v_cvt_pk_bf16_f32", MI355_CHK0, MI355_CHK1, MI355_RW); }
+  } else {
+    if constexpr (CHK == 1) { MI355_PAIR_PV("f16", "v_cvt_pk_f16_f32", MI355_CHF0, MI355_CHF1, MI355_WO); }
+    else { MI355_PAIR_PV("f16", "v_cvt_pk_f16_f32", MI355_CHK0, MI355_CHK1, MI355_RW); }
+  }
+#undef MI355_PAIR_PV
+#endif
 }
 
 }  // namespace
@@ -468,6 +556,77 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_pipe_kernel(AttnArgs p) {
       tlast = a3;
     }
   };
+  // The full phase (S, X and PV all present: every phase of the main loop) with each pair of MFMA slots as one
+  // assembly statement (pair_s / pair_pv): same schedule as `phase`, same fragment sequence and loads.
+  auto phase_full = [&](auto PAR_, int u) {
+    constexpr int par = decltype(PAR_)::value;
+    using HK = std::integral_constant<int, par ^ 1>;
+    using HN = std::integral_constant<int, par>;
+    const int j = u >> 1;
+    auto request = [&](auto Q_) {
+      constexpr int q = decltype(Q_)::value;
+      if constexpr (q < 8) read_k(std::integral_constant<int, q>{}, HK{}, kf[q % NF]);
+      else if constexpr (q < 16) read_v(std::integral_constant<int, q - 8>{}, HK{}, vf[(q - 8) % NF]);
+      else read_k(std::integral_constant<int, q - 16>{}, HN{}, kf[(q - 16) % NF]);
+    };
+    auto behind = [](int q) { int n = 0; for (int i = q + 1; i <= q + FD; i++) n += (i >= 8 && i < 16) ? 2 : 1; return n; };
+    if constexpr (par == 1) aim_k(j + 3);
+    const unsigned long long a0 = stamp();
+    x_head(PAR_);
+    float dummy0 = 0.f, dummy1 = 0.f;
+    // pair g = 0 .. 15: slots 2 g and 2 g + 1; elements [tile 0, g], [tile 1, g] are finished, [tile 0, g + 1], [tile 1, g + 1] started
+    auto run_pair = [&](auto G_) {
+      constexpr int g = decltype(G_)::value, n = g & 7;
+      constexpr bool cvt = (g & 1) == 1;
+      float sA = s[par][0][g], sB = s[par][1][g];
+      float sC = g < 15 ? s[par][0][g < 15 ? g + 1 : 0] : dummy0, sD = g < 15 ? s[par][1][g < 15 ? g + 1 : 0] : dummy1;
+      const float sP0 = s[par][0][g > 0 ? g - 1 : 0], sP1 = s[par][1][g > 0 ? g - 1 : 0];
+      int w0 = 0, w1 = 0;
+      request(std::integral_constant<int, g + FD>{});
+      if constexpr (g < 8) {
+        pair_s<BF, g == 0, cvt, behind(g)>(s[par ^ 1][0], s[par ^ 1][1], kf[n % NF], qf[0][n], qf[1][n], mb[0], mb[1], l_i[0], l_i[1],
+                                           sA, sB, sC, sD, sP0, sP1, w0, w1, qk_scale, m_i[0], m_i[1]);
+      } else {
+        constexpr int t = n >> 2, c = n & 3, k = g - 8;
+        const i32x4 vfrag = __builtin_shufflevector(vf[n % NF][0], vf[n % NF][1], 0, 1, 2, 3);
+        pair_pv<BF, cvt, (k == 0 ? 1 : 2), behind(g)>(oacc[c][0], oacc[c][1], vfrag, pf[par ^ 1][0][t], pf[par ^ 1][1][t], l_i[0], l_i[1],
+                                                      sA, sB, sC, sD, sP0, sP1, w0, w1, qk_scale, m_i[0], m_i[1], mxl[0], mxl[1],
+                                                      s[par ^ 1][0][2 * k], s[par ^ 1][0][2 * k + 1], s[par ^ 1][1][2 * k], s[par ^ 1][1][2 * k + 1]);
+      }
+      s[par][1][g] = sB;
+      if constexpr (g < 15) { s[par][0][g + 1] = sC; s[par][1][g + 1] = sD; }
+      else { dummy0 = sC; dummy1 = sD; }
+      if constexpr (cvt) { pf[par][0][g >> 3][(g & 7) >> 1] = w0; pf[par][1][g >> 3][(g & 7) >> 1] = w1; }
+      if constexpr (par == 1 && g >= 4 && g < 8) {
+        if constexpr ((MI355_ATTN_PIPE_KO & 8) == 0) load_k(std::integral_constant<int, (g >= 4 && g < 8 ? g - 4 : 0)>{}, F{});
+      }
+      if constexpr (par == 0 && g >= 8 && g < 12) {
+        if constexpr ((MI355_ATTN_PIPE_KO & 8) == 0) load_v(std::integral_constant<int, (g >= 8 && g < 12 ? g - 8 : 0)>{}, F{});
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    static_for<8>([&](auto N_) { run_pair(N_); });
+    const unsigned long long a1 = stamp();
+    if constexpr (par == 0) {
+      wait_vmcnt<GROUP>();
+      __builtin_amdgcn_sched_barrier(0);
+      block_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+      set_kslot(j + 1);
+      aim_v(j + 2);
+    }
+    const unsigned long long a2 = stamp();
+    static_for<8>([&](auto N_) { run_pair(std::integral_constant<int, 8 + decltype(N_)::value>{}); });
+    over[0] = __builtin_amdgcn_ballot_w64(mxl[0] > thr[0]);
+    over[1] = __builtin_amdgcn_ballot_w64(mxl[1] > thr[1]);
+    if constexpr (par == 0) set_vslot(j);
+    if constexpr (MI355_ATTN_PIPE_TIMING != 0) {
+      unsigned long long a3 = stamp(), b0 = a0, b1 = a1, b2 = a2;
+      asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(b0), "+s"(b1), "+s"(b2), "+s"(a3) :: "memory");
+      tsum[0] += b1 - b0; tsum[1] += b2 - b1; tsum[2] += a3 - b2; tsum[4] += 1;
+      tlast = a3;
+    }
+  };
   // the cold work between two phases: the accumulators' pending rescale, the raise that the scores of S(u+1) ask
   // for, and the bias tiles of S(u+2) where that sub-step meets the diagonal
   auto between = [&](int u, bool more_s) {
@@ -528,9 +687,9 @@ __global__ __launch_bounds__(256, 1) void attn_fwd_pipe_kernel(AttnArgs p) {
   between(0, true);
   int u = 1;
   for (; u + 1 < L; u += 2) {
-    phase(I1{}, T{}, T{}, T{}, u);
+    if constexpr (MI355_ATTN_PIPE_FUSED_SLOTS) phase_full(I1{}, u); else phase(I1{}, T{}, T{}, T{}, u);
     between(u, true);
-    phase(I0{}, T{}, T{}, T{}, u + 1);
+    if constexpr (MI355_ATTN_PIPE_FUSED_SLOTS) phase_full(I0{}, u + 1); else phase(I0{}, T{}, T{}, T{}, u + 1);
     between(u + 1, true);
   }
   phase(I1{}, F{}, T{}, T{}, u);         // u == L
