@@ -12,6 +12,7 @@ import pytest
 import torch
 
 import triton_amd
+from triton_amd import _lib
 from oracle import formats, gemm
 from util import bits_equal, from_np, randn_rounded, to_np, set_knob
 
@@ -236,10 +237,11 @@ def test_fp8_raw_code_inputs_like_reference_test(gpu):
     assert np.allclose(c, ref, rtol=0.01, atol=0.01)
 
 
-def test_fp8_row_major_b_uses_the_strided_kernel_and_fp8_output(gpu):
+def test_fp8_row_major_b_of_unaligned_rows_and_fp8_output(gpu):
+    # (rows of 72 bytes are not whole 16-byte chunks: the strided kernel, whose sums are in fp32 order of k)
     rng = np.random.default_rng(8)
     ca = formats.encode_fp8(rng.standard_normal((64, 96)).astype(np.float32), "e4m3")
-    cb = formats.encode_fp8(rng.standard_normal((96, 80)).astype(np.float32), "e4m3")    # [K, N] row-major
+    cb = formats.encode_fp8(rng.standard_normal((96, 72)).astype(np.float32), "e4m3")    # [K, N] row-major
     tab = formats.fp8_table("e4m3")
     ta = torch.from_numpy(ca).to(gpu).view(torch.float8_e4m3fn)
     tb = torch.from_numpy(cb).to(gpu).view(torch.float8_e4m3fn)
@@ -253,23 +255,61 @@ def test_fp8_row_major_b_uses_the_strided_kernel_and_fp8_output(gpu):
     assert triton_amd.matmul_like_input(a16, b16).dtype == torch.float16
 
 
-def test_large_row_major_fp8_b_is_put_k_major_by_the_host_wrapper(gpu):
-    # 03:378-380 pre-transposes b on the host for fp8; `matmul` does the same for a large row-major fp8 B, so the
-    # product runs on the fp8 MFMAs (told apart from the strided kernel by time) and equals the K-major call
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+@pytest.mark.parametrize("shape", [(128, 128, 64), (256, 256, 256), (300, 208, 144), (100, 16, 48), (512, 768, 1040), (1024, 2048, 512),
+                                   (2304, 2560, 320)])
+def test_row_major_fp8_b_runs_the_mfma_kernels_bit_exactly(gpu, fmt, tdt, shape):
+    # `matmul(a, b)` with b stored [K, N] (what tutorial 03 passes before its fp8 special case, 03:378-380): the C ABI
+    # transposes the B tile on its way out of LDS.  Small integers as operands: every sum is exact in fp32, so the
+    # product equals numpy's and the K-major call's bit for bit - edge tiles, K tails (K % 64 != 0) and both tile sizes.
+    M, N, K = shape
+    rng = np.random.default_rng(M * 7 + N * 3 + K)
+    xa = rng.integers(-4, 5, size=(M, K)).astype(np.float32)
+    xb = rng.integers(-4, 5, size=(K, N)).astype(np.float32)
+    ta = torch.from_numpy(formats.encode_fp8(xa, fmt)).to(gpu).view(tdt)
+    tb = torch.from_numpy(formats.encode_fp8(xb, fmt)).to(gpu).view(tdt)                   # [K, N] row-major
+    got = triton_amd.matmul(ta, tb, out_dtype=torch.float32)
+    assert np.array_equal(to_np(got), xa.astype(np.float64) @ xb.astype(np.float64))
+    assert torch.equal(got, triton_amd.matmul(ta, tb.t().contiguous().t(), out_dtype=torch.float32))
+    # a pitch wider than the row (a column slice of a larger matrix)
+    wide = torch.zeros(K, N + 48, dtype=torch.uint8, device=gpu).view(tdt)
+    wide[:, 16:16 + N] = tb
+    assert torch.equal(triton_amd.matmul(ta, wide[:, 16:16 + N], out_dtype=torch.float32), got)
+
+
+def test_large_row_major_fp8_b_runs_on_the_fp8_mfmas_inside_the_c_abi(gpu):
+    # 03:378-380 pre-transposes b on the host for fp8; here mi355_gemm itself takes the row-major B (no copy of B in
+    # the wrapper): told apart from the strided kernel by time, equal to the K-major call bit for bit (the same
+    # products summed in the same order: both forms walk K in 64-byte steps with the same lane assignment)
     n = 4096
     g = torch.Generator(device="cpu").manual_seed(12)
     a = (torch.randn(n, n, generator=g) * 0.5).to(torch.float8_e4m3fn).to(gpu)
     b = (torch.randn(n, n, generator=g) * 0.5).to(torch.float8_e4m3fn).to(gpu)     # [K, N] row-major
-    want = triton_amd.matmul(a, b.t().contiguous().t(), out_dtype=torch.bfloat16)
-    got = triton_amd.matmul(a, b, out_dtype=torch.bfloat16)
+    got = torch.empty(n, n, dtype=torch.bfloat16, device=gpu)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def call():
+        rc = lib.mi355_gemm(a.data_ptr(), b.data_ptr(), got.data_ptr(), n, n, n, a.stride(0), a.stride(1), b.stride(0), b.stride(1),
+                            got.stride(0), got.stride(1), _lib.F8E4M3, _lib.BF16, None, None, _lib.ACT_NONE, stream)
+        assert rc == 0, rc
+
+    call()
     torch.cuda.synchronize()
     ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     ev0.record()
-    got = triton_amd.matmul(a, b, out_dtype=torch.bfloat16)
+    call()
     ev1.record()
     torch.cuda.synchronize()
-    assert torch.equal(got, want)
-    assert ev0.elapsed_time(ev1) < 5.0, ev0.elapsed_time(ev1)
+    ms = ev0.elapsed_time(ev1)
+    print(f"mi355_gemm, row-major e4m3 B, 4096^3: {ms:.3f} ms = {2 * n ** 3 / ms / 1e9:.0f} TFLOP/s")
+    assert ms < 1.0, ms
+    rows = [0, 255, 2048, 4095]
+    ref = a[rows].double() @ b.double()
+    err = (got[rows].double() - ref).abs().max().item()
+    print(f"max abs error against fp64 on 4 rows: {err:.3e}")
+    assert torch.allclose(got[rows].double(), ref, rtol=1e-2, atol=0.02)      # (bf16 results: half an ulp is 2^-9 of the value)
+    assert torch.equal(triton_amd.matmul(a, b, out_dtype=torch.bfloat16), got)
 
 
 @pytest.mark.parametrize("tile", [None, 6])

@@ -163,7 +163,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const bool out_ok = true;   // every output type of the ABI has a store in the MFMA epilogues (fp8: hardware conversion, saturating)
   const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
-  const bool b_nmajor = !is8 && sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
+  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
   // the tile copies address 256 rows of an operand with 32-bit byte offsets from a 64-bit tile base
   const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
   const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && knob(knobs().force_strided, 0) == 0;
@@ -254,9 +254,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     if (use && gemm_skinny_ok(sk, y_kmajor, x_kmajor, es))
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
-  if (is8 && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && w128_ok && gemm_wave128_ok(p, true, in_dtype)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, tile, stream);
+  if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && b_kmajor && tile == 6 && w128_ok) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)
   if (tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);

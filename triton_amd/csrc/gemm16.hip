@@ -9,6 +9,7 @@ struct Cfg16 {
   using Operand = V8;
   static constexpr int kSteps = 2, kChunks = 1;
   static constexpr bool kRowMajorB = true, kScaled = false;
+  static constexpr int kElemBytes = 2;
   static constexpr int kStepsPerScaleDword = 1;
   // no block scales: placeholders so that generic code naming them compiles
   __device__ static int scale_dword_offset(int) { return 0; }

@@ -1,7 +1,8 @@
 // fp8 (e4m3fn / e5m2) instantiation of the tiled MFMA GEMM core: 64 elements per K step, one
-// 32x32x64 f8f6f4 MFMA sub-step, both operands K-major (the layout the reference uses for fp8:
-// `matmul(a, b.T)` with b stored [N, K], python/tutorials/03-matrix-multiplication.py:378-382,
-// python/tutorials/09-persistent-matmul.py:396-407).
+// 32x32x64 f8f6f4 MFMA sub-step.  Every kernel form takes both operands K-major (the layout the reference uses
+// for fp8: `matmul(a, b.T)` with b stored [N, K], python/tutorials/03-matrix-multiplication.py:378-382,
+// python/tutorials/09-persistent-matmul.py:396-407); a row-major B[K, N] (what `matmul(a, b)` passes without that
+// host-side transpose) runs the one-barrier-per-step form, which transposes it on its way out of LDS.
 #include "gemm_core.h"
 #include "formats.h"
 
@@ -11,7 +12,8 @@ template <int FMT>  // 0 = e4m3fn, 1 = e5m2 (cbsz / blgp encoding of the instruc
 struct Cfg8 {
   using Operand = i32x8;
   static constexpr int kSteps = 1, kChunks = 2;
-  static constexpr bool kRowMajorB = false, kScaled = false;
+  static constexpr bool kRowMajorB = true, kScaled = false;   // (row-major B: the one-barrier-per-step kernel only)
+  static constexpr int kElemBytes = 1;
   static constexpr int kStepsPerScaleDword = 1;
   // no block scales: placeholders so that generic code naming them compiles
   __device__ static int scale_dword_offset(int) { return 0; }
@@ -125,7 +127,12 @@ int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
   return (int)hipGetLastError();
 }
 
-int gemm8_launch(const GemmArgs& p, bool e5m2, int tile, hipStream_t stream) {
+int gemm8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int tile, hipStream_t stream) {
+  if (!b_kmajor) {
+    // 128x128 tiles (two workgroups per CU) where the dispatcher chose them, 256x256 tiles otherwise
+    if (tile == 1) return e5m2 ? launch_gemm<Cfg8<1>, 128, 128, 2, 2, false, 4>(p, stream) : launch_gemm<Cfg8<0>, 128, 128, 2, 2, false, 4>(p, stream);
+    return e5m2 ? launch_gemm<Cfg8<1>, 256, 256, 2, 4, false, 4>(p, stream) : launch_gemm<Cfg8<0>, 256, 256, 2, 4, false, 4>(p, stream);
+  }
   return e5m2 ? launch_gemm_tile<Cfg8<1>, true>(p, tile, stream) : launch_gemm_tile<Cfg8<0>, true>(p, tile, stream);
 }
 

@@ -13,7 +13,7 @@
 //     multiplied (the younger ones stay in flight);
 //   * LDS rows are XOR-swizzled for the 64-bank LDS so that ds_read_b128 / ds_read_b64_tr_b16
 //     are conflict free;
-//   * a row-major 16-bit B[K,N] is transposed on the fly by the LDS transpose read; a K-major B
+//   * a row-major 16-bit or fp8 B[K,N] is transposed on the fly by the LDS transpose reads; a K-major B
 //     (the `b.T` view the reference passes for fp8, :378-382) uses plain 128-bit reads;
 //   * 32x32 MFMA tiles with the operands swapped, so every lane owns 4 consecutive columns of
 //     one C row and stores them with one instruction;
@@ -23,7 +23,9 @@
 //   kSteps            MFMA sub-steps per 64-byte K step
 //   kChunks           16-byte LDS chunks one lane feeds into one MFMA operand (1 or 2)
 //   chunk(ks, g, c)   which 16-byte chunk (0..3) of the row lane-group g reads for sub-step ks
-//   kRowMajorB        whether the transpose-read path for a row-major B exists (16-bit only)
+//   kRowMajorB        whether a transpose-read path for a row-major B exists (16-bit: every kernel form; fp8: the
+//                     one-barrier-per-step form)
+//   kElemBytes        bytes per element of a row-major B (2 or 1; unused without kRowMajorB)
 //   kScaled           block-scaled: per-row e8m0 scales ride along (MX)
 //   Operand           register type of one MFMA operand
 //   mma<ks>(...)      the MFMA itself
@@ -55,23 +57,34 @@ struct TileCopyK {
   __device__ static int chunk(int lane, int r) { return (lane % CPR) ^ kswz(r); }  // logical chunk fetched
 };
 
-// Row-major [RBK/2 x BN] 16-bit tile of B (rows are k, BN*2 bytes each, a multiple of the
-// 256-byte bank sweep).  A transpose read is served 32 lanes at a time: two 16-lane groups that
-// address the same 4 consecutive k rows and two neighbouring 32-byte groups of columns.  The
-// 32-byte group index is XORed with 2 * (k & 3), which spreads those 4 rows x 64 bytes over all
-// banks.
-template <int BN, int NW>
+// Row-major [RBK/EB x BN] tile of B with elements of EB bytes (rows are k, BN*EB bytes each).
+// 16-bit: a transpose read is served 32 lanes at a time: two 16-lane groups that address the same 4
+// consecutive k rows and two neighbouring 32-byte groups of columns.  The 32-byte group index is XORed
+// with 2 * (k & 3), which spreads those 4 rows x 64 bytes over all banks.
+// 8-bit: a transpose read (ds_read_b64_tr_b8: within 16 lanes, lane 2 r + h addresses the 8 bytes of columns
+// 8 h .. 8 h + 7 of row r; lane j receives column j of the 8 rows) covers, per 32 lanes, 8 consecutive k rows of
+// two neighbouring 16-byte chunks.  The chunk index is XORed with twice the row's number among the rows that
+// share a 16-byte bank column (every row when a row is a whole 256-byte bank sweep, every second when it is half
+// of one), which puts those 16 pieces on 16 different bank groups.
+template <int BN, int NW, int EB = 2>
 struct TileCopyKN {
-  static constexpr int kRows = RBK / 2;
-  static constexpr int kChunksPerRow = BN / 8;             // 16-byte chunks per k row
+  static constexpr int kRows = RBK / EB;
+  static constexpr int kChunksPerRow = BN * EB / 16;       // 16-byte chunks per k row
   static constexpr int kRowsPerInst = 64 / kChunksPerRow;  // k rows moved by one wave instruction
   static constexpr int kIters = kRows / kRowsPerInst / NW;
+  static constexpr int kRowsPerSweep = 256 / (BN * EB) > 0 ? 256 / (BN * EB) : 1;
   static_assert(kRowsPerInst >= 1 && kIters >= 1, "tile too small for this wave count");
+  static_assert(EB == 2 || ((7 / kRowsPerSweep) << 1) < kChunksPerRow, "the 8-bit swizzle needs that many chunks per row");
   __device__ static int row(int wave, int lane, int i) { return (i * NW + wave) * kRowsPerInst + lane / kChunksPerRow; }
+  __device__ static int swz8(int r) { return ((r & 7) / kRowsPerSweep) << 1; }
   __device__ static int col16(int lane, int r) {  // logical 16-byte chunk this lane fetches
     int pc16 = lane % kChunksPerRow;
-    int lc32 = (pc16 >> 1) ^ ((r & 3) << 1);
-    return lc32 * 2 + (pc16 & 1);
+    if constexpr (EB == 1) {
+      return pc16 ^ swz8(r);
+    } else {
+      int lc32 = (pc16 >> 1) ^ ((r & 3) << 1);
+      return lc32 * 2 + (pc16 & 1);
+    }
   }
 };
 
@@ -188,13 +201,14 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
   constexpr int NW = WM * WN, TM = BM / WM, TN = BN / WN, MT = TM / 32, NT = TN / 32;
   constexpr int A_BYTES = BM * RBK, B_BYTES = BN * RBK, STAGE = A_BYTES + B_BYTES;
   constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
-  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs a transpose read");
+  constexpr int EB = Cfg::kElemBytes == 1 ? 1 : 2;   // element size of a row-major B (16-bit or fp8)
   using CopyA = TileCopyK<BM, NW>;
   using CopyBk = TileCopyK<BN, NW>;
-  using CopyBn = TileCopyKN<BN, NW>;
+  using CopyBn = TileCopyKN<BN, NW, EB>;
   constexpr int ITA = CopyA::kIters;
   constexpr int ITB = B_KMAJOR ? CopyBk::kIters : CopyBn::kIters;
-  constexpr int KROWS = RBK / 2;  // k rows of a row-major 16-bit B tile
+  constexpr int KROWS = RBK / EB;  // k rows of a row-major B tile
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -218,9 +232,9 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
       srcB[i] = p.B + (int64_t)gr * p.ldb + CopyBk::chunk(lane, r) * 16;
     } else {
       int r = CopyBn::row(wave, lane, i);
-      int n = n0 + CopyBn::col16(lane, r) * 8;
-      n = n < p.N ? n : p.N - 8;  // N % 8 == 0 on this path: clamp whole chunks
-      srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
+      int nb = n0 * EB + CopyBn::col16(lane, r) * 16;   // byte column of the chunk
+      nb = nb < p.N * EB ? nb : p.N * EB - 16;          // rows of whole chunks on this path: clamp whole chunks
+      srcB[i] = p.B + (int64_t)r * p.ldb + nb;
     }
   }
   const int64_t stepA = RBK, stepB = B_KMAJOR ? (int64_t)RBK : KROWS * p.ldb;
@@ -270,8 +284,11 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
   // Per-lane LDS byte offsets of the MFMA operands inside one stage.
   //   K-major operand (A always, B when B_KMAJOR): lane reads row (l%32) and the 16-byte
   //   chunk(s) Cfg::chunk(ks, l/32, c), swizzled; 32-row sub-tiles add t * 32 * RBK.
-  //   Row-major B: transpose read, lane i of a 16-lane group q addresses k row
+  //   Row-major 16-bit B: transpose read, lane i of a 16-lane group q addresses k row
   //   16*ks + 8*(q/2) + i/4 (+4 for the second half) and 32-byte group (n/16) ^ 2*(k & 3).
+  //   Row-major fp8 B: four transpose reads of 8 k rows each - rows 16 (q/2) + {0, 8, 32, 40} + i/2, the K positions
+  //   of the two chunks (q/2, 2 + q/2) that the A operand of the same lane group holds - of the 16-byte chunk
+  //   (n/16) ^ swz8(k), half i & 1; k & 7 and with it the swizzle are the same for all four.
   const int l32 = lane & 31, g = lane >> 5;
   const int i16 = lane & 15, q = lane >> 4;
   unsigned offA[KS][NC], offB[KS][NC];
@@ -283,7 +300,14 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
       offB[ks][c] = A_BYTES + kmajor_off(wn * TN + l32, Cfg::chunk(ks, g, c));
     }
   unsigned offBn[NT];
-  {
+  if constexpr (EB == 1) {
+    int k = (q >> 1) * 16 + (i16 >> 1);
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+      int c16 = (wn * TN + t * 32) / 16 + (q & 1);
+      offBn[t] = A_BYTES + k * BN + ((c16 ^ CopyBn::swz8(k)) << 4) + (i16 & 1) * 8;
+    }
+  } else {
     // k row without the ks / +4 terms; (k & 3) is the same for every ks and both halves
     int k = (q >> 1) * 8 + (i16 >> 2);
 #pragma unroll
@@ -315,6 +339,16 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
       constexpr int t = decltype(T_)::value;
       if constexpr (B_KMAJOR) {
         f.b[t] = read_operand(base, offB[ks], std::integral_constant<int, t * 32 * RBK>{});
+      } else if constexpr (EB == 1) {
+        static_assert(KS == 1 && NC == 2, "the fp8 transpose read feeds one 64-byte sub-step");
+        i32x2 r0 = lds_read_tr8_b64<0>(base + offBn[t]);
+        i32x2 r1 = lds_read_tr8_b64<8 * BN>(base + offBn[t]);
+        i32x2 r2 = lds_read_tr8_b64<32 * BN>(base + offBn[t]);
+        i32x2 r3 = lds_read_tr8_b64<40 * BN>(base + offBn[t]);
+        i32x4 lo = __builtin_shufflevector(r0, r1, 0, 1, 2, 3);
+        i32x4 hi = __builtin_shufflevector(r2, r3, 0, 1, 2, 3);
+        i32x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        f.b[t] = __builtin_bit_cast(Operand, both);
       } else {
         constexpr int imm = ks * 16 * BN * 2;
         i32x2 lo = lds_read_tr16_b64<imm>(base + offBn[t]);
@@ -324,7 +358,7 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
       }
     });
   };
-  constexpr int kReadsPerStep = MT * NC + NT * (B_KMAJOR ? NC : 2);
+  constexpr int kReadsPerStep = MT * NC + NT * (B_KMAJOR ? NC : (EB == 1 ? 4 : 2));
   auto use_frags = [&](Frags& f) {
 #pragma unroll
     for (int t = 0; t < MT; t++) lds_use(f.a[t]);
@@ -601,7 +635,7 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
   constexpr int SC_BYTES = Cfg::kScaled ? (BM + BN) * 4 : 0;
   constexpr int STAGE = A_BYTES + B_BYTES + SC_BYTES;
   constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
-  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  static_assert(B_KMAJOR || (Cfg::kRowMajorB && Cfg::kElemBytes == 2), "row-major B: the 16-bit transpose read only in this kernel");
   static_assert(!Cfg::kScaled || (BM == 256 && BN == 256), "scale copies assume 64 rows per wave");
   using CopyA = TileCopyK<BM, NW>;
   using CopyBk = TileCopyK<BN, NW>;
@@ -878,7 +912,7 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
   constexpr int SPG = 4 * Cfg::kStepsPerScaleDword;
   constexpr int SC_SLOT = (BM + BN) * 16;
   constexpr int KS = Cfg::kSteps, NC = Cfg::kChunks;
-  static_assert(B_KMAJOR || Cfg::kRowMajorB, "row-major B needs the 16-bit transpose read");
+  static_assert(B_KMAJOR || (Cfg::kRowMajorB && Cfg::kElemBytes == 2), "row-major B: the 16-bit transpose read only in this kernel");
   using CopyA = TileCopyK<BM, NW>;
   using CopyBk = TileCopyK<BN, NW>;
   using CopyBn = TileCopyKN<BN, NW>;

@@ -18,6 +18,7 @@ struct CfgMxfp4 {
   static constexpr int kSteps = 2, kChunks = 1;
   static constexpr int kStepsPerScaleDword = 1;  // 4 scale bytes per row and K step
   static constexpr bool kRowMajorB = false, kScaled = true;
+  static constexpr int kElemBytes = 1;
   // lane group g reads scale blocks 2g, 2g+1 of the step (16 bytes = 32 elements each), one per sub-step
   __device__ static constexpr int chunk(int ks, int g, int) { return g * 2 + ks; }
   // the step has 4 scale bytes per row; move bytes 2g, 2g+1 to positions 0, 1 (selector = ks)
@@ -44,6 +45,7 @@ struct CfgMxfp8 {
   static constexpr int kSteps = 1, kChunks = 2;
   static constexpr int kStepsPerScaleDword = 2;  // 2 scale bytes per row and K step
   static constexpr bool kRowMajorB = false, kScaled = true;
+  static constexpr int kElemBytes = 1;
   // register half c is scale block c of the step; lane group g holds its 16-byte half g
   __device__ static constexpr int chunk(int, int g, int c) { return 2 * c + g; }
   // the step has 2 scale bytes per row; lane group g supplies the scale of block g in byte 0

@@ -134,10 +134,11 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
             b = torch.nn.functional.pad(as_bytes(b), (0, 0, 0, pad)).view(b.dtype)
         K += pad        # (the launch metadata below keeps the caller's K)
     if (in_dt in (_lib.F8E4M3, _lib.F8E5M2) and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
-            and K % 16 == 0 and M * N * K >= 1 << 24):
-        # fp8 MFMAs want both operands K-contiguous: a row-major fp8 B is put into that layout first, as the
-        # reference does on the host for its fp8 case ("pre-transpose b for efficiency", 03:378-380) - one
-        # pass over B instead of the strided kernel (the C ABI itself runs whatever layout it is given)
+            and (N % 16 != 0 or b.stride(0) % 16 != 0 or b.data_ptr() % 16 != 0) and K % 16 == 0 and M * N * K >= 1 << 24):
+        # A row-major fp8 B runs on the fp8 MFMAs inside the C ABI when its rows are whole 16-byte chunks.  One that is
+        # not (N or the pitch not a multiple of 16) would take the strided kernel: it is put K-major first, as the
+        # reference does on the host for its fp8 case ("pre-transpose b for efficiency", 03:378-380) - K-major rows
+        # are K bytes long, which are whole chunks here.
         b = b.t().contiguous().t()
     pa, keep_a = _scale_ptr(a_scale, device)
     pb, keep_b = _scale_ptr(b_scale, device)
