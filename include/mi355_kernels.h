@@ -265,7 +265,8 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
  * fp8 forward (dtype MI355_F8E5M2 as in the reference's fp8 benchmark, :609-614, or MI355_F8E4M3):
  * q, k and o as above, v transposed in memory (stride 1 along N_CTX, a multiple of 16 along D:
  * what `v.permute(0,1,3,2).contiguous().permute(0,1,3,2)` yields); P is rounded to the fp8 type
- * before the second product (:66-67) and o is written in the fp8 type.  There is no fp8 backward.
+ * before the second product (:66-67) and o is written in the fp8 type; the same five head dims (16 and 32: rows
+ * of D bytes, and D rows of V^T).  There is no fp8 backward.
  */
 int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* Mlse,
                    int Z, int H, int N_CTX, int D,

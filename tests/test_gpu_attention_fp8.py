@@ -38,7 +38,8 @@ def _code_distance(got_codes, ref_vals, fmt):
 
 @pytest.mark.parametrize("fmt", ["e5m2", "e4m3"])
 @pytest.mark.parametrize("causal", [True, False])
-@pytest.mark.parametrize("shape", [(1, 2, 128, 64), (1, 2, 256, 128), (2, 3, 512, 128), (1, 1, 384, 64), (1, 2, 384, 128)])
+@pytest.mark.parametrize("shape", [(1, 2, 128, 64), (1, 2, 256, 128), (2, 3, 512, 128), (1, 1, 384, 64), (1, 2, 384, 128),
+                                   (1, 2, 256, 16), (2, 2, 384, 32), (1, 2, 256, 256), (2, 1, 384, 256)])   # (all five head dims of 06:447)
 def test_fp8_forward_against_oracle(gpu, fmt, causal, shape):
     (q, k, v), (tq, tk, tv) = _fp8_inputs(sum(shape), shape, fmt, gpu)
     sm_scale = shape[-1] ** -0.5
@@ -74,11 +75,12 @@ def test_fp8_forward_eight_wave_variant_gives_the_same_codes(gpu, causal, monkey
     assert np.array_equal(base, wide)
 
 
-def test_fp8_forward_exact_case_uniform_attention(gpu):
+@pytest.mark.parametrize("D", [16, 32, 64, 128, 256])
+def test_fp8_forward_exact_case_uniform_attention(gpu, D):
     # q = 0: every score is 0, P = 1 exactly in any format, O = mean over keys of V (causal: running mean).
     # With V constant along the keys of each column the mean is that constant: exact in fp8.
-    Z, H, N, D = 1, 2, 256, 128
-    rng = np.random.default_rng(0)
+    Z, H, N = 1, 2, 256
+    rng = np.random.default_rng(D)
     col = formats.fp8_table("e5m2")[formats.encode_fp8(rng.normal(0, 1, (Z, H, 1, D)).astype(np.float32), "e5m2")]
     v = np.broadcast_to(col, (Z, H, N, D)).astype(np.float32)
     tq = torch.zeros(Z, H, N, D, device=gpu, dtype=torch.float8_e5m2)

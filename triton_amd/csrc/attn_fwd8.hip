@@ -1,5 +1,6 @@
-// Fused flash-attention forward for fp8 inputs (e5m2 as in the reference, or e4m3fn), head_dim 128
-// or 64: q, k [Z,H,N,D] with D contiguous, v with N contiguous (the reference transposes V in
+// Fused flash-attention forward for fp8 inputs (e5m2 as in the reference, or e4m3fn), head_dim 256, 128
+// or 64, and 32 or 16 as a padded form of 64 (python/tutorials/06-fused-attention.py:447 admits these five for every
+// type): q, k [Z,H,N,D] with D contiguous, v with N contiguous (the reference transposes V in
 // memory for fp8, python/tutorials/06-fused-attention.py:609-614 and :127-135), o in the input
 // type, M in fp32.  Same algorithm and rounding points as the 16-bit kernel (attn_fwd.hip): S in
 // fp32 from an fp8 x fp8 MFMA, softmax in fp32 in the exp2 domain, P rounded to the fp8 type before
@@ -15,6 +16,7 @@
 //     64-bank LDS and these access patterns.
 #include "common.h"
 #include "launch.h"
+#include "attn_tiles.h"
 
 namespace mi355 {
 
@@ -27,8 +29,13 @@ __device__ __forceinline__ f32x16 mfma_f8(i32x8 a, i32x8 b, f32x16 c) {
 #endif
 }
 
-template <int FMT, int D, int NW>
-__global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd8_kernel(AttnArgs p) {
+// PAD (D = 64 only): the tensors hold p.d_real = 16 or 32 bytes per row of q, k, o and that many rows of V^T; the
+// missing columns are zeros that never exist in memory - the Q fragments are zero-filled in registers, the K / V^T
+// tiles in LDS are zeroed once and only the chunks present are ever loaded, and only the first d_real columns of O are
+// stored.  Zero columns add nothing to the scores and give zero columns of O: what a HEAD_DIM d_real kernel computes.
+template <int FMT, int D, int NW, bool PAD = false>
+__global__ __launch_bounds__(NW * 64, NW == 4 && D <= 128 ? 2 : 1) void attn_fwd8_kernel(AttnArgs p) {
+  static_assert(!PAD || D == 64, "the padded form is the 64-column one");
   constexpr int BM = NW * 32, BN = 64;
   constexpr int KSQ = D / 64;          // MFMA k-steps of S^T
   constexpr int DT = D / 32;           // 32-row tiles of O^T
@@ -67,41 +74,54 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd8_kernel(Att
     const char* src = qbase + (int64_t)r * qpitch + g * 32;
 #pragma unroll
     for (int ks = 0; ks < KSQ; ks++) {
-      i32x4 lo = *(const i32x4*)(src + ks * 64), hi = *(const i32x4*)(src + ks * 64 + 16);
+      i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+      if (!PAD || ks * 64 + g * 32 < p.d_real) lo = *(const i32x4*)(src + ks * 64);
+      if (!PAD || ks * 64 + g * 32 + 16 < p.d_real) hi = *(const i32x4*)(src + ks * 64 + 16);
       qf[ks] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     }
   }
 
-  // swizzles: K rows of D bytes (D = 128: two rows per 256-byte bank sweep), V^T rows of 64 bytes
+  // swizzles: K rows of D bytes (D = 128: two rows per 256-byte bank sweep, D = 256: one), V^T rows of 64 bytes
   // (a ds_read_b128 is served 16 lanes at a time; with the permuted key order those are key rows
   //  0-7 and 16-23, or 8-15 and 24-31, of a 32-row tile - the XOR value must separate exactly those)
   auto kswz8 = [](int row) {
-    return D == 128 ? (((row >> 1) & 3) | (((row >> 4) & 1) << 2)) : (((row >> 2) & 1) | (((row >> 4) & 1) << 1));
+    return D == 256 ? ((row & 7) | (((row >> 4) & 1) << 3))
+         : D == 128 ? (((row >> 1) & 3) | (((row >> 4) & 1) << 2)) : (((row >> 2) & 1) | (((row >> 4) & 1) << 1));
   };
   auto vswz8 = [](int row) { return (row >> 2) & 3; };
 
   // direct loads: one wave instruction moves 1 KiB = 1024/D K rows or 16 V^T rows
   // (scalar tile base + 32-bit lane offset: the host bounds the row pitches)
   unsigned offK[KINST], offV[VINST];
+  bool presentK[KINST], presentV[VINST];
 #pragma unroll
   for (int i = 0; i < KINST; i++) {
     const int r = (i * NW + wave) * (1024 / D) + lane / KCH;
-    offK[i] = (unsigned)(r * kpitch) + (((lane % KCH) ^ kswz8(r)) << 4);
+    const int chunk = (lane % KCH) ^ kswz8(r);
+    offK[i] = (unsigned)(r * kpitch) + (chunk << 4);
+    presentK[i] = !PAD || chunk * 16 < p.d_real;
   }
 #pragma unroll
   for (int i = 0; i < VINST; i++) {
     const int r = (i * NW + wave) * 16 + lane / 4;   // d row
     offV[i] = (unsigned)(r * vpitch) + (((lane % 4) ^ vswz8(r)) << 4);
+    presentV[i] = !PAD || r < p.d_real;
   }
   const unsigned lds_base = lds_addr(lds);
+  if constexpr (PAD) {
+    lds_zero(lds, 2 * STAGE, tid, NW * 64);
+    __syncthreads();
+  }
   auto issue_kv = [&](int j, int stage) {
     const unsigned kd = lds_base + stage * STAGE, vd = kd + KTILE;
     const char* ksrc = kbase + (int64_t)j * BN * kpitch;
     const char* vsrc = vbase + (int64_t)j * BN;
 #pragma unroll
-    for (int i = 0; i < KINST; i++) async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
+    for (int i = 0; i < KINST; i++)
+      if (presentK[i]) async_copy16_sbase(ksrc, offK[i], kd + (i * NW + wave) * 1024);
 #pragma unroll
-    for (int i = 0; i < VINST; i++) async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
+    for (int i = 0; i < VINST; i++)
+      if (presentV[i]) async_copy16_sbase(vsrc, offV[i], vd + (i * NW + wave) * 1024);
   };
 
   // per-lane LDS offsets.  K operand of tile row l32 = 8a + 4b + e is key row 16b + 4a + e
@@ -262,32 +282,34 @@ __global__ __launch_bounds__(NW * 64, NW == 4 ? 2 : 1) void attn_fwd8_kernel(Att
           w[rg] = pack4_fp8<FMT>(oacc[c][rg * 4] * inv, oacc[c][rg * 4 + 1] * inv, oacc[c][rg * 4 + 2] * inv, oacc[c][rg * 4 + 3] * inv);
         swap32_regs(w[0], w[2]);
         swap32_regs(w[1], w[3]);
-        *(i32x4*)(dst + c * 32) = i32x4{w[0], w[2], w[1], w[3]};
+        if (!PAD || c * 32 + g * 16 < p.d_real) *(i32x4*)(dst + c * 32) = i32x4{w[0], w[2], w[1], w[3]};
       }
     }
   }
 }
 
-template <int FMT, int D, int NW>
+template <int FMT, int D, int NW, bool PAD = false>
 static int launch_fwd8(const AttnArgs& p, hipStream_t stream) {
   constexpr int BM = NW * 32;
   constexpr int smem = 2 * 2 * 64 * D;
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd8_kernel<FMT, D, NW>,
+    hipError_t e = hipFuncSetAttribute((const void*)attn_fwd8_kernel<FMT, D, NW, PAD>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int nqb = (p.N + BM - 1) / BM;
-  attn_fwd8_kernel<FMT, D, NW><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
+  attn_fwd8_kernel<FMT, D, NW, PAD><<<dim3(nqb * p.Z * p.H), dim3(NW * 64), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 template <int FMT>
 static int launch_fwd8_fmt(const AttnArgs& p, hipStream_t stream) {
   // variant 2: eight waves (256 query rows per K/V stream), head_dim 128 only
+  if (p.D == 256) return launch_fwd8<FMT, 256, 4>(p, stream);   // (one workgroup per CU: 128 accumulator registers per lane)
   if (p.D == 128) return p.variant == 2 ? launch_fwd8<FMT, 128, 8>(p, stream) : launch_fwd8<FMT, 128, 4>(p, stream);
+  if (p.d_real < p.D) return launch_fwd8<FMT, 64, 4, true>(p, stream);    // head dims 16 / 32
   return launch_fwd8<FMT, 64, 4>(p, stream);
 }
 

@@ -466,12 +466,12 @@ int mi355_dequant(const uint8_t* codes, float* out, int64_t n, int fmt, void* st
   return dequant_launch(codes, out, n, fmt, (hipStream_t)stream_);
 }
 
-static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype, bool allow_256 = false) {
+static int attn_common(AttnArgs& p, int Z, int H, int N_CTX, int D, int dtype) {
   if (Z <= 0 || H <= 0 || N_CTX <= 0) return MI355_EINVAL;
   if (dtype != MI355_F16 && dtype != MI355_BF16) return MI355_EDTYPE;
-  // head_dim 256 and the padded forms of head dims 16 / 32: 16-bit forward and backward (not the fp8 forward)
-  const bool small = allow_256 && (D == 16 || D == 32);
-  if (D != 64 && D != 128 && !(allow_256 && D == 256) && !small) return MI355_ESHAPE;
+  // head_dim 256 and the padded forms of head dims 16 / 32: the forward kernels of every type and the backward
+  const bool small = D == 16 || D == 32;
+  if (D != 64 && D != 128 && D != 256 && !small) return MI355_ESHAPE;
   if (N_CTX % 128 != 0) return MI355_ESHAPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
   // 16 / 32: the 64-column kernels, which pad with zeros on the fly (loads, LDS tiles and stores know d_real)
@@ -507,7 +507,7 @@ int mi355_attn_fwd(const void* q, const void* k, const void* v, void* o, float* 
     p.variant = knob(knobs().attn_fwd_variant, 1);  // fp8: four waves, two workgroups per CU (eight waves measured 6-12 % slower)
     return attn_fwd8_launch(p, dtype == MI355_F8E5M2, (hipStream_t)stream_);
   }
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
   if (rc) return rc;
   if (!copy_strides(sq, p.sq) || !copy_strides(sk, p.sk) || !copy_strides(sv, p.sv) || !copy_strides(so, p.so))
     return MI355_EINVAL;
@@ -530,7 +530,7 @@ int mi355_attn_bwd_preprocess(const void* o, const void* d_o, float* delta,
                               int Z, int H, int N_CTX, int D, const int64_t* stride, int dtype, void* stream_) {
   if (!o || !d_o || !delta) return MI355_EINVAL;
   AttnArgs p{};
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
   if (rc) return rc;
   if (!copy_strides(stride, p.so)) return MI355_EINVAL;
   if (!attn_stride_ok(p.so, o, D) || !aligned(d_o, 16)) return MI355_ESTRIDE;
@@ -546,7 +546,7 @@ int mi355_attn_bwd(const void* q, const void* k, const void* v, const void* d_o,
                    float sm_scale, int causal, int dtype, void* stream_) {
   if (!q || !k || !v || !d_o || !Mlse || !delta || !dq || !dk || !dv) return MI355_EINVAL;
   AttnArgs p{};
-  int rc = attn_common(p, Z, H, N_CTX, D, dtype, true);
+  int rc = attn_common(p, Z, H, N_CTX, D, dtype);
   if (rc) return rc;
   if (!copy_strides(stride, p.sq)) return MI355_EINVAL;
   if (!attn_stride_ok(p.sq, q, D) || !aligned(k, 16) || !aligned(v, 16) || !aligned(d_o, 16) ||
