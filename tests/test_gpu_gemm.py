@@ -493,6 +493,30 @@ def test_four_wave_kernel_k_tails_are_bit_exact(gpu, monkeypatch, dtype, layout,
         assert bits_equal(own, gemm.matmul_closed_form(a, b, out_dtype=dtype)), (K, dtype, layout, programs, "own type")
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_four_wave_fp8_kernel_k_tails_are_bit_exact(gpu, monkeypatch, fmt, tdt, programs):
+    # K bytes not a multiple of 256 in the four-wave fp8 kernel: what is left behind the last pair of 128-byte K steps
+    # (16 .. 240 bytes) follows as one or two steps whose fragments come straight from global memory, zeros beyond K.
+    # Every class of tail (one and two steps; a lane group's first chunk only, both, neither), one and several tiles
+    # per program (the tail runs while the stages and half of the fragment registers already hold the next tile's
+    # first K steps), every epilogue that has the form (fp32: general; fp16, bf16: lean).  Integer data: exact sums.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(fmt))
+    M, N = 768, 512
+    for K in (272, 320, 336, 384, 400, 448, 496, 1008, 2064):
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+        ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
+        tb = torch.from_numpy(formats.encode_fp8(b, fmt)).to(gpu).view(tdt).t()          # K-major B
+        want = a.astype(np.float64) @ b.astype(np.float64).T
+        assert np.array_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), want), (K, fmt, programs)
+        for out, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=out))
+            assert bits_equal(got, gemm.matmul_closed_form(a, b.T, out_dtype=name)), (K, fmt, programs, name)
+
+
 @pytest.mark.parametrize("layout", ["row_major_b", "k_major_b"])
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 def test_uneven_k_8192x8192x8176(gpu, dtype, layout):

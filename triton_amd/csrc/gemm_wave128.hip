@@ -479,6 +479,17 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_grouped_kernel(GroupedArg
 // places the two halves directly in the eight-register operand and waits for each fragment just
 // before its first use); the direct global->LDS loads stay invisible to its bookkeeping.
 // ---------------------------------------------------------------------------------------------
+// The tail's fragments come from ordinary loads and moves that the compiler schedules; the MFMAs that read them are
+// assembly it cannot see into: everything that writes these registers has completed behind this statement (the values
+// pass through it) and two idle cycles separate the last such write from the first MFMA.
+template <int NA, int NB>
+__device__ __forceinline__ void settle_operands(i32x8 (&a)[NA], i32x8 (&b)[NB]) {
+#if MI355_DEVICE_PASS
+  static_assert(NA == 4 && NB == 8, "four A fragments and the first four of the B set");
+  asm volatile("s_nop 1" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3]), "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+#endif
+}
+
 template <int FMT>
 __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4& c) {
 #if MI355_DEVICE_PASS
@@ -488,7 +499,12 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 }
 
 // EPI: 0 = general epilogue, 2 = with the addend, 3 / 4 = lean epilogue writing fp16 / bf16
-template <int FMT, int EPI>
+// TAIL: K bytes need not be a multiple of 256 (of 16 still): the main loop does the whole pairs of K steps, and what is
+// left of each row (16 .. 240 bytes, the same for every tile) follows as one or two K steps whose fragments every lane
+// loads straight from global memory - the same two chunks per 128-byte step as from LDS, zeros beyond K, the masked
+// tail of the reference's loop (python/tutorials/03-matrix-multiplication.py:297-298) - into the fragment registers
+// that the pipeline has free at that point (it already holds the next tile's first B and A fragments in the others).
+template <int FMT, int EPI, bool TAIL = false>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -507,7 +523,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
-  const int nk = p.k_bytes / ROWB;
+  const int nk = TAIL ? p.k_bytes / (2 * ROWB) * 2 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
   asm volatile("" : "+s"(nk_last));
 
@@ -655,6 +671,43 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       step(I1{}, I1{}, touch_a(), touch_b()); advance();
       if (kt + 2 >= nk_last) mfma_retire();
     }
+    if constexpr (TAIL) {
+      // (free here: a1 and the B set 1 - the last step read the next tile's first fragments into a0 and the B set 0)
+      const int k_main = nk * ROWB, tail = p.k_bytes - k_main;
+      int tm = pm * BM + wm * 128, tn = pn * BN + wn * 128, tl = l16, tk = kg;
+      asm volatile("" : "+s"(tm), "+s"(tn), "+v"(tl), "+v"(tk));   // (keeps this address arithmetic out of the K loop)
+      // a scalar base per fragment and one 32-bit lane offset per operand (gemm_wave128_f8_ok bounds 128 rows plus K)
+      const char* const tA = p.A + (int64_t)tm * p.lda + k_main;
+      const char* const tB = p.B + (int64_t)tn * p.ldb + k_main;
+      const unsigned offA = (unsigned)tl * (unsigned)p.lda + tk * 16, offB = (unsigned)tl * (unsigned)p.ldb + tk * 16;
+      for (int h = 0; h * ROWB < tail; h++) {
+        const bool lo_ok = h * ROWB + tk * 16 < tail, hi_ok = h * ROWB + 64 + tk * 16 < tail;
+        auto frag = [&](const char* src, unsigned off) {
+          i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+          if (lo_ok) lo = *(const i32x4*)(src + h * ROWB + (uint64_t)off);
+          if (hi_ok) hi = *(const i32x4*)(src + h * ROWB + 64 + (uint64_t)off);
+          return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        // (a quarter of the wave's tile at a time - four B and four A fragments: with all eight B fragments at once the
+        // compiler spills lane offsets of the K loop across the tail and reloads them in front of the loop, behind
+        // the wait there, so that their first use inside the loop would drain every load, in every step)
+        static_for<4>([&](auto Q_) {
+          constexpr int bh = decltype(Q_)::value / 2, ah = decltype(Q_)::value % 2;
+          if constexpr (ah == 0) {
+#pragma unroll
+            for (int t = 0; t < MH; t++) b[1][t] = frag(tB + (int64_t)(bh * MH + t) * 16 * p.ldb, offB);
+          }
+#pragma unroll
+          for (int t = 0; t < MH; t++) a1[t] = frag(tA + (int64_t)(ah * MH + t) * 16 * p.lda, offA);
+          settle_operands(a1, b[1]);
+          static_for<MH * MH>([&](auto N_) {
+            constexpr int n = decltype(N_)::value, i = n / MH, j = n % MH;
+            mfma16_f8<FMT>(b[1][j], a1[i], acc[ah * MH + i][bh * MH + j]);
+          });
+        });
+        mfma_retire();   // (inside the loop's block, like the main loop's: see mfma_retire)
+      }
+    }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
@@ -670,27 +723,41 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #endif
 }
 
-template <int FMT, int EPI>
+template <int FMT, int EPI, bool TAIL = false>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 1024;   // (two stages and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_f8_kernel<FMT, EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_f8_kernel<FMT, EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
+  if (p.k_bytes % 256 != 0) {   // (gemm_wave128_f8_ok: no addend then)
+    const int lean = lean_epilogue_type(p);
+    if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3, true>(p, stream) : launch_wave128_f8<0, 3, true>(p, stream);
+    if (lean == 2) return e5m2 ? launch_wave128_f8<1, 4, true>(p, stream) : launch_wave128_f8<0, 4, true>(p, stream);
+    return e5m2 ? launch_wave128_f8<1, 0, true>(p, stream) : launch_wave128_f8<0, 0, true>(p, stream);
+  }
   if (p.aux) return e5m2 ? launch_wave128_f8<1, 2>(p, stream) : launch_wave128_f8<0, 2>(p, stream);
   const int lean = lean_epilogue_type(p);
   if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3>(p, stream) : launch_wave128_f8<0, 3>(p, stream);
   if (lean == 2) return e5m2 ? launch_wave128_f8<1, 4>(p, stream) : launch_wave128_f8<0, 4>(p, stream);
   return e5m2 ? launch_wave128_f8<1, 0>(p, stream) : launch_wave128_f8<0, 0>(p, stream);
+}
+
+// fp8 (K-major B): whole tiles, at least one pair of 128-byte K steps; what is left behind the last pair is the TAIL
+// form's, which exists without the addend
+bool gemm_wave128_f8_ok(const GemmArgs& p) {
+  if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 16 == 0 && p.k_bytes >= 256)) return false;
+  if (p.k_bytes % 256 != 0 && p.aux) return false;
+  return p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
 }
 
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
