@@ -54,6 +54,43 @@ def test_mxfp4_exact_sums_are_bitwise(gpu, shape):
     assert bits_equal(_run(gpu, a, sa, b, sb, "mxfp4", torch.bfloat16), formats.round_bf16(ref32))
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
+def test_four_wave_kernels_k_tails_are_bit_exact(gpu, monkeypatch, fmt, programs):
+    # K not a multiple of 1024 in the four-wave kernels: what is left behind the last whole group of K steps follows in
+    # steps whose fragments and scale bytes come straight from global memory, zeros beyond K.  Every class of tail
+    # (one block, part of a step, whole steps, all but one block), one and several tiles per program (the tail runs
+    # while the stages and half of the registers hold the next tile's first steps), each epilogue (fp32: general;
+    # bf16, fp16: lean).  Exact data (fp4 values, or small integers as e4m3, with scales 1/2, 1, 2: every partial sum
+    # is exact in fp32), so the results carry the oracle's bits.  The scale rows are slices of wider ones: the
+    # 16-byte scale loads of these kernels need a pitch that is a multiple of 16.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(fmt))
+    M, N = 768, 512
+    t = lambda x: torch.from_numpy(x).to(gpu)
+    for K in (1024 + 32, 1024 + 96, 1024 + 128, 1024 + 320, 1536, 2048 + 480, 1024 + 992, 3072 + 64):
+        if fmt == "mxfp4":
+            a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
+        else:
+            a = formats.encode_fp8(rng.integers(-4, 5, size=(M, K)).astype(np.float32), "e4m3")
+            b = formats.encode_fp8(rng.integers(-4, 5, size=(N, K)).astype(np.float32), "e4m3")
+            sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+            sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
+        pitch = -(-(K // 32) // 16) * 16
+        wa = torch.full((M, pitch), 0xFF, dtype=torch.uint8, device=gpu)      # (NaN scales beyond K: never read)
+        wb = torch.full((N, pitch), 0xFF, dtype=torch.uint8, device=gpu)
+        wa[:, :K // 32] = t(sa)
+        wb[:, :K // 32] = t(sb)
+        ta, tb = t(a), t(b)
+        if fmt == "mxfp8":
+            ta, tb = ta.view(torch.float8_e4m3fn), tb.view(torch.float8_e4m3fn)
+        for out, rnd in ((torch.float32, lambda x: x), (torch.bfloat16, formats.round_bf16), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+            got = to_np(triton_amd.mx_matmul(ta, wa[:, :K // 32], tb, wb[:, :K // 32], fmt, out_dtype=out))
+            assert bits_equal(got, rnd(ref32)), (fmt, K, programs, out)
+
+
 def test_scale_blocks_are_applied_per_row_and_per_32_elements(gpu):
     # all-ones data; one scale byte raised: exactly one row (or column) of C changes by 32 * (2^d - 1)
     M = N = 128; K = 512

@@ -433,11 +433,22 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   const int cus = device_info().cus > 0 ? device_info().cus : 256;
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
   int tile = (tiles256 * 2 >= cus) ? (tiles256 % cus == 0 ? 5 : 4) : 1;
-  // MXFP4 with whole 256x256 tiles, K a multiple of 1024 and at least half a round of tiles: four waves of
+  // MXFP4 with whole 256x256 tiles, K at least 1024 and at least half a round of tiles: four waves of
   // scaled 16x16x128 MFMAs (8192^3: 4000-4050 vs 3340-3640 TFLOP/s for the persistent eight-wave kernel)
-  if (fmt == MI355_MXFP4 && tiles256 * 2 >= cus && gemm_wave128_mxfp4_ok(p)) tile = 6;
+  // K beyond the last whole group of K steps (four 128-byte steps for MXFP4, eight for MXFP8) is those kernels' tail
+  // form, whose steps are not pipelined: one costs about 3.5 (MXFP4) / 7 (MXFP8) steps of the main loop (8192 x 8192 x
+  // 8704: MXFP4 3890 vs 3540 TFLOP/s for the eight-wave kernel, MXFP8 2110 vs 2100; x 4608: 3230 vs 3280 and 1740 vs
+  // 2040).  It is chosen where the tail is short against the main loop - and wherever the eight-wave kernels cannot take
+  // the product at all (K bytes not a multiple of 64: 8192 x 8192 x 8224 ran the one-thread-per-output kernel, 700 ms).
+  auto tail_pays = [&](int group_bytes, int cost) {
+    const int tail = p.k_bytes % group_bytes;
+    if (tail == 0) return true;
+    const bool eight_wave_runs = p.k_bytes % 64 == 0 && lds_a % 4 == 0 && lds_b % 4 == 0 && aligned(sA, 4) && aligned(sB, 4);
+    return !eight_wave_runs || (int64_t)((tail + 127) / 128) * cost <= (int64_t)(p.k_bytes - tail) / 128;
+  };
+  if (fmt == MI355_MXFP4 && tiles256 * 2 >= cus && gemm_wave128_mxfp4_ok(p) && tail_pays(512, 9)) tile = 6;
   // (MXFP8 likewise: 2530-2570 vs 2110-2240)
-  if (fmt == MI355_MXFP8 && tiles256 * 2 >= cus && gemm_wave128_mxfp8_ok(p)) tile = 6;
+  if (fmt == MI355_MXFP8 && tiles256 * 2 >= cus && gemm_wave128_mxfp8_ok(p) && tail_pays(1024, 21)) tile = 6;
   tile = knob(knobs().tile, tile);
   p.num_programs = knob(knobs().programs, cus);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);

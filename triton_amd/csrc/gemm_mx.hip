@@ -98,6 +98,10 @@ __global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4
 }
 
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
+  // 6: four waves of scaled 16x16x128 MFMAs (whole 256x256 tiles, K at least 1024, any multiple of the scale block:
+  // what is left behind the last whole group of K steps is the tail form's)
+  if (tile == 6 && fmt == 0 && gemm_wave128_mxfp4_ok(p)) return gemm_wave128_mxfp4_launch(p, stream);
+  if (tile == 6 && fmt != 0 && gemm_wave128_mxfp8_ok(p)) return gemm_wave128_mxfp8_launch(p, stream);
   const bool whole_tiles = p.k_bytes % RBK == 0;
   const bool scales_aligned = p.lds_a % 4 == 0 && p.lds_b % 4 == 0 && ((uintptr_t)p.sA % 4) == 0 && ((uintptr_t)p.sB % 4) == 0;
   if (!whole_tiles || !scales_aligned || tile < 0) {
@@ -105,9 +109,6 @@ int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
     mx_gemm_simple_kernel<<<grid, dim3(256), 0, stream>>>(p, fmt == 0);
     return (int)hipGetLastError();
   }
-  // 6: MXFP4 on four waves of scaled 16x16x128 MFMAs (whole tiles, K a multiple of 1024)
-  if (tile == 6 && fmt == 0 && gemm_wave128_mxfp4_ok(p)) return gemm_wave128_mxfp4_launch(p, stream);
-  if (tile == 6 && fmt != 0 && gemm_wave128_mxfp8_ok(p)) return gemm_wave128_mxfp8_launch(p, stream);
   return fmt == 0 ? launch_gemm_tile<CfgMxfp4, true>(p, tile, stream) : launch_gemm_tile<CfgMxfp8, true>(p, tile, stream);
 }
 

@@ -13,6 +13,27 @@ __device__ __forceinline__ void mfma16_mxfp8(const i32x8& a, const i32x8& b, f32
                : "+a"(c) : "v"(a), "v"(b), "v"(sa), "v"(sb));
 #endif
 }
+// The tails' fragments and scales come from ordinary loads and moves that the compiler schedules; the MFMAs that read
+// them are assembly it cannot see into: everything that writes these registers has completed behind this statement (the
+// values pass through it) and two idle cycles separate the last such write from the first MFMA.
+template <typename R>
+__device__ __forceinline__ void settle_one(R& r) {
+#if MI355_DEVICE_PASS
+  asm volatile("" : "+v"(r));
+#endif
+}
+template <typename... R>
+__device__ __forceinline__ void settle_pass(R&... r) {
+  (settle_one(r), ...);
+}
+template <typename... R>
+__device__ __forceinline__ void settle_tail(R&... r) {
+#if MI355_DEVICE_PASS
+  settle_pass(r...);
+  asm volatile("s_nop 1" ::: "memory");
+  settle_pass(r...);
+#endif
+}
 #ifndef MXFP8_CHUNK
 #define MXFP8_CHUNK(kg, c) ((kg) + 4 * (c))
 #endif
@@ -21,7 +42,11 @@ __device__ __forceinline__ void mfma16_mxfp8(const i32x8& a, const i32x8& b, f32
 // 128 elements = four scale blocks, the scales travel 16 bytes per row (four K steps) per direct load into a
 // two-slot LDS ring like those of the MXFP4 kernel below.
 // EPI: 0 = general epilogue, 3 / 4 = lean epilogue (gemm_epilogue16_lean) writing fp16 / bf16
-template <int EPI>
+// TAIL: K need not be a multiple of 1024 (of 32 still, the scale block): the main loop does the whole groups of eight K
+// steps, and what is left of each row (32 .. 992 bytes, the same for every tile) follows in K steps whose fragments and
+// scale bytes every lane loads straight from global memory - zeros (and the scale 1) beyond K - into the registers that
+// the pipeline has free at that point, a quarter of the wave's tile at a time.
+template <int EPI, bool TAIL = false>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -41,7 +66,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
-  const int nk = p.k_bytes / ROWB;
+  const int nk = TAIL ? p.k_bytes / (8 * ROWB) * 8 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
   asm volatile("" : "+s"(nk_last));
 
@@ -225,6 +250,60 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       static_for<8>([&](auto U_) { step(U_, fk); advance(); });
       if (kt + 8 >= nk_last) mfma_retire();
     }
+    if constexpr (TAIL) {
+      // (free here: a1, the B set 1 and the scale set 1 - the last step read the next tile's first fragments and scales
+      // into the others)
+      const int k_main = nk * ROWB, tail = p.k_bytes - k_main;
+      int tm = pm * BM + wm * 128, tn = pn * BN + wn * 128, tl = l16, tk = kg;
+      asm volatile("" : "+s"(tm), "+s"(tn), "+v"(tl), "+v"(tk));   // (keeps this address arithmetic out of the K loop)
+      // a scalar base per fragment and one 32-bit lane offset per operand (gemm_wave128_mxfp8_ok bounds them)
+      const char* const tA = p.A + (int64_t)tm * p.lda + k_main;
+      const char* const tB = p.B + (int64_t)tn * p.ldb + k_main;
+      const uint8_t* const tSA = p.sA + (int64_t)tm * p.lds_a + k_main / 32;
+      const uint8_t* const tSB = p.sB + (int64_t)tn * p.lds_b + k_main / 32;
+      unsigned offA = (unsigned)tl * (unsigned)p.lda + tk * 16, offB = (unsigned)tl * (unsigned)p.ldb + tk * 16;
+      unsigned offSA = (unsigned)tl * (unsigned)p.lds_a + tk, offSB = (unsigned)tl * (unsigned)p.lds_b + tk;
+      for (int h = 0; h * ROWB < tail; h++) {
+        // chunk tk (low registers) and chunk 4 + tk (high registers) of the step; the scale of its block tk
+        const bool lo_ok = h * ROWB + tk * 16 < tail, hi_ok = h * ROWB + 64 + tk * 16 < tail, sc_ok = h * ROWB + tk * 32 < tail;
+        auto frag = [&](const char* src, unsigned off) {
+          i32x4 lo = {0, 0, 0, 0}, hi = {0, 0, 0, 0};
+          if (lo_ok) lo = *(const i32x4*)(src + h * ROWB + (uint64_t)off);
+          if (hi_ok) hi = *(const i32x4*)(src + h * ROWB + 64 + (uint64_t)off);
+          return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        auto scale = [&](const uint8_t* src, unsigned off) {
+          int v = 127;   // (2^0: multiplies zeros)
+          if (sc_ok) v = src[h * 4 + (uint64_t)off];
+          return v;
+        };
+        static_for<4>([&](auto Q_) {
+          constexpr int bh = decltype(Q_)::value / 2, ah = decltype(Q_)::value % 2;
+          // (the offsets pass through an assembly statement, which stays behind the MFMAs of the quarter before: the
+          // compiler cannot start this quarter's loads earlier and so needs no second set of registers for them)
+          asm volatile("" : "+v"(offA), "+v"(offB), "+v"(offSA), "+v"(offSB));
+          if constexpr (ah == 0) {
+#pragma unroll
+            for (int t = 0; t < MH; t++) {
+              b[1][t] = frag(tB + (int64_t)(bh * MH + t) * 16 * p.ldb, offB);
+              sb[1][t] = scale(tSB + (int64_t)(bh * MH + t) * 16 * p.lds_b, offSB);
+            }
+          }
+#pragma unroll
+          for (int t = 0; t < MH; t++) {
+            a1[t] = frag(tA + (int64_t)(ah * MH + t) * 16 * p.lda, offA);
+            sa[1][t] = scale(tSA + (int64_t)(ah * MH + t) * 16 * p.lds_a, offSA);
+          }
+          settle_tail(a1[0], a1[1], a1[2], a1[3], b[1][0], b[1][1], b[1][2], b[1][3],
+                      sa[1][0], sa[1][1], sa[1][2], sa[1][3], sb[1][0], sb[1][1], sb[1][2], sb[1][3]);
+          static_for<MH * MH>([&](auto N_) {
+            constexpr int n = decltype(N_)::value, i = n / MH, j = n % MH;
+            mfma16_mxfp8(b[1][j], a1[i], acc[ah * MH + i][bh * MH + j], sb[1][j], sa[1][i]);
+          });
+        });
+        mfma_retire();   // (inside the loop's block, like the main loop's: see mfma_retire)
+      }
+    }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
@@ -241,30 +320,33 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
 }
 
 bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
-  // whole tiles, K steps in groups of eight (K a multiple of 1024), scale rows that a 16-byte load can fetch
-  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 1024 == 0 && p.k_bytes >= 1024 &&
+  // whole tiles, at least one group of eight K steps (K >= 1024; what is left behind the last group: the TAIL form),
+  // scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 32 == 0 && p.k_bytes >= 1024 &&
          p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
          p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
          p.lds_a * 64 + p.k_bytes / 32 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 32 < (1ll << 31);
 }
 
-template <int EPI>
+template <int EPI, bool TAIL = false>
 static int launch_wave128_mxfp8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp8_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp8_kernel<EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
+  if (p.k_bytes % 1024 != 0)
+    return lean == 1 ? launch_wave128_mxfp8<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4, true>(p, stream) : launch_wave128_mxfp8<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp8<3>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4>(p, stream) : launch_wave128_mxfp8<0>(p, stream);
 }
 
@@ -293,7 +375,11 @@ __device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32
 }
 
 // EPI: 0 = general epilogue, 3 / 4 = lean epilogue (gemm_epilogue16_lean) writing fp16 / bf16
-template <int EPI>
+// TAIL: K need not be a multiple of 1024 (of 32 still, the scale block): the main loop does the whole groups of four K
+// steps, and what is left of each row (16 .. 496 bytes, the same for every tile) follows in K steps whose fragments and
+// scale bytes every lane loads straight from global memory - zeros (and the scale 1) beyond K - into the fragment and
+// scale registers that the pipeline has free at that point.
+template <int EPI, bool TAIL = false>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
@@ -313,7 +399,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
   int pm, pn;
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
-  const int nk = p.k_bytes / ROWB;
+  const int nk = TAIL ? p.k_bytes / (4 * ROWB) * 4 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
   asm volatile("" : "+s"(nk_last));
 
@@ -509,6 +595,56 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       step(I3{}, fk); advance();
       if (kt + 4 >= nk_last) mfma_retire();
     }
+    if constexpr (TAIL) {
+      // (free here: the fragment set 1 and the scale set 1 - the last step read the next tile's first fragments and
+      // scales into the sets 0)
+      const int k_main = nk * ROWB, tail = p.k_bytes - k_main;
+      int tm = pm * BM + wm * 128, tn = pn * BN + wn * 128, tl = l16, tk = kg;
+      asm volatile("" : "+s"(tm), "+s"(tn), "+v"(tl), "+v"(tk));   // (keeps this address arithmetic out of the K loop)
+      // a scalar base per fragment and one 32-bit lane offset per operand (gemm_wave128_mxfp4_ok bounds them)
+      const char* const tA = p.A + (int64_t)tm * p.lda + k_main;
+      const char* const tB = p.B + (int64_t)tn * p.ldb + k_main;
+      const uint8_t* const tSA = p.sA + (int64_t)tm * p.lds_a + k_main / 16;
+      const uint8_t* const tSB = p.sB + (int64_t)tn * p.lds_b + k_main / 16;
+      const unsigned offA = (unsigned)tl * (unsigned)p.lda + tk * 32, offB = (unsigned)tl * (unsigned)p.ldb + tk * 32;
+      const unsigned offSA = (unsigned)tl * (unsigned)p.lds_a + tk * 2, offSB = (unsigned)tl * (unsigned)p.lds_b + tk * 2;
+      for (int h = 0; h * ROWB < tail; h++) {
+        // the blocks 2 tk (sub-step 0) and 2 tk + 1 (sub-step 1) of the step; their scales in bytes 0 and 1
+        const bool ok0 = h * ROWB + tk * 32 < tail, ok1 = h * ROWB + tk * 32 + 16 < tail;
+        auto scale = [&](const uint8_t* src, unsigned off) {
+          int v0 = 127, v1 = 127;   // (2^0: multiplies zeros)
+          if (ok0) v0 = src[h * 8 + (uint64_t)off];
+          if (ok1) v1 = src[h * 8 + 1 + (uint64_t)off];
+          return v0 | (v1 << 8);
+        };
+#pragma unroll
+        for (int t = 0; t < MT; t++) sa[1][t] = scale(tSA + (int64_t)t * 16 * p.lds_a, offSA);
+#pragma unroll
+        for (int t = 0; t < NT; t++) sb[1][t] = scale(tSB + (int64_t)t * 16 * p.lds_b, offSB);
+        static_for<KS>([&](auto KS_) {
+          constexpr int ks = decltype(KS_)::value;
+          const bool ok = ks == 0 ? ok0 : ok1;
+          auto frag = [&](const char* src, unsigned off) {
+            i32x4 v = {0, 0, 0, 0};
+            if (ok) v = *(const i32x4*)(src + h * ROWB + ks * 16 + (uint64_t)off);
+            return v;
+          };
+#pragma unroll
+          for (int t = 0; t < MT; t++) f[1].a[t] = frag(tA + (int64_t)t * 16 * p.lda, offA);
+#pragma unroll
+          for (int t = 0; t < NT; t++) f[1].b[t] = frag(tB + (int64_t)t * 16 * p.ldb, offB);
+          settle_pass(sa[1][0], sa[1][1], sa[1][2], sa[1][3], sa[1][4], sa[1][5], sa[1][6], sa[1][7],
+                      sb[1][0], sb[1][1], sb[1][2], sb[1][3], sb[1][4], sb[1][5], sb[1][6], sb[1][7]);
+          settle_tail(f[1].a[0], f[1].a[1], f[1].a[2], f[1].a[3], f[1].a[4], f[1].a[5], f[1].a[6], f[1].a[7],
+                      f[1].b[0], f[1].b[1], f[1].b[2], f[1].b[3], f[1].b[4], f[1].b[5], f[1].b[6], f[1].b[7]);
+          static_for<NM>([&](auto N_) {
+            constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
+            mfma16_mxfp4<ks>(f[1].b[j], f[1].a[i], acc[i][j], sb[1][j], sa[1][i]);
+          });
+        });
+        mfma_retire();   // (inside the loop's block, like the main loop's: see mfma_retire)
+      }
+    }
     mfma_drain(acc);
     int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
@@ -525,30 +661,33 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
 }
 
 bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
-  // whole tiles, K steps in groups of four (K a multiple of 1024 elements), scale rows that a 16-byte load can fetch
-  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 512 == 0 && p.k_bytes >= 512 &&
+  // whole tiles, at least one group of four K steps (K >= 1024 elements; what is left behind the last group: the TAIL
+  // form), scale rows that a 16-byte load can fetch
+  return p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 16 == 0 && p.k_bytes >= 512 &&
          p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
          p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
          p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
 }
 
-template <int EPI>
+template <int EPI, bool TAIL = false>
 static int launch_wave128_mxfp4(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp4_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp4_kernel<EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
+  if (p.k_bytes % 512 != 0)
+    return lean == 1 ? launch_wave128_mxfp4<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4, true>(p, stream) : launch_wave128_mxfp4<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp4<3>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4>(p, stream) : launch_wave128_mxfp4<0>(p, stream);
 }
 
