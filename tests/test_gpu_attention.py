@@ -148,8 +148,8 @@ def test_unsupported_configurations_raise(gpu):
     q = torch.zeros(1, 1, 100, 64, dtype=torch.float16, device=gpu)
     with pytest.raises(ValueError):          # N_CTX must be a multiple of 128 here (the reference asserts it in backward, 06:494)
         triton_amd.attention(q, q, q, True, 0.5)
-    q8 = torch.zeros(1, 1, 128, 32, dtype=torch.float8_e5m2, device=gpu)
-    with pytest.raises(ValueError):          # fp8 forward: head dims 64 and 128 only
+    q8 = torch.zeros(1, 1, 192, 32, dtype=torch.float8_e5m2, device=gpu)
+    with pytest.raises(ValueError):          # fp8 forward: the same rule
         triton_amd.attention(q8, q8, q8.permute(0, 1, 3, 2).contiguous().permute(0, 1, 3, 2), True, 0.5)
     q48 = torch.zeros(1, 1, 128, 48, dtype=torch.float16, device=gpu)
     with pytest.raises(AssertionError):      # the reference's own assert (06:447)

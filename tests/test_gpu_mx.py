@@ -32,7 +32,7 @@ def _run(gpu, a, sa, b, sb, fmt, out_dtype):
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
 @pytest.mark.parametrize("shape", [(128, 128, 256), (512, 512, 512), (300, 200, 1024), (1024, 1024, 1024),
-                                   (64, 64, 96), (33, 70, 32), (256, 256, 2048)])
+                                   (64, 64, 96), (33, 70, 32), (256, 256, 2048), (300, 200, 1056), (128, 128, 160), (512, 256, 4064)])
 def test_against_oracle(gpu, fmt, shape):
     # config 5 distribution: codes uniform, scale exponents 2^-4 .. 2^4
     M, N, K = shape
@@ -43,7 +43,8 @@ def test_against_oracle(gpu, fmt, shape):
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * max(1.0, scale / 64))
 
 
-@pytest.mark.parametrize("shape", [(256, 256, 1024), (128, 384, 4096), (130, 70, 256), (64, 64, 96)])
+@pytest.mark.parametrize("shape", [(256, 256, 1024), (128, 384, 4096), (130, 70, 256), (64, 64, 96), (256, 512, 1056), (130, 70, 288),
+                                   (64, 64, 32), (300, 260, 2016)])     # (K / 32 odd: scale rows of odd pitch, a partial last K step)
 def test_mxfp4_exact_sums_are_bitwise(gpu, shape):
     # fp4 values are multiples of 1/2 with |x| <= 6 and scales 2^-1..2^1: every product is a multiple
     # of 2^-4, every partial sum over K <= 4096 stays below 2^20 -> exact in fp32 in any order
@@ -144,10 +145,11 @@ def test_full_size_8192_sampled_rows(gpu, fmt):
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max() / 64)
 
 
-@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4, 5, 6])
 @pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
 def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile):
-    # MI355_GEMM_TILE forces one kernel (ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves,
+    # MI355_GEMM_TILE forces one kernel (-1: the one-thread-per-output kernel, an independent second implementation;
+    # ping-pong, 128x128, one-barrier, pipelined 4 / 8 waves,
     # persistent) for shapes the size heuristic would give to another; K = 1536 covers three 16-byte
     # scale groups per row in the pipelined kernels (an odd number: the two-slot scale ring changes
     # parity from tile to tile in the persistent form, two programs for six and twelve tiles),
@@ -155,7 +157,7 @@ def test_every_kernel_variant_is_exact_on_exact_sums(gpu, monkeypatch, fmt, tile
     # 256x256 tiles and K a multiple of 1024 (the last two shapes: one and two groups of four K steps), else 5.
     set_knob(monkeypatch, "MI355_GEMM_TILE", str(tile))
     set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", "2")
-    rng = np.random.default_rng(tile)
+    rng = np.random.default_rng(tile + 1)
     for (M, N, K) in [(512, 256, 1536), (300, 520, 1056), (768, 512, 1536), (768, 1024, 1024), (512, 256, 2048)]:
         if fmt == "mxfp4":
             a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)

@@ -69,7 +69,7 @@ void load_knobs() {
   Knobs k;
   k.force_strided = read_env("MI355_GEMM_FORCE_STRIDED", 0);
   k.group_m = read_env("MI355_GEMM_GROUP_M", 1);
-  k.tile = read_env("MI355_GEMM_TILE", 0);
+  k.tile = read_env("MI355_GEMM_TILE", -1);   // (-1: the block-scaled products' one-thread-per-output kernel)
   k.programs = read_env("MI355_GEMM_PROGRAMS", 1);
   k.skinny = read_env("MI355_GEMM_SKINNY", 0);
   k.grouped_big_min = read_env("MI355_GROUPED_BIG_MIN", 1);

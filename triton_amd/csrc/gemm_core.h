@@ -463,10 +463,23 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
     fill = fill + 1 == NS ? 0 : fill + 1;
   }
   // K tail (K bytes % RBK != 0): one more tile, zero-filled past K, outside the pipelined loop.
-  // (Block-scaled operands always come in whole tiles.)
+  // (Block-scaled operands: whole scale blocks; the scales of the blocks past K read as 2^0.)
   if (nfull * RBK < p.k_bytes) {
     block_barrier();  // every wave is done with the ring
     guarded_tile(nfull, lds);
+    if constexpr (Cfg::kScaled) {
+      const int nblocks = (p.k_bytes - nfull * RBK) / Cfg::kBlockBytes;
+#pragma unroll
+      for (int t = 0; t < MT; t++) {
+        int r = min(m0 + wm * TM + t * 32 + l32, p.M - 1);
+        sa[t] = Cfg::load_scale_tail(p.sA + (int64_t)r * p.lds_a, nfull, g, nblocks);
+      }
+#pragma unroll
+      for (int t = 0; t < NT; t++) {
+        int r = min(n0 + wn * TN + t * 32 + l32, p.N - 1);
+        sb[t] = Cfg::load_scale_tail(p.sB + (int64_t)r * p.lds_b, nfull, g, nblocks);
+      }
+    }
     wait_all();
     __syncthreads();
     compute_tile(lds);

@@ -22,9 +22,21 @@ struct CfgMxfp4 {
   // lane group g reads scale blocks 2g, 2g+1 of the step (16 bytes = 32 elements each), one per sub-step
   __device__ static constexpr int chunk(int ks, int g, int) { return g * 2 + ks; }
   // the step has 4 scale bytes per row; move bytes 2g, 2g+1 to positions 0, 1 (selector = ks)
+  // (scale rows of any pitch: the four bytes need not be aligned - the compiler emits what the target allows)
   __device__ static int load_scale(const uint8_t* row, int kt, int g) {
-    return (int)(*(const uint32_t*)(row + kt * 4) >> (16 * g));
+    uint32_t v;
+    __builtin_memcpy(&v, row + kt * 4, 4);
+    return (int)(v >> (16 * g));
   }
+  // the last, partial step: `nblocks` (1 .. 3) scale bytes exist; the others become 2^0, next to zero-filled operands
+  __device__ static int load_scale_tail(const uint8_t* row, int kt, int g, int nblocks) {
+    uint32_t v = 0x7F7F7F7Fu;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (i < nblocks) v = (v & ~(0xFFu << (8 * i))) | ((uint32_t)row[kt * 4 + i] << (8 * i));
+    return (int)(v >> (16 * g));
+  }
+  static constexpr int kBlockBytes = 16;   // operand bytes per scale block
   __device__ static int scale_dword_offset(int kt) { return kt * 4; }          // dword copied to LDS for step kt
   __device__ static int scale_fixup(int v, int, int g) { return (int)((unsigned)v >> (16 * g)); }
   template <int ks>
@@ -50,8 +62,15 @@ struct CfgMxfp8 {
   __device__ static constexpr int chunk(int, int g, int c) { return 2 * c + g; }
   // the step has 2 scale bytes per row; lane group g supplies the scale of block g in byte 0
   __device__ static int load_scale(const uint8_t* row, int kt, int g) {
-    return (int)(*(const uint16_t*)(row + kt * 2)) >> (8 * g);
+    uint16_t v;
+    __builtin_memcpy(&v, row + kt * 2, 2);
+    return (int)v >> (8 * g);
   }
+  // the last, partial step holds one scale block; the other becomes 2^0, next to zero-filled operands
+  __device__ static int load_scale_tail(const uint8_t* row, int kt, int g, int) {
+    return (int)((uint32_t)row[kt * 2] | 0x7F00u) >> (8 * g);
+  }
+  static constexpr int kBlockBytes = 32;   // operand bytes per scale block
   // the dword holding the scales of steps kt and kt^1; bytes 2*(kt&1) + g
   __device__ static int scale_dword_offset(int kt) { return (kt >> 1) * 4; }
   __device__ static int scale_fixup(int v, int kt, int g) { return (int)((unsigned)v >> (16 * (kt & 1) + 8 * g)); }
@@ -65,8 +84,8 @@ struct CfgMxfp8 {
   }
 };
 
-// Any shape / pitch: one thread per output, decode-and-FMA in fp32.  Used when K is not a
-// whole number of 64-byte steps or the scale rows are not dword aligned.
+// Any shape / pitch: one thread per output, decode-and-FMA in fp32.  Runs only on request (a negative tile number):
+// an independent second implementation for the tests.
 __global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4) {
   int n = blockIdx.x * 16 + threadIdx.x % 16, m = blockIdx.y * 16 + threadIdx.x / 16;
   if (m >= p.M || n >= p.N) return;
@@ -102,13 +121,17 @@ int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
   // what is left behind the last whole group of K steps is the tail form's)
   if (tile == 6 && fmt == 0 && gemm_wave128_mxfp4_ok(p)) return gemm_wave128_mxfp4_launch(p, stream);
   if (tile == 6 && fmt != 0 && gemm_wave128_mxfp8_ok(p)) return gemm_wave128_mxfp8_launch(p, stream);
-  const bool whole_tiles = p.k_bytes % RBK == 0;
-  const bool scales_aligned = p.lds_a % 4 == 0 && p.lds_b % 4 == 0 && ((uintptr_t)p.sA % 4) == 0 && ((uintptr_t)p.sB % 4) == 0;
-  if (!whole_tiles || !scales_aligned || tile < 0) {
+  if (tile < 0) {
     dim3 grid((p.N + 15) / 16, (p.M + 15) / 16);
     mx_gemm_simple_kernel<<<grid, dim3(256), 0, stream>>>(p, fmt == 0);
     return (int)hipGetLastError();
   }
+  // K not a whole number of 64-byte steps, or scale rows that are not dword aligned (a contiguous scale matrix whose
+  // K / 32 is not a multiple of four): the one-barrier-per-step kernels, which read their scales with loads of any
+  // alignment and finish a partial last step themselves
+  const bool whole_tiles = p.k_bytes % RBK == 0;
+  const bool scales_aligned = p.lds_a % 4 == 0 && p.lds_b % 4 == 0 && ((uintptr_t)p.sA % 4) == 0 && ((uintptr_t)p.sB % 4) == 0;
+  if (!whole_tiles || !scales_aligned) tile = tile == 1 ? 1 : 2;
   return fmt == 0 ? launch_gemm_tile<CfgMxfp4, true>(p, tile, stream) : launch_gemm_tile<CfgMxfp8, true>(p, tile, stream);
 }
 
