@@ -337,7 +337,9 @@ enum {
   MI355_BURN_FP8_32X32X64 = 2,
   MI355_BURN_FP8_16X16X128 = 3,
   MI355_BURN_FP4_32X32X64 = 4,
-  MI355_BURN_FP4_16X16X128 = 5
+  MI355_BURN_FP4_16X16X128 = 5,
+  MI355_BURN_MXFP4_32X32X64 = 6,    /* the block-scaled forms of the two fp4 shapes (one e8m0 scale per lane and operand) */
+  MI355_BURN_MXFP4_16X16X128 = 7
 };
 int mi355_mfma_burn(float* sink, int shape, int random_operands, int iters, int waves_per_simd, void* stream);
 

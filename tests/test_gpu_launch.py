@@ -176,7 +176,7 @@ def test_clock_and_mfma_burn_probes(gpu):
     ticks = torch.zeros(2, device=gpu, dtype=torch.int64)
     stream = torch.cuda.current_stream().cuda_stream
     side = torch.cuda.Stream(device=gpu)
-    for shape in range(6):
+    for shape in range(8):
         for rnd in (0, 1):
             assert lib.mi355_mfma_burn(sink.data_ptr(), shape, rnd, 200, 1, stream) == 0
     assert lib.mi355_clock_probe(ticks.data_ptr(), 2000, side.cuda_stream) == 0   # 2 ms next to the queued burns
@@ -185,7 +185,7 @@ def test_clock_and_mfma_burn_probes(gpu):
     cyc, real = ticks.tolist()
     mhz = cyc / real * lib.mi355_query(_lib.Q_WALL_CLOCK_KHZ) / 1e3
     assert 90 < mhz < 2600, mhz
-    for bad in ((0, 0, 0, 100, 1), (sink.data_ptr(), 6, 0, 100, 1), (sink.data_ptr(), 0, 0, 0, 1), (sink.data_ptr(), 0, 0, 100, 3)):
+    for bad in ((0, 0, 0, 100, 1), (sink.data_ptr(), 8, 0, 100, 1), (sink.data_ptr(), 0, 0, 0, 1), (sink.data_ptr(), 0, 0, 100, 3)):
         assert lib.mi355_mfma_burn(*bad, stream) == -1
 
 
@@ -197,7 +197,7 @@ def test_power_probe_module_reports_every_leg(gpu, capsys):
     import json
 
     rec = json.loads(capsys.readouterr().out)
-    assert len(rec["legs"]) == 12 and all(leg["tflops"] > 100 for leg in rec["legs"])
+    assert len(rec["legs"]) == 16 and all(leg["tflops"] > 100 for leg in rec["legs"])
     # the constant-operand legs are never slower than the random ones by more than noise (less switching, same work)
     by = {(leg["shape"], leg["operands"]): leg["tflops"] for leg in rec["legs"]}
     assert by[("bf16 16x16x32", "constant")] > 0.9 * by[("bf16 16x16x32", "random")]

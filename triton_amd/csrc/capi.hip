@@ -462,7 +462,7 @@ int mi355_clock_probe(uint64_t* ticks, int duration_us, void* stream_) {
 }
 
 int mi355_mfma_burn(float* sink, int shape, int random_operands, int iters, int waves_per_simd, void* stream_) {
-  if (!sink || !aligned(sink, 4) || shape < MI355_BURN_BF16_32X32X16 || shape > MI355_BURN_FP4_16X16X128) return MI355_EINVAL;
+  if (!sink || !aligned(sink, 4) || shape < MI355_BURN_BF16_32X32X16 || shape > MI355_BURN_MXFP4_16X16X128) return MI355_EINVAL;
   if (iters <= 0 || iters > (1 << 24) || waves_per_simd < 1 || waves_per_simd > 2) return MI355_EINVAL;
   if (!device_info().gfx950) return MI355_EDEVICE;
   return mfma_burn_launch(sink, shape, random_operands != 0, iters, waves_per_simd, device_info().cus > 0 ? device_info().cus : 256,

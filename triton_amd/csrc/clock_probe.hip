@@ -66,17 +66,21 @@ __device__ inline unsigned burn_e4m3_quad(unsigned& s) {
 }
 
 template <int SHAPE>
-__device__ __forceinline__ void burn_mfma32(f32x16& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4) {
+__device__ __forceinline__ void burn_mfma32(f32x16& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4, int sa, int sb) {
 #if MI355_DEVICE_PASS
-  if constexpr (SHAPE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
+  if constexpr (SHAPE == 6)
+    asm volatile("v_mfma_scale_f32_32x32x64_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4), "v"(sa), "v"(sb));
+  else if constexpr (SHAPE == 0) asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
   else if constexpr (SHAPE == 2) asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   else asm volatile("v_mfma_f32_32x32x64_f8f6f4 %0, %1, %2, %0 cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4));
 #endif
 }
 template <int SHAPE>
-__device__ __forceinline__ void burn_mfma16(f32x4& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4) {
+__device__ __forceinline__ void burn_mfma16(f32x4& c, const burn_i32x8& a, const burn_i32x8& b, const i32x4& a4, const i32x4& b4, int sa, int sb) {
 #if MI355_DEVICE_PASS
-  if constexpr (SHAPE == 1) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
+  if constexpr (SHAPE == 7)
+    asm volatile("v_mfma_scale_f32_16x16x128_f8f6f4 %0, %1, %2, %0, %3, %4 op_sel_hi:[0,0,0] cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4), "v"(sa), "v"(sb));
+  else if constexpr (SHAPE == 1) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a4), "v"(b4));
   else if constexpr (SHAPE == 3) asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   else asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0 cbsz:4 blgp:4" : "+a"(c) : "v"(a4), "v"(b4));
 #endif
@@ -90,9 +94,9 @@ __device__ __forceinline__ void burn_settle(V& c) {
 #endif
 }
 __device__ __forceinline__ void burn_settle_operands(burn_i32x8& a0, burn_i32x8& a1, burn_i32x8& b0, burn_i32x8& b1,
-                                                     i32x4& c0, i32x4& c1, i32x4& d0, i32x4& d1) {
+                                                     i32x4& c0, i32x4& c1, i32x4& d0, i32x4& d1, int& sa, int& sb) {
 #if MI355_DEVICE_PASS
-  asm volatile("s_nop 1" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1), "+v"(c0), "+v"(c1), "+v"(d0), "+v"(d1));
+  asm volatile("s_nop 1" : "+v"(a0), "+v"(a1), "+v"(b0), "+v"(b1), "+v"(c0), "+v"(c1), "+v"(d0), "+v"(d1), "+v"(sa), "+v"(sb));
 #endif
 }
 template <typename V>
@@ -125,10 +129,13 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
   // The MFMAs are issued as assembly with the accumulators pinned to accumulation registers, as the GEMM kernels
   // issue theirs (left to the register allocator, the chains of four-register tiles were rotated through
   // architectural registers in every round, at half the rate).  16-bit and fp4 operands are four registers, fp8 eight.
+  // block scales of the scaled fp4 legs (e8m0 in byte 0): 2^-4 .. 2^4, or 1
+  s = burn_rnd(s);
+  int sa = random_operands ? 123 + (int)(s % 9u) : 127, sb = random_operands ? 123 + (int)((s >> 8) % 9u) : 127;
   float total = 0.f;
   i32x4 a4[2] = {__builtin_shufflevector(a[0], a[0], 0, 1, 2, 3), __builtin_shufflevector(a[1], a[1], 0, 1, 2, 3)};
   i32x4 b4[2] = {__builtin_shufflevector(b[0], b[0], 0, 1, 2, 3), __builtin_shufflevector(b[1], b[1], 0, 1, 2, 3)};
-  if constexpr (SHAPE == 0 || SHAPE == 2 || SHAPE == 4) {         // 32 x 32 tiles: four chains of 16 registers
+  if constexpr (SHAPE == 0 || SHAPE == 2 || SHAPE == 4 || SHAPE == 6) {         // 32 x 32 tiles: four chains of 16 registers
     f32x16 acc[4];
 #pragma unroll
     for (int c = 0; c < 4; c++)
@@ -136,10 +143,10 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
       for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
 #pragma unroll
     for (int c = 0; c < 4; c++) burn_settle(acc[c]);
-    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1]);
+    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1], sa, sb);
     for (int i = 0; i < iters; i++) {
 #pragma unroll
-      for (int u = 0; u < 8; u++) burn_mfma32<SHAPE>(acc[u & 3], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);
+      for (int u = 0; u < 8; u++) burn_mfma32<SHAPE>(acc[u & 3], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1], sa, sb);
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");          // the last MFMAs retire before their results are read
 #pragma unroll
@@ -156,10 +163,10 @@ __global__ __launch_bounds__(256) void mfma_burn_kernel(float* sink, int iters, 
       for (int r = 0; r < 4; r++) acc[c][r] = 0.f;
 #pragma unroll
     for (int c = 0; c < 8; c++) burn_settle(acc[c]);
-    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1]);
+    burn_settle_operands(a[0], a[1], b[0], b[1], a4[0], a4[1], b4[0], b4[1], sa, sb);
     for (int i = 0; i < iters; i++) {
 #pragma unroll
-      for (int u = 0; u < 16; u++) burn_mfma16<SHAPE>(acc[u & 7], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1]);
+      for (int u = 0; u < 16; u++) burn_mfma16<SHAPE>(acc[u & 7], a[u & 1], b[(u >> 1) & 1], a4[u & 1], b4[(u >> 1) & 1], sa, sb);
     }
     asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
 #pragma unroll
@@ -185,6 +192,8 @@ int mfma_burn_launch(float* sink, int shape, int random_operands, int iters, int
     case 3: hipLaunchKernelGGL(mfma_burn_kernel<3>, grid, block, 0, stream, sink, iters, random_operands); break;
     case 4: hipLaunchKernelGGL(mfma_burn_kernel<4>, grid, block, 0, stream, sink, iters, random_operands); break;
     case 5: hipLaunchKernelGGL(mfma_burn_kernel<5>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 6: hipLaunchKernelGGL(mfma_burn_kernel<6>, grid, block, 0, stream, sink, iters, random_operands); break;
+    case 7: hipLaunchKernelGGL(mfma_burn_kernel<7>, grid, block, 0, stream, sink, iters, random_operands); break;
     default: return -1;
   }
   return (int)hipGetLastError();

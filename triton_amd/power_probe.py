@@ -2,7 +2,7 @@
 
 Runs the library's bare MFMA loops (`mi355_mfma_burn`: one MFMA shape issued back to back from registers on every
 SIMD, no memory traffic) for a sustained period each - 16-bit 32x32x16 and 16x16x32, fp8 32x32x64 and 16x16x128,
-fp4 likewise; pseudo-random and constant operands - and prints, per leg, the rate from device events next to the
+fp4 likewise, and the block-scaled forms of the fp4 shapes; pseudo-random and constant operands - and prints, per leg, the rate from device events next to the
 board power and shader clock that the driver reports meanwhile (hwmon power1_average / power1_input and
 power1_cap, pp_dpm_sclk).  The nominal peaks (2.5 / 5 / 10.1 PFLOP/s) assume 2.4 GHz on every CU; under the
 power cap the clock settles where the kernel's energy per flop puts it, and the figures printed here are what a
@@ -27,6 +27,8 @@ SHAPES = [  # (name, enum of include/mi355_kernels.h, flop per wave and round, n
     ("fp8 16x16x128", 3, 16 * 65536, 5000.0),
     ("fp4 32x32x64", 4, 8 * 131072, 10100.0),
     ("fp4 16x16x128", 5, 16 * 65536, 10100.0),
+    ("mxfp4 32x32x64", 6, 8 * 131072, 10100.0),
+    ("mxfp4 16x16x128", 7, 16 * 65536, 10100.0),
 ]
 
 
