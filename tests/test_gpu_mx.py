@@ -7,7 +7,7 @@ import torch
 
 import triton_amd
 from oracle import formats, mx
-from util import bits_equal, to_np, set_knob
+from util import bits_equal, report_error, to_np, set_knob
 
 pytestmark = pytest.mark.gpu
 
@@ -40,6 +40,7 @@ def test_against_oracle(gpu, fmt, shape):
     ref = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="bf16")
     got = _run(gpu, a, sa, b, sb, fmt, torch.bfloat16)
     scale = np.abs(ref).max()
+    report_error(f"{fmt} {shape}", got, ref)
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * max(1.0, scale / 64))
 
 
@@ -142,6 +143,8 @@ def test_full_size_8192_sampled_rows(gpu, fmt):
     rows = [0, 255, 256, 4097, 8191]
     ref = mx.mx_matmul(a[rows], sa[rows], b, sb, fmt, out_dtype="bf16")
     got = to_np(c[rows])
+    # (the working bar for MX is rtol = 3e-2; the absolute term, a 2000th of the largest output, only covers outputs near 0)
+    report_error(f"{fmt} 8192^3, bf16 out, 5 rows", got, ref)
     assert np.allclose(got, ref, rtol=3e-2, atol=3e-2 * np.abs(ref).max() / 64)
 
 

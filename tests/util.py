@@ -37,3 +37,17 @@ def set_knob(monkeypatch, name: str, value) -> None:
 
     monkeypatch.setenv(name, str(value))
     _lib.load().mi355_refresh_env()
+
+
+def report_error(tag: str, got: np.ndarray, ref: np.ndarray) -> float:
+    """Print (pytest -s / on failure) and return the largest |got - ref| as a fraction of max |ref|, next to the largest
+    element-wise relative error over the outputs that are at least 1 % of the largest one: what the fp8 / MX tests
+    actually observe under their rtol = 3e-2 bar."""
+    got = np.asarray(got, dtype=np.float64); ref = np.asarray(ref, dtype=np.float64)
+    top = float(np.abs(ref).max())
+    d = np.abs(got - ref)
+    big = np.abs(ref) >= 0.01 * top
+    rel_big = float((d[big] / np.abs(ref[big])).max()) if big.any() else 0.0
+    frac = float(d.max() / top) if top > 0 else 0.0
+    print(f"{tag}: max |err| = {d.max():.3e} = {frac:.2e} of max |ref| ({top:.3g}); max relative error over outputs >= 1 % of it: {rel_big:.2e}")
+    return frac
