@@ -349,10 +349,11 @@ int mi355_gemm_epilogue(const void* A, const void* B, void* C, int M, int N, int
   if (softmax && out_dtype != MI355_F16 && out_dtype != MI355_BF16 && out_dtype != MI355_F32) return MI355_EDTYPE;
   // a row that fits one tile: product, addend, activation and softmax in ONE launch, on the fp32 accumulator,
   // one rounding at the store - what the reference's single tile does
-  // (that kernel is one workgroup per 128 rows with an unpipelined K loop, built for the small, latency-bound
-  // products of the reference's test: larger ones - more than 2^21 elements of A by default,
-  // MI355_ROWFUSED_MAX_MK - take the tiled GEMM and the softmax as a second launch)
-  const int64_t rowfused_max = (int64_t)knob(knobs().rowfused_max_mk, 1 << 21);
+  // (that kernel is one workgroup per 128 rows with operands of any strides, built for the small products of the
+  // reference's test, where the single rounding is the point: on time the tiled GEMM plus a softmax launch wins at every
+  // size - flushed caches, bf16: 32^3 10.8 against 9.3 us, 128 x 256 x 128 50 / 13, 1024 x 256 x 256 59 / 14, 8192 x 256 x 256
+  // 59 / 19, 256 x 256 x 2048 237 / 33 - and takes over beyond 2^18 elements of A by default, MI355_ROWFUSED_MAX_MK)
+  const int64_t rowfused_max = (int64_t)knob(knobs().rowfused_max_mk, 1 << 18);
   if (softmax && N <= 256 && (in_dtype == MI355_F16 || in_dtype == MI355_BF16) && (int64_t)M * K <= rowfused_max) {
     if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
     if (addend && addend_dtype != MI355_F16 && addend_dtype != MI355_BF16 && addend_dtype != MI355_F32) return MI355_EDTYPE;
