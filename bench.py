@@ -515,6 +515,21 @@ def main():
                 rec["data"] = info["data"]
             extra[name] = rec
             del fn
+        # What this board's matrix pipes sustain with nothing but MFMAs of the shapes the GEMMs above are built from, on
+        # pseudo-random operands, under the same power limit (triton_amd/power_probe.py over mi355_mfma_burn; 0.4 s per
+        # shape): the ceiling that the nominal peaks of `roofline.peak` / `frac_of_peak` do not know about.
+        from triton_amd import power_probe
+
+        sampler = power_probe.BoardSampler()
+        sink = torch.zeros(4, device=dev, dtype=torch.float32)
+        ceiling = {}
+        for key, want, ref in (("bf16_16x16x32", "bf16 16x16x32", out["value"]), ("fp8_16x16x128", "fp8 16x16x128", extra.get("fp8_e4m3_gemm_8192", {}).get("tflops")),
+                               ("mxfp4_16x16x128", "mxfp4 16x16x128", extra.get("mxfp4_gemm_8192", {}).get("tflops"))):
+            name, shape, flop_per_round, _ = next(x for x in power_probe.SHAPES if x[0] == want)
+            r = power_probe.burn(lib, sink, stream, shape, flop_per_round, True, 0.4, 1, lib.mi355_query(_lib.Q_CU_COUNT), sampler)
+            r["gemm_of_this_ceiling"] = round(ref / r["tflops"], 3) if ref else None
+            ceiling[key] = r
+        extra["bare_mfma_ceiling_random_operands"] = ceiling
         out["extra"] = extra
 
     if not args.no_cpu:
