@@ -1,7 +1,7 @@
 """Benchmark of the hot path on one MI355X.
 
 `python bench.py --gpus 1 --steps K --warmup W` times K back-to-back launches of the headline
-workload (bf16 GEMM 8192^3, BASELINE config 2) with inputs resident in HBM, and prints ONE JSON
+workload (bf16 GEMM 8192^3, benchmark configuration 2) with inputs resident in HBM, and prints ONE JSON
 line: TFLOP/s (work = 2*M*N*K as in python/tutorials/03-matrix-multiplication.py:437), the MFMA
 roofline fraction of the GEMM kernel from per-launch device events, and the CPU oracle timed on
 the host cores.  The other workloads of the path (fp8 / MX GEMM, attention forward / backward)

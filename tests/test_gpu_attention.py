@@ -158,7 +158,7 @@ def test_unsupported_configurations_raise(gpu):
 
 @pytest.mark.parametrize("causal", [True, False])
 def test_full_size_config3_sampled_heads(gpu, causal):
-    # BASELINE config 3: Z=4, H=32, N=4096, D=128 bf16, sm_scale = 1/sqrt(128); two heads are checked
+    # benchmark configuration 3: Z=4, H=32, N=4096, D=128 bf16, sm_scale = 1/sqrt(128); two heads are checked
     # in full against the restated tile programs in bf16 at rtol = atol = 1e-2 and the fp64 closed form
     # (forward and all three gradients)
     Z, H, N, D = 4, 32, 4096, 128

@@ -23,7 +23,7 @@ GOLD_FMT = json.load(open(os.path.join(HERE, "golden", "formats.json")))
 
 
 def test_config1_fp16_512_matches_tiled_oracle(gpu):
-    # BASELINE config 1: seed 0, 512^3 fp16, the oracle runs the reference tile program 64x64x32 / GROUP_M 8
+    # benchmark configuration 1: seed 0, 512^3 fp16, the oracle runs the reference tile program 64x64x32 / GROUP_M 8
     rng = np.random.default_rng(0)
     a = randn_rounded(rng, (512, 512), "fp16")
     b = randn_rounded(rng, (512, 512), "fp16")
@@ -404,7 +404,7 @@ def test_mfma_decodes_every_fp8_code_exactly(gpu, fmt, tdt):
 
 
 def test_full_size_8192_bf16_sampled_rows_and_exact_permutation(gpu):
-    # BASELINE config 2 at full size: (a) sampled rows against the fp64 closed form, (b) B = signed
+    # benchmark configuration 2 at full size: (a) sampled rows against the fp64 closed form, (b) B = signed
     # permutation makes every output one exactly-representable product -> bitwise
     n = 8192
     g = torch.Generator(device="cpu").manual_seed(0)
@@ -456,7 +456,7 @@ def _sampled_rows_check(gpu, M, N, K, dtype, seed, layout="row_major_b"):
 
 @pytest.mark.parametrize("n", [2048, 3072, 4096, 5120, 6144, 7168])
 def test_config2_sweep_sizes_bf16(gpu, n):
-    # BASELINE config 2 sweeps square sizes 1024 .. 8192 (1024 and 8192 have tests of their own): 5120, 6144
+    # benchmark configuration 2 sweeps square sizes 1024 .. 8192 (1024 and 8192 have tests of their own): 5120, 6144
     # and 7168 are the sizes whose tiles do not divide by the CU count, so the persistent programs walk ragged
     # rounds of tiles as one stream of K steps
     _sampled_rows_check(gpu, n, n, n, "bf16", seed=n)
@@ -525,7 +525,7 @@ def test_uneven_k_8192x8192x8176(gpu, dtype, layout):
 
 
 def test_full_size_8192_fp8_sampled_rows_and_k_major_bf16(gpu):
-    # BASELINE config 4 at full size (e4m3fn codes with per-tensor scales, bf16 out), sampled rows against the
+    # benchmark configuration 4 at full size (e4m3fn codes with per-tensor scales, bf16 out), sampled rows against the
     # dequantised fp64 product; and config 2 with B stored K-major (the `b.T` view), sampled rows
     n = 8192
     g = torch.Generator(device="cpu").manual_seed(1)

@@ -134,7 +134,7 @@ def test_mfma_decodes_every_fp4_code_and_scale_exactly(gpu):
 
 @pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
 def test_full_size_8192_sampled_rows(gpu, fmt):
-    # BASELINE config 5 at full size, checked on sampled rows against the fp64 oracle
+    # benchmark configuration 5 at full size, checked on sampled rows against the fp64 oracle
     n = 8192
     a, sa, b, sb = _operands(np.random.default_rng(0), n, n, n, fmt)
     t = lambda x: torch.from_numpy(x).to(gpu)

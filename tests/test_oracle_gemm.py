@@ -50,7 +50,7 @@ def test_single_nonzero_checks_tile_addressing_and_edge_wrap():
 
 
 def test_config1_512_fp16_within_reference_tolerance():
-    # BASELINE config 1: 512^3 fp16, tiles 64x64x32, GROUP_M = 8; tolerance of 03:368 (atol 1e-2, rtol 0)
+    # benchmark configuration 1: 512^3 fp16, tiles 64x64x32, GROUP_M = 8; tolerance of 03:368 (atol 1e-2, rtol 0)
     rng = np.random.default_rng(0)
     a = formats.round_fp16(rng.standard_normal((512, 512)).astype(np.float32))
     b = formats.round_fp16(rng.standard_normal((512, 512)).astype(np.float32))
