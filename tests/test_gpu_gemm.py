@@ -277,6 +277,31 @@ def test_row_major_fp8_b_runs_the_mfma_kernels_bit_exactly(gpu, fmt, tdt, shape)
     assert torch.equal(triton_amd.matmul(ta, wide[:, 16:16 + N], out_dtype=torch.float32), got)
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_four_wave_fp8_kernel_with_a_row_major_b_is_bit_exact(gpu, monkeypatch, fmt, tdt, programs):
+    # the four-wave fp8 kernel's form for B[K, N]: 128 k rows of 256 bytes per stage, fragments by 8-bit transpose reads.
+    # Whole tiles and pairs of K steps; one and several tiles per program; every epilogue the form has (fp32: general;
+    # fp16, bf16: lean); a pitch wider than the row.  Integer data: the bits of the exact product and of the K-major call.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", "6")
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(fmt))
+    for (M, N, K, pad) in [(256, 256, 256, 0), (768, 512, 512, 0), (512, 768, 1280, 64), (256, 1024, 2048, 16)]:
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+        ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
+        wide = torch.zeros(K, N + pad, dtype=torch.uint8, device=gpu).view(tdt)
+        wide[:, :N] = torch.from_numpy(formats.encode_fp8(b, fmt)).to(gpu).view(tdt)
+        tb = wide[:, :N]                                                                    # [K, N], pitch N + pad
+        want = a.astype(np.float64) @ b.astype(np.float64)
+        got32 = triton_amd.matmul(ta, tb, out_dtype=torch.float32)
+        assert np.array_equal(to_np(got32), want), (M, N, K, fmt, programs)
+        assert torch.equal(got32, triton_amd.matmul(ta, tb.t().contiguous().t(), out_dtype=torch.float32))
+        for out, name in ((torch.float16, "fp16"), (torch.bfloat16, "bf16")):
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=out))
+            assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype=name)), (M, N, K, fmt, programs, name)
+
+
 def test_large_row_major_fp8_b_runs_on_the_fp8_mfmas_inside_the_c_abi(gpu):
     # 03:378-380 pre-transposes b on the host for fp8; here mi355_gemm itself takes the row-major B (no copy of B in
     # the wrapper): told apart from the strided kernel by time, equal to the K-major call bit for bit (the same

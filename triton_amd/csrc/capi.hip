@@ -205,7 +205,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // (an epilogue addend: instantiations of their own)
   // (fp8 from three quarters of a round: at 144 tiles the eight-wave kernel is 4-7 % ahead - 3072^3 1520 vs
   // 1450, 3072x3072x8192 2040 vs 1890 TFLOP/s -, at 196 tiles the four-wave one by 2 %, at 225 by 13 %)
-  const bool w128_ok = is8 ? b_kmajor && gemm_wave128_f8_ok(p) : gemm_wave128_ok(p, b_kmajor, in_dtype);
+  const bool w128_ok = is8 ? gemm_wave128_f8_ok(p, b_kmajor) : gemm_wave128_ok(p, b_kmajor, in_dtype);
   if (tiles256 * (is8 ? 4 : 2) >= cus * (is8 ? 3 : 1) && w128_ok) tile = 6;
   tile = tile_arg >= 0 ? tile_arg : knob(knobs().tile, tile);
   // 16-bit products whose 256 x 256 tiles fill the last round of CUs badly (or whose M is a multiple of 192 only): the
@@ -255,7 +255,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && w128_ok) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && tile == 6 && w128_ok) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)

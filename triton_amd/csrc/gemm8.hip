@@ -1,5 +1,6 @@
 // fp8 (e4m3fn / e5m2) instantiation of the tiled MFMA GEMM core: 64 elements per K step, one
-// 32x32x64 f8f6f4 MFMA sub-step.  Every kernel form takes both operands K-major (the layout the reference uses
+// 32x32x64 f8f6f4 MFMA sub-step (large products with whole tiles run the four-wave kernel of gemm_wave128.hip instead,
+// either B layout).  Every kernel form here takes both operands K-major (the layout the reference uses
 // for fp8: `matmul(a, b.T)` with b stored [N, K], python/tutorials/03-matrix-multiplication.py:378-382,
 // python/tutorials/09-persistent-matmul.py:396-407); a row-major B[K, N] (what `matmul(a, b)` passes without that
 // host-side transpose) runs the one-barrier-per-step form, which transposes it on its way out of LDS.

@@ -504,8 +504,16 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 // loads straight from global memory - the same two chunks per 128-byte step as from LDS, zeros beyond K, the masked
 // tail of the reference's loop (python/tutorials/03-matrix-multiplication.py:297-298) - into the fragment registers
 // that the pipeline has free at that point (it already holds the next tile's first B and A fragments in the others).
-template <int FMT, int EPI, bool TAIL = false>
+// B_KMAJOR = false: B is row-major [K, N].  Its stage holds the K step's 128 k rows of 256 bytes (wave w loads the rows
+// 32 w .. 32 w + 31, four per load); the 16-byte chunk c of row k lives in chunk c ^ g(k), g(k) = (k & 7) | 8 ((k >> 4) & 1),
+// and a B fragment is four 8-bit transpose reads (ds_read_b64_tr_b8: within 16 lanes, lane 2 r + h addresses the bytes
+// 8 h .. 8 h + 7 of row r, lane j receives column j of the 8 rows) of the rows 16 kg + {0, 8, 64, 72} + l16 / 2 - the K
+// positions of the two chunks that the A fragment of the same lane group holds, in the same order.  g is the same for
+// the four reads of a lane (they differ in bits 3 and 6 of k), so a fragment has one address and four immediates;
+// the 8 rows x 2 chunks that a half-wave reads fall on 16 different bank groups.
+template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
+  static_assert(B_KMAJOR || !TAIL, "the K tail loads K-contiguous fragments");
 #if MI355_DEVICE_PASS
   constexpr int BM = 256, BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
@@ -535,8 +543,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   for (int q = 0; q < 8; q++) {
     const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
     voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
-    voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
+    if constexpr (B_KMAJOR) {
+      voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
+    } else {
+      // load q of the wave: k rows 4 q .. 4 q + 3 of its 32 (lane i: row i / 16, physical chunk i % 16)
+      const unsigned kr = 4 * q + (lane >> 4), g = (kr & 7) | (((kr >> 4) & 1) << 3);
+      voffB[q] = kr * (unsigned)p.ldb + (((lane & 15) ^ g) * 16) - (unsigned)((q - 4) * 1024);
+    }
   }
+  const int64_t kstepB = B_KMAJOR ? (int64_t)ROWB : (int64_t)ROWB * p.ldb;   // bytes from one K step of B to the next
   // scalar bases of the K step the loads are fetching (two K steps ahead of the MFMAs)
   const char* fA;
   const char* fB;
@@ -546,13 +561,16 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
   const char* pA = nullptr;
   const char* pB = nullptr;
-  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
+  // (row-major B: the K step's 128 rows of 256 bytes are 256 lines, line L = half L & 1 of row L / 2)
+  const unsigned voffPA = (lane & 15) * (unsigned)p.lda;
+  const unsigned voffPB = B_KMAJOR ? (lane & 7) * (unsigned)p.ldb : ((lane & 7) >> 1) * (unsigned)p.ldb + (lane & 1) * 128;
   auto set_fill_tile = [&](int fm, int fn) {
     fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
-    fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
+    fB = B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb : p.B + (int64_t)fn * BN + (int64_t)(wave * 32) * p.ldb;
     if constexpr (PF) {
       pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
-      pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
+      pB = B_KMAJOR ? p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb
+                    : p.B + (int64_t)fn * BN + (int64_t)((fm & 7) * 16 + wave * 4) * p.ldb;
     }
   };
   set_fill_tile(pm, pn);
@@ -580,6 +598,28 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     i32x4 hi = *(LDS_PTR(const i32x4))(base[1] + off);
     return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
   };
+  // row-major B: the address of fragment 0 in stage 0; fragment t is the chunk index XOR t (t < 8 and the term of
+  // wn, 8, touch different bits than each other, g any of them)
+  unsigned trB = 0;
+  if constexpr (!B_KMAJOR) {
+    const unsigned kr = 16 * kg + (l16 >> 1), g = (kr & 7) | (((kr >> 4) & 1) << 3);
+    trB = lds0 + A_BYTES + kr * BN + (((wn * 8) ^ g) << 4) + (l16 & 1) * 8;
+  }
+  auto read_b = [&](auto T_, auto SO_) {   // B fragment t of the stage at byte offset SO
+    constexpr int t = decltype(T_)::value, so = decltype(SO_)::value;
+    if constexpr (B_KMAJOR) {
+      return read_frag(fragB, so + t * 16 * ROWB);
+    } else {
+      const unsigned ad = (trB ^ (unsigned)(t << 4)) + so;
+      typedef int i32x2v __attribute__((ext_vector_type(2)));
+      const i32x2v r0 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS_PTR(i32x2v))(uintptr_t)ad);
+      const i32x2v r1 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS_PTR(i32x2v))(uintptr_t)(ad + 8 * BN));
+      const i32x2v r2 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS_PTR(i32x2v))(uintptr_t)(ad + 64 * BN));
+      const i32x2v r3 = __builtin_amdgcn_ds_read_tr8_b64_v2i32((LDS_PTR(i32x2v))(uintptr_t)(ad + 72 * BN));
+      const i32x4 lo = __builtin_shufflevector(r0, r1, 0, 1, 2, 3), hi = __builtin_shufflevector(r2, r3, 0, 1, 2, 3);
+      return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  };
   i32x8 a0[MH], a1[MH], b[2][NT];
 
   f32x4 acc[MT][NT];
@@ -593,24 +633,23 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
   static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + kstepB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
-  fB += 2 * ROWB;
+  fB += 2 * kstepB;
   if constexpr (PF) {
     // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
     // the loop's waits leave outstanding from the first step on
     const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
     touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, lds0 + 2 * STAGE + wave * 256);
-    touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
+    touch_line_sbase<false, 8>(pB + k2 * kstepB, voffPB, 0u);
     touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
-    touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
+    touch_line_sbase<false, 8>(pB + k3 * kstepB, voffPB, 0u);
     pA += 2 * ROWB;
-    pB += 2 * ROWB;
+    pB += 2 * kstepB;
   }
   wait_vmcnt<16 + (PF ? 4 : 0)>();
   block_barrier();
-#pragma unroll
-  for (int t = 0; t < NT; t++) b[0][t] = read_frag(fragB, t * 16 * ROWB);
+  static_for<NT>([&](auto T_) { b[0][decltype(T_)::value] = read_b(T_, std::integral_constant<int, 0>{}); });
 #pragma unroll
   for (int t = 0; t < MH; t++) a0[t] = read_frag(fragA, t * 16 * ROWB);
 
@@ -633,7 +672,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     static_for<MH * NT>([&](auto N_) {
       constexpr int n = decltype(N_)::value, i = n / NT, j = n % NT;
       mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
-      if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
+      if constexpr (n < NT) b[nxt][n] = read_b(std::integral_constant<int, n>{}, std::integral_constant<int, sn>{});
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
       if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
@@ -650,11 +689,11 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   int fk = 2, ftile = tile;
   // the lines to touch: K step fk + PFD of the fill tile, or (past its end) the step being fetched anyway
   auto touch_a = [&]() { return PF ? pA + (fk + PFD < nk ? PFD * ROWB : 0) : nullptr; };
-  auto touch_b = [&]() { return PF ? pB + (fk + PFD < nk ? PFD * ROWB : 0) : nullptr; };
+  auto touch_b = [&]() { return PF ? pB + (fk + PFD < nk ? PFD * kstepB : (int64_t)0) : nullptr; };
   auto advance = [&]() {
     fA += ROWB;
-    fB += ROWB;
-    if constexpr (PF) { pA += ROWB; pB += ROWB; }
+    fB += kstepB;
+    if constexpr (PF) { pA += ROWB; pB += kstepB; }
     if (++fk == nk) {
       fk = 0;
       if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
@@ -723,22 +762,28 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #endif
 }
 
-template <int FMT, int EPI, bool TAIL = false>
+template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
   constexpr int smem = 2 * 2 * 256 * 128 + 1024;   // (two stages and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
   const int tiles = (p.M / 256) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_f8_kernel<FMT, EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
-int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
+int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, hipStream_t stream) {
+  if (!b_kmajor) {   // (gemm_wave128_f8_ok: whole pairs of K steps, no addend)
+    const int lean = lean_epilogue_type(p);
+    if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3, false, false>(p, stream) : launch_wave128_f8<0, 3, false, false>(p, stream);
+    if (lean == 2) return e5m2 ? launch_wave128_f8<1, 4, false, false>(p, stream) : launch_wave128_f8<0, 4, false, false>(p, stream);
+    return e5m2 ? launch_wave128_f8<1, 0, false, false>(p, stream) : launch_wave128_f8<0, 0, false, false>(p, stream);
+  }
   if (p.k_bytes % 256 != 0) {   // (gemm_wave128_f8_ok: no addend then)
     const int lean = lean_epilogue_type(p);
     if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3, true>(p, stream) : launch_wave128_f8<0, 3, true>(p, stream);
@@ -752,12 +797,15 @@ int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, hipStream_t stream) {
   return e5m2 ? launch_wave128_f8<1, 0>(p, stream) : launch_wave128_f8<0, 0>(p, stream);
 }
 
-// fp8 (K-major B): whole tiles, at least one pair of 128-byte K steps; what is left behind the last pair is the TAIL
-// form's, which exists without the addend
-bool gemm_wave128_f8_ok(const GemmArgs& p) {
+// fp8: whole tiles, at least one pair of 128-byte K steps; with a K-major B, what is left behind the last pair is the
+// TAIL form's, which exists without the addend
+bool gemm_wave128_f8_ok(const GemmArgs& p, bool b_kmajor) {
   if (!(p.M % 256 == 0 && p.N % 256 == 0 && p.k_bytes % 16 == 0 && p.k_bytes >= 256)) return false;
   if (p.k_bytes % 256 != 0 && p.aux) return false;
-  return p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
+  if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
+  if (b_kmajor) return p.ldb * 8 + p.k_bytes < (1ll << 31);
+  // row-major B: whole pairs of K steps, no addend; 32 rows plus a tile row within 32-bit lane offsets
+  return p.k_bytes % 256 == 0 && !p.aux && p.ldb % 16 == 0 && p.ldb * 32 + 256 < (1ll << 32);
 }
 
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
