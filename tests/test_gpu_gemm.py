@@ -696,6 +696,32 @@ def test_fused_addends_in_the_four_wave_fp8_kernel(gpu, monkeypatch, fmt, tdt):
             assert bits_equal(got, gemm.dot_epilogue(a, b, add=add_np)), (fmt, add_dt, add_np.shape)
 
 
+@pytest.mark.parametrize("tile", [None, 0, 1, 2, 3, 4, 5, 6, 7])
+def test_row_major_fp8_b_under_every_tile_choice_with_addend_activation_and_fp8_output(gpu, monkeypatch, tile):
+    # whatever kernel the tuning knob asks for, a row-major fp8 B ends on a kernel that has the layout (the four-wave
+    # one for 6, the 128x128 tiles for 1, the 256x256 one-barrier-per-step tiles otherwise); epilogues with an addend,
+    # leaky_relu and an fp8 result go through the tile kernels' general epilogue.  Integer data: exact, and bit-equal
+    # to the K-major call of the same product.
+    if tile is not None:
+        set_knob(monkeypatch, "MI355_GEMM_TILE", tile)
+    M, N, K = 512, 768, 512
+    rng = np.random.default_rng(3 if tile is None else tile)
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+    z = rng.integers(-4, 5, size=(M, N)).astype(np.float32)
+    ta = torch.from_numpy(formats.encode_fp8(a, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+    tb = torch.from_numpy(formats.encode_fp8(b, "e4m3")).to(gpu).view(torch.float8_e4m3fn)     # [K, N] row-major
+    tbk = tb.t().contiguous().t()
+    tz = torch.from_numpy(z).to(gpu)
+    assert np.array_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32)), a.astype(np.float64) @ b.astype(np.float64))
+    got = triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=tz, activation="leaky_relu")
+    assert bits_equal(to_np(got), gemm.dot_epilogue(a, b, add=z, activation="leaky_relu"))
+    assert torch.equal(got, triton_amd.matmul(ta, tbk, out_dtype=torch.float32, add=tz, activation="leaky_relu"))
+    out8 = triton_amd.matmul(ta, tb, out_dtype=torch.float8_e4m3fn, a_scale=0.125)
+    assert torch.equal(out8.view(torch.uint8), triton_amd.matmul(ta, tbk, out_dtype=torch.float8_e4m3fn, a_scale=0.125).view(torch.uint8))
+    assert np.array_equal(out8.view(torch.uint8).cpu().numpy(), formats.encode_fp8((a @ b) * 0.125, "e4m3"))
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512),
                                    (1024, 32, 256)])
