@@ -25,7 +25,9 @@
  * enum value or the meaning of an argument is added; a binding built for version V works with any library that
  * reports at least V.  (1: GEMM, MX GEMM, attention, dequant; 2: stream-K with and without a workspace, chained
  * product, clock probe, environment refresh, MI355_ESCRATCH, head dims 16 / 32 / 256 in the backward, fp8 output
- * of the MFMA epilogues; 3: MFMA burn probe, per-device properties.) */
+ * of the MFMA epilogues; 3: MFMA burn probe with its block-scaled shapes, per-device properties, fp8 attention forward at
+ * head dims 16 / 32 / 256, a row-major fp8 B on the MFMA kernels, block-scaled products with any K that is a multiple of
+ * 32 and scale rows of any pitch on the MFMA kernels.) */
 #define MI355_ABI_VERSION 3
 
 #ifdef __cplusplus
@@ -88,8 +90,8 @@ enum {
  *   python/tutorials/09-persistent-matmul.py:48-102 (kernel), :105-138 (`matmul`, fp8e4nv)
  * i.e. what the generated launcher third_party/amd/backend/driver.py:326-377 does for them.
  * Same arguments as the kernel: three pointers, M N K, six strides (any strides are accepted;
- * the MFMA path needs a unit stride on one axis of each operand, anything else runs a
- * slower strided kernel on the GPU), plus ACTIVATION.  in_dtype is the type of A and B
+ * the MFMA path needs a unit stride on one axis of each operand and rows of whole 16-byte chunks -
+ * either layout of B for every type -, anything else runs a slower strided kernel on the GPU), plus ACTIVATION.  in_dtype is the type of A and B
  * (they must match, python/triton/language/semantic.py:1355).  a_scale / b_scale are
  * optional device pointers to one fp32 each (NULL = 1.0): per-tensor dequantisation
  * scales for fp8 inputs, applied to the fp32 accumulator before activation and cast.
@@ -112,8 +114,9 @@ int mi355_gemm(const void* A, const void* B, void* C,
  * 5 = the eight-wave pipelined kernel as persistent programs (one per CU, MI355_GEMM_PROGRAMS
  * overrides) that walk their tiles as one stream of K steps, the schedule of
  * python/tutorials/09-persistent-matmul.py:141-190, 6 = four waves of 128x128 from 16x16x32
- * (fp8: 16x16x128) MFMAs on 256x256 tiles (whole tiles, K at least 128 elements - fp8: K bytes a multiple of 256 -, a row-major B with a
- * pitch that is a multiple of 512 bytes, fp8 with a K-major B; the heuristic's choice for such products from
+ * (fp8: 16x16x128) MFMAs on 256x256 tiles (whole tiles, K at least 128 elements - fp8: at least 256 bytes, any multiple of 16 with a
+ * K-major B, a multiple of 256 with a row-major one -, a row-major 16-bit B with a pitch that is a multiple of 512 bytes; the
+ * heuristic's choice for such products from
  * 128 tiles on, fp8 from 192; with more tiles than MI355_GEMM_PROGRAMS, default the CU count, its programs
  * take ceil(tiles / programs) tiles each as one stream of K steps)
  * (a kernel that does not exist for the dtype or shape falls back to the nearest one).  group_m: the
