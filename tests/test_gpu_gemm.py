@@ -937,6 +937,26 @@ def test_four_wave_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, dt
     assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got), "tiles of 256 rows"
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_four_wave_fp8_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, fmt, tdt, programs):
+    # the fp8 form of the same tiles (K-major B, 16-bit C): six A fragments per wave, 14 loads per K step; one and
+    # several tiles per program.  Integer data: the bits of the exact product, and of the 256-row tiles' result.
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(fmt))
+    for (M, N, K) in [(192, 256, 256), (1536, 1024, 1280), (3072, 768, 512), (576, 512, 2048)]:
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+        ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
+        tb = torch.from_numpy(formats.encode_fp8(b, fmt)).to(gpu).view(tdt).t()
+        for out, name in ((torch.bfloat16, "bf16"), (torch.float16, "fp16")):
+            set_knob(monkeypatch, "MI355_GEMM_TILE_M", "192")
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=out))
+            assert bits_equal(got, gemm.matmul_closed_form(a, b.T, out_dtype=name)), (M, N, K, fmt, programs, name)
+            set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
+            assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=out)), got)
+
+
 def test_3072_cubed_takes_the_192_row_tiles_and_matches_sampled_rows(gpu):
     # 144 tiles of 256 x 256 for 256 CUs, 192 tiles of 192 x 256: the size heuristic picks the latter
     rng = np.random.default_rng(11)

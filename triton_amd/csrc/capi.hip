@@ -219,6 +219,20 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 192;
     }
   }
+  // fp8 likewise (K-major B, 16-bit C), from three quarters of a round of the 192-row tiles on.  Flushed do_bench, e4m3,
+  // 256-row choice / 192-row tiles: 3072^3 (144 / 192 tiles) 1100 / 1565 TFLOP/s, 3072 x 3072 x 8192 1365 / 2145, 2304 x
+  // 4096 x 4096 1220 / 1785, 4608 x 4096 x 4096 (288 / 384) 1600 / 2070, 6144^3 (576 / 768) 2510 / 2805, 1536 x 8192 x 8192
+  // (192 / 256) 2100 / 2680; not taken where they fill worse: 3840 x 3840 x 4096 (225 / 300) 2270 / 1530, 5376 x 5120 x
+  // 4096 (420 / 560) 2185 / 1995
+  if (is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 192) && gemm_wave128_f8_192_ok(p, b_kmajor)) {
+    auto fill = [&](long t) { return t <= 0 ? 0.0 : (double)t / (double)(((t + cus - 1) / cus) * cus); };
+    const long tiles192 = (long)(M / 192) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    if (want == 192 || (want == 0 && tiles192 * 4 >= cus * 3 && (tile != 6 || fill(tiles192) > fill(tiles256) + 0.08))) {
+      tile = 6;
+      p.tile_m = 192;
+    }
+  }
   // and on tiles of 128 x 256 where the 256 x 256 tiles are too few for their kernel (less than half a round) but these
   // fill most of one round (2560^3: 100 and 200 tiles; 716 -> 825 TFLOP/s against the 128 x 128 tiles)
   if (!is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 128) && p.tile_m == 0 &&
@@ -255,7 +269,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && w128_ok) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
+  if (is8 && tile == 6 && (p.tile_m == 192 || w128_ok)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)

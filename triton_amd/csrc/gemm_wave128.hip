@@ -511,13 +511,17 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 // positions of the two chunks that the A fragment of the same lane group holds, in the same order.  g is the same for
 // the four reads of a lane (they differ in bits 3 and 6 of k), so a fragment has one address and four immediates;
 // the 8 rows x 2 chunks that a half-wave reads fall on 16 different bank groups.
-template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true>
+// BM = 192: tiles of 192 x 256 (a wave: 96 x 128, six A fragments), for products whose 256 x 256 tiles fill the last
+// round of CUs badly - as in the 16-bit kernel; lean epilogue, whole pairs of K steps.
+template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
+  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
   static_assert(B_KMAJOR || !TAIL, "the K tail loads K-contiguous fragments");
 #if MI355_DEVICE_PASS
-  constexpr int BM = 256, BN = 256, ROWB = 128;
-  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
-  constexpr int MT = 8, NT = 8, MH = MT / 2;
+  constexpr int BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
+  constexpr int MT = BM / 32, NT = 8, MH = MT / 2;
+  constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
@@ -538,11 +542,11 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   // ---- direct loads, exactly as in the 16-bit kernel (the tiles are the same bytes): a lane offset per load,
   // one scalar base per operand that moves with the K step being fetched
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[8], voffB[8];
+  unsigned voffA[LA], voffB[8];
 #pragma unroll
   for (int q = 0; q < 8; q++) {
     const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
-    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    if (q < LA) voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
     if constexpr (B_KMAJOR) {
       voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
     } else {
@@ -562,21 +566,22 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   const char* pA = nullptr;
   const char* pB = nullptr;
   // (row-major B: the K step's 128 rows of 256 bytes are 256 lines, line L = half L & 1 of row L / 2)
-  const unsigned voffPA = (lane & 15) * (unsigned)p.lda;
+  const unsigned voffPA = (lane % (BM / 16)) * (unsigned)p.lda;
   const unsigned voffPB = B_KMAJOR ? (lane & 7) * (unsigned)p.ldb : ((lane & 7) >> 1) * (unsigned)p.ldb + (lane & 1) * 128;
   auto set_fill_tile = [&](int fm, int fn) {
-    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fA = p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda;
     fB = B_KMAJOR ? p.B + ((int64_t)fn * BN + wave * 64) * p.ldb : p.B + (int64_t)fn * BN + (int64_t)(wave * 32) * p.ldb;
     if constexpr (PF) {
-      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * (BM / 4) + wave * (BM / 16)) * p.lda;
       pB = B_KMAJOR ? p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb
                     : p.B + (int64_t)fn * BN + (int64_t)((fm & 7) * 16 + wave * 4) * p.ldb;
     }
   };
   set_fill_tile(pm, pn);
+  auto load_of = [](int slot) constexpr { return slot < LA ? slot : 8 + slot - LA; };   // load slot -> j (A: 0 .. LA-1, B: 8 .. 15)
   auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned dst = stage_base + (j < 8 ? wave * (LA * 1024) : A_BYTES + wave * 8192) + 4096;
     if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
     else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
@@ -589,7 +594,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #pragma unroll
     for (int c = 0; c < 2; c++) {
       const unsigned slot = ((kg + 4 * c) ^ s) * 16;
-      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * 128 + l16) * ROWB + slot;
+      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * (BM / 2) + l16) * ROWB + slot;
       fragB[c] = (LDS_PTR(const char))lds_raw + A_BYTES + (wn * 128 + l16) * ROWB + slot;
     }
   }
@@ -632,22 +637,22 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   zero_acc();
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
-  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + kstepB, lds0 + STAGE, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA, fB, lds0, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA + ROWB, fB + kstepB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * kstepB;
   if constexpr (PF) {
     // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
     // the loop's waits leave outstanding from the first step on
     const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
-    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, lds0 + 2 * STAGE + wave * 256);
+    touch_line_sbase<true, BM / 16>(pA + k2 * ROWB, voffPA, lds0 + 2 * STAGE + wave * 256);
     touch_line_sbase<false, 8>(pB + k2 * kstepB, voffPB, 0u);
-    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, BM / 16>(pA + k3 * ROWB, voffPA, 0u);
     touch_line_sbase<false, 8>(pB + k3 * kstepB, voffPB, 0u);
     pA += 2 * ROWB;
     pB += 2 * kstepB;
   }
-  wait_vmcnt<16 + (PF ? 4 : 0)>();
+  wait_vmcnt<NLOADS + (PF ? 4 : 0)>();
   block_barrier();
   static_for<NT>([&](auto T_) { b[0][decltype(T_)::value] = read_b(T_, std::integral_constant<int, 0>{}); });
 #pragma unroll
@@ -674,11 +679,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
       if constexpr (n < NT) b[nxt][n] = read_b(std::integral_constant<int, n>{}, std::integral_constant<int, sn>{});
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
-      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs: the last two go into even slots)
+      constexpr int HALF = MH * NT, EXTRA = NLOADS > HALF / 2 ? NLOADS - HALF / 2 : 0;
+      if constexpr (n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      if constexpr (EXTRA > 0 && n % 2 == 0 && n >= HALF - 2 * EXTRA)
+        issue(std::integral_constant<int, load_of(HALF / 2 + (n - (HALF - 2 * EXTRA)) / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (PF) {
-      touch_line_sbase<true, 16>(tA, voffPA, lds0 + 2 * STAGE + wave * 256);
+      touch_line_sbase<true, BM / 16>(tA, voffPA, lds0 + 2 * STAGE + wave * 256);
       touch_line_sbase<false, 8>(tB, voffPB, 0u);
     }
   };
@@ -748,7 +757,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       }
     }
     mfma_drain(acc);
-    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    int em = pm * BM + wm * (BM / 2), en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
@@ -762,22 +771,26 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 #endif
 }
 
-template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true>
+template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
 static int launch_wave128_f8(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + 1024;   // (two stages and the 1 KiB that the L2 touches land in)
+  constexpr int smem = 2 * (BM + 256) * 128 + 1024;   // (two stages and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int tiles = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / BM) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_f8_kernel<FMT, EPI, TAIL, B_KMAJOR, BM><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, hipStream_t stream) {
+  if (p.tile_m == 192) {   // (gemm_wave128_f8_192_ok: K-major B, lean epilogue, whole pairs of K steps)
+    if (lean_epilogue_type(p) == 1) return e5m2 ? launch_wave128_f8<1, 3, false, true, 192>(p, stream) : launch_wave128_f8<0, 3, false, true, 192>(p, stream);
+    return e5m2 ? launch_wave128_f8<1, 4, false, true, 192>(p, stream) : launch_wave128_f8<0, 4, false, true, 192>(p, stream);
+  }
   if (!b_kmajor) {   // (gemm_wave128_f8_ok: whole pairs of K steps, no addend)
     const int lean = lean_epilogue_type(p);
     if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3, false, false>(p, stream) : launch_wave128_f8<0, 3, false, false>(p, stream);
@@ -806,6 +819,13 @@ bool gemm_wave128_f8_ok(const GemmArgs& p, bool b_kmajor) {
   if (b_kmajor) return p.ldb * 8 + p.k_bytes < (1ll << 31);
   // row-major B: whole pairs of K steps, no addend; 32 rows plus a tile row within 32-bit lane offsets
   return p.k_bytes % 256 == 0 && !p.aux && p.ldb % 16 == 0 && p.ldb * 32 + 256 < (1ll << 32);
+}
+
+// fp8 on tiles of 192 x 256: M a multiple of 192, K-major B, whole pairs of K steps, a 16-bit C through the lean epilogue
+bool gemm_wave128_f8_192_ok(const GemmArgs& p, bool b_kmajor) {
+  if (!(b_kmajor && p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  if (lean_epilogue_type(p) == 0) return false;
+  return p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
 }
 
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype) {
