@@ -93,6 +93,33 @@ def test_four_wave_kernels_k_tails_are_bit_exact(gpu, monkeypatch, fmt, programs
             assert bits_equal(got, rnd(ref32)), (fmt, K, programs, out)
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
+def test_four_wave_kernels_on_tiles_of_192_rows_are_bit_exact(gpu, monkeypatch, fmt, programs):
+    # M a multiple of 192: the four-wave block-scaled kernels also run on tiles of 192 x 256 (six A fragments per wave,
+    # 48 rows of operands and scales per wave and load group; chosen by themselves where those tiles fill the CUs
+    # better, forced here), one and several tiles per program, K of one to several scale-load groups.  Exact data
+    # with scales 1/2, 1, 2: the oracle's bits, and those of the 256-row tiles.
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    rng = np.random.default_rng(programs + len(fmt))
+    t = lambda x: torch.from_numpy(x).to(gpu)
+    for (M, N, K) in [(192, 256, 1024), (1536, 1024, 2048), (3072, 768, 1024), (576, 512, 5120)]:
+        if fmt == "mxfp4":
+            a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
+        else:
+            a = formats.encode_fp8(rng.integers(-4, 5, size=(M, K)).astype(np.float32), "e4m3")
+            b = formats.encode_fp8(rng.integers(-4, 5, size=(N, K)).astype(np.float32), "e4m3")
+            sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+            sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
+        for out, rnd in ((torch.bfloat16, formats.round_bf16), (torch.float16, lambda x: x.astype(np.float16).astype(np.float32))):
+            set_knob(monkeypatch, "MI355_GEMM_TILE_M", "192")
+            got = _run(gpu, a, sa, b, sb, fmt, out)
+            assert bits_equal(got, rnd(ref32)), (fmt, M, N, K, programs, out)
+            set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
+            assert bits_equal(_run(gpu, a, sa, b, sb, fmt, out), got)
+
+
 def test_scale_blocks_are_applied_per_row_and_per_32_elements(gpu):
     # all-ones data; one scale byte raised: exactly one row (or column) of C changes by 32 * (2^d - 1)
     M = N = 128; K = 512

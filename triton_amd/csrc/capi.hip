@@ -461,9 +461,27 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
     const bool eight_wave_runs = p.k_bytes % 64 == 0 && lds_a % 4 == 0 && lds_b % 4 == 0 && aligned(sA, 4) && aligned(sB, 4);
     return !eight_wave_runs || (int64_t)((tail + 127) / 128) * cost <= (int64_t)(p.k_bytes - tail) / 128;
   };
-  if (fmt == MI355_MXFP4 && tiles256 * 2 >= cus && gemm_wave128_mxfp4_ok(p) && tail_pays(512, 9)) tile = 6;
+  // (below half a round of tiles the four-wave kernels still win where K is long - flushed do_bench, four-wave / 128 x 128
+  // tiles: MXFP4 2048 x 2048 x 4096 1010 / 745 TFLOP/s, 1024 x 1024 x 4096 240 / 198, MXFP8 2048 x 2048 x 4096 636 / 407,
+  // 1536 x 1536 x 2048 278 / 219 - and lose where it is short: MXFP4 2048 x 2048 x 1024 427 / 504, 1024^3 117 / 139)
+  const bool enough = tiles256 * 2 >= cus || (tiles256 >= 16 && p.k_bytes >= 1024);
+  if (fmt == MI355_MXFP4 && enough && gemm_wave128_mxfp4_ok(p) && tail_pays(512, 9)) tile = 6;
   // (MXFP8 likewise: 2530-2570 vs 2110-2240)
-  if (fmt == MI355_MXFP8 && tiles256 * 2 >= cus && gemm_wave128_mxfp8_ok(p) && tail_pays(1024, 21)) tile = 6;
+  if (fmt == MI355_MXFP8 && enough && gemm_wave128_mxfp8_ok(p) && tail_pays(1024, 21)) tile = 6;
+  // the same kernels on tiles of 192 x 256 where those fill the CUs better (as for the 16-bit and fp8 products).  Flushed
+  // do_bench, 256-row choice / 192-row tiles, MXFP4: 3072^3 1750 / 2100 TFLOP/s, 4608 x 4096 x 4096 2475 / 2885, 6144^3
+  // 3725 / 3970, 1536 x 8192 x 8192 3205 / 3780, 1536 x 2048 x 8192 880 / 1080; MXFP8: 1255 / 1420, 1480 / 1830, 2275 / 2520,
+  // 1945 / 2345, 519 / 630; not taken where they fill worse (3840 x 3840 x 4096: 3080 / 2230)
+  if ((knobs().tile == UNSET || knobs().tile_m == 192) && gemm_wave128_mx_192_ok(p, fmt == MI355_MXFP4 ? 512 : 1024)) {
+    auto fill = [&](long t) { return t <= 0 ? 0.0 : (double)t / (double)(((t + cus - 1) / cus) * cus); };
+    const long tiles192 = (long)(M / 192) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    const bool enough192 = tiles192 * 2 >= cus || (tiles192 >= 16 && p.k_bytes >= 1024);
+    if (want == 192 || (want == 0 && enough192 && (tile != 6 || fill(tiles192) > fill(tiles256) * 1.1))) {
+      tile = 6;
+      p.tile_m = 192;
+    }
+  }
   tile = knob(knobs().tile, tile);
   p.num_programs = knob(knobs().programs, cus);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);

@@ -46,13 +46,16 @@ __device__ __forceinline__ void settle_tail(R&... r) {
 // steps, and what is left of each row (32 .. 992 bytes, the same for every tile) follows in K steps whose fragments and
 // scale bytes every lane loads straight from global memory - zeros (and the scale 1) beyond K - into the registers that
 // the pipeline has free at that point, a quarter of the wave's tile at a time.
-template <int EPI, bool TAIL = false>
+// BM = 192: tiles of 192 x 256, as in the MXFP4 kernel below.
+template <int EPI, bool TAIL = false, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
+  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
-  constexpr int BM = 256, BN = 256, ROWB = 128;
-  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
-  constexpr int MT = 8, NT = 8, MH = MT / 2;
-  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
+  constexpr int BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
+  constexpr int MT = BM / 32, NT = 8, MH = MT / 2;
+  constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (256 + BN) * 16;     // scale ring behind the two stages (A part: room for 256 rows)
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
@@ -74,11 +77,11 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   // (a lane offset per load - row, chunk, and the instruction offset taken back out - and one scalar base per
   // operand that moves with the K step being fetched)
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[8], voffB[8];
+  unsigned voffA[LA], voffB[8];
 #pragma unroll
   for (int q = 0; q < 8; q++) {
     const unsigned chunk = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
-    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    if (q < LA) voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
     voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
   // scalar bases of the tile the loads are fetching (two K steps ahead of the MFMAs)
@@ -92,22 +95,23 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
   const char* pA = nullptr;
   const char* pB = nullptr;
-  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
+  const unsigned voffPA = (lane % (BM / 16)) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
   const unsigned touch_lds = lds0 + SC_BASE + 2 * SC_SLOT + wave * 256;
   auto set_fill_tile = [&](int fm, int fn) {
-    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fA = p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda;
     fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
     if constexpr (PF) {
-      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * (BM / 4) + wave * (BM / 16)) * p.lda;
       pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
     }
-    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * (BM / 4)) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
   set_fill_tile(pm, pn);
+  auto load_of = [](int slot) constexpr { return slot < LA ? slot : 8 + slot - LA; };   // load slot -> j (A: 0 .. LA-1, B: 8 .. 15)
   auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned dst = stage_base + (j < 8 ? wave * (LA * 1024) : A_BYTES + wave * 8192) + 4096;
     if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
     else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
@@ -115,14 +119,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   // ---- scale loads: wave w fetches the 16 scale bytes (four K steps) of rows 64 w .. 64 w + 63 of A and of B
   const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
   auto issue_scales = [&](int g, auto SETTLE_) {   // group g of four K steps of the fill tile -> slot g & 1 (K steps come in eights)
-    const unsigned slot = lds0 + SC_BASE + (g & 1) * SC_SLOT + wave * 1024;
-    async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)g * 16, slot);
-    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)g * 16, slot + BM * 16);
+    const unsigned slot = lds0 + SC_BASE + (g & 1) * SC_SLOT;
+    // (192-row tiles: a wave fetches the scales of its 48 A rows, the lanes beyond sit the load out)
+    if (BM == 256 || lane < BM / 4) async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)g * 16, slot + wave * (BM / 4) * 16);
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)g * 16, slot + 256 * 16 + wave * 1024);
   };
   // scales of a K step: lane group kg supplies block kg of its row, fetched as one byte (ds_read_u8: it arrives in
   // byte 0, the position the MFMA's selector names, so no shift), one read per two MFMAs
-  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + kg;
-  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + kg;
+  const unsigned adrSA = lds0 + SC_BASE + (wm * (BM / 2) + l16) * 16 + kg;
+  const unsigned adrSB = lds0 + SC_BASE + 256 * 16 + (wn * 128 + l16) * 16 + kg;
   int sa[2][MT], sb[2][NT];
   auto read_scale = [&](auto OP_, auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 3) * 4
     constexpr int op = decltype(OP_)::value, set = decltype(SET_)::value, off = decltype(OFF_)::value;
@@ -146,7 +151,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
 #pragma unroll
     for (int c = 0; c < 2; c++) {
       const unsigned slot = ((MXFP8_CHUNK(kg, c)) ^ s) * 16;
-      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * 128 + l16) * ROWB + slot;
+      fragA[c] = (LDS_PTR(const char))lds_raw + (wm * (BM / 2) + l16) * ROWB + slot;
       fragB[c] = (LDS_PTR(const char))lds_raw + A_BYTES + (wn * 128 + l16) * ROWB + slot;
     }
   }
@@ -168,22 +173,22 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
 
   // ---- prologue: both stages requested, B and the first four A fragments of stage 0 read
   issue_scales(0, std::true_type{});
-  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA, fB, lds0, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * ROWB;
   if constexpr (PF) {
     // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
     // the loop's waits leave outstanding from the first step on
     const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
-    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, touch_lds);
+    touch_line_sbase<true, BM / 16>(pA + k2 * ROWB, voffPA, touch_lds);
     touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
-    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, BM / 16>(pA + k3 * ROWB, voffPA, 0u);
     touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
     pA += 2 * ROWB;
     pB += 2 * ROWB;
   }
-  wait_vmcnt<16 + (PF ? 4 : 0)>();
+  wait_vmcnt<NLOADS + (PF ? 4 : 0)>();
   block_barrier();
   static_for<MT + NT>([&](auto OP_) { read_scale(OP_, std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{}); });
   lds_wait<0>();
@@ -212,16 +217,26 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       mfma16_mxfp8(b[cur][j], a1[i], acc[MH + i][j], sb[cur][j], sa[cur][MH + i]);
       if constexpr (n < NT) b[nxt][n] = read_frag(fragB, sn + n * 16 * ROWB);
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
-      if constexpr (n % 2 == 0)
-        read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, nxt>{}, std::integral_constant<int, (UN >> 2) * SC_SLOT + (UN & 3) * 4>{});
-      if constexpr (n % 2 == 1) issue(std::integral_constant<int, n / 2>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      // (the next step's scales: one read per two MFMAs, or - 192-row tiles, 14 reads for 24 MFMAs - one per MFMA)
+      constexpr int HALF = MH * NT, NSC = MT + NT, EXTRA = NLOADS > HALF / 2 ? NLOADS - HALF / 2 : 0;
+      using OffNext = std::integral_constant<int, (UN >> 2) * SC_SLOT + (UN & 3) * 4>;
+      if constexpr (HALF >= 2 * NSC) {
+        if constexpr (n % 2 == 0) read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, nxt>{}, OffNext{});
+      } else {
+        if constexpr (n < NSC) read_scale(std::integral_constant<int, n>{}, std::integral_constant<int, nxt>{}, OffNext{});
+      }
+      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs: the last two go into even slots)
+      if constexpr (n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      if constexpr (EXTRA > 0 && n % 2 == 0 && n >= HALF - 2 * EXTRA)
+        issue(std::integral_constant<int, load_of(HALF / 2 + (n - (HALF - 2 * EXTRA)) / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       // (the scales of the K steps fk .. fk + 3 are requested in the third step of every four, into the slot whose
       // last reader was the read for the step before this one)
-      if constexpr ((U & 3) == 2 && n == 16) issue_scales(fk >> 2, std::false_type{});
+      // (between the last A load and the first B load, which sets M0 for its group again)
+      if constexpr ((U & 3) == 2 && n == 2 * LA) issue_scales(fk >> 2, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (PF) {
-      touch_line_sbase<true, 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
+      touch_line_sbase<true, BM / 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
       touch_line_sbase<false, 8>(pB + (fk + PFD < nk ? PFD * ROWB : 0), voffPB, 0u);
     }
     lds_wait<0>();
@@ -305,7 +320,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       }
     }
     mfma_drain(acc);
-    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    int em = pm * BM + wm * (BM / 2), en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
@@ -328,23 +343,25 @@ bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
          p.lds_a * 64 + p.k_bytes / 32 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 32 < (1ll << 31);
 }
 
-template <int EPI, bool TAIL = false>
+template <int EPI, bool TAIL = false, int BM = 256>
 static int launch_wave128_mxfp8(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
+  constexpr int smem = 2 * (BM + 256) * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_kernel<EPI, TAIL, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int tiles = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / BM) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp8_kernel<EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp8_kernel<EPI, TAIL, BM><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
+  if (p.tile_m == 192)   // (gemm_wave128_mx_192_ok: lean epilogue, whole groups of K steps)
+    return lean == 1 ? launch_wave128_mxfp8<3, false, 192>(p, stream) : launch_wave128_mxfp8<4, false, 192>(p, stream);
   if (p.k_bytes % 1024 != 0)
     return lean == 1 ? launch_wave128_mxfp8<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4, true>(p, stream) : launch_wave128_mxfp8<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp8<3>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4>(p, stream) : launch_wave128_mxfp8<0>(p, stream);
@@ -379,13 +396,18 @@ __device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32
 // steps, and what is left of each row (16 .. 496 bytes, the same for every tile) follows in K steps whose fragments and
 // scale bytes every lane loads straight from global memory - zeros (and the scale 1) beyond K - into the fragment and
 // scale registers that the pipeline has free at that point.
-template <int EPI, bool TAIL = false>
+// BM = 192: tiles of 192 x 256 (a wave: 96 x 128, six A fragments, 48 of the tile's A rows and scale rows to fetch), for
+// products whose 256 x 256 tiles fill the last round of CUs badly; lean epilogue, K steps in whole groups.
+template <int EPI, bool TAIL = false, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
+  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
-  constexpr int BM = 256, BN = 256, ROWB = 128;
-  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB
-  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (BM + BN) * 16;      // scale ring behind the two stages
-  constexpr int MT = 8, NT = 8, KS = 2, NM = MT * NT, NRD = MT + NT;
+  constexpr int BN = 256, ROWB = 128;
+  constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
+  constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (256 + BN) * 16;     // scale ring behind the two stages (A part: room for 256 rows)
+  constexpr int MT = BM / 32, NT = 8, KS = 2, NM = MT * NT, NRD = MT + NT;
+  constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
+  constexpr int EVERY = NM / 16;                                    // MFMAs per load slot: 4 (64 MFMAs) or 3 (48)
   extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
@@ -407,14 +429,14 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   // (a lane offset per load - row, chunk, and the instruction offset taken back out - and one scalar base per
   // operand that moves with the K step being fetched)
   const unsigned drow = lane >> 3, dslot = lane & 7;
-  unsigned voffA[8], voffB[8];
+  unsigned voffA[LA], voffB[8];
 #pragma unroll
   for (int q = 0; q < 8; q++) {
     // (LDS slot s of a row takes the row's chunk 2 (s & 3) + (s >> 2): the fragment reads keep their conflict-free
     // slots 4 ks + kg and find the chunks 2 kg + ks there - the two scale blocks of a lane are then neighbours)
     const unsigned slot = dslot ^ (((q & 1) * 4 + (lane >> 4)) & 7);
     const unsigned chunk = 2 * (slot & 3) + (slot >> 2);
-    voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
+    if (q < LA) voffA[q] = (drow + 8 * q) * (unsigned)p.lda + chunk * 16 - (unsigned)((q - 4) * 1024);
     voffB[q] = (drow + 8 * q) * (unsigned)p.ldb + chunk * 16 - (unsigned)((q - 4) * 1024);
   }
   // scalar bases (operands and scales) of the tile the loads are fetching, two K steps ahead of the MFMAs
@@ -428,31 +450,33 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   constexpr int PFD = MI355_W128_PREFETCH_DISTANCE;
   const char* pA = nullptr;
   const char* pB = nullptr;
-  const unsigned voffPA = (lane & 15) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
+  const unsigned voffPA = (lane % (BM / 16)) * (unsigned)p.lda, voffPB = (lane & 7) * (unsigned)p.ldb;
   const unsigned touch_lds = lds0 + SC_BASE + 2 * SC_SLOT + wave * 256;
   auto set_fill_tile = [&](int fm, int fn) {
-    fA = p.A + ((int64_t)fm * BM + wave * 64) * p.lda;
+    fA = p.A + ((int64_t)fm * BM + wave * (BM / 4)) * p.lda;
     fB = p.B + ((int64_t)fn * BN + wave * 64) * p.ldb;
     if constexpr (PF) {
-      pA = p.A + ((int64_t)fm * BM + (fn & 3) * 64 + wave * 16) * p.lda;
+      pA = p.A + ((int64_t)fm * BM + (fn & 3) * (BM / 4) + wave * (BM / 16)) * p.lda;
       pB = p.B + ((int64_t)fn * BN + (fm & 7) * 32 + wave * 8) * p.ldb;
     }
-    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * 64) * p.lds_a;
+    gSA = (const char*)p.sA + ((int64_t)fm * BM + wave * (BM / 4)) * p.lds_a;
     gSB = (const char*)p.sB + ((int64_t)fn * BN + wave * 64) * p.lds_b;
   };
   set_fill_tile(pm, pn);
+  auto load_of = [](int slot) constexpr { return slot < LA ? slot : 8 + slot - LA; };   // load slot -> j (A: 0 .. LA-1, B: 8 .. 15)
   auto issue = [&](auto J_, const char* srcA, const char* srcB, unsigned stage_base, auto SETTLE_) {
     constexpr int j = decltype(J_)::value, q = j & 7, ioff = (q - 4) * 1024;
-    const unsigned dst = stage_base + (j < 8 ? 0 : A_BYTES) + wave * 8192 + 4096;
+    const unsigned dst = stage_base + (j < 8 ? wave * (LA * 1024) : A_BYTES + wave * 8192) + 4096;
     if constexpr (j < 8) async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcA, voffA[q], dst);
     else async_copy16_sbase_off<ioff, q == 0, decltype(SETTLE_)::value>(srcB, voffB[q], dst);
   };
-  // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of rows 64 w .. 64 w + 63 of A and of B
+  // ---- scale loads: wave w fetches the 16 scale bytes (K steps 2 h, 2 h + 1) of its BM / 4 rows of A (192-row tiles: the
+  // lanes beyond row 47 sit the load out) and of rows 64 w .. 64 w + 63 of B
   const unsigned voffSA = lane * (unsigned)p.lds_a, voffSB = lane * (unsigned)p.lds_b;
   auto issue_scales = [&](int h, auto SETTLE_) {   // pair h of K steps of the fill tile -> slot h & 1 (K steps come in fours, so
-    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT + wave * 1024;   // the slots alternate across tiles too)
-    async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)h * 16, slot);
-    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)h * 16, slot + BM * 16);
+    const unsigned slot = lds0 + SC_BASE + (h & 1) * SC_SLOT;   // the slots alternate across tiles too)
+    if (BM == 256 || lane < BM / 4) async_copy16_sbase<decltype(SETTLE_)::value>(gSA, voffSA + (unsigned)h * 16, slot + wave * (BM / 4) * 16);
+    async_copy16_sbase<decltype(SETTLE_)::value>(gSB, voffSB + (unsigned)h * 16, slot + 256 * 16 + wave * 1024);
   };
 
   // ---- fragment reads: lane (l16, kg) of sub-step ks wants chunk 2 kg + ks of row l16 (+ 16 t)
@@ -462,7 +486,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
 #pragma unroll
     for (int ks = 0; ks < KS; ks++) {
       const unsigned slot = ((4 * ks + kg) ^ s) * 16;
-      adrA[ks] = lds0 + (wm * 128 + l16) * ROWB + slot;
+      adrA[ks] = lds0 + (wm * (BM / 2) + l16) * ROWB + slot;
       adrB[ks] = lds0 + A_BYTES + (wn * 128 + l16) * ROWB + slot;
     }
   }
@@ -481,8 +505,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   // scales: lane (r, kg) multiplies block 2 kg of its row in sub-step 0 and block 2 kg + 1 in sub-step 1: ONE 16-bit
   // read per fragment and K step fetches both (bytes 0 and 1 of the register, which the MFMA's compile-time selector
   // names: no shift), into the register set of the step's parity, read during the second half of the step before.
-  const unsigned adrSA = lds0 + SC_BASE + (wm * 128 + l16) * 16 + 2 * kg;
-  const unsigned adrSB = lds0 + SC_BASE + BM * 16 + (wn * 128 + l16) * 16 + 2 * kg;
+  const unsigned adrSA = lds0 + SC_BASE + (wm * (BM / 2) + l16) * 16 + 2 * kg;
+  const unsigned adrSB = lds0 + SC_BASE + 256 * 16 + (wn * 128 + l16) * 16 + 2 * kg;
   int sa[2][MT], sb[2][NT];
   auto read_scale = [&](auto OP_, auto SET_, auto OFF_) {   // OFF: slot * SC_SLOT + (K step & 1) * 8
     constexpr int op = decltype(OP_)::value, set = decltype(SET_)::value, off = decltype(OFF_)::value;
@@ -508,22 +532,22 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   using I0 = std::integral_constant<int, 0>; using I1 = std::integral_constant<int, 1>;
   using T = std::true_type; using F = std::false_type;
   issue_scales(0, std::true_type{});
-  static_for<16>([&](auto J_) { issue(J_, fA, fB, lds0, std::true_type{}); });
-  static_for<16>([&](auto J_) { issue(J_, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA, fB, lds0, std::true_type{}); });
+  static_for<NLOADS>([&](auto L_) { issue(std::integral_constant<int, load_of(decltype(L_)::value)>{}, fA + ROWB, fB + ROWB, lds0 + STAGE, std::true_type{}); });
   fA += 2 * ROWB;
   fB += 2 * ROWB;
   if constexpr (PF) {
     // the lines of K steps 2 and 3 (the loop's touches begin with step 2 + PFD); also the two youngest loads that
     // the loop's waits leave outstanding from the first step on
     const int k2 = min(2, nk - 1), k3 = min(3, nk - 1);
-    touch_line_sbase<true, 16>(pA + k2 * ROWB, voffPA, touch_lds);
+    touch_line_sbase<true, BM / 16>(pA + k2 * ROWB, voffPA, touch_lds);
     touch_line_sbase<false, 8>(pB + k2 * ROWB, voffPB, 0u);
-    touch_line_sbase<false, 16>(pA + k3 * ROWB, voffPA, 0u);
+    touch_line_sbase<false, BM / 16>(pA + k3 * ROWB, voffPA, 0u);
     touch_line_sbase<false, 8>(pB + k3 * ROWB, voffPB, 0u);
     pA += 2 * ROWB;
     pB += 2 * ROWB;
   }
-  wait_vmcnt<16 + (PF ? 4 : 0)>();
+  wait_vmcnt<NLOADS + (PF ? 4 : 0)>();
   block_barrier();
   static_for<NRD>([&](auto OP_) { read_one(OP_, I0{}, I0{}, f[0]); });
   static_for<NRD>([&](auto OP_) { read_scale(OP_, I0{}, I0{}); });
@@ -551,15 +575,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       mfma16_mxfp4<1>(f[1].b[j], f[1].a[i], acc[i][j], sb[P][j], sa[P][i]);
       if constexpr (n % 2 == 0 && n / 2 < NRD) read_one(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, I0{}, f[0]);
       if constexpr (n % 2 == 1 && n / 2 < NRD) read_scale(std::integral_constant<int, n / 2>{}, std::integral_constant<int, P ^ 1>{}, OffNext{});
-      if constexpr (n % 4 == 1) issue(std::integral_constant<int, n / 4>{}, fA, fB, lds0 + P * STAGE, std::false_type{});   // one per 64 cycles
+      if constexpr (n % EVERY == 1 && n / EVERY < NLOADS) issue(std::integral_constant<int, load_of(n / EVERY)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});   // one per 64 (48) cycles
       // (the scales of the K steps fk, fk + 1 are requested in the even steps, into the slot that the pair
       // two steps back used: its last readers were the reads of that pair's second step, in its sub-step 0)
       // (after the last operand load: the eight loads of an operand share the M0 value that the first one sets)
-      if constexpr (P == 0 && n == 62) issue_scales(fk >> 1, std::false_type{});
+      if constexpr (P == 0 && n == NM - 2) issue_scales(fk >> 1, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (PF) {
-      touch_line_sbase<true, 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
+      touch_line_sbase<true, BM / 16>(pA + (fk + PFD < nk ? PFD * ROWB : 0), voffPA, touch_lds);
       touch_line_sbase<false, 8>(pB + (fk + PFD < nk ? PFD * ROWB : 0), voffPB, 0u);
     }
     // everything requested above has landed before the registers are touched again
@@ -646,7 +670,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
       }
     }
     mfma_drain(acc);
-    int em = pm * BM + wm * 128, en = pn * BN + wn * 128, el = l16, ek = kg;
+    int em = pm * BM + wm * (BM / 2), en = pn * BN + wn * 128, el = l16, ek = kg;
     asm volatile("" : "+s"(em), "+s"(en), "+v"(el), "+v"(ek));   // (keeps the epilogue's address arithmetic out of the K loop)
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
@@ -660,6 +684,15 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
 #endif
 }
 
+// the block-scaled forms on tiles of 192 x 256: M a multiple of 192, whole groups of K steps (`group_bytes` of a row: 512
+// for MXFP4, 1024 for MXFP8), a 16-bit C through the lean epilogue
+bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes) {
+  return p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % group_bytes == 0 && p.k_bytes >= group_bytes && lean_epilogue_type(p) != 0 &&
+         p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
+         p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
+         p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
+}
+
 bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
   // whole tiles, at least one group of four K steps (K >= 1024 elements; what is left behind the last group: the TAIL
   // form), scale rows that a 16-byte load can fetch
@@ -669,23 +702,25 @@ bool gemm_wave128_mxfp4_ok(const GemmArgs& p) {
          p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
 }
 
-template <int EPI, bool TAIL = false>
+template <int EPI, bool TAIL = false, int BM = 256>
 static int launch_wave128_mxfp4(const GemmArgs& p, hipStream_t stream) {
-  constexpr int smem = 2 * 2 * 256 * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
+  constexpr int smem = 2 * (BM + 256) * 128 + 2 * 512 * 16 + 1024;   // (stages, scale ring and the 1 KiB that the L2 touches land in)
   static bool attr_set = false;
   if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI, TAIL>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_kernel<EPI, TAIL, BM>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return (int)e;
     attr_set = true;
   }
-  const int tiles = (p.M / 256) * (p.N / 256);
+  const int tiles = (p.M / BM) * (p.N / 256);
   const int grid = wave128_grid(tiles, p.num_programs);
-  gemm_wave128_mxfp4_kernel<EPI, TAIL><<<dim3(grid), dim3(256), smem, stream>>>(p);
+  gemm_wave128_mxfp4_kernel<EPI, TAIL, BM><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
 }
 
 int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
+  if (p.tile_m == 192)   // (gemm_wave128_mx_192_ok: lean epilogue, whole groups of K steps)
+    return lean == 1 ? launch_wave128_mxfp4<3, false, 192>(p, stream) : launch_wave128_mxfp4<4, false, 192>(p, stream);
   if (p.k_bytes % 512 != 0)
     return lean == 1 ? launch_wave128_mxfp4<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4, true>(p, stream) : launch_wave128_mxfp4<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp4<3>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4>(p, stream) : launch_wave128_mxfp4<0>(p, stream);
