@@ -214,7 +214,12 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     auto fill = [&](long t) { return t <= 0 ? 0.0 : (double)t / (double)(((t + cus - 1) / cus) * cus); };
     const long tiles192 = (long)(M / 192) * (N / 256);
     const int want = knob(knobs().tile_m, 0);
-    if (want == 192 || (want == 0 && tiles192 * 2 >= cus && (tile != 6 || fill(tiles192) > fill(tiles256) + 0.08))) {
+    // (below half a round of 256-row tiles the 128-row tiles further down may fill better still: 3072 x 2048 x 4096 bf16,
+    // 128 tiles of 192 rows 734 TFLOP/s, 192 tiles of 128 rows 815)
+    const long tiles128 = (long)(M / 128) * (N / 256);
+    const bool rather128 = tile == 1 && M % 128 == 0 && tiles128 <= cus && fill(tiles128) > fill(tiles192) &&
+                           gemm_wave128_192_ok(p, b_kmajor, in_dtype, 128);
+    if (want == 192 || (want == 0 && !rather128 && tiles192 * 2 >= cus && (tile != 6 || fill(tiles192) > fill(tiles256) + 0.08))) {
       tile = 6;
       p.tile_m = 192;
     }
@@ -234,12 +239,13 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     }
   }
   // and on tiles of 128 x 256 where the 256 x 256 tiles are too few for their kernel (less than half a round) but these
-  // fill most of one round (2560^3: 100 and 200 tiles; 716 -> 825 TFLOP/s against the 128 x 128 tiles)
+  // fill more than half of one round (2560^3: 100 and 200 tiles; 716 -> 825 TFLOP/s against the 128 x 128 tiles; 2304 x
+  // 2048 x 8192, 144 tiles: 650 -> 692; at half a round the 128 x 128 tiles stay ahead, 2048 x 2048 x 4096: 627 vs 569)
   if (!is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 128) && p.tile_m == 0 &&
       gemm_wave128_192_ok(p, b_kmajor, in_dtype, 128)) {
     const long tiles128 = (long)(M / 128) * (N / 256);
     const int want = knob(knobs().tile_m, 0);
-    if (want == 128 || (want == 0 && tile == 1 && tiles128 * 10 >= cus * 7 && tiles128 <= cus)) {
+    if (want == 128 || (want == 0 && tile == 1 && tiles128 * 16 >= cus * 9 && tiles128 <= cus)) {
       tile = 6;
       p.tile_m = 128;
     }
