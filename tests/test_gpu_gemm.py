@@ -940,11 +940,12 @@ def test_four_wave_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, dt
 @pytest.mark.parametrize("programs", [3, 256])
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
 def test_four_wave_fp8_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, fmt, tdt, programs):
-    # the fp8 form of the same tiles (K-major B, 16-bit C): six A fragments per wave, 14 loads per K step; one and
-    # several tiles per program.  Integer data: the bits of the exact product, and of the 256-row tiles' result.
+    # the fp8 form of the same tiles (K-major B, 16-bit C): six A fragments per wave, 14 loads per K step (128 rows:
+    # four and 12); one and several tiles per program.  Integer data: the bits of the exact product, and of the
+    # 256-row tiles' result.
     set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
     rng = np.random.default_rng(programs + len(fmt))
-    for (M, N, K) in [(192, 256, 256), (1536, 1024, 1280), (3072, 768, 512), (576, 512, 2048)]:
+    for (M, N, K) in [(192, 256, 256), (1536, 1024, 1280), (3072, 768, 512), (576, 512, 2048), (384, 256, 768)]:
         a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
         b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
         ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
@@ -955,6 +956,9 @@ def test_four_wave_fp8_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch
             assert bits_equal(got, gemm.matmul_closed_form(a, b.T, out_dtype=name)), (M, N, K, fmt, programs, name)
             set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
             assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=out)), got)
+            if M % 128 == 0:
+                set_knob(monkeypatch, "MI355_GEMM_TILE_M", "128")
+                assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=out)), got), "tiles of 128 rows"
 
 
 def test_3072_cubed_takes_the_192_row_tiles_and_matches_sampled_rows(gpu):

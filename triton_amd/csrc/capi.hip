@@ -250,6 +250,16 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 128;
     }
   }
+  // fp8 likewise (measured: see the design notes' table of shapes)
+  if (is8 && tile_arg < 0 && (knobs().tile == UNSET || knobs().tile_m == 128) && p.tile_m == 0 &&
+      gemm_wave128_f8_192_ok(p, b_kmajor, 128)) {
+    const long tiles128 = (long)(M / 128) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    if (want == 128 || (want == 0 && tile == 1 && tiles128 * 16 >= cus * 9 && tiles128 <= cus)) {
+      tile = 6;
+      p.tile_m = 128;
+    }
+  }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;
@@ -275,7 +285,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
-  if (is8 && tile == 6 && (p.tile_m == 192 || w128_ok)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
+  if (is8 && tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || w128_ok)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)

@@ -512,10 +512,12 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 // the four reads of a lane (they differ in bits 3 and 6 of k), so a fragment has one address and four immediates;
 // the 8 rows x 2 chunks that a half-wave reads fall on 16 different bank groups.
 // BM = 192: tiles of 192 x 256 (a wave: 96 x 128, six A fragments), for products whose 256 x 256 tiles fill the last
-// round of CUs badly - as in the 16-bit kernel; lean epilogue, whole pairs of K steps.
+// round of CUs badly - as in the 16-bit kernel; lean epilogue, whole pairs of K steps.  BM = 128: tiles of 128 x 256 (a
+// wave: 64 x 128, four A fragments; twelve loads for the sixteen MFMAs of a half step), for products with too few
+// 256 x 256 tiles for this kernel.
 template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
-  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
+  static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
   static_assert(B_KMAJOR || !TAIL, "the K tail loads K-contiguous fragments");
 #if MI355_DEVICE_PASS
   constexpr int BN = 256, ROWB = 128;
@@ -679,11 +681,12 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
       mfma16_f8<FMT>(b[cur][j], a1[i], acc[MH + i][j]);
       if constexpr (n < NT) b[nxt][n] = read_b(std::integral_constant<int, n>{}, std::integral_constant<int, sn>{});
       if constexpr (n >= NT && n < NT + MH) a0[n - NT] = read_frag(fragA, sn + (n - NT) * 16 * ROWB);
-      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs: the last two go into even slots)
-      constexpr int HALF = MH * NT, EXTRA = NLOADS > HALF / 2 ? NLOADS - HALF / 2 : 0;
-      if constexpr (n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
-      if constexpr (EXTRA > 0 && n % 2 == 0 && n >= HALF - 2 * EXTRA)
-        issue(std::integral_constant<int, load_of(HALF / 2 + (n - (HALF - 2 * EXTRA)) / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs, the 128-row tile 12 for 16: from MFMA R
+      // on every MFMA is followed by one.  The loads stay in slot order - A, then B - because only the first of each
+      // operand sets M0.)
+      constexpr int HALF = MH * NT, EXTRA = NLOADS > HALF / 2 ? NLOADS - HALF / 2 : 0, R = HALF - 2 * EXTRA;
+      if constexpr (n < R && n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      if constexpr (n >= R) issue(std::integral_constant<int, load_of(R / 2 + n - R)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (PF) {
@@ -791,6 +794,10 @@ int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, hipStrea
     if (lean_epilogue_type(p) == 1) return e5m2 ? launch_wave128_f8<1, 3, false, true, 192>(p, stream) : launch_wave128_f8<0, 3, false, true, 192>(p, stream);
     return e5m2 ? launch_wave128_f8<1, 4, false, true, 192>(p, stream) : launch_wave128_f8<0, 4, false, true, 192>(p, stream);
   }
+  if (p.tile_m == 128) {   // (the same conditions)
+    if (lean_epilogue_type(p) == 1) return e5m2 ? launch_wave128_f8<1, 3, false, true, 128>(p, stream) : launch_wave128_f8<0, 3, false, true, 128>(p, stream);
+    return e5m2 ? launch_wave128_f8<1, 4, false, true, 128>(p, stream) : launch_wave128_f8<0, 4, false, true, 128>(p, stream);
+  }
   if (!b_kmajor) {   // (gemm_wave128_f8_ok: whole pairs of K steps, no addend)
     const int lean = lean_epilogue_type(p);
     if (lean == 1) return e5m2 ? launch_wave128_f8<1, 3, false, false>(p, stream) : launch_wave128_f8<0, 3, false, false>(p, stream);
@@ -821,9 +828,10 @@ bool gemm_wave128_f8_ok(const GemmArgs& p, bool b_kmajor) {
   return p.k_bytes % 256 == 0 && !p.aux && p.ldb % 16 == 0 && p.ldb * 32 + 256 < (1ll << 32);
 }
 
-// fp8 on tiles of 192 x 256: M a multiple of 192, K-major B, whole pairs of K steps, a 16-bit C through the lean epilogue
-bool gemm_wave128_f8_192_ok(const GemmArgs& p, bool b_kmajor) {
-  if (!(b_kmajor && p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+// fp8 on tiles of 192 x 256 (128 x 256): M a multiple of 192 (128), K-major B, whole pairs of K steps, a 16-bit C through
+// the lean epilogue
+bool gemm_wave128_f8_192_ok(const GemmArgs& p, bool b_kmajor, int tile_m) {
+  if (!(b_kmajor && p.M % tile_m == 0 && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
   if (lean_epilogue_type(p) == 0) return false;
   return p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
 }
