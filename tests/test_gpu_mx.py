@@ -103,7 +103,7 @@ def test_four_wave_kernels_on_tiles_of_192_rows_are_bit_exact(gpu, monkeypatch, 
     set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
     rng = np.random.default_rng(programs + len(fmt))
     t = lambda x: torch.from_numpy(x).to(gpu)
-    for (M, N, K) in [(192, 256, 1024), (1536, 1024, 2048), (3072, 768, 1024), (576, 512, 5120)]:
+    for (M, N, K) in [(192, 256, 1024), (1536, 1024, 2048), (3072, 768, 1024), (576, 512, 5120), (384, 256, 3072)]:
         if fmt == "mxfp4":
             a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
         else:
@@ -118,6 +118,9 @@ def test_four_wave_kernels_on_tiles_of_192_rows_are_bit_exact(gpu, monkeypatch, 
             assert bits_equal(got, rnd(ref32)), (fmt, M, N, K, programs, out)
             set_knob(monkeypatch, "MI355_GEMM_TILE_M", "256")
             assert bits_equal(_run(gpu, a, sa, b, sb, fmt, out), got)
+            if M % 128 == 0:   # (tiles of 128 x 256: four A fragments, 32 rows per wave and load group)
+                set_knob(monkeypatch, "MI355_GEMM_TILE_M", "128")
+                assert bits_equal(_run(gpu, a, sa, b, sb, fmt, out), got), "tiles of 128 rows"
 
 
 def test_scale_blocks_are_applied_per_row_and_per_32_elements(gpu):

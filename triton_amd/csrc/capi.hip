@@ -484,11 +484,24 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
   if (fmt == MI355_MXFP4 && enough && gemm_wave128_mxfp4_ok(p) && tail_pays(512, 9)) tile = 6;
   // (MXFP8 likewise: 2530-2570 vs 2110-2240)
   if (fmt == MI355_MXFP8 && enough && gemm_wave128_mxfp8_ok(p) && tail_pays(1024, 21)) tile = 6;
-  // the same kernels on tiles of 192 x 256 where those fill the CUs better (as for the 16-bit and fp8 products).  Flushed
+  // the same kernels on tiles of 128 x 256 wherever those fit one round of CUs (from 16 on): flushed do_bench, best of
+  // the other forms / 128-row tiles, MXFP4: 1024^3 141 / 162 TFLOP/s, 2048 x 2048 x 1024 503 / 600, 2048 x 2048 x 4096 1012 /
+  // 1309, 1536 x 2048 x 8192 1071 / 1216, 3072 x 2048 x 4096 1661 / 1854, 2304 x 2048 x 8192 1606 / 1795; MXFP8: 92 / 127,
+  // 360 / 491, 644 / 856, 627 / 754, 1072 / 1244, 947 / 1120; beyond one round they lose (3072^3, 288 tiles: MXFP4 2084 for
+  // the 192-row tiles / 1555, 4096^3 3209 / 2834)
+  if ((knobs().tile == UNSET || knobs().tile_m == 128) && gemm_wave128_mx_192_ok(p, fmt == MI355_MXFP4 ? 512 : 1024, 128)) {
+    const long tiles128 = (long)(M / 128) * (N / 256);
+    const int want = knob(knobs().tile_m, 0);
+    if (want == 128 || (want == 0 && tiles128 >= 16 && tiles128 <= cus)) {
+      tile = 6;
+      p.tile_m = 128;
+    }
+  }
+  // and on tiles of 192 x 256 where those fill the CUs better (as for the 16-bit and fp8 products).  Flushed
   // do_bench, 256-row choice / 192-row tiles, MXFP4: 3072^3 1750 / 2100 TFLOP/s, 4608 x 4096 x 4096 2475 / 2885, 6144^3
   // 3725 / 3970, 1536 x 8192 x 8192 3205 / 3780, 1536 x 2048 x 8192 880 / 1080; MXFP8: 1255 / 1420, 1480 / 1830, 2275 / 2520,
   // 1945 / 2345, 519 / 630; not taken where they fill worse (3840 x 3840 x 4096: 3080 / 2230)
-  if ((knobs().tile == UNSET || knobs().tile_m == 192) && gemm_wave128_mx_192_ok(p, fmt == MI355_MXFP4 ? 512 : 1024)) {
+  if ((knobs().tile == UNSET || knobs().tile_m == 192) && p.tile_m == 0 && gemm_wave128_mx_192_ok(p, fmt == MI355_MXFP4 ? 512 : 1024)) {
     auto fill = [&](long t) { return t <= 0 ? 0.0 : (double)t / (double)(((t + cus - 1) / cus) * cus); };
     const long tiles192 = (long)(M / 192) * (N / 256);
     const int want = knob(knobs().tile_m, 0);

@@ -119,8 +119,8 @@ __global__ __launch_bounds__(256) void mx_gemm_simple_kernel(GemmArgs p, int fp4
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream) {
   // 6: four waves of scaled 16x16x128 MFMAs (whole 256x256 tiles, K at least 1024, any multiple of the scale block:
   // what is left behind the last whole group of K steps is the tail form's)
-  if (tile == 6 && fmt == 0 && (p.tile_m == 192 || gemm_wave128_mxfp4_ok(p))) return gemm_wave128_mxfp4_launch(p, stream);
-  if (tile == 6 && fmt != 0 && (p.tile_m == 192 || gemm_wave128_mxfp8_ok(p))) return gemm_wave128_mxfp8_launch(p, stream);
+  if (tile == 6 && fmt == 0 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_mxfp4_ok(p))) return gemm_wave128_mxfp4_launch(p, stream);
+  if (tile == 6 && fmt != 0 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_mxfp8_ok(p))) return gemm_wave128_mxfp8_launch(p, stream);
   if (tile < 0) {
     dim3 grid((p.N + 15) / 16, (p.M + 15) / 16);
     mx_gemm_simple_kernel<<<grid, dim3(256), 0, stream>>>(p, fmt == 0);

@@ -49,7 +49,7 @@ __device__ __forceinline__ void settle_tail(R&... r) {
 // BM = 192: tiles of 192 x 256, as in the MXFP4 kernel below.
 template <int EPI, bool TAIL = false, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
-  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
+  static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
   constexpr int BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
@@ -225,14 +225,16 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
       } else {
         if constexpr (n < NSC) read_scale(std::integral_constant<int, n>{}, std::integral_constant<int, nxt>{}, OffNext{});
       }
-      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs: the last two go into even slots)
-      if constexpr (n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
-      if constexpr (EXTRA > 0 && n % 2 == 0 && n >= HALF - 2 * EXTRA)
-        issue(std::integral_constant<int, load_of(HALF / 2 + (n - (HALF - 2 * EXTRA)) / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       // (the scales of the K steps fk .. fk + 3 are requested in the third step of every four, into the slot whose
       // last reader was the read for the step before this one)
       // (between the last A load and the first B load, which sets M0 for its group again)
       if constexpr ((U & 3) == 2 && n == 2 * LA) issue_scales(fk >> 2, std::false_type{});
+      // (one load per two MFMAs; the 192-row tile has 14 loads for its 24 MFMAs, the 128-row tile 12 for 16: from MFMA R
+      // on every MFMA is followed by one.  The loads stay in slot order - A, then B - because only the first of each
+      // operand sets M0.)
+      constexpr int R = HALF - 2 * EXTRA;
+      if constexpr (n < R && n % 2 == 1 && n / 2 < NLOADS) issue(std::integral_constant<int, load_of(n / 2)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
+      if constexpr (n >= R) issue(std::integral_constant<int, load_of(R / 2 + n - R)>{}, fA, fB, lds0 + P * STAGE, std::false_type{});
       if constexpr (n % 2 == 1) __builtin_amdgcn_sched_barrier(0);
     });
     if constexpr (PF) {
@@ -362,6 +364,8 @@ int gemm_wave128_mxfp8_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
   if (p.tile_m == 192)   // (gemm_wave128_mx_192_ok: lean epilogue, whole groups of K steps)
     return lean == 1 ? launch_wave128_mxfp8<3, false, 192>(p, stream) : launch_wave128_mxfp8<4, false, 192>(p, stream);
+  if (p.tile_m == 128)
+    return lean == 1 ? launch_wave128_mxfp8<3, false, 128>(p, stream) : launch_wave128_mxfp8<4, false, 128>(p, stream);
   if (p.k_bytes % 1024 != 0)
     return lean == 1 ? launch_wave128_mxfp8<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4, true>(p, stream) : launch_wave128_mxfp8<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp8<3>(p, stream) : lean == 2 ? launch_wave128_mxfp8<4>(p, stream) : launch_wave128_mxfp8<0>(p, stream);
@@ -400,7 +404,7 @@ __device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32
 // products whose 256 x 256 tiles fill the last round of CUs badly; lean epilogue, K steps in whole groups.
 template <int EPI, bool TAIL = false, int BM = 256>
 __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
-  static_assert(BM == 256 || (BM == 192 && !TAIL && (EPI == 3 || EPI == 4)), "192-row tiles: lean epilogue, no K tail");
+  static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
   constexpr int BN = 256, ROWB = 128;
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
@@ -686,8 +690,8 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
 
 // the block-scaled forms on tiles of 192 x 256: M a multiple of 192, whole groups of K steps (`group_bytes` of a row: 512
 // for MXFP4, 1024 for MXFP8), a 16-bit C through the lean epilogue
-bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes) {
-  return p.M % 192 == 0 && p.N % 256 == 0 && p.k_bytes % group_bytes == 0 && p.k_bytes >= group_bytes && lean_epilogue_type(p) != 0 &&
+bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes, int tile_m) {
+  return p.M % tile_m == 0 && p.N % 256 == 0 && p.k_bytes % group_bytes == 0 && p.k_bytes >= group_bytes && lean_epilogue_type(p) != 0 &&
          p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31) &&
          p.lds_a % 16 == 0 && p.lds_b % 16 == 0 && ((uintptr_t)p.sA | (uintptr_t)p.sB) % 16 == 0 &&
          p.lds_a * 64 + p.k_bytes / 16 < (1ll << 31) && p.lds_b * 64 + p.k_bytes / 16 < (1ll << 31);
@@ -721,6 +725,8 @@ int gemm_wave128_mxfp4_launch(const GemmArgs& p, hipStream_t stream) {
   const int lean = lean_epilogue_type(p);
   if (p.tile_m == 192)   // (gemm_wave128_mx_192_ok: lean epilogue, whole groups of K steps)
     return lean == 1 ? launch_wave128_mxfp4<3, false, 192>(p, stream) : launch_wave128_mxfp4<4, false, 192>(p, stream);
+  if (p.tile_m == 128)
+    return lean == 1 ? launch_wave128_mxfp4<3, false, 128>(p, stream) : launch_wave128_mxfp4<4, false, 128>(p, stream);
   if (p.k_bytes % 512 != 0)
     return lean == 1 ? launch_wave128_mxfp4<3, true>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4, true>(p, stream) : launch_wave128_mxfp4<0, true>(p, stream);
   return lean == 1 ? launch_wave128_mxfp4<3>(p, stream) : lean == 2 ? launch_wave128_mxfp4<4>(p, stream) : launch_wave128_mxfp4<0>(p, stream);

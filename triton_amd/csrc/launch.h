@@ -113,7 +113,7 @@ bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int til
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype);
 bool gemm_wave128_f8_ok(const GemmArgs& p, bool b_kmajor);
 bool gemm_wave128_f8_192_ok(const GemmArgs& p, bool b_kmajor, int tile_m = 192);   // tiles of 192 x 256 / 128 x 256
-bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes);   // in_dtype: C ABI code of the operands' type
+bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes, int tile_m = 192);   // in_dtype: C ABI code of the operands' type
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream);
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, hipStream_t stream);
 bool gemm_wave128_mxfp4_ok(const GemmArgs& p);
