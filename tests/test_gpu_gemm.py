@@ -937,6 +937,40 @@ def test_four_wave_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, dt
     assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got), "tiles of 256 rows"
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("kmajor", [False, True])
+@pytest.mark.parametrize("programs", [3, 256])
+def test_two_tile_heights_in_one_launch_are_bit_exact(gpu, monkeypatch, dtype, kmajor, programs):
+    # the upper rows of C on 256-row tiles and the lower ones on 192-row tiles, one launch (chosen by itself for tile
+    # counts that fill the last round of CUs badly, forced here): one tile of each kind, several of each per program,
+    # more programs than tiles of either kind.  Small integers make every sum exact.
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    for (rows256, M, N, K) in [(256, 448, 256, 256), (256, 1216, 512, 512), (1280, 2240, 768, 1280), (768, 960, 1024, 384)]:
+        rng = np.random.default_rng(M + N + K + programs)
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ta, tb = from_np(a, dtype, gpu), from_np(b, dtype, gpu)
+        if kmajor:
+            tb = tb.t().contiguous().t()
+        ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+        set_knob(monkeypatch, "MI355_GEMM_MIXED_ROWS", rows256)
+        got = to_np(triton_amd.matmul(ta, tb))
+        assert bits_equal(got, to_np(from_np(ref, dtype, gpu))), (rows256, M, N, K)
+        set_knob(monkeypatch, "MI355_GEMM_MIXED_ROWS", 0)
+        assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got)
+
+
+def test_5120_cubed_takes_two_tile_heights_and_matches_sampled_rows(gpu):
+    # 400 tiles of 256 x 256 for 256 CUs: the size heuristic splits M into 2816 rows of 256-row and 2304 of 192-row tiles
+    rng = np.random.default_rng(12)
+    n = 5120
+    a, b = randn_rounded(rng, (n, n), "bf16", 1.0), randn_rounded(rng, (n, n), "bf16", 1.0)
+    got = to_np(triton_amd.matmul(from_np(a, "bf16", gpu), from_np(b, "bf16", gpu)))
+    rows = np.concatenate([rng.choice(n, size=20, replace=False), [0, 2815, 2816, 3007, 3008, n - 1]])
+    ref = a[rows].astype(np.float64) @ b.astype(np.float64)
+    assert np.allclose(got[rows], ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+
+
 @pytest.mark.parametrize("programs", [3, 256])
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
 def test_four_wave_fp8_kernel_on_tiles_of_192_rows_is_bit_exact(gpu, monkeypatch, fmt, tdt, programs):

@@ -2,6 +2,8 @@
 // family / tile selection, launch.  Plays the role of the generated launcher of the reference
 // (third_party/amd/backend/driver.py:326-377): pointers and scalars in, one asynchronous
 // launch on the caller's stream out, an integer status back.
+#include <algorithm>
+#include <cmath>
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 #include <string.h>
@@ -51,7 +53,7 @@ const DeviceInfo& device_info() {
 constexpr int UNSET = INT_MIN;
 struct Knobs {
   int force_strided, group_m, tile, programs, skinny, grouped_big_min, grouped_wave128_min_k, grouped_chunk,
-      attn_fwd_variant, attn_programs, lean_epilogue, tile_m, rowfused_max_mk;
+      attn_fwd_variant, attn_programs, lean_epilogue, tile_m, rowfused_max_mk, mixed_rows;
 };
 Knobs g_knobs;
 std::atomic<int> g_knobs_ready{0};
@@ -80,6 +82,7 @@ void load_knobs() {
   k.lean_epilogue = read_env("MI355_GEMM_LEAN_EPILOGUE", 0);
   k.tile_m = read_env("MI355_GEMM_TILE_M", 0);
   k.rowfused_max_mk = read_env("MI355_ROWFUSED_MAX_MK", 0);
+  k.mixed_rows = read_env("MI355_GEMM_MIXED_ROWS", 0);
   g_knobs = k;
   g_knobs_ready.store(1, std::memory_order_release);
 }
@@ -260,6 +263,41 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 128;
     }
   }
+  // 16-bit products of more than one round of tiles whose last round is badly filled: the upper rows on 256-row tiles
+  // and the lower ones on 192-row tiles in ONE launch (gemm_wave128_mixed_kernel), split so that the busiest program
+  // has the least to do.  A 192-row tile is counted as 0.78 of a 256-row one (3072^3 on 192 of them against 4096^3 on 256
+  // tiles, per tile and K step).  Flushed do_bench, bf16: 5120^3 (400 tiles; 220 + 240) and 7168^3 (784; 112 + 896) - see
+  // the design notes.  MI355_GEMM_MIXED_ROWS forces the rows of the 256-row part (0 = never).
+  int mixed_rows = 0;
+  if (!is8 && tile_arg < 0 && knobs().tile == UNSET && knobs().tile_m == UNSET && N % 256 == 0) {
+    const int want = knob(knobs().mixed_rows, -1);
+    const int nn = N / 256, P = cus;
+    if (want > 0) {
+      if (gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, want)) mixed_rows = want;
+    } else if (want < 0 && tile == 6 && p.tile_m == 0 && tiles256 > cus && M % 256 == 0) {
+      auto count = [&](long tiles, int b) { return b < tiles ? (tiles - b + P - 1) / P : 0; };   // tiles b, b + P, ... below `tiles`
+      double one_height = (double)((tiles256 + P - 1) / P), best = 1e30;   // in units of a 256-row tile's time
+      if (M % 192 == 0) one_height = std::min(one_height, 0.78 * (double)(((long)(M / 192) * nn + P - 1) / P));
+      auto busiest = [&](int a) {
+        const long n256 = (long)a * nn, n192 = (long)((M - a * 256) / 192) * nn;
+        double worst = 0;
+        for (int b = 0; b < P; b++) worst = std::max(worst, (double)count(n256, b) + 0.78 * (double)count(n192, P - 1 - b));
+        return worst;
+      };
+      for (int a = 1; a * 256 < M; a++)
+        if ((M - a * 256) % 192 == 0) best = std::min(best, busiest(a));
+      // among the splits within 7 % of the best one, the one whose two parts are closest in work (measured: 5120^3 1164 /
+      // 1280 / 1325 TFLOP/s for 100 + 400 / 160 + 320 / 220 + 240 tiles, which this count rates the same)
+      int best_rows = 0;
+      double best_gap = 1e30;
+      for (int a = 1; a * 256 < M; a++) {
+        if ((M - a * 256) % 192 != 0 || busiest(a) > 1.07 * best) continue;
+        const double gap = std::abs((double)a * nn - 0.78 * (double)((M - a * 256) / 192) * nn);
+        if (gap < best_gap) { best_gap = gap; best_rows = a * 256; }
+      }
+      if (best_rows > 0 && best < 0.95 * one_height && gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, best_rows)) mixed_rows = best_rows;
+    }
+  }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
   if (p.num_programs > cus) p.num_programs = cus;       // (the stream-K workspace is sized for one program per CU)
   p.workspace = workspace;
@@ -289,6 +327,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)
+  if (mixed_rows > 0) return gemm_wave128_mixed_launch(p, mixed_rows, in_dtype == MI355_BF16, b_kmajor, stream);
   if (tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }

@@ -410,6 +410,38 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_kernel(GemmArgs p) {
 #endif
 }
 
+// Two tile heights in one launch, for tile counts that fill the last round of CUs badly and an M that is no multiple
+// of 192: the first `rows256` rows of C on tiles of 256 x 256, the rows below on tiles of 192 x 256.  Every program walks
+// its 256-row tiles (b, b + G, ...) and then its 192-row tiles, which are dealt from the other end (G - 1 - b, ...), so
+// that the programs with one tile fewer in the first part are the ones with one more in the second; a program moves on
+// by itself, nobody waits for the first part as a whole - which is what two launches would do.  5120^3 on 256 CUs: 400
+// tiles are two rounds of which the second is 56 % full; 220 tiles of 256 rows + 240 of 192 are one tile of each per
+// program.  (Lean epilogue, whole pairs of K steps: gemm_wave128_mixed_ok.)
+template <typename V8, bool B_KMAJOR>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mixed_kernel(GemmArgs p, int rows256) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
+  const int G = gridDim.x, nn = p.N / 256;
+  {
+    GemmArgs q = p;
+    q.M = rows256;
+    if ((int)blockIdx.x < (rows256 / 256) * nn) gemm_wave128_tiles<V8, B_KMAJOR, true, 3, false, 256>(q, blockIdx.x, G, lds0);
+  }
+  // (every wave has waited for its own loads; the stages are laid out differently from here on, so no wave may
+  // request its first loads of the second part while another's last loads of the first part could still land)
+  block_barrier();
+  {
+    GemmArgs q = p;
+    q.A = p.A + (int64_t)rows256 * p.lda;
+    q.C = p.C + (int64_t)rows256 * p.ldc * 2;
+    q.M = p.M - rows256;
+    const int j = G - 1 - (int)blockIdx.x;
+    if (j < (q.M / 192) * nn) gemm_wave128_tiles<V8, B_KMAJOR, true, 3, false, 192>(q, j, G, lds0);
+  }
+#endif
+}
+
 // Grouped GEMM (python/tutorials/08-grouped-gemm.py:64-140: pointers, sizes and leading dimensions of the
 // problems in device arrays, row-major B) for groups made of whole 256x256 tiles: gridDim.x workgroups walk
 // the tiles of all problems, numbered problem after problem; a tile is one run of the stream above (its
@@ -870,6 +902,35 @@ static int launch_wave128(const GemmArgs& p, hipStream_t stream) {
   const int grid = wave128_grid(tiles, p.num_programs);
   gemm_wave128_kernel<V8, B_KMAJOR, EPI, TAIL, BM><<<dim3(grid), dim3(256), smem, stream>>>(p);
   return (int)hipGetLastError();
+}
+
+template <typename V8, bool B_KMAJOR>
+static int launch_wave128_mixed(const GemmArgs& p, int rows256, hipStream_t stream) {
+  constexpr int smem = 2 * (256 + 256) * 128 + 1024;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mixed_kernel<V8, B_KMAJOR>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = p.num_programs > 0 ? p.num_programs : 256;
+  gemm_wave128_mixed_kernel<V8, B_KMAJOR><<<dim3(grid), dim3(256), smem, stream>>>(p, rows256);
+  return (int)hipGetLastError();
+}
+
+int gemm_wave128_mixed_launch(const GemmArgs& p, int rows256, bool bf16, bool b_kmajor, hipStream_t stream) {
+  if (bf16) return b_kmajor ? launch_wave128_mixed<bf16x8, true>(p, rows256, stream) : launch_wave128_mixed<bf16x8, false>(p, rows256, stream);
+  return b_kmajor ? launch_wave128_mixed<f16x8, true>(p, rows256, stream) : launch_wave128_mixed<f16x8, false>(p, rows256, stream);
+}
+
+// the first `rows256` rows on 256-row tiles and the rest on 192-row tiles: both parts non-empty and whole, and what the
+// 192-row tiles ask for (whole pairs of K steps, C in the operands' type through the lean epilogue)
+bool gemm_wave128_mixed_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int rows256) {
+  if (!(rows256 > 0 && rows256 < p.M && rows256 % 256 == 0 && (p.M - rows256) % 192 == 0)) return false;
+  if (!(p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  if (!((in_dtype == 0 || in_dtype == 1) && lean_epilogue_type(p) == in_dtype + 1)) return false;
+  if (p.lda * 8 + p.k_bytes >= (1ll << 31)) return false;
+  return b_kmajor ? p.ldb * 8 + p.k_bytes < (1ll << 31) : (p.ldb % 512 == 0 && (int64_t)p.K * p.ldb + 512 < (1ll << 31));
 }
 
 template <typename V8>
