@@ -960,6 +960,25 @@ def test_two_tile_heights_in_one_launch_are_bit_exact(gpu, monkeypatch, dtype, k
         assert bits_equal(to_np(triton_amd.matmul(ta, tb)), got)
 
 
+@pytest.mark.parametrize("programs", [3, 256])
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_two_tile_heights_in_one_launch_are_bit_exact_for_fp8(gpu, monkeypatch, fmt, tdt, programs):
+    # the fp8 form of the same launch (K-major B, 16-bit C)
+    set_knob(monkeypatch, "MI355_GEMM_PROGRAMS", programs)
+    for (rows256, M, N, K) in [(256, 448, 256, 256), (256, 1216, 512, 1024), (1280, 2240, 768, 1280), (768, 960, 1024, 512)]:
+        rng = np.random.default_rng(M + N + K + programs + len(fmt))
+        a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+        b = rng.integers(-3, 4, size=(N, K)).astype(np.float32)
+        ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
+        tb = torch.from_numpy(formats.encode_fp8(b, fmt)).to(gpu).view(tdt).t()
+        for out, name in ((torch.bfloat16, "bf16"), (torch.float16, "fp16")):
+            set_knob(monkeypatch, "MI355_GEMM_MIXED_ROWS", rows256)
+            got = to_np(triton_amd.matmul(ta, tb, out_dtype=out))
+            assert bits_equal(got, gemm.matmul_closed_form(a, b.T, out_dtype=name)), (rows256, M, N, K, fmt, programs, name)
+            set_knob(monkeypatch, "MI355_GEMM_MIXED_ROWS", 0)
+            assert bits_equal(to_np(triton_amd.matmul(ta, tb, out_dtype=out)), got)
+
+
 def test_5120_cubed_takes_two_tile_heights_and_matches_sampled_rows(gpu):
     # 400 tiles of 256 x 256 for 256 CUs: the size heuristic splits M into 2816 rows of 256-row and 2304 of 192-row tiles
     rng = np.random.default_rng(12)

@@ -263,17 +263,20 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 128;
     }
   }
-  // 16-bit products of more than one round of tiles whose last round is badly filled: the upper rows on 256-row tiles
+  // 16-bit and fp8 products of more than one round of tiles whose last round is badly filled: the upper rows on 256-row tiles
   // and the lower ones on 192-row tiles in ONE launch (gemm_wave128_mixed_kernel), split so that the busiest program
   // has the least to do.  A 192-row tile is counted as 0.78 of a 256-row one (3072^3 on 192 of them against 4096^3 on 256
   // tiles, per tile and K step).  Flushed do_bench, bf16: 5120^3 (400 tiles; 220 + 240) and 7168^3 (784; 112 + 896) - see
   // the design notes.  MI355_GEMM_MIXED_ROWS forces the rows of the 256-row part (0 = never).
   int mixed_rows = 0;
-  if (!is8 && tile_arg < 0 && knobs().tile == UNSET && knobs().tile_m == UNSET && N % 256 == 0) {
+  auto mixed_ok = [&](int rows256) {
+    return is8 ? gemm_wave128_f8_mixed_ok(p, b_kmajor, rows256) : gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, rows256);
+  };
+  if (tile_arg < 0 && knobs().tile == UNSET && knobs().tile_m == UNSET && N % 256 == 0) {
     const int want = knob(knobs().mixed_rows, -1);
     const int nn = N / 256, P = cus;
     if (want > 0) {
-      if (gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, want)) mixed_rows = want;
+      if (mixed_ok(want)) mixed_rows = want;
     } else if (want < 0 && tile == 6 && p.tile_m == 0 && tiles256 > cus && M % 256 == 0) {
       auto count = [&](long tiles, int b) { return b < tiles ? (tiles - b + P - 1) / P : 0; };   // tiles b, b + P, ... below `tiles`
       double one_height = (double)((tiles256 + P - 1) / P), best = 1e30;   // in units of a 256-row tile's time
@@ -295,7 +298,7 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
         const double gap = std::abs((double)a * nn - 0.78 * (double)((M - a * 256) / 192) * nn);
         if (gap < best_gap) { best_gap = gap; best_rows = a * 256; }
       }
-      if (best_rows > 0 && best < 0.95 * one_height && gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, best_rows)) mixed_rows = best_rows;
+      if (best_rows > 0 && best < 0.95 * one_height && mixed_ok(best_rows)) mixed_rows = best_rows;
     }
   }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
@@ -323,11 +326,12 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
   }
   if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
+  if (is8 && mixed_rows > 0) return gemm_wave128_f8_mixed_launch(p, mixed_rows, in_dtype == MI355_F8E5M2, stream);
   if (is8 && tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || w128_ok)) return gemm_wave128_f8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, stream);
   if (is8) return gemm8_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, tile, stream);
   // 6: four waves, 128x128 of C per wave from 16x16x32 MFMAs (whole tiles)
   // (a tile height of 192 / 128 rows was set above only after gemm_wave128_192_ok had accepted the shape for it)
-  if (mixed_rows > 0) return gemm_wave128_mixed_launch(p, mixed_rows, in_dtype == MI355_BF16, b_kmajor, stream);
+  if (mixed_rows > 0 && !is8) return gemm_wave128_mixed_launch(p, mixed_rows, in_dtype == MI355_BF16, b_kmajor, stream);
   if (tile == 6 && (p.tile_m == 192 || p.tile_m == 128 || gemm_wave128_ok(p, b_kmajor, in_dtype))) return gemm_wave128_launch(p, in_dtype == MI355_BF16, b_kmajor, stream);
   return gemm16_launch(p, in_dtype == MI355_BF16, b_kmajor, tile, stream);
 }

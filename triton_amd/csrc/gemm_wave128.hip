@@ -547,8 +547,9 @@ __device__ __forceinline__ void mfma16_f8(const i32x8& a, const i32x8& b, f32x4&
 // round of CUs badly - as in the 16-bit kernel; lean epilogue, whole pairs of K steps.  BM = 128: tiles of 128 x 256 (a
 // wave: 64 x 128, four A fragments; twelve loads for the sixteen MFMAs of a half step), for products with too few
 // 256 x 256 tiles for this kernel.
+// The calling workgroup computes the tiles `tile`, `tile + tile_step`, ... of the problem with the LDS at `lds_raw`.
 template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
-__global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_wave128_f8_tiles(const GemmArgs& p, int tile, const int tile_step, LDS_PTR(char) const lds_raw) {
   static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
   static_assert(B_KMAJOR || !TAIL, "the K tail loads K-contiguous fragments");
 #if MI355_DEVICE_PASS
@@ -556,7 +557,6 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
   constexpr int A_BYTES = BM * ROWB, STAGE = A_BYTES + BN * ROWB;  // 64 KiB (56 KiB)
   constexpr int MT = BM / 32, NT = 8, MH = MT / 2;
   constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
-  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -566,8 +566,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
 
   const int num_m = p.M / BM, num_n = p.N / BN;
   const int ntiles = num_m * num_n;
-  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
-  int pm, pn;
+  int pm, pn;   // (the tiles are computed as one stream of K steps)
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = TAIL ? p.k_bytes / (2 * ROWB) * 2 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
@@ -740,7 +739,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     if constexpr (PF) { pA += ROWB; pB += kstepB; }
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      if (ftile + tile_step < ntiles) ftile += tile_step;
       int fm, fn;
       grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
       set_fill_tile(fm, fn);
@@ -797,13 +796,73 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT, EPI == 2>(acc, p, em, en, el, ek);
-    tile += gridDim.x;
+    tile += tile_step;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
     zero_acc();
   }
   wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 #endif
+}
+
+// Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
+template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_f8_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  gemm_wave128_f8_tiles<FMT, EPI, TAIL, B_KMAJOR, BM>(p, blockIdx.x, gridDim.x, (LDS_PTR(char))lds_raw);
+#endif
+}
+
+// Two tile heights in one launch, as gemm_wave128_mixed_kernel: the first `rows256` rows of C on tiles of 256 x 256, the
+// rows below on tiles of 192 x 256 dealt from the other end of the grid (K-major B, lean epilogue, whole pairs of K steps).
+template <int FMT, int EPI>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_f8_mixed_kernel(GemmArgs p, int rows256) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const int G = gridDim.x, nn = p.N / 256;
+  {
+    GemmArgs q = p;
+    q.M = rows256;
+    if ((int)blockIdx.x < (rows256 / 256) * nn) gemm_wave128_f8_tiles<FMT, EPI, false, true, 256>(q, blockIdx.x, G, (LDS_PTR(char))lds_raw);
+  }
+  block_barrier();   // (the stages are laid out differently from here on: see gemm_wave128_mixed_kernel)
+  {
+    GemmArgs q = p;
+    q.A = p.A + (int64_t)rows256 * p.lda;
+    q.C = p.C + (int64_t)rows256 * p.ldc * 2;
+    q.M = p.M - rows256;
+    const int j = G - 1 - (int)blockIdx.x;
+    if (j < (q.M / 192) * nn) gemm_wave128_f8_tiles<FMT, EPI, false, true, 192>(q, j, G, (LDS_PTR(char))lds_raw);
+  }
+#endif
+}
+
+template <int FMT, int EPI>
+static int launch_wave128_f8_mixed(const GemmArgs& p, int rows256, hipStream_t stream) {
+  constexpr int smem = 2 * (256 + 256) * 128 + 1024;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_f8_mixed_kernel<FMT, EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = p.num_programs > 0 ? p.num_programs : 256;
+  gemm_wave128_f8_mixed_kernel<FMT, EPI><<<dim3(grid), dim3(256), smem, stream>>>(p, rows256);
+  return (int)hipGetLastError();
+}
+
+int gemm_wave128_f8_mixed_launch(const GemmArgs& p, int rows256, bool e5m2, hipStream_t stream) {
+  if (lean_epilogue_type(p) == 1) return e5m2 ? launch_wave128_f8_mixed<1, 3>(p, rows256, stream) : launch_wave128_f8_mixed<0, 3>(p, rows256, stream);
+  return e5m2 ? launch_wave128_f8_mixed<1, 4>(p, rows256, stream) : launch_wave128_f8_mixed<0, 4>(p, rows256, stream);
+}
+
+// fp8: the first `rows256` rows on 256-row tiles and the rest on 192-row tiles, under the conditions of the 192-row tiles
+bool gemm_wave128_f8_mixed_ok(const GemmArgs& p, bool b_kmajor, int rows256) {
+  if (!(rows256 > 0 && rows256 < p.M && rows256 % 256 == 0 && (p.M - rows256) % 192 == 0)) return false;
+  if (!(b_kmajor && p.N % 256 == 0 && p.k_bytes % 256 == 0 && p.k_bytes >= 256)) return false;
+  if (lean_epilogue_type(p) == 0) return false;
+  return p.lda * 8 + p.k_bytes < (1ll << 31) && p.ldb * 8 + p.k_bytes < (1ll << 31);
 }
 
 template <int FMT, int EPI, bool TAIL = false, bool B_KMAJOR = true, int BM = 256>
