@@ -94,6 +94,38 @@ const Knobs& knobs() {
 
 int knob(int value, int dflt) { return value == UNSET ? dflt : value; }
 
+// Two tile heights in one launch (gemm_wave128_mixed_kernel and its fp8 / block-scaled forms): the rows of C to give to
+// the 256-row tiles, the rest going to 192-row tiles, for a product of M rows and nn tile columns on P programs - or 0
+// when no split is rated 5 % better than one tile height.  A split is rated by its busiest program (tiles b, b + P, ...
+// of the first part and P - 1 - b, ... of the second; a 192-row tile counted as 0.78 of a 256-row one: 3072^3 on 192
+// of them against 4096^3 on 256 tiles, per tile and K step); among the splits within 7 % of the best, the one whose two
+// parts are closest in work is taken (measured: 5120^3 bf16 1164 / 1280 / 1325 TFLOP/s for 100 + 400 / 160 + 320 / 220 +
+// 240 tiles, which the count rates the same).
+int mixed_split(int M, int nn, int P) {
+  if (M % 256 != 0 || nn <= 0 || P <= 0) return 0;
+  auto count = [&](long tiles, int b) { return b < tiles ? (tiles - b + P - 1) / P : 0; };
+  const long tiles256 = (long)(M / 256) * nn;
+  double one_height = (double)((tiles256 + P - 1) / P), best = 1e30;   // in units of a 256-row tile's time
+  if (M % 192 == 0) one_height = std::min(one_height, 0.78 * (double)(((long)(M / 192) * nn + P - 1) / P));
+  auto busiest = [&](int a) {
+    const long n256 = (long)a * nn, n192 = (long)((M - a * 256) / 192) * nn;
+    double worst = 0;
+    for (int b = 0; b < P; b++) worst = std::max(worst, (double)count(n256, b) + 0.78 * (double)count(n192, P - 1 - b));
+    return worst;
+  };
+  for (int a = 1; a * 256 < M; a++)
+    if ((M - a * 256) % 192 == 0) best = std::min(best, busiest(a));
+  if (!(best < 0.95 * one_height)) return 0;
+  int best_rows = 0;
+  double best_gap = 1e30;
+  for (int a = 1; a * 256 < M; a++) {
+    if ((M - a * 256) % 192 != 0 || busiest(a) > 1.07 * best) continue;
+    const double gap = std::abs((double)a * nn - 0.78 * (double)((M - a * 256) / 192) * nn);
+    if (gap < best_gap) { best_gap = gap; best_rows = a * 256; }
+  }
+  return best_rows;
+}
+
 bool aligned(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
 int elem_size(int dtype) {
@@ -263,11 +295,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
       p.tile_m = 128;
     }
   }
-  // 16-bit and fp8 products of more than one round of tiles whose last round is badly filled: the upper rows on 256-row tiles
-  // and the lower ones on 192-row tiles in ONE launch (gemm_wave128_mixed_kernel), split so that the busiest program
-  // has the least to do.  A 192-row tile is counted as 0.78 of a 256-row one (3072^3 on 192 of them against 4096^3 on 256
-  // tiles, per tile and K step).  Flushed do_bench, bf16: 5120^3 (400 tiles; 220 + 240) and 7168^3 (784; 112 + 896) - see
-  // the design notes.  MI355_GEMM_MIXED_ROWS forces the rows of the 256-row part (0 = never).
+  // 16-bit and fp8 products of more than one round of tiles whose last round is badly filled: the upper rows on 256-row
+  // tiles and the lower ones on 192-row tiles in ONE launch, split by mixed_split.  MI355_GEMM_MIXED_ROWS forces the rows
+  // of the 256-row part (0 = never).
   int mixed_rows = 0;
   auto mixed_ok = [&](int rows256) {
     return is8 ? gemm_wave128_f8_mixed_ok(p, b_kmajor, rows256) : gemm_wave128_mixed_ok(p, b_kmajor, in_dtype, rows256);
@@ -278,27 +308,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
     if (want > 0) {
       if (mixed_ok(want)) mixed_rows = want;
     } else if (want < 0 && tile == 6 && p.tile_m == 0 && tiles256 > cus && M % 256 == 0) {
-      auto count = [&](long tiles, int b) { return b < tiles ? (tiles - b + P - 1) / P : 0; };   // tiles b, b + P, ... below `tiles`
-      double one_height = (double)((tiles256 + P - 1) / P), best = 1e30;   // in units of a 256-row tile's time
-      if (M % 192 == 0) one_height = std::min(one_height, 0.78 * (double)(((long)(M / 192) * nn + P - 1) / P));
-      auto busiest = [&](int a) {
-        const long n256 = (long)a * nn, n192 = (long)((M - a * 256) / 192) * nn;
-        double worst = 0;
-        for (int b = 0; b < P; b++) worst = std::max(worst, (double)count(n256, b) + 0.78 * (double)count(n192, P - 1 - b));
-        return worst;
-      };
-      for (int a = 1; a * 256 < M; a++)
-        if ((M - a * 256) % 192 == 0) best = std::min(best, busiest(a));
-      // among the splits within 7 % of the best one, the one whose two parts are closest in work (measured: 5120^3 1164 /
-      // 1280 / 1325 TFLOP/s for 100 + 400 / 160 + 320 / 220 + 240 tiles, which this count rates the same)
-      int best_rows = 0;
-      double best_gap = 1e30;
-      for (int a = 1; a * 256 < M; a++) {
-        if ((M - a * 256) % 192 != 0 || busiest(a) > 1.07 * best) continue;
-        const double gap = std::abs((double)a * nn - 0.78 * (double)((M - a * 256) / 192) * nn);
-        if (gap < best_gap) { best_gap = gap; best_rows = a * 256; }
-      }
-      if (best_rows > 0 && best < 0.95 * one_height && mixed_ok(best_rows)) mixed_rows = best_rows;
+      const int rows = mixed_split(M, nn, P);
+      if (rows > 0 && mixed_ok(rows)) mixed_rows = rows;
     }
   }
   p.num_programs = knob(knobs().programs, cus);  // persistent and stream-K forms (tile 5 / 7): one workgroup per CU
@@ -554,8 +565,16 @@ int mi355_mx_gemm(const uint8_t* A, const uint8_t* sA, const uint8_t* B, const u
       p.tile_m = 192;
     }
   }
-  tile = knob(knobs().tile, tile);
   p.num_programs = knob(knobs().programs, cus);
+  // and on both tile heights in one launch, as for the 16-bit and fp8 products
+  if (knobs().tile == UNSET && knobs().tile_m == UNSET && N % 256 == 0) {
+    const int want = knob(knobs().mixed_rows, -1), group = fmt == MI355_MXFP4 ? 512 : 1024;
+    int rows = 0;
+    if (want > 0) rows = want;
+    else if (want < 0 && tile == 6 && p.tile_m == 0 && tiles256 > cus) rows = mixed_split(M, N / 256, cus);
+    if (rows > 0 && gemm_wave128_mx_mixed_ok(p, group, rows)) return gemm_wave128_mx_mixed_launch(p, fmt == MI355_MXFP4 ? 0 : 1, rows, (hipStream_t)stream_);
+  }
+  tile = knob(knobs().tile, tile);
   return mx_gemm_launch(p, fmt, tile, (hipStream_t)stream_);
 }
 

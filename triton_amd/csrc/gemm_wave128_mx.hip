@@ -48,7 +48,7 @@ __device__ __forceinline__ void settle_tail(R&... r) {
 // the pipeline has free at that point, a quarter of the wave's tile at a time.
 // BM = 192: tiles of 192 x 256, as in the MXFP4 kernel below.
 template <int EPI, bool TAIL = false, int BM = 256>
-__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_wave128_mxfp8_tiles(const GemmArgs& p, int tile, const int tile_step, LDS_PTR(char) const lds_raw) {
   static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
   constexpr int BN = 256, ROWB = 128;
@@ -56,7 +56,6 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
   constexpr int MT = BM / 32, NT = 8, MH = MT / 2;
   constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
   constexpr int SC_BASE = 2 * STAGE, SC_SLOT = (256 + BN) * 16;     // scale ring behind the two stages (A part: room for 256 rows)
-  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -66,8 +65,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
 
   const int num_m = p.M / BM, num_n = p.N / BN;
   const int ntiles = num_m * num_n;
-  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
-  int pm, pn;
+  int pm, pn;   // (the tiles tile, tile + tile_step, ... are computed as one stream of K steps)
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = TAIL ? p.k_bytes / (8 * ROWB) * 8 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
@@ -255,7 +253,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
     if constexpr (PF) { pA += ROWB; pB += ROWB; }
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      if (ftile + tile_step < ntiles) ftile += tile_step;
       int fm, fn;
       grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
       set_fill_tile(fm, fn);
@@ -327,13 +325,61 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) 
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
-    tile += gridDim.x;
+    tile += tile_step;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
     zero_acc();
   }
   wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 #endif
+}
+
+// Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
+template <int EPI, bool TAIL = false, int BM = 256>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  gemm_wave128_mxfp8_tiles<EPI, TAIL, BM>(p, blockIdx.x, gridDim.x, (LDS_PTR(char))lds_raw);
+#endif
+}
+
+// Two tile heights in one launch, as for the 16-bit and fp8 products: the first `rows256` rows of C on tiles of 256 x 256,
+// the rows below (their operand and scale rows) on tiles of 192 x 256 dealt from the other end of the grid.
+template <int EPI>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp8_mixed_kernel(GemmArgs p, int rows256) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const int G = gridDim.x, nn = p.N / 256;
+  {
+    GemmArgs q = p;
+    q.M = rows256;
+    if ((int)blockIdx.x < (rows256 / 256) * nn) gemm_wave128_mxfp8_tiles<EPI, false, 256>(q, blockIdx.x, G, (LDS_PTR(char))lds_raw);
+  }
+  block_barrier();   // (the stages are laid out differently from here on; every wave has waited for its own loads)
+  {
+    GemmArgs q = p;
+    q.A = p.A + (int64_t)rows256 * p.lda;
+    q.sA = p.sA + (int64_t)rows256 * p.lds_a;
+    q.C = p.C + (int64_t)rows256 * p.ldc * 2;
+    q.M = p.M - rows256;
+    const int j = G - 1 - (int)blockIdx.x;
+    if (j < (q.M / 192) * nn) gemm_wave128_mxfp8_tiles<EPI, false, 192>(q, j, G, (LDS_PTR(char))lds_raw);
+  }
+#endif
+}
+
+template <int EPI>
+static int launch_wave128_mxfp8_mixed(const GemmArgs& p, int rows256, hipStream_t stream) {
+  constexpr int smem = 2 * (256 + 256) * 128 + 2 * 512 * 16 + 1024;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp8_mixed_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = p.num_programs > 0 ? p.num_programs : 256;
+  gemm_wave128_mxfp8_mixed_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p, rows256);
+  return (int)hipGetLastError();
 }
 
 bool gemm_wave128_mxfp8_ok(const GemmArgs& p) {
@@ -403,7 +449,7 @@ __device__ __forceinline__ void mfma16_mxfp4(const i32x4& a, const i32x4& b, f32
 // BM = 192: tiles of 192 x 256 (a wave: 96 x 128, six A fragments, 48 of the tile's A rows and scale rows to fetch), for
 // products whose 256 x 256 tiles fill the last round of CUs badly; lean epilogue, K steps in whole groups.
 template <int EPI, bool TAIL = false, int BM = 256>
-__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
+__device__ __forceinline__ void gemm_wave128_mxfp4_tiles(const GemmArgs& p, int tile, const int tile_step, LDS_PTR(char) const lds_raw) {
   static_assert(BM == 256 || ((BM == 192 || BM == 128) && !TAIL && (EPI == 3 || EPI == 4)), "192- and 128-row tiles: lean epilogue, no K tail");
 #if MI355_DEVICE_PASS
   constexpr int BN = 256, ROWB = 128;
@@ -412,7 +458,6 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
   constexpr int MT = BM / 32, NT = 8, KS = 2, NM = MT * NT, NRD = MT + NT;
   constexpr int LA = BM / 32, NLOADS = LA + 8;                      // direct loads per wave and K step: A, then B
   constexpr int EVERY = NM / 16;                                    // MFMAs per load slot: 4 (64 MFMAs) or 3 (48)
-  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
   const unsigned lds0 = lds_addr((LDS_PTR(const void))lds_raw);
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -422,8 +467,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
 
   const int num_m = p.M / BM, num_n = p.N / BN;
   const int ntiles = num_m * num_n;
-  int tile = blockIdx.x;   // this workgroup computes the tiles tile, tile + gridDim.x, ... as one stream of K steps
-  int pm, pn;
+  int pm, pn;   // (the tiles tile, tile + tile_step, ... are computed as one stream of K steps)
   grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
   const int nk = TAIL ? p.k_bytes / (4 * ROWB) * 4 : p.k_bytes / ROWB;
   int nk_last = nk;   // the same number, but opaque: see mfma_retire
@@ -608,7 +652,7 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     if constexpr (PF) { pA += ROWB; pB += ROWB; }
     if (++fk == nk) {
       fk = 0;
-      if (ftile + (int)gridDim.x < ntiles) ftile += gridDim.x;
+      if (ftile + tile_step < ntiles) ftile += tile_step;
       int fm, fn;
       grouped_tile(xcd_remap(ftile, ntiles), num_m, num_n, p.group_m, fm, fn);
       set_fill_tile(fm, fn);
@@ -679,13 +723,76 @@ __global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) 
     if constexpr (EPI == 3) gemm_epilogue16_lean<MT, NT, _Float16>(acc, p, em, en, el, ek);
     else if constexpr (EPI == 4) gemm_epilogue16_lean<MT, NT, __bf16>(acc, p, em, en, el, ek);
     else gemm_epilogue16<MT, NT>(acc, p, em, en, el, ek);
-    tile += gridDim.x;
+    tile += tile_step;
     if (tile >= ntiles) break;
     grouped_tile(xcd_remap(tile, ntiles), num_m, num_n, p.group_m, pm, pn);
     zero_acc();
   }
   wait_vmcnt<0>();  // nothing may still be writing LDS when the workgroup ends
 #endif
+}
+
+// Workgroup b computes the tiles b, b + gridDim.x, ... (the grid: wave128_grid).
+template <int EPI, bool TAIL = false, int BM = 256>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_kernel(GemmArgs p) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  gemm_wave128_mxfp4_tiles<EPI, TAIL, BM>(p, blockIdx.x, gridDim.x, (LDS_PTR(char))lds_raw);
+#endif
+}
+
+// Two tile heights in one launch, as for the 16-bit and fp8 products: the first `rows256` rows of C on tiles of 256 x 256,
+// the rows below (their operand and scale rows) on tiles of 192 x 256 dealt from the other end of the grid.
+template <int EPI>
+__global__ __launch_bounds__(256, 1) void gemm_wave128_mxfp4_mixed_kernel(GemmArgs p, int rows256) {
+#if MI355_DEVICE_PASS
+  extern __shared__ __attribute__((aligned(1024))) char lds_raw[];
+  const int G = gridDim.x, nn = p.N / 256;
+  {
+    GemmArgs q = p;
+    q.M = rows256;
+    if ((int)blockIdx.x < (rows256 / 256) * nn) gemm_wave128_mxfp4_tiles<EPI, false, 256>(q, blockIdx.x, G, (LDS_PTR(char))lds_raw);
+  }
+  block_barrier();   // (the stages are laid out differently from here on; every wave has waited for its own loads)
+  {
+    GemmArgs q = p;
+    q.A = p.A + (int64_t)rows256 * p.lda;
+    q.sA = p.sA + (int64_t)rows256 * p.lds_a;
+    q.C = p.C + (int64_t)rows256 * p.ldc * 2;
+    q.M = p.M - rows256;
+    const int j = G - 1 - (int)blockIdx.x;
+    if (j < (q.M / 192) * nn) gemm_wave128_mxfp4_tiles<EPI, false, 192>(q, j, G, (LDS_PTR(char))lds_raw);
+  }
+#endif
+}
+
+template <int EPI>
+static int launch_wave128_mxfp4_mixed(const GemmArgs& p, int rows256, hipStream_t stream) {
+  constexpr int smem = 2 * (256 + 256) * 128 + 2 * 512 * 16 + 1024;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_wave128_mxfp4_mixed_kernel<EPI>, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int grid = p.num_programs > 0 ? p.num_programs : 256;
+  gemm_wave128_mxfp4_mixed_kernel<EPI><<<dim3(grid), dim3(256), smem, stream>>>(p, rows256);
+  return (int)hipGetLastError();
+}
+
+// fmt: 0 = MXFP4, else MXFP8 (gemm_wave128_mx_mixed_ok: lean epilogue)
+int gemm_wave128_mx_mixed_launch(const GemmArgs& p, int fmt, int rows256, hipStream_t stream) {
+  const int lean = lean_epilogue_type(p);
+  if (fmt == 0) return lean == 1 ? launch_wave128_mxfp4_mixed<3>(p, rows256, stream) : launch_wave128_mxfp4_mixed<4>(p, rows256, stream);
+  return lean == 1 ? launch_wave128_mxfp8_mixed<3>(p, rows256, stream) : launch_wave128_mxfp8_mixed<4>(p, rows256, stream);
+}
+
+// the first `rows256` rows on 256-row tiles and the rest on 192-row tiles, under the conditions of the 192-row tiles
+bool gemm_wave128_mx_mixed_ok(const GemmArgs& p, int group_bytes, int rows256) {
+  if (!(rows256 > 0 && rows256 < p.M && rows256 % 256 == 0 && (p.M - rows256) % 192 == 0)) return false;
+  GemmArgs q = p;
+  q.M = 768;   // (a multiple of both tile heights: the other conditions of gemm_wave128_mx_192_ok)
+  return gemm_wave128_mx_192_ok(q, group_bytes, 192);
 }
 
 // the block-scaled forms on tiles of 192 x 256: M a multiple of 192, whole groups of K steps (`group_bytes` of a row: 512

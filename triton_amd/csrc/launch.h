@@ -117,6 +117,8 @@ int gemm_wave128_mixed_launch(const GemmArgs& p, int rows256, bool bf16, bool b_
 bool gemm_wave128_f8_mixed_ok(const GemmArgs& p, bool b_kmajor, int rows256);
 int gemm_wave128_f8_mixed_launch(const GemmArgs& p, int rows256, bool e5m2, hipStream_t stream);
 bool gemm_wave128_f8_192_ok(const GemmArgs& p, bool b_kmajor, int tile_m = 192);   // tiles of 192 x 256 / 128 x 256
+bool gemm_wave128_mx_mixed_ok(const GemmArgs& p, int group_bytes, int rows256);
+int gemm_wave128_mx_mixed_launch(const GemmArgs& p, int fmt, int rows256, hipStream_t stream);   // fmt: 0 = MXFP4, else MXFP8
 bool gemm_wave128_mx_192_ok(const GemmArgs& p, int group_bytes, int tile_m = 192);   // in_dtype: C ABI code of the operands' type
 int gemm_wave128_launch(const GemmArgs& p, bool bf16, bool b_kmajor, hipStream_t stream);
 int gemm_wave128_f8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, hipStream_t stream);
