@@ -881,6 +881,25 @@ def test_lean_and_general_epilogue_of_the_four_wave_kernels_agree_bit_for_bit(gp
             assert bits_equal(results[name, "1"], results[name, "0"]), name
 
 
+@pytest.mark.parametrize("dtype", ["bf16", "fp16"])
+@pytest.mark.parametrize("N", [1004, 1001])
+def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_k_major_copy(gpu, dtype, N):
+    # rows of a row-major B that are not 16-byte multiples cannot be loaded by the MFMA kernels; the wrapper puts such a
+    # B K-major (one copy) instead of leaving the product to the strided kernel.  Integer-valued operands: exact sums,
+    # so the result is the strided kernel's bit for bit, in a C of the caller's shape.
+    rng = np.random.default_rng(N)
+    M, K = 512, 768
+    ai = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    bi = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    got = triton_amd.matmul(from_np(ai, dtype, gpu), from_np(bi, dtype, gpu), out_dtype=torch.float32)
+    assert got.shape == (M, N) and got.is_contiguous()
+    assert bits_equal(to_np(got), (ai.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))
+    a, b = randn_rounded(rng, (M, K), dtype, 1.0), randn_rounded(rng, (K, N), dtype, 1.0)
+    got = to_np(triton_amd.matmul(from_np(a, dtype, gpu), from_np(b, dtype, gpu)))
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    assert np.allclose(got, ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+
+
 @pytest.mark.parametrize("case", ["bf16 row-major B", "fp16 K-major B", "fp8"])
 def test_k_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_zero_padding(gpu, case):
     # rows that are not 16-byte multiples cannot be loaded by the MFMA kernels; the wrapper appends the zeros that the
