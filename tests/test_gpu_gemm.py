@@ -63,6 +63,59 @@ def test_unaligned_shapes_take_the_strided_kernel(gpu, shape):
     assert np.allclose(c, gemm.matmul_tiled(a, b, 64, 64, 32, 8, out_dtype="fp16"), rtol=1e-2, atol=1e-2)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3", "e5m2"])
+def test_masked_mfma_kernel_against_the_fp32_fma_kernel_on_odd_shapes_and_strides(gpu, monkeypatch, dtype):
+    # Operands that the tiled kernels do not take run 64 x 64 tiles on MFMAs with masked loads; the older kernel of fp32
+    # FMAs (MI355_GEMM_FORCE_STRIDED=2) is a second implementation.  Integer-valued data: every sum is exact, so the
+    # two - and the closed form - agree bit for bit, whatever the order of the sums.  Shapes with a single row or
+    # column, K below and across the 32-element step, rows that start at odd addresses, B in all three layouts
+    # (row-major, K-major, neither axis contiguous), C with a column stride.
+    from triton_amd import _lib
+
+    rng = np.random.default_rng(len(dtype) + ord(dtype[-1]))
+    tdt = {"fp16": torch.float16, "bf16": torch.bfloat16, "e4m3": torch.float8_e4m3fn, "e5m2": torch.float8_e5m2}[dtype]
+    abi = {"fp16": _lib.F16, "bf16": _lib.BF16, "e4m3": _lib.F8E4M3, "e5m2": _lib.F8E5M2}[dtype]
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    for (M, N, K) in [(1, 1, 1), (2047, 1, 1024), (1, 1100, 257), (100, 100, 512), (512, 33, 100), (65, 129, 31), (37, 19, 7),
+                      (130, 250, 100), (64, 64, 33), (300, 70, 1000)]:
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+
+        def dev(x):
+            t = torch.from_numpy(x).to(gpu)
+            return t.to(tdt)
+
+        ta = dev(a)
+        for layout in ("row-major", "K-major", "neither", "odd base"):
+            if layout == "row-major":
+                tb = dev(b)
+            elif layout == "K-major":
+                tb = dev(b).t().contiguous().t()
+            elif layout == "neither":
+                tb = torch.zeros(K, 3 * N, dtype=torch.float32, device=gpu).to(tdt)
+                tb[:, ::3] = dev(b)
+                tb = tb[:, ::3]
+            else:
+                flat = torch.zeros(K * N + 1, dtype=torch.float32, device=gpu).to(tdt)
+                flat[1:] = dev(b).reshape(-1)
+                tb = flat[1:].view(K, N)
+            outs = []
+            for force in ("1", "2"):
+                set_knob(monkeypatch, "MI355_GEMM_FORCE_STRIDED", force)
+                cbuf = torch.full((M, 2 * N), 7.0, dtype=torch.float32, device=gpu)
+                c = cbuf[:, ::2]                                      # column stride 2
+                rc = lib.mi355_gemm(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), M, N, K, ta.stride(0), ta.stride(1),
+                                    tb.stride(0), tb.stride(1), c.stride(0), c.stride(1), abi, _lib.F32, 0, 0, _lib.ACT_NONE, stream)
+                assert rc == 0
+                torch.cuda.synchronize()
+                assert torch.all(cbuf[:, 1::2] == 7.0), "columns between the outputs untouched"
+                outs.append(c.cpu().numpy())
+            assert bits_equal(outs[0], ref), (dtype, M, N, K, layout)
+            assert bits_equal(outs[1], ref), (dtype, M, N, K, layout, "fp32 FMA kernel")
+
+
 def test_arbitrary_strides_on_b_and_c_views(gpu):
     rng = np.random.default_rng(12)
     a = randn_rounded(rng, (96, 64), "fp16")

@@ -206,7 +206,8 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   if (!fast) {
     GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype,
                       aux, aux_sm, aux_sn, aux_dtype};
-    return gemm_strided_launch(s, stream);
+    // (MI355_GEMM_FORCE_STRIDED=2: the fp32-FMA kernel, a second implementation kept for tests)
+    return knob(knobs().force_strided, 0) == 2 ? gemm_strided_launch(s, stream) : gemm_masked_launch(s, stream);
   }
 
   GemmArgs p{};

@@ -130,7 +130,8 @@ bool gemm8_skinny_ok(const GemmArgs& p);  // M <= 32, K a multiple of 256
 int gemm8_skinny_launch(const GemmArgs& p, bool e5m2, hipStream_t stream);
 bool gemm_skinny_ok(const SkinnyArgs& p, bool y_kmajor, bool x_kmajor, int elem_bytes);
 int gemm_skinny_launch(const SkinnyArgs& p, int kind, bool y_kmajor, bool x_kmajor, hipStream_t stream);
-int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);
+int gemm_strided_launch(const GemmStridedArgs& p, hipStream_t stream);   // fp32 FMAs, one thread per 4 x 4 outputs (a second implementation for tests)
+int gemm_masked_launch(const GemmStridedArgs& p, hipStream_t stream);    // 64 x 64 tiles on MFMAs with masked loads: any strides and sizes
 int mx_gemm_launch(const GemmArgs& p, int fmt, int tile, hipStream_t stream);
 int attn_fwd_launch(const AttnArgs& p, bool bf16, hipStream_t stream);
 bool attn_fwd_pipe_ok(const AttnArgs& p);
