@@ -636,12 +636,15 @@ def test_decode_shape_m16(gpu):
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(16, 256, 512), (64, 128, 1024), (33, 96, 64), (1, 32, 32), (7, 2048, 4096),
-                                   (256, 64, 512), (128, 32, 256), (1024, 16, 2048), (96, 40, 96)])
+                                   (256, 64, 512), (128, 32, 256), (1024, 16, 2048), (96, 40, 96),
+                                   (100, 2048, 512), (128, 2048, 256), (65, 4096, 128), (2048, 128, 512), (2048, 96, 256),
+                                   (2048, 100, 256)])
 def test_skinny_16bit_kernel_is_bit_exact_on_integers(gpu, monkeypatch, dtype, shape):
     # at most 64 rows on one side (shapes of python/test/regression/test_performance.py:36-44): the
     # streaming kernel (K split over the waves of a workgroup) for row-major and K-major B; M > 64
     # with N <= 64 takes it with the operands swapped (a row-major B then needs N = 32 or 64; the
-    # other cases here fall through to the tile kernels).  Every partial sum is an exact integer,
+    # other cases here fall through to the tile kernels); 65 .. 128 rows against at least 2048 on the other
+    # side run as two launches, 64 rows and the rest.  Every partial sum is an exact integer,
     # so the result does not depend on how K is split.
     M, N, K = shape
     rng = np.random.default_rng(M + 3 * N + 7 * K)
@@ -777,12 +780,12 @@ def test_row_major_fp8_b_under_every_tile_choice_with_addend_activation_and_fp8_
 
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("shape", [(64, 64, 64), (128, 128, 64), (512, 768, 256), (300, 200, 136), (100, 70, 50), (16, 256, 512),
-                                   (1024, 32, 256)])
+                                   (1024, 32, 256), (100, 2048, 64), (2048, 128, 64)])
 def test_fused_epilogues_of_the_reference_dot_test(gpu, dtype, shape):
     # add-matrix / add-rows / add-cols / softmax / chain-dot (python/test/unit/language/test_core.py:3128-3145)
-    # through mi355_gemm_epilogue: MFMA tile kernels, the strided kernel (100, 70, 50) and two skinny
+    # through mi355_gemm_epilogue: MFMA tile kernels, the any-stride kernel (100, 70, 50) and four skinny
     # shapes (the streaming kernels add the addend in their own epilogue; the second one runs with the
-    # operands swapped).  Integer data: bit-exact.
+    # operands swapped, the last two as two launches of 64 rows and the rest).  Integer data: bit-exact.
     M, N, K = shape
     rng = np.random.default_rng(M + N + K)
     a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
@@ -936,10 +939,10 @@ def test_lean_and_general_epilogue_of_the_four_wave_kernels_agree_bit_for_bit(gp
 
 @pytest.mark.parametrize("dtype", ["bf16", "fp16"])
 @pytest.mark.parametrize("N", [1004, 1001])
-def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_k_major_copy(gpu, dtype, N):
-    # rows of a row-major B that are not 16-byte multiples cannot be loaded by the MFMA kernels; the wrapper puts such a
-    # B K-major (one copy) instead of leaving the product to the strided kernel.  Integer-valued operands: exact sums,
-    # so the result is the strided kernel's bit for bit, in a C of the caller's shape.
+def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_padded_pitch(gpu, dtype, N):
+    # rows of a row-major B that do not start on 16-byte boundaries cannot be loaded by the MFMA kernels; the wrapper
+    # copies such a B into rows of a padded pitch instead of leaving the product to the any-stride kernel.
+    # Integer-valued operands: exact sums, so the result is that kernel's bit for bit, in a C of the caller's shape.
     rng = np.random.default_rng(N)
     M, K = 512, 768
     ai = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
@@ -951,6 +954,29 @@ def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_k_major_c
     got = to_np(triton_amd.matmul(from_np(a, dtype, gpu), from_np(b, dtype, gpu)))
     ref = a.astype(np.float64) @ b.astype(np.float64)
     assert np.allclose(got, ref, rtol=1e-2, atol=1e-2 * np.abs(ref).max())
+    # a B that already lives in a buffer with a padded pitch (rows start on 16-byte boundaries, N is no multiple) is
+    # taken as it is: the last chunk of a row reaches into the padding - filled with NaN here, which must not show
+    wide = torch.full((K, N + 16 - N % 8), float("nan"), dtype=torch.float32, device=gpu).to(from_np(bi, dtype, gpu).dtype)
+    wide[:, :N] = from_np(bi, dtype, gpu)
+    got = triton_amd.matmul(from_np(ai, dtype, gpu), wide[:, :N], out_dtype=torch.float32)
+    assert bits_equal(to_np(got), (ai.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))
+
+
+@pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
+def test_row_major_fp8_b_with_n_not_a_multiple_of_16_in_a_padded_pitch(gpu, fmt, tdt):
+    # the fp8 case of the same: N = 1000 in rows of 1008 bytes, and through the wrapper's padding copy (pitch 1000)
+    rng = np.random.default_rng(41)
+    M, N, K = 512, 1000, 768
+    a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    b = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+    ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)
+    tb = torch.from_numpy(formats.encode_fp8(b, fmt)).to(gpu).view(tdt)
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    wide = torch.full((K, 1008), 0x7f if fmt == "e4m3" else 0x7e, dtype=torch.uint8, device=gpu)    # NaN codes
+    wide[:, :N] = tb.view(torch.uint8)
+    for bb in (tb, wide.view(tdt)[:, :N]):
+        got = triton_amd.matmul(ta, bb, out_dtype=torch.float32)
+        assert got.shape == (M, N) and bits_equal(to_np(got), ref), bb.stride()
 
 
 @pytest.mark.parametrize("case", ["bf16 row-major B", "fp16 K-major B", "fp8"])

@@ -198,7 +198,9 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const bool out_ok = true;   // every output type of the ABI has a store in the MFMA epilogues (fp8: hardware conversion, saturating)
   const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
-  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= N && N % vec == 0 && aligned(B, 16);
+  // (a row-major B: rows of whole 16-byte chunks - N itself need not be one: the last chunk of a row then reaches into
+  // the padding that the pitch provides, and the columns beyond N are never stored)
+  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
   // the tile copies address 256 rows of an operand with 32-bit byte offsets from a 64-bit tile base
   const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
   const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && knob(knobs().force_strided, 0) == 0;
@@ -318,24 +320,45 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   p.workspace = workspace;
   const bool skinny_allowed = tile_arg < 0 && knob(knobs().skinny, 1);  // an explicit tile means a tile kernel
   if (skinny_allowed) {
-    // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side)
+    // at most 64 rows on one side: stream the other operand once (X = small side, Y = streamed side).  65 .. 128 rows
+    // against a streamed side of at least 2048: two such launches, 64 rows and the rest - the tile kernels have too
+    // few tiles there (flushed do_bench, bf16, tile kernel / two launches: 2048 x 128 x 4096 50.6 / 39.1 us, 8192 x 128 x
+    // 8192 117 / 95, 128 x 8192 x 8192 124 / 102; with 256 rows the tiles win, 115 / 147).
     SkinnyArgs sk{};
     sk.K = K; sk.C = (char*)C; sk.a_scale = a_scale; sk.b_scale = b_scale;
     sk.activation = activation; sk.out_dtype = out_dtype; sk.cus = device_info().cus;
     bool use = false, y_kmajor = false, x_kmajor = true;
-    if (M <= 64) {
-      sk.X = (const char*)A; sk.Y = (const char*)B; sk.S = M; sk.L = N;
+    int small = 0;
+    if (M <= 64 || (M <= 128 && N >= 2048)) {
+      sk.X = (const char*)A; sk.Y = (const char*)B; small = M; sk.L = N;
       sk.x_pitch = p.lda; sk.y_pitch = p.ldb; sk.cs = scm; sk.cl = scn;
       sk.aux = aux; sk.aux_ss = aux_sm; sk.aux_sl = aux_sn; sk.aux_dtype = aux_dtype;
       y_kmajor = b_kmajor; use = true;
-    } else if (N <= 64) {
-      sk.X = (const char*)B; sk.Y = (const char*)A; sk.S = N; sk.L = M;
+    } else if (N <= 64 || (N <= 128 && M >= 2048)) {
+      sk.X = (const char*)B; sk.Y = (const char*)A; small = N; sk.L = M;
       sk.x_pitch = p.ldb; sk.y_pitch = p.lda; sk.cs = scn; sk.cl = scm;
       sk.aux = aux; sk.aux_ss = aux_sn; sk.aux_sl = aux_sm; sk.aux_dtype = aux_dtype;
       y_kmajor = true; x_kmajor = b_kmajor; use = true;
     }
-    if (use && gemm_skinny_ok(sk, y_kmajor, x_kmajor, es))
-      return gemm_skinny_launch(sk, in_dtype, y_kmajor, x_kmajor, stream);
+    if (use) {
+      SkinnyArgs part[2] = {sk, sk};
+      part[0].S = small < 64 ? small : 64;
+      part[1].S = small - part[0].S;
+      // (the second part starts 64 rows of X further: K-contiguous rows 64 pitches, S-contiguous rows 64 elements on)
+      part[1].X = sk.X + (x_kmajor ? 64 * sk.x_pitch : (int64_t)64 * es);
+      part[1].C = sk.C + 64 * sk.cs * elem_size(out_dtype);
+      if (aux) part[1].aux = (const char*)aux + 64 * sk.aux_ss * elem_size(aux_dtype);
+      const int nparts = part[1].S > 0 ? 2 : 1;
+      bool ok = true;
+      for (int i = 0; i < nparts; i++) ok = ok && gemm_skinny_ok(part[i], y_kmajor, x_kmajor, es);
+      if (ok) {
+        for (int i = 0; i < nparts; i++) {
+          const int rc = gemm_skinny_launch(part[i], in_dtype, y_kmajor, x_kmajor, stream);
+          if (rc != 0) return rc;
+        }
+        return MI355_OK;
+      }
+    }
   }
   if (is8 && b_kmajor && !aux && gemm8_skinny_ok(p) && skinny_allowed) return gemm8_skinny_launch(p, in_dtype == MI355_F8E5M2, stream);
   if (is8 && mixed_rows > 0) return gemm_wave128_f8_mixed_launch(p, mixed_rows, in_dtype == MI355_F8E5M2, stream);

@@ -233,7 +233,10 @@ __device__ __forceinline__ void gemm_tile_body(const GemmArgs& p, const int pm, 
     } else {
       int r = CopyBn::row(wave, lane, i);
       int nb = n0 * EB + CopyBn::col16(lane, r) * 16;   // byte column of the chunk
-      nb = nb < p.N * EB ? nb : p.N * EB - 16;          // rows of whole chunks on this path: clamp whole chunks
+      // (clamp whole chunks; the last chunk of a row may reach beyond N into the row's padding: the C ABI takes a
+      // row-major B only with a pitch that covers N rounded up to whole chunks)
+      const int nbytes = (p.N * EB + 15) / 16 * 16;
+      nb = nb < nbytes ? nb : nbytes - 16;
       srcB[i] = p.B + (int64_t)r * p.ldb + nb;
     }
   }
@@ -690,7 +693,8 @@ __global__ __launch_bounds__(512, 1) void gemm_pp_kernel(GemmArgs p) {
     } else {
       int r = CopyBn::row(wave, lane, i);
       int n = n0 + CopyBn::col16(lane, r) * 8;
-      n = n < p.N ? n : p.N - 8;
+      const int npad = (p.N + 7) / 8 * 8;   // (the last chunk may reach into the row's padding, see gemm_tile_body)
+      n = n < npad ? n : npad - 8;
       srcB[i] = p.B + (int64_t)r * p.ldb + (int64_t)n * 2;
     }
   }
@@ -994,7 +998,8 @@ __global__ __launch_bounds__(2 * WN * 64, 1) void gemm_w4_kernel(GemmArgs p) {
     } else {
       int r = CopyBn::row(wave, lane, i);
       int n = n0 + CopyBn::col16(lane, r) * 8;
-      n = (n < p.N ? n : p.N - 8) - n0;
+      const int npad = (p.N + 7) / 8 * 8;   // (the last chunk may reach into the row's padding, see gemm_tile_body)
+      n = (n < npad ? n : npad - 8) - n0;
       offGB[i] = (unsigned)r * (unsigned)p.ldb + (unsigned)n * 2;
     }
   }

@@ -135,13 +135,14 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         K += pad        # (the launch metadata below keeps the caller's K)
     vec = 16 // _ELEM_BYTES[in_dt] if in_dt != _lib.F32 else 0
     if (vec and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
-            and (N % vec != 0 or b.stride(0) % vec != 0 or b.data_ptr() % 16 != 0) and K % vec == 0 and M * N * K >= 1 << 24):
-        # A row-major B runs on the MFMAs inside the C ABI when its rows are whole 16-byte chunks.  One that is not (N
-        # or the pitch not a multiple of 16 bytes) would take the strided kernel (8100 x 8100 x 8192 bf16: 48 TFLOP/s):
-        # it is put K-major first, as the reference does on the host for its fp8 case ("pre-transpose b for
-        # efficiency", 03:378-380) - K-major rows are K elements long, which are whole chunks here (the same shape:
-        # 885 TFLOP/s, the copy included).
-        b = b.t().contiguous().t()
+            and (b.stride(0) % vec != 0 or b.data_ptr() % 16 != 0) and K % vec == 0 and M * N * K >= 1 << 24):
+        # A row-major B runs on the MFMAs inside the C ABI when its rows START on 16-byte boundaries (N itself need not
+        # be a multiple: the last chunk of a row then reaches into the padding that the pitch provides).  One whose
+        # pitch is not a multiple of 16 bytes would take the any-stride kernel (8100 x 8100 x 8192 bf16: 48 TFLOP/s on
+        # the old kernel of that path): its rows are copied into a buffer with a padded pitch first - one plain copy,
+        # as the reference spends one on its fp8 case ("pre-transpose b for efficiency", 03:378-380).
+        as_bytes = (lambda t: t.view(torch.uint8)) if _ELEM_BYTES[in_dt] == 1 else (lambda t: t)
+        b = torch.nn.functional.pad(as_bytes(b), (0, -N % vec)).view(b.dtype)[:, :N]
     pa, keep_a = _scale_ptr(a_scale, device)
     pb, keep_b = _scale_ptr(b_scale, device)
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
