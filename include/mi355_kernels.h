@@ -90,8 +90,9 @@ enum {
  *   python/tutorials/09-persistent-matmul.py:48-102 (kernel), :105-138 (`matmul`, fp8e4nv)
  * i.e. what the generated launcher third_party/amd/backend/driver.py:326-377 does for them.
  * Same arguments as the kernel: three pointers, M N K, six strides (any strides are accepted;
- * the MFMA path needs a unit stride on one axis of each operand and rows of whole 16-byte chunks -
- * either layout of B for every type -, anything else runs a slower strided kernel on the GPU), plus ACTIVATION.  in_dtype is the type of A and B
+ * the tiled MFMA kernels need a unit stride on one axis of each operand and rows that start on 16-byte boundaries -
+ * either layout of B for every type; K a multiple of 16 bytes, N any size when a row-major B's pitch covers N rounded up
+ * to 16 bytes -, anything else runs a slower MFMA kernel of 64x64 tiles with masked element loads), plus ACTIVATION.  in_dtype is the type of A and B
  * (they must match, python/triton/language/semantic.py:1355).  a_scale / b_scale are
  * optional device pointers to one fp32 each (NULL = 1.0): per-tensor dequantisation
  * scales for fp8 inputs, applied to the fp32 accumulator before activation and cast.
@@ -121,7 +122,7 @@ int mi355_gemm(const void* A, const void* B, void* C,
  * take ceil(tiles / programs) tiles each as one stream of K steps)
  * (a kernel that does not exist for the dtype or shape falls back to the nearest one).  group_m: the
  * reference's GROUP_SIZE_M (:265-273), 0 = default 8.  Operands without 16-byte rows run the
- * strided kernel whatever `tile` says.
+ * masked any-stride kernel whatever `tile` says.
  */
 int mi355_gemm_tuned(const void* A, const void* B, void* C,
                      int M, int N, int K,

@@ -944,7 +944,7 @@ def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_padded_pi
     # copies such a B into rows of a padded pitch instead of leaving the product to the any-stride kernel.
     # Integer-valued operands: exact sums, so the result is that kernel's bit for bit, in a C of the caller's shape.
     rng = np.random.default_rng(N)
-    M, K = 512, 768
+    M, K = 1024, 1536       # (large enough for the wrapper to copy: 2^30 multiply-adds)
     ai = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
     bi = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
     got = triton_amd.matmul(from_np(ai, dtype, gpu), from_np(bi, dtype, gpu), out_dtype=torch.float32)
@@ -966,7 +966,7 @@ def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_padded_pi
 def test_row_major_fp8_b_with_n_not_a_multiple_of_16_in_a_padded_pitch(gpu, fmt, tdt):
     # the fp8 case of the same: N = 1000 in rows of 1008 bytes, and through the wrapper's padding copy (pitch 1000)
     rng = np.random.default_rng(41)
-    M, N, K = 512, 1000, 768
+    M, N, K = 1024, 1000, 1536
     a = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
     b = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
     ta = torch.from_numpy(formats.encode_fp8(a, fmt)).to(gpu).view(tdt)

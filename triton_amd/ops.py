@@ -119,12 +119,15 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         return c
     if K == 0:
         return c.zero_()
-    if (in_dt != _lib.F32 and (K * _ELEM_BYTES[in_dt]) % 16 != 0 and M * N * K >= 1 << 24
+    if (in_dt != _lib.F32 and (K * _ELEM_BYTES[in_dt]) % 16 != 0 and M * N * K >= 1 << 30
             and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)):
         # Rows of A that are not a multiple of 16 bytes long do not start on 16-byte boundaries, which every MFMA
         # kernel's loads need: the C ABI then runs its strided kernel (4096 x 4096 x 4100 bf16: 43 TFLOP/s).  The
         # reference masks the K tail to zero (03:297-298); appending those zeros to K here - one copy of each
-        # operand - gives the same sums on the fast kernels (the same shape: 1000 TFLOP/s).
+        # operand - gives the same sums on the fast kernels (the same shape: 1000 TFLOP/s).  Below about 2^30
+        # multiply-adds the any-stride MFMA kernel is as fast or faster than the copies plus the tile kernels (flushed
+        # do_bench, bf16, that kernel / padded: 2048 x 100 x 100 12 / 27 us, 2047 x 257 x 257 16 / 32, 1024 x 1024 x 1000 23 / 23,
+        # 1024 x 1024 x 4100 107 / 70).
         pad = -K % (16 // _ELEM_BYTES[in_dt])
         as_bytes = (lambda t: t.view(torch.uint8)) if _ELEM_BYTES[in_dt] == 1 else (lambda t: t)
         a = torch.nn.functional.pad(as_bytes(a), (0, pad)).view(a.dtype)
@@ -135,7 +138,7 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         K += pad        # (the launch metadata below keeps the caller's K)
     vec = 16 // _ELEM_BYTES[in_dt] if in_dt != _lib.F32 else 0
     if (vec and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
-            and (b.stride(0) % vec != 0 or b.data_ptr() % 16 != 0) and K % vec == 0 and M * N * K >= 1 << 24):
+            and (b.stride(0) % vec != 0 or b.data_ptr() % 16 != 0) and K % vec == 0 and M * N * K >= 1 << 30):
         # A row-major B runs on the MFMAs inside the C ABI when its rows START on 16-byte boundaries (N itself need not
         # be a multiple: the last chunk of a row then reaches into the padding that the pitch provides).  One whose
         # pitch is not a multiple of 16 bytes would take the any-stride kernel (8100 x 8100 x 8192 bf16: 48 TFLOP/s on
