@@ -962,6 +962,23 @@ def test_n_not_a_multiple_of_16_bytes_takes_the_fast_kernels_through_a_padded_pi
     assert bits_equal(to_np(got), (ai.astype(np.float64) @ bi.astype(np.float64)).astype(np.float32))
 
 
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4, 5])
+def test_padded_pitch_row_major_b_under_every_tile_kernel(gpu, monkeypatch, tile):
+    # N = 2052 in rows of 2056 elements (NaN in the padding), enough tiles for the large-product kernels: every tile
+    # kernel clamps its last chunk of a B row to N rounded up to whole chunks.  Integer data: exact.
+    set_knob(monkeypatch, "MI355_GEMM_TILE", tile)
+    rng = np.random.default_rng(50 + tile)
+    M, N, K = 1024, 2052, 320
+    a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    for dtype in ("bf16", "fp16"):
+        wide = torch.full((K, N + 4), float("nan"), dtype=torch.float32, device=gpu).to(from_np(b, dtype, gpu).dtype)
+        wide[:, :N] = from_np(b, dtype, gpu)
+        got = triton_amd.matmul(from_np(a, dtype, gpu), wide[:, :N], out_dtype=torch.float32)
+        assert bits_equal(to_np(got), ref), (tile, dtype)
+
+
 @pytest.mark.parametrize("fmt,tdt", [("e4m3", torch.float8_e4m3fn), ("e5m2", torch.float8_e5m2)])
 def test_row_major_fp8_b_with_n_not_a_multiple_of_16_in_a_padded_pitch(gpu, fmt, tdt):
     # the fp8 case of the same: N = 1000 in rows of 1008 bytes, and through the wrapper's padding copy (pitch 1000)
