@@ -27,8 +27,9 @@
  * product, clock probe, environment refresh, MI355_ESCRATCH, head dims 16 / 32 / 256 in the backward, fp8 output
  * of the MFMA epilogues; 3: MFMA burn probe with its block-scaled shapes, per-device properties, fp8 attention forward at
  * head dims 16 / 32 / 256, a row-major fp8 B on the MFMA kernels, block-scaled products with any K that is a multiple of
- * 32 and scale rows of any pitch on the MFMA kernels.) */
-#define MI355_ABI_VERSION 3
+ * 32 and scale rows of any pitch on the MFMA kernels; 4: mi355_gemm_splitk, a row-major B whose N is not a multiple of
+ * 16 bytes inside a padded pitch on the tile kernels.) */
+#define MI355_ABI_VERSION 4
 
 #ifdef __cplusplus
 extern "C" {
@@ -132,6 +133,26 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C,
                      int in_dtype, int out_dtype,
                      const float* a_scale, const float* b_scale,
                      int activation, int tile, int group_m, void* stream);
+
+/* mi355_gemm with K split over `splits` workgroups per tile (0 = chosen by size: one workgroup per CU, at least sixteen
+ * 64-byte K steps each, at most 32; none from half a round of 128x128 tiles on): for products of few tiles with a long K - one row of tiles against a long
+ * weight, a small square against a long K -, where one workgroup per tile leaves most of the device idle and a few
+ * K steps of loads in flight are all that hides the memory latency.  The reference's kernel has no such form
+ * (python/tutorials/03-matrix-multiplication.py:241-316 gives every tile to one program); the contract is the same
+ * C = act((a_scale * b_scale) * A @ B) with fp32 accumulation and one rounding, the partial sums added in split order.
+ * Two launches: the tile kernel on 128x128 tiles into fp32 slices of `workspace`, then the sum and the epilogue.
+ * workspace: device memory of at least splits * M * N * 4 bytes (32 * M * N * 4 always suffices for splits = 0),
+ * 16-byte aligned, contents irrelevant; two calls that overlap in time need different workspaces.  Operands that the
+ * tile kernels do not take, or a K too short to split, run as mi355_gemm (the workspace is then not touched).
+ */
+int mi355_gemm_splitk(const void* A, const void* B, void* C,
+                      int M, int N, int K,
+                      int64_t stride_am, int64_t stride_ak,
+                      int64_t stride_bk, int64_t stride_bn,
+                      int64_t stride_cm, int64_t stride_cn,
+                      int in_dtype, int out_dtype,
+                      const float* a_scale, const float* b_scale,
+                      int activation, int splits, void* workspace, size_t workspace_bytes, void* stream);
 
 /* mi355_gemm with a stream-K schedule: one program per CU, and the programs split ALL K steps of ALL
  * 256x256 tiles evenly, so a tile count that is not a multiple of the CU count (or smaller than it:

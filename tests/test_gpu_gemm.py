@@ -1185,3 +1185,74 @@ def test_skinny_kernel_with_64_columns_per_workgroup_is_bit_exact(gpu, dtype, sh
     assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32")), (dtype, shape)
     got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32, add=td))
     assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32") + d), (dtype, shape, "addend")
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3"])
+@pytest.mark.parametrize("splits", [0, 2, 3, 7, 32])
+def test_split_k_is_bit_exact_on_integers(gpu, dtype, splits):
+    # mi355_gemm_splitk through the C ABI: `splits` workgroups per 128x128 tile, fp32 partial tiles in the workspace,
+    # a second launch adds them in split order and does the epilogue.  Integer data: every partial sum is exact, so
+    # any split gives the bits of the closed form.  Shapes: partial tiles on both sides, a K that is not a multiple
+    # of the split, a K with a tail below one 64-byte step, one tile only; both layouts of B; a strided C.
+    lib = _lib.load()
+    rng = np.random.default_rng(23 + splits)
+    abi = {"fp16": _lib.F16, "bf16": _lib.BF16, "e4m3": _lib.F8E4M3}[dtype]
+    for (M, N, K) in [(256, 256, 4096), (130, 96, 8192), (384, 200, 2096), (128, 128, 16384), (512, 640, 1056)]:
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        ref = gemm.matmul_closed_form(a, b, out_dtype="fp32")
+        if dtype == "e4m3":
+            ta = torch.from_numpy(formats.encode_fp8(a, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+            tbs = [torch.from_numpy(formats.encode_fp8(np.ascontiguousarray(b.T), "e4m3")).to(gpu).view(torch.float8_e4m3fn).t()]
+            if N % 16 == 0:
+                tbs.append(torch.from_numpy(formats.encode_fp8(b, "e4m3")).to(gpu).view(torch.float8_e4m3fn))
+        else:
+            ta = from_np(a, dtype, gpu)
+            tbs = [from_np(np.ascontiguousarray(b.T), dtype, gpu).t()]
+            if N % 8 == 0:
+                tbs.append(from_np(b, dtype, gpu))
+        ws = torch.full((32 * M * N,), float("nan"), dtype=torch.float32, device=gpu)   # (contents must not matter)
+        for tb in tbs:
+            cbuf = torch.full((M, N + 5), 7.0, dtype=torch.float32, device=gpu)
+            c = cbuf[:, :N]
+            rc = lib.mi355_gemm_splitk(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), M, N, K, ta.stride(0), ta.stride(1),
+                                       tb.stride(0), tb.stride(1), c.stride(0), c.stride(1), abi, _lib.F32, None, None,
+                                       _lib.ACT_NONE, splits, ws.data_ptr(), ws.numel() * 4, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, (rc, dtype, splits, M, N, K)
+            assert bits_equal(to_np(c), ref), (dtype, splits, M, N, K, tb.stride())
+            assert bool((cbuf[:, N:] == 7.0).all())
+
+
+def test_split_k_epilogue_and_the_route_from_matmul(gpu, monkeypatch):
+    # the epilogue of the second launch (scales, leaky_relu, one rounding to the output type) against the closed form,
+    # and matmul() itself: with the split switched off it must give the same bits on integers and agree to 1e-2 on
+    # random data; a workspace that is too small is refused before any launch
+    lib = _lib.load()
+    rng = np.random.default_rng(5)
+    M, N, K = 256, 384, 8192
+    a, b = randn_rounded(rng, (M, K), "bf16"), randn_rounded(rng, (K, N), "bf16")
+    ta, tb = from_np(a, "bf16", gpu), from_np(b, "bf16", gpu)
+    ref = gemm.matmul_closed_form(a, b, out_dtype="bf16", activation="leaky_relu")
+    got = to_np(triton_amd.matmul(ta, tb, activation="leaky_relu"))
+    assert np.allclose(got, ref, rtol=1e-2, atol=1e-2)
+    set_knob(monkeypatch, "MI355_GEMM_SPLITK", "0")
+    plain = to_np(triton_amd.matmul(ta, tb, activation="leaky_relu"))
+    assert np.allclose(plain, ref, rtol=1e-2, atol=1e-2)
+    monkeypatch.delenv("MI355_GEMM_SPLITK")
+    ai = rng.integers(-3, 4, size=(M, K)).astype(np.float32)
+    bi = rng.integers(-3, 4, size=(K, N)).astype(np.float32)
+    tai, tbi = from_np(ai, "fp16", gpu), from_np(bi, "fp16", gpu)
+    refi = gemm.matmul_closed_form(ai, bi, out_dtype="fp32")
+    assert bits_equal(to_np(triton_amd.matmul(tai, tbi, out_dtype=torch.float32)), refi)
+    # fp8 with per-tensor scales and an fp8 output: the scales multiply the sum of the slices once
+    qa = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    qb = rng.integers(-2, 3, size=(N, K)).astype(np.float32)
+    tqa = torch.from_numpy(formats.encode_fp8(qa, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+    tqb = torch.from_numpy(formats.encode_fp8(qb, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+    got8 = to_np(triton_amd.matmul(tqa, tqb.t(), a_scale=0.5, b_scale=0.25, out_dtype=torch.bfloat16))
+    assert bits_equal(got8, formats.round_to((qa @ qb.T) * 0.125, "bf16"))
+    c = torch.empty((M, N), dtype=torch.bfloat16, device=gpu)
+    ws = torch.empty(M * N, dtype=torch.float32, device=gpu)
+    rc = lib.mi355_gemm_splitk(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), M, N, K, K, 1, N, 1, N, 1, _lib.BF16, _lib.BF16,
+                               None, None, _lib.ACT_NONE, 4, ws.data_ptr(), ws.numel() * 4, torch.cuda.current_stream().cuda_stream)
+    assert rc == -1   # MI355_EINVAL

@@ -24,7 +24,7 @@ Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORK
 I64x4 = c_int64 * 4
 
 # MI355_ABI_VERSION of include/mi355_kernels.h that this binding was written for
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 # name -> (restype, argtypes); kept in one table so tests can check it against the header
 SIGNATURES = {
@@ -34,6 +34,9 @@ SIGNATURES = {
     "mi355_gemm_tuned": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                  c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "mi355_gemm_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                  c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
+                                  c_int, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p, c_size_t, c_void_p]),
     "mi355_gemm_streamk": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                    c_int64, c_int64, c_int64, c_int64, c_int64, c_int64,
                                    c_int, c_int, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p]),

@@ -388,6 +388,52 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C, int M, int N, int K,
                    activation, nullptr, 0, 0, 0, tile, group_m, stream_);
 }
 
+int mi355_gemm_splitk(const void* A, const void* B, void* C, int M, int N, int K,
+                      int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
+                      int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,
+                      int activation, int splits, void* workspace, size_t workspace_bytes, void* stream_) {
+  if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0 || splits < 0) return MI355_EINVAL;
+  if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
+  if (in_dtype < MI355_F16 || in_dtype > MI355_F8E5M2) return MI355_EDTYPE;
+  if (out_dtype < MI355_F16 || out_dtype > MI355_F32) return MI355_EDTYPE;
+  if (!device_info().gfx950) return MI355_EDEVICE;
+  const int es = elem_size(in_dtype), vec = 16 / es;
+  // what the tile kernels ask of the operands (as in mi355_gemm); anything else, or nothing to split: the plain call
+  const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
+  const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
+  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
+  const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
+  const int64_t k_bytes = (int64_t)K * es;
+  const int ksteps = (int)((k_bytes + 63) / 64);
+  const int cus = device_info().cus > 0 ? device_info().cus : 256;
+  if (splits == 0) {
+    // a workgroup per CU, at least sixteen K steps each, at most 32 slices to add up; nothing to gain from half a round
+    // of tiles on or below 64 K steps (measured: see ops.py::_splitk_splits)
+    const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    splits = tiles * 2 > cus || ksteps < 64 ? 1 : (int)std::min<long>(std::min<long>(cus / tiles, ksteps / 16), 32);
+  }
+  const int per = splits >= 2 ? (ksteps + splits - 1) / splits : ksteps;
+  const int used = (ksteps + per - 1) / per;   // (no split is left empty)
+  if (!(a_ok && (b_kmajor || b_nmajor) && pitch_ok) || used < 2 || knob(knobs().force_strided, 0) != 0)
+    return mi355_gemm(A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, in_dtype, out_dtype, a_scale, b_scale, activation, stream_);
+  if (!workspace || !aligned(workspace, 16) || workspace_bytes < (size_t)used * M * N * sizeof(float)) return MI355_EINVAL;
+  hipStream_t stream = (hipStream_t)stream_;
+  GemmArgs p{};
+  p.A = (const char*)A; p.B = (const char*)B; p.C = (char*)C;
+  p.M = M; p.N = N; p.K = K; p.k_bytes = (int)k_bytes;
+  p.lda = sam * es;
+  p.ldb = (b_kmajor ? sbn : sbk) * es;
+  p.group_m = knob(knobs().group_m, 8);
+  p.workspace = (float*)workspace;
+  const int rc = es == 1 ? gemm8_splitk_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, used, per * 64, stream)
+                         : gemm16_splitk_launch(p, in_dtype == MI355_BF16, b_kmajor, used, per * 64, stream);
+  if (rc != 0) return rc;
+  GemmStridedArgs out{};
+  out.C = C; out.M = M; out.N = N; out.scm = scm; out.scn = scn;
+  out.a_scale = a_scale; out.b_scale = b_scale; out.activation = activation; out.out_dtype = out_dtype;
+  return splitk_reduce_launch(out, (const float*)workspace, used, stream);
+}
+
 int mi355_gemm_streamk(const void* A, const void* B, void* C, int M, int N, int K,
                        int64_t sam, int64_t sak, int64_t sbk, int64_t sbn, int64_t scm, int64_t scn,
                        int in_dtype, int out_dtype, const float* a_scale, const float* b_scale,

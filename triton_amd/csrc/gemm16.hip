@@ -29,6 +29,15 @@ int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStre
                   : launch_gemm_tile<Cfg16<f16x8>, false>(p, tile, stream);
 }
 
+int gemm16_splitk_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream) {
+  if (bf16) {
+    return b_kmajor ? launch_gemm_splitk<Cfg16<bf16x8>, true>(p, splits, chunk_bytes, stream)
+                    : launch_gemm_splitk<Cfg16<bf16x8>, false>(p, splits, chunk_bytes, stream);
+  }
+  return b_kmajor ? launch_gemm_splitk<Cfg16<f16x8>, true>(p, splits, chunk_bytes, stream)
+                  : launch_gemm_splitk<Cfg16<f16x8>, false>(p, splits, chunk_bytes, stream);
+}
+
 int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream) {
   return bf16 ? launch_gemm_grouped<Cfg16<bf16x8>, __bf16>(ga, nprog, nprog_big, stream)
               : launch_gemm_grouped<Cfg16<f16x8>, _Float16>(ga, nprog, nprog_big, stream);

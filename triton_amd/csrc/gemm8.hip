@@ -137,4 +137,9 @@ int gemm8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int tile, hipStrea
   return e5m2 ? launch_gemm_tile<Cfg8<1>, true>(p, tile, stream) : launch_gemm_tile<Cfg8<0>, true>(p, tile, stream);
 }
 
+int gemm8_splitk_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream) {
+  if (b_kmajor) return e5m2 ? launch_gemm_splitk<Cfg8<1>, true>(p, splits, chunk_bytes, stream) : launch_gemm_splitk<Cfg8<0>, true>(p, splits, chunk_bytes, stream);
+  return e5m2 ? launch_gemm_splitk<Cfg8<1>, false>(p, splits, chunk_bytes, stream) : launch_gemm_splitk<Cfg8<0>, false>(p, splits, chunk_bytes, stream);
+}
+
 }  // namespace mi355

@@ -502,6 +502,47 @@ __global__ __launch_bounds__(WM * WN * 64, 1) void gemm_kernel(GemmArgs p) {
   gemm_tile_body<Cfg, BM, BN, WM, WN, B_KMAJOR, NS>(p, pm, pn, (LDS_PTR(char))smem);
 }
 
+// Split-K for products of few tiles with a long K (one row of tiles against a long weight, a small square against a
+// long K): workgroup z * tiles + t multiplies the K bytes [z * chunk, z * chunk + chunk) of tile t and leaves the fp32
+// partial tile in slice z of the workspace ([splits][M][N] floats); splitk_reduce_kernel adds the slices and does the
+// epilogue.  The one-workgroup-per-tile kernel keeps two to four K steps of loads in flight per workgroup, which with
+// a handful of workgroups is a small fraction of what the memory system needs to be busy.
+template <typename Cfg, int BM, int BN, int WM, int WN, bool B_KMAJOR, int NS>
+__global__ __launch_bounds__(WM * WN * 64, 1) void gemm_splitk_kernel(GemmArgs p, int chunk_bytes) {
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int num_m = (p.M + BM - 1) / BM, num_n = (p.N + BN - 1) / BN, tiles = num_m * num_n;
+  const int z = blockIdx.x / tiles;
+  int pm, pn;
+  grouped_tile(xcd_remap(blockIdx.x % tiles, tiles), num_m, num_n, p.group_m, pm, pn);
+  GemmArgs q = p;
+  const int k0 = z * chunk_bytes;
+  q.k_bytes = p.k_bytes - k0 < chunk_bytes ? p.k_bytes - k0 : chunk_bytes;   // (the host leaves no split empty)
+  q.K = q.k_bytes / Cfg::kElemBytes;
+  q.A = p.A + k0;
+  q.B = B_KMAJOR ? p.B + k0 : p.B + (int64_t)(k0 / Cfg::kElemBytes) * p.ldb;
+  q.C = (char*)(p.workspace + (int64_t)z * p.M * p.N);
+  q.ldc = p.N; q.scn = 1; q.out_dtype = 4;   // fp32 partial sums, dense rows
+  q.c_vec_ok = p.N % 4 == 0;                 // (the workspace is 16-byte aligned)
+  q.a_scale = nullptr; q.b_scale = nullptr; q.activation = 0; q.aux = nullptr;
+  gemm_tile_body<Cfg, BM, BN, WM, WN, B_KMAJOR, NS>(q, pm, pn, (LDS_PTR(char))smem);
+}
+
+template <typename Cfg, bool B_KMAJOR>
+static int launch_gemm_splitk(const GemmArgs& p, int splits, int chunk_bytes, hipStream_t stream) {
+  constexpr int BM = 128, BN = 128, NS = 4;
+  constexpr int smem = NS * (BM + BN) * RBK;
+  static bool attr_set = false;
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute((const void*)gemm_splitk_kernel<Cfg, BM, BN, 2, 2, B_KMAJOR, NS>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return (int)e;
+    attr_set = true;
+  }
+  const int tiles = ((p.M + BM - 1) / BM) * ((p.N + BN - 1) / BN);
+  gemm_splitk_kernel<Cfg, BM, BN, 2, 2, B_KMAJOR, NS><<<dim3(tiles * splits), dim3(256), smem, stream>>>(p, chunk_bytes);
+  return (int)hipGetLastError();
+}
+
 // ---------------------------------------------------------------------------------------------
 // Grouped GEMM: a fixed number of workgroups walks the tiles of `group_size` independent
 // problems C_g = A_g @ B_g, whose pointers, sizes and leading dimensions live in device arrays -

@@ -109,6 +109,11 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int tile, hipStream_t stream);
+// split-K on 128x128 tiles: `splits` chunks of `chunk_bytes` of every operand row (whole K steps of 64 bytes), fp32
+// partial tiles into p.workspace ([splits][M][N]); splitk_reduce_launch adds them up and does the epilogue
+int gemm16_splitk_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream);
+int gemm8_splitk_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream);
+int splitk_reduce_launch(const GemmStridedArgs& out, const float* workspace, int splits, hipStream_t stream);   // A, B, K, in_dtype of `out` unused
 bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int tile_m = 192);   // the same for tiles of 192 x 256 / 128 x 256
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype);
 bool gemm_wave128_f8_ok(const GemmArgs& p, bool b_kmajor);

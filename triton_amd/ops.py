@@ -10,6 +10,8 @@ and device (the duck typing of the reference launcher, third_party/amd/backend/d
 """
 from __future__ import annotations
 
+import os
+
 import math
 
 import torch
@@ -88,6 +90,34 @@ def _scale_ptr(s, device):
     return s.data_ptr(), s
 
 
+_cu_count = {}   # device index -> compute units
+
+
+def _splitk_splits(device, M, N, k_bytes):
+    """Number of K splits for `matmul` (0 = none): products with less than half a round of 128x128 tiles and a long K
+    give every tile to several workgroups (`mi355_gemm_splitk`) - one workgroup per CU, at least sixteen 64-byte K steps
+    each, at most 32 slices and 64 MiB of fp32 partial sums.  Shapes with at most 64 rows on a side (and up to 128
+    against a long other side) stay with the streaming kernels."""
+    if os.environ.get("MI355_GEMM_SPLITK", "1") == "0":
+        return 0
+    small, large = min(M, N), max(M, N)
+    if small <= 64 or (small <= 128 and large >= 2048):
+        return 0
+    idx = device.index if device.index is not None else torch.cuda.current_device()
+    cus = _cu_count.get(idx)
+    if cus is None:
+        cus = _cu_count[idx] = max(1, _lib.load().mi355_query(_lib.Q_CU_COUNT))
+    tiles = -(-M // 128) * -(-N // 128)
+    ksteps = -(-k_bytes // 64)
+    if tiles * 2 > cus or ksteps < 64:
+        return 0
+    # one workgroup per CU, at least 16 K steps each (flushed do_bench, bf16, us by number of splits - 1 / 2 / 4 / 8 / 16 /
+    # 32: 256 x 256 x 4096 51 / 34 / 24 / 20 / 19 / 23, 1024 x 1024 x 4096 52 / 38 / 30 / 36 / 49 / 71, 256 x 8192 x 8192 117 / 81 / 89 /
+    # 99 / 122 / 189, 256 x 1024 x 8192 97 / 59 / 39 / 28 / 27 / 35; 1024^3, 32 steps: 18 / 21 / 23 - not split)
+    splits = min(cus // tiles, ksteps // 16, 32, (64 << 20) // (4 * M * N))
+    return splits if splits >= 2 else 0
+
+
 def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, add=None, softmax=False):
     """C = softmax_rows?(act((a_scale*b_scale) * A @ B + add)) with fp32 accumulation.
 
@@ -151,6 +181,19 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
     stream = _stream()
     md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K_caller, _ELEM_BYTES[in_dt]))
+    if add is None and not softmax and in_dt != _lib.F32 and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
+        splits = _splitk_splits(device, M, N, K * _ELEM_BYTES[in_dt])
+        if splits:
+            # few tiles, long K: every tile's K range is shared out (the fp32 partial sums live in a buffer from
+            # torch's caching allocator, which orders its reuse on this stream)
+            ws = torch.empty(splits * M * N, dtype=torch.float32, device=device)
+            rc = _lib.load().mi355_gemm_splitk(
+                a.data_ptr(), b.data_ptr(), c.data_ptr(), M, N, K,
+                a.stride(0), a.stride(1), b.stride(0), b.stride(1), c.stride(0), c.stride(1),
+                in_dt, _TORCH_TO_ABI[out_dtype], pa, pb, act, splits, ws.data_ptr(), ws.numel() * 4, stream)
+            _lib.check(rc, "mi355_gemm_splitk")
+            hooks.exit(md)
+            return c
     ext = _lib.ext()
     if ext is not None and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
         # the PyTorch-ROCm extension: tensors in, torch's current stream taken in C++, one C-ABI call
