@@ -3,7 +3,8 @@
 `warmup` / `rep` milliseconds worth of calls, every timed call preceded by a write over a buffer
 larger than the last-level cache and bracketed by its own pair of device events.
 
-`do_bench` keeps the reference's signature, defaults and return conventions.  The flush buffer is 512 MB here:
+`do_bench` keeps the reference's signature, defaults and return conventions; `do_bench_cudagraph`
+(python/triton/testing.py:19-82) is the same measurement from inside a captured HIP graph.  The flush buffer is 512 MB here:
 MI355X's memory-side cache holds 256 MB, the size the reference clears.
 
 `Benchmark`, `perf_report` and `Mark.run` (python/triton/testing.py:214-388) are the sweep harness that the
@@ -71,6 +72,55 @@ def do_bench(fn, warmup=25, rep=100, grad_to_none=None, quantiles=None, fast_flu
     if quantiles is not None:
         out = torch.quantile(times, torch.tensor(quantiles, dtype=torch.float)).tolist()
         return out[0] if len(out) == 1 else out
+    return getattr(torch, return_mode)(times).item()
+
+
+def do_bench_cudagraph(fn, rep=20, grad_to_none=None, return_mode="mean"):
+    """`do_bench` without host overhead between the calls (python/triton/testing.py:19-82, same signature and protocol):
+    `fn` is captured into a HIP graph, first once for an estimate, then `rep` ms worth of calls unrolled in one graph,
+    which is replayed ten times; the result is the time per call in ms over those replays (`return_mode`).  No cache
+    flush between the calls.  Must run on a side stream, like the reference's (a capture on the default stream is
+    refused); `fn` has been called once outside any capture before the first one, so first-call set-up never lands in
+    a graph.  The operators of this package record kernels only (no runtime allocation or memset inside the library)."""
+    assert return_mode in _RETURN_MODES
+    import torch
+
+    if torch.cuda.current_stream() == torch.cuda.default_stream():
+        raise RuntimeError("Cannot capture graph in default stream. Please use side stream in benchmark code.")
+
+    def reset_grads():
+        if grad_to_none is not None:
+            for x in grad_to_none:
+                x.grad = None
+
+    def capture(calls):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for _ in range(calls):
+                reset_grads()
+                fn()
+        torch.cuda.synchronize()
+        return graph
+
+    def replay_ms(graph):
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        graph.replay()
+        end.record()
+        torch.cuda.synchronize()
+        return begin.elapsed_time(end)
+
+    fn()
+    torch.cuda.synchronize()
+    if grad_to_none is not None:
+        for x in grad_to_none:
+            x.detach_()
+            x.requires_grad_(True)
+            x.grad = None
+    estimate_ms = replay_ms(capture(1))
+    n_repeat = max(1, int(rep / estimate_ms))
+    graph = capture(n_repeat)
+    times = torch.tensor([replay_ms(graph) / n_repeat for _ in range(10)], dtype=torch.float)
     return getattr(torch, return_mode)(times).item()
 
 
