@@ -1256,3 +1256,38 @@ def test_split_k_epilogue_and_the_route_from_matmul(gpu, monkeypatch):
     rc = lib.mi355_gemm_splitk(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), M, N, K, K, 1, N, 1, N, 1, _lib.BF16, _lib.BF16,
                                None, None, _lib.ACT_NONE, 4, ws.data_ptr(), ws.numel() * 4, torch.cuda.current_stream().cuda_stream)
     assert rc == -1   # MI355_EINVAL
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3"])
+def test_random_shapes_through_the_default_dispatch_are_bit_exact(gpu, dtype):
+    # Whatever kernel the size heuristics pick - four-wave tiles of three heights, two heights in one launch, 128x128
+    # tiles, split-K, skinny, masked, padded pitches - the product of small integers has exactly representable partial
+    # sums, so the result must be the closed form's bits (rounded once where the output is 16-bit).  Seeded shapes
+    # around the heuristics' thresholds: multiples of 64 .. 256 with and without a ragged remainder, both B layouts.
+    rng = np.random.default_rng({"fp16": 101, "bf16": 202, "e4m3": 303}[dtype])
+    base = [64, 128, 192, 256, 320, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2304, 2560, 3072]
+    ks = [64, 128, 256, 320, 512, 1024, 1040, 2048, 4096, 8192]
+    for case in range(26):
+        M = int(rng.choice(base)) + int(rng.choice([0, 0, 0, 8, -8, 16, 1]))
+        N = int(rng.choice(base)) + int(rng.choice([0, 0, 0, 8, -8, 16, 3]))
+        K = int(rng.choice(ks)) + int(rng.choice([0, 0, 0, 8, 16, -16]))
+        if M * N * K > 3072 * 3072 * 2048:   # (keeps the numpy reference to a fraction of a second per case)
+            K = max(64, (3072 * 3072 * 2048 // (M * N)) // 64 * 64)
+        kmajor = bool(rng.integers(0, 2))
+        a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
+        exact = a @ b                          # fp32 sums of integers below 2^24: exact in any order
+        if dtype == "e4m3":
+            ta = torch.from_numpy(formats.encode_fp8(a, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+            if kmajor:
+                tb = torch.from_numpy(formats.encode_fp8(np.ascontiguousarray(b.T), "e4m3")).to(gpu).view(torch.float8_e4m3fn).t()
+            else:
+                tb = torch.from_numpy(formats.encode_fp8(b, "e4m3")).to(gpu).view(torch.float8_e4m3fn)
+            out = [torch.float32, torch.bfloat16, torch.float16][case % 3]
+        else:
+            ta = from_np(a, dtype, gpu)
+            tb = from_np(np.ascontiguousarray(b.T), dtype, gpu).t() if kmajor else from_np(b, dtype, gpu)
+            out = [torch.float32, None][case % 2]
+        got = triton_amd.matmul(ta, tb) if out is None else triton_amd.matmul(ta, tb, out_dtype=out)
+        name = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16", None: dtype}[out]
+        assert bits_equal(to_np(got), formats.round_to(exact, name)), (dtype, case, M, N, K, kmajor, name)
