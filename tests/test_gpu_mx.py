@@ -275,3 +275,33 @@ def test_mxfp8_with_freshly_uploaded_operands_is_bit_exact_every_time(gpu, monke
         if len(churn) > 8:
             churn.pop(0)
         assert bits_equal(_run(gpu, a, sa, b, sb, "mxfp8", torch.float32), ref), rep
+
+
+@pytest.mark.parametrize("fmt", ["mxfp4", "mxfp8"])
+def test_random_shapes_through_the_default_dispatch_are_bit_exact(gpu, fmt):
+    # Whatever kernel the size heuristics pick (four-wave tiles of three heights, two heights in one launch, their K
+    # tails, the eight-wave kernels, partial tiles): exact data - fp4 values or small integers as e4m3, scales 1/2, 1,
+    # 2 - make every partial sum exact in fp32, so the results carry the oracle's bits.  Seeded shapes around the
+    # thresholds of the heuristics.
+    rng = np.random.default_rng({"mxfp4": 11, "mxfp8": 12}[fmt])
+    base = [64, 128, 192, 256, 384, 512, 768, 1024, 1280, 1536, 2048, 2304, 2560, 3072]
+    ks = [32, 64, 256, 512, 1024, 1056, 2048, 2048 + 480, 4096]
+    t = lambda x: torch.from_numpy(x).to(gpu)
+    for case in range(22):
+        M = int(rng.choice(base)) + int(rng.choice([0, 0, 0, 8, -8, 1]))
+        N = int(rng.choice(base)) + int(rng.choice([0, 0, 0, 16, -8, 3]))
+        K = int(rng.choice(ks))
+        if M * N * K > 2560 * 2560 * 2048:   # (keeps the numpy oracle to about a second per case)
+            K = max(32, (2560 * 2560 * 2048 // (M * N)) // 32 * 32)
+        if fmt == "mxfp4":
+            a, sa, b, sb = _operands(rng, M, N, K, fmt, lo=126, hi=129)
+        else:
+            a = formats.encode_fp8(rng.integers(-4, 5, size=(M, K)).astype(np.float32), "e4m3")
+            b = formats.encode_fp8(rng.integers(-4, 5, size=(N, K)).astype(np.float32), "e4m3")
+            sa = rng.integers(126, 129, size=(M, K // 32)).astype(np.uint8)
+            sb = rng.integers(126, 129, size=(N, K // 32)).astype(np.uint8)
+        ref32 = mx.mx_matmul(a, sa, b, sb, fmt, out_dtype="fp32")
+        out = [torch.bfloat16, torch.float32, torch.float16][case % 3]
+        got = to_np(triton_amd.mx_matmul(t(a), t(sa), t(b), t(sb), fmt, out_dtype=out))
+        name = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16"}[out]
+        assert bits_equal(got, formats.round_to(ref32, name)), (fmt, case, M, N, K, name)
