@@ -91,4 +91,4 @@ def test_do_bench_cudagraph_times_a_captured_call(gpu):
     torch.cuda.current_stream().wait_stream(side)
     ms_events = do_bench(fn, warmup=5, rep=20, return_mode="median")
     print(f"4096^3 bf16: {ms_graph:.4f} ms per call inside a graph, {ms_events:.4f} ms flushed with events")
-    assert 0.05 < ms_graph < 1.0 and 0.5 < ms_graph / ms_events < 1.5
+    assert 0.05 < ms_graph < 1.0 and 0.3 < ms_graph / ms_events < 2.0
