@@ -20,7 +20,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 # dense MFMA peaks of MI355X in TFLOP/s (published, without sparsity) and HBM3E bandwidth in GB/s
-PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4": 10100.0}
+PEAK = {"bf16": 2500.0, "fp16": 2500.0, "fp8": 5000.0, "mxfp8": 5000.0, "mxfp4": 10100.0, "fp32": 157.3}
 HBM_GBPS = 8000.0
 
 # HBM-side bytes per launch of the 8192^3 bf16 GEMM kernel.  NOT read in this run (hardware counters need
@@ -262,6 +262,21 @@ def secondary_workloads(lib, dev, n):
         fn = lambda: triton_amd.matmul(a8, b8.t(), out_dtype=torch.bfloat16, a_scale=sa8, b_scale=sb8)
         return fn, flops, "flops", {"peak": "fp8", "clock": True, "data": "N(0,1) scaled to amax 448, e4m3fn, per-tensor fp32 scales"}, 60
     W["fp8_e4m3_gemm_8192"] = fp8_gemm
+
+    # fp32 operands on the fp32 MFMAs (the `ieee` precision of `tl.dot`): N(0, 1), K-major B as the kernel takes it,
+    # fp32 out; 7 ms per launch, so a handful of launches
+    def fp32_gemm():
+        a32 = torch.randn(n, n, device=dev)
+        b32 = torch.randn(n, n, device=dev)      # [N, K]: b32.t() is the K-major [K, N] operand
+        c32 = torch.empty(n, n, device=dev)
+
+        def fn():
+            rc = lib.mi355_gemm(a32.data_ptr(), b32.data_ptr(), c32.data_ptr(), n, n, n, n, 1, 1, n, n, 1,
+                                _lib.F32, _lib.F32, None, None, 0, stream)
+            assert rc == 0, rc
+
+        return fn, flops, "flops", {"peak": "fp32", "data": "N(0,1) fp32, K-major B, fp32 out"}, 8
+    W["fp32_gemm_8192"] = fp32_gemm
 
     def fp8_decode():
         b8, _ = quantize_e4m3(torch.randn(n, n, device=dev))

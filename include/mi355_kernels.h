@@ -28,8 +28,8 @@
  * of the MFMA epilogues; 3: MFMA burn probe with its block-scaled shapes, per-device properties, fp8 attention forward at
  * head dims 16 / 32 / 256, a row-major fp8 B on the MFMA kernels, block-scaled products with any K that is a multiple of
  * 32 and scale rows of any pitch on the MFMA kernels; 4: mi355_gemm_splitk, a row-major B whose N is not a multiple of
- * 16 bytes inside a padded pitch on the tile kernels.) */
-#define MI355_ABI_VERSION 4
+ * 16 bytes inside a padded pitch on the tile kernels; 5: fp32 operands in mi355_gemm.) */
+#define MI355_ABI_VERSION 5
 
 #ifdef __cplusplus
 extern "C" {
@@ -41,7 +41,7 @@ enum {
   MI355_BF16 = 1,   /* bf16                        */
   MI355_F8E4M3 = 2, /* fp8e4nv  (OCP e4m3fn)       */
   MI355_F8E5M2 = 3, /* fp8e5    (OCP e5m2)         */
-  MI355_F32 = 4     /* fp32 (output only)          */
+  MI355_F32 = 4     /* fp32 (outputs; operands of mi355_gemm / _tuned / _epilogue) */
 };
 
 /* MX element formats for mi355_mx_gemm */
@@ -94,7 +94,10 @@ enum {
  * the tiled MFMA kernels need a unit stride on one axis of each operand and rows that start on 16-byte boundaries -
  * either layout of B for every type; K a multiple of 16 bytes, N any size when a row-major B's pitch covers N rounded up
  * to 16 bytes -, anything else runs a slower MFMA kernel of 64x64 tiles with masked element loads), plus ACTIVATION.  in_dtype is the type of A and B
- * (they must match, python/triton/language/semantic.py:1355).  a_scale / b_scale are
+ * (they must match, python/triton/language/semantic.py:1355): fp16, bf16, fp8e4nv, fp8e5 or fp32.  fp32 operands are
+ * multiplied exactly on the fp32 MFMAs (the `ieee` input precision of `tl.dot`, semantic.py:1322-1410; what the
+ * reference's CPU path computes, python/triton/runtime/interpreter.py:542-549) when A's rows and B's columns are
+ * K-contiguous and start on 16-byte boundaries with K a multiple of 4, and by an fp32 FMA kernel otherwise.  a_scale / b_scale are
  * optional device pointers to one fp32 each (NULL = 1.0): per-tensor dequantisation
  * scales for fp8 inputs, applied to the fp32 accumulator before activation and cast.
  */

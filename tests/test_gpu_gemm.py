@@ -1258,13 +1258,13 @@ def test_split_k_epilogue_and_the_route_from_matmul(gpu, monkeypatch):
     assert rc == -1   # MI355_EINVAL
 
 
-@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3"])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3", "fp32"])
 def test_random_shapes_through_the_default_dispatch_are_bit_exact(gpu, dtype):
     # Whatever kernel the size heuristics pick - four-wave tiles of three heights, two heights in one launch, 128x128
     # tiles, split-K, skinny, masked, padded pitches - the product of small integers has exactly representable partial
     # sums, so the result must be the closed form's bits (rounded once where the output is 16-bit).  Seeded shapes
     # around the heuristics' thresholds: multiples of 64 .. 256 with and without a ragged remainder, both B layouts.
-    rng = np.random.default_rng({"fp16": 101, "bf16": 202, "e4m3": 303}[dtype])
+    rng = np.random.default_rng({"fp16": 101, "bf16": 202, "e4m3": 303, "fp32": 404}[dtype])
     base = [64, 128, 192, 256, 320, 384, 512, 640, 768, 1024, 1280, 1536, 2048, 2304, 2560, 3072]
     ks = [64, 128, 256, 320, 512, 1024, 1040, 2048, 4096, 8192]
     for case in range(26):
@@ -1289,5 +1289,67 @@ def test_random_shapes_through_the_default_dispatch_are_bit_exact(gpu, dtype):
             tb = from_np(np.ascontiguousarray(b.T), dtype, gpu).t() if kmajor else from_np(b, dtype, gpu)
             out = [torch.float32, None][case % 2]
         got = triton_amd.matmul(ta, tb) if out is None else triton_amd.matmul(ta, tb, out_dtype=out)
-        name = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16", None: dtype}[out]
+        name = {torch.float32: "fp32", torch.bfloat16: "bf16", torch.float16: "fp16", None: "fp16" if dtype == "fp32" else dtype}[out]
         assert bits_equal(to_np(got), formats.round_to(exact, name)), (dtype, case, M, N, K, kmajor, name)
+
+
+@pytest.mark.parametrize("kmajor", [True, False])
+def test_fp32_operands_are_multiplied_exactly(gpu, kmajor):
+    # fp32 inputs: `tl.dot` of fp32 blocks accumulates exact fp32 products in fp32 (the interpreter's np.matmul in fp32,
+    # python/triton/runtime/interpreter.py:542-549).  Integers beyond what any 16-bit type holds (|x| <= 3000, so a
+    # detour through fp16 / bf16 would show) with sums that stay below 2^24: the result is the closed form's bits,
+    # on the MFMA tiles (K-major B through the C ABI, a row-major B through the wrapper's transposing copy), on the
+    # any-stride kernel (small products, K not a multiple of 4, a row-major B through the C ABI) and for every output
+    # type; then N(0,1) data against the fp64 product at fp32 accuracy.
+    lib = _lib.load()
+    rng = np.random.default_rng(41 + kmajor)
+    for (M, N, K) in [(256, 256, 64), (128, 128, 16), (300, 200, 72), (512, 384, 130), (2048, 2048, 256), (1024, 3072, 512), (64, 64, 4)]:
+        a = rng.integers(-3000, 3001, size=(M, K)).astype(np.float32)
+        b = rng.integers(-1, 2, size=(K, N)).astype(np.float32)
+        ref = a.astype(np.float64) @ b.astype(np.float64)
+        assert np.abs(ref).max() < 2 ** 24
+        ta = torch.from_numpy(a).to(gpu)
+        tb = torch.from_numpy(np.ascontiguousarray(b.T)).to(gpu).t() if kmajor else torch.from_numpy(b).to(gpu)
+        got = triton_amd.matmul(ta, tb, out_dtype=torch.float32)
+        assert bits_equal(to_np(got), ref.astype(np.float32)), (M, N, K, kmajor)
+        # the C ABI itself, with the strides as they are
+        c = torch.full((M, N + 3), 7.0, dtype=torch.float32, device=gpu)
+        cv = c[:, :N]
+        rc = lib.mi355_gemm(ta.data_ptr(), tb.data_ptr(), cv.data_ptr(), M, N, K, ta.stride(0), ta.stride(1), tb.stride(0), tb.stride(1),
+                            cv.stride(0), cv.stride(1), _lib.F32, _lib.F32, None, None, _lib.ACT_NONE, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0 and bits_equal(to_np(cv), ref.astype(np.float32)) and bool((c[:, N:] == 7.0).all()), (M, N, K, kmajor)
+    # the reference wrapper's own output type (03:338: fp16 whatever the inputs) and the activation
+    a = rng.integers(-8, 9, size=(384, 96)).astype(np.float32)
+    b = rng.integers(-8, 9, size=(96, 256)).astype(np.float32)
+    ta, tb = torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu)
+    got = triton_amd.matmul(ta, tb, activation="leaky_relu")
+    assert got.dtype == torch.float16
+    assert bits_equal(to_np(got), gemm.matmul_closed_form(a, b, activation="leaky_relu", out_dtype="fp16"))
+    # random data: fp32 products and sums against fp64
+    a = rng.normal(size=(1024, 2048)).astype(np.float32)
+    b = rng.normal(size=(2048, 768)).astype(np.float32)
+    ta = torch.from_numpy(a).to(gpu)
+    tb = torch.from_numpy(np.ascontiguousarray(b.T)).to(gpu).t() if kmajor else torch.from_numpy(b).to(gpu)
+    got = to_np(triton_amd.matmul(ta, tb, out_dtype=torch.float32))
+    ref = a.astype(np.float64) @ b.astype(np.float64)
+    err = report_error(f"fp32 1024 x 768 x 2048 kmajor={kmajor}", got, ref)
+    assert err < 1e-5
+    # every tile form of the fp32 kernel on whole and partial tiles, through mi355_gemm_tuned: the same bits on integers
+    a = rng.integers(-300, 301, size=(768, 264)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(264, 520)).astype(np.float32)
+    ta, tb = torch.from_numpy(a).to(gpu), torch.from_numpy(np.ascontiguousarray(b.T)).to(gpu).t()
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    for tile in (0, 1, 2, 3, 4, 5, 6):
+        c = torch.empty(768, 520, dtype=torch.float32, device=gpu)
+        rc = lib.mi355_gemm_tuned(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), 768, 520, 264, 264, 1, 1, 264, 520, 1, _lib.F32, _lib.F32,
+                                  None, None, _lib.ACT_NONE, tile, 8, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0 and bits_equal(to_np(c), ref), tile
+    a = rng.integers(-300, 301, size=(512, 1024)).astype(np.float32)
+    b = rng.integers(-2, 3, size=(1024, 768)).astype(np.float32)
+    ta, tb = torch.from_numpy(a).to(gpu), torch.from_numpy(np.ascontiguousarray(b.T)).to(gpu).t()
+    ref = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+    for tile in (2, 4, 5):   # (whole tiles and rings of K steps: the persistent form runs as such)
+        c = torch.empty(512, 768, dtype=torch.float32, device=gpu)
+        rc = lib.mi355_gemm_tuned(ta.data_ptr(), tb.data_ptr(), c.data_ptr(), 512, 768, 1024, 1024, 1, 1, 1024, 768, 1, _lib.F32, _lib.F32,
+                                  None, None, _lib.ACT_NONE, tile, 8, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0 and bits_equal(to_np(c), ref), tile

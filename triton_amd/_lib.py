@@ -24,7 +24,7 @@ Q_ABI_VERSION, Q_CU_COUNT, Q_IS_GFX950, Q_LDS_BYTES, Q_CLOCK_KHZ, Q_STREAMK_WORK
 I64x4 = c_int64 * 4
 
 # MI355_ABI_VERSION of include/mi355_kernels.h that this binding was written for
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 # name -> (restype, argtypes); kept in one table so tests can check it against the header
 SIGNATURES = {

@@ -187,11 +187,12 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0) return MI355_EINVAL;
   if (aux && aux_dtype != MI355_F16 && aux_dtype != MI355_BF16 && aux_dtype != MI355_F32) return MI355_EDTYPE;
   if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
-  if (in_dtype < MI355_F16 || in_dtype > MI355_F8E5M2) return MI355_EDTYPE;
+  if (in_dtype < MI355_F16 || in_dtype > MI355_F32) return MI355_EDTYPE;
   if (out_dtype < MI355_F16 || out_dtype > MI355_F32) return MI355_EDTYPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
   hipStream_t stream = (hipStream_t)stream_;
   const int es = elem_size(in_dtype);
+  const bool is32 = in_dtype == MI355_F32;   // fp32 operands: fp32 MFMAs with a K-major B, the any-stride FMA kernel otherwise
   const bool is8 = es == 1;
   const int vec = 16 / es;  // elements per 16-byte chunk
 
@@ -200,11 +201,16 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
   // (a row-major B: rows of whole 16-byte chunks - N itself need not be one: the last chunk of a row then reaches into
   // the padding that the pitch provides, and the columns beyond N are never stored)
-  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
+  const bool b_nmajor = !is32 && sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
   // the tile copies address 256 rows of an operand with 32-bit byte offsets from a 64-bit tile base
   const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
   const bool fast = pitch_ok && out_ok && a_ok && (b_kmajor || b_nmajor) && knob(knobs().force_strided, 0) == 0;
 
+  if (!fast && is32) {
+    GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype,
+                      aux, aux_sm, aux_sn, aux_dtype};
+    return gemm_strided_launch(s, stream);   // (the masked MFMA kernel converts to 16 bits on its way through LDS: not for fp32)
+  }
   if (!fast) {
     GemmStridedArgs s{A, B, C, M, N, K, sam, sak, sbk, sbn, scm, scn, a_scale, b_scale, activation, in_dtype, out_dtype,
                       aux, aux_sm, aux_sn, aux_dtype};
@@ -231,6 +237,18 @@ static int gemm_impl(const void* A, const void* B, void* C, int M, int N, int K,
   // 256x256 tiles once they fill half of the CUs, 128x128 tiles (two workgroups per CU) below that
   // (bf16, 144 tiles: 912 vs 651 TFLOP/s; 100 tiles: 654 vs 715)
   const long tiles256 = (long)((M + 255) / 256) * ((N + 255) / 256);
+  if (is32) {
+    p.num_programs = std::min(knob(knobs().programs, cus), cus);
+    // fp32 products are bound by the fp32 MFMA rate alone (1/16 of the bf16 rate on the same bytes), so what counts is
+    // how evenly the tiles fill the CUs: 256x256 tiles (pipelined kernel: 8192^3 152 TFLOP/s, 4096^3 149; one barrier per
+    // step 141 / 139) against 128x128 tiles, two workgroups per CU, at about 0.9 of that rate (137 / 135; 2048^3: 102
+    // against 36 for its 64 large tiles)
+    auto fill = [&](long t, long slots) { return (double)t / (double)(((t + slots - 1) / slots) * slots); };
+    const long tiles128 = (long)((M + 127) / 128) * ((N + 127) / 128);
+    const bool large = fill(tiles256, cus) >= 0.9 * fill(tiles128, 2 * cus);
+    const int t32 = tile_arg >= 0 ? tile_arg : knob(knobs().tile, large ? (tiles256 % cus == 0 ? 5 : 4) : 1);
+    return gemm32_launch(p, t32 == 6 || t32 == 7 ? 4 : t32, stream);   // (the four-wave 16x16 kernels and stream-K have no fp32 form)
+  }
   // large problems run the software-pipelined 8-wave kernel
   // (5 = the persistent form of the pipelined kernel; it falls back to 4 for edge tiles or a K tail)
   // persistent only when every program gets the same number of tiles: with a remainder the hardware's

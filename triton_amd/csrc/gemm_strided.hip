@@ -14,7 +14,8 @@ __device__ __forceinline__ float load_elem(const void* p, int64_t idx, int dtype
     case 0: return (float)((const _Float16*)p)[idx];
     case 1: return (float)((const __bf16*)p)[idx];
     case 2: return e4m3_to_f32(((const uint8_t*)p)[idx]);
-    default: return e5m2_to_f32(((const uint8_t*)p)[idx]);
+    case 3: return e5m2_to_f32(((const uint8_t*)p)[idx]);
+    default: return ((const float*)p)[idx];
   }
 }
 

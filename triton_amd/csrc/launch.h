@@ -109,6 +109,7 @@ int gemm_wave128_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, hip
 int gemm16_grouped_launch(const GroupedArgs& ga, bool bf16, int nprog, int nprog_big, hipStream_t stream);
 int gemm16_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int tile, hipStream_t stream);
 int gemm8_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int tile, hipStream_t stream);
+int gemm32_launch(const GemmArgs& p, int tile, hipStream_t stream);   // fp32 operands, K-major B; tile as for gemm16_launch
 // split-K on 128x128 tiles: `splits` chunks of `chunk_bytes` of every operand row (whole K steps of 64 bytes), fp32
 // partial tiles into p.workspace ([splits][M][N]); splitk_reduce_launch adds them up and does the epilogue
 int gemm16_splitk_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream);

@@ -124,7 +124,8 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     Same contract as the reference wrapper (03:330-348): A must be contiguous, B may have any
     strides (the reference passes `b.T` for fp8, 03:378-382), the result is fp16 for fp16 / fp8
     inputs.  Extensions, all keyword-only and defaulting to the reference behaviour: bf16
-    inputs give a bf16 result, `out_dtype` overrides the result type, `a_scale` / `b_scale`
+    inputs give a bf16 result, fp32 inputs (exact fp32 products on the fp32 MFMAs, the `ieee` precision of `tl.dot`) an
+    fp16 one like the reference's `c = accumulator.to(tl.float16)`, `out_dtype` overrides the result type, `a_scale` / `b_scale`
     are per-tensor fp32 dequantisation scales; `add` (fp16 / bf16 / fp32, broadcastable to
     [M, N]: a matrix, an [M, 1] column = the reference's add-rows, a [1, N] / [N] row = its
     add-cols) and `softmax` are the fused epilogues of the reference's dot test
@@ -166,6 +167,11 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
         else:
             b = torch.nn.functional.pad(as_bytes(b), (0, 0, 0, pad)).view(b.dtype)
         K += pad        # (the launch metadata below keeps the caller's K)
+    if (in_dt == _lib.F32 and isinstance(b, torch.Tensor) and b.stride(0) != 1 and K % 4 == 0 and M * N * K >= 1 << 24):
+        # fp32 operands run on the fp32 MFMAs with a K-major B only (the LDS transpose reads stop at 16-bit elements): a
+        # row-major B is put K-major first - one transposing copy, 1 / M of the product's work -; small products and a K
+        # that is not a multiple of four elements take the any-stride kernel of the C ABI as they are
+        b = b.t().contiguous().t()
     vec = 16 // _ELEM_BYTES[in_dt] if in_dt != _lib.F32 else 0
     if (vec and isinstance(b, torch.Tensor) and b.stride(1) == 1 and b.stride(0) != 1
             and (b.stride(0) % vec != 0 or b.data_ptr() % 16 != 0) and K % vec == 0 and M * N * K >= 1 << 30):
