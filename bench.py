@@ -275,7 +275,7 @@ def secondary_workloads(lib, dev, n):
                                 _lib.F32, _lib.F32, None, None, 0, stream)
             assert rc == 0, rc
 
-        return fn, flops, "flops", {"peak": "fp32", "data": "N(0,1) fp32, K-major B, fp32 out"}, 8
+        return fn, flops, "flops", {"peak": "fp32", "clock": True, "data": "N(0,1) fp32, K-major B, fp32 out"}, 8
     W["fp32_gemm_8192"] = fp32_gemm
 
     def fp8_decode():
