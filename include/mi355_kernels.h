@@ -145,7 +145,8 @@ int mi355_gemm_tuned(const void* A, const void* B, void* C,
  * C = act((a_scale * b_scale) * A @ B) with fp32 accumulation and one rounding, the partial sums added in split order.
  * Two launches: the tile kernel on 128x128 tiles into fp32 slices of `workspace`, then the sum and the epilogue.
  * workspace: device memory of at least splits * M * N * 4 bytes (32 * M * N * 4 always suffices for splits = 0),
- * 16-byte aligned, contents irrelevant; two calls that overlap in time need different workspaces.  Operands that the
+ * 16-byte aligned, contents irrelevant; two calls that overlap in time need different workspaces.  fp32 operands (K-major B)
+ * are split too, and sooner: their products are bound by the fp32 MFMA rate alone, so idle CUs are all that counts.  Operands that the
  * tile kernels do not take, or a K too short to split, run as mi355_gemm (the workspace is then not touched).
  */
 int mi355_gemm_splitk(const void* A, const void* B, void* C,

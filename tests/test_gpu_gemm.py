@@ -1187,7 +1187,7 @@ def test_skinny_kernel_with_64_columns_per_workgroup_is_bit_exact(gpu, dtype, sh
     assert bits_equal(got, gemm.matmul_closed_form(a, b, out_dtype="fp32") + d), (dtype, shape, "addend")
 
 
-@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3"])
+@pytest.mark.parametrize("dtype", ["fp16", "bf16", "e4m3", "fp32"])
 @pytest.mark.parametrize("splits", [0, 2, 3, 7, 32])
 def test_split_k_is_bit_exact_on_integers(gpu, dtype, splits):
     # mi355_gemm_splitk through the C ABI: `splits` workgroups per 128x128 tile, fp32 partial tiles in the workspace,
@@ -1196,7 +1196,7 @@ def test_split_k_is_bit_exact_on_integers(gpu, dtype, splits):
     # of the split, a K with a tail below one 64-byte step, one tile only; both layouts of B; a strided C.
     lib = _lib.load()
     rng = np.random.default_rng(23 + splits)
-    abi = {"fp16": _lib.F16, "bf16": _lib.BF16, "e4m3": _lib.F8E4M3}[dtype]
+    abi = {"fp16": _lib.F16, "bf16": _lib.BF16, "e4m3": _lib.F8E4M3, "fp32": _lib.F32}[dtype]
     for (M, N, K) in [(256, 256, 4096), (130, 96, 8192), (384, 200, 2096), (128, 128, 16384), (512, 640, 1056)]:
         a = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
         b = rng.integers(-2, 3, size=(K, N)).astype(np.float32)
@@ -1210,7 +1210,7 @@ def test_split_k_is_bit_exact_on_integers(gpu, dtype, splits):
             ta = from_np(a, dtype, gpu)
             tbs = [from_np(np.ascontiguousarray(b.T), dtype, gpu).t()]
             if N % 8 == 0:
-                tbs.append(from_np(b, dtype, gpu))
+                tbs.append(from_np(b, dtype, gpu))     # (fp32: no tile kernel for a row-major B - the plain call's any-stride kernel)
         ws = torch.full((32 * M * N,), float("nan"), dtype=torch.float32, device=gpu)   # (contents must not matter)
         for tb in tbs:
             cbuf = torch.full((M, N + 5), 7.0, dtype=torch.float32, device=gpu)

@@ -412,14 +412,15 @@ int mi355_gemm_splitk(const void* A, const void* B, void* C, int M, int N, int K
                       int activation, int splits, void* workspace, size_t workspace_bytes, void* stream_) {
   if (!A || !B || !C || M <= 0 || N <= 0 || K <= 0 || splits < 0) return MI355_EINVAL;
   if (activation != MI355_ACT_NONE && activation != MI355_ACT_LEAKY_RELU) return MI355_EINVAL;
-  if (in_dtype < MI355_F16 || in_dtype > MI355_F8E5M2) return MI355_EDTYPE;
+  if (in_dtype < MI355_F16 || in_dtype > MI355_F32) return MI355_EDTYPE;
   if (out_dtype < MI355_F16 || out_dtype > MI355_F32) return MI355_EDTYPE;
   if (!device_info().gfx950) return MI355_EDEVICE;
   const int es = elem_size(in_dtype), vec = 16 / es;
   // what the tile kernels ask of the operands (as in mi355_gemm); anything else, or nothing to split: the plain call
   const bool a_ok = sak == 1 && sam % vec == 0 && sam >= K && aligned(A, 16) && K % vec == 0;
   const bool b_kmajor = sbk == 1 && sbn % vec == 0 && sbn >= K && aligned(B, 16);
-  const bool b_nmajor = sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
+  const bool is32 = in_dtype == MI355_F32;   // (fp32 operands: the fp32 MFMAs, K-major B only)
+  const bool b_nmajor = !is32 && sbn == 1 && sbk % vec == 0 && sbk >= (N + vec - 1) / vec * vec && aligned(B, 16);
   const bool pitch_ok = (int64_t)sam * es < (1 << 23) && (b_kmajor ? (int64_t)sbn * es < (1 << 23) : (int64_t)sbk * es < (1 << 26));
   const int64_t k_bytes = (int64_t)K * es;
   const int ksteps = (int)((k_bytes + 63) / 64);
@@ -429,6 +430,9 @@ int mi355_gemm_splitk(const void* A, const void* B, void* C, int M, int N, int K
     // of tiles on or below 64 K steps (measured: see ops.py::_splitk_splits)
     const long tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
     splits = tiles * 2 > cus || ksteps < 64 ? 1 : (int)std::min<long>(std::min<long>(cus / tiles, ksteps / 16), 32);
+    // (fp32: bound by the fp32 MFMA rate alone, 2048 cycles per K step of a 128x128 tile - whatever puts more CUs to work
+    // wins, down to eight K steps a slice; 1024^3: 74 -> 24 us)
+    if (is32) splits = tiles >= cus || ksteps < 16 ? 1 : (int)std::min<long>(std::min<long>((2 * cus + tiles - 1) / tiles, ksteps / 8), 32);
   }
   const int per = splits >= 2 ? (ksteps + splits - 1) / splits : ksteps;
   const int used = (ksteps + per - 1) / per;   // (no split is left empty)
@@ -443,8 +447,9 @@ int mi355_gemm_splitk(const void* A, const void* B, void* C, int M, int N, int K
   p.ldb = (b_kmajor ? sbn : sbk) * es;
   p.group_m = knob(knobs().group_m, 8);
   p.workspace = (float*)workspace;
-  const int rc = es == 1 ? gemm8_splitk_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, used, per * 64, stream)
-                         : gemm16_splitk_launch(p, in_dtype == MI355_BF16, b_kmajor, used, per * 64, stream);
+  const int rc = is32    ? gemm32_splitk_launch(p, used, per * 64, stream)
+                 : es == 1 ? gemm8_splitk_launch(p, in_dtype == MI355_F8E5M2, b_kmajor, used, per * 64, stream)
+                           : gemm16_splitk_launch(p, in_dtype == MI355_BF16, b_kmajor, used, per * 64, stream);
   if (rc != 0) return rc;
   GemmStridedArgs out{};
   out.C = C; out.M = M; out.N = N; out.scm = scm; out.scn = scn;

@@ -34,4 +34,8 @@ int gemm32_launch(const GemmArgs& p, int tile, hipStream_t stream) {
   return launch_gemm_tile<Cfg32, true>(p, tile, stream);
 }
 
+int gemm32_splitk_launch(const GemmArgs& p, int splits, int chunk_bytes, hipStream_t stream) {
+  return launch_gemm_splitk<Cfg32, true>(p, splits, chunk_bytes, stream);
+}
+
 }  // namespace mi355

@@ -114,6 +114,7 @@ int gemm32_launch(const GemmArgs& p, int tile, hipStream_t stream);   // fp32 op
 // partial tiles into p.workspace ([splits][M][N]); splitk_reduce_launch adds them up and does the epilogue
 int gemm16_splitk_launch(const GemmArgs& p, bool bf16, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream);
 int gemm8_splitk_launch(const GemmArgs& p, bool e5m2, bool b_kmajor, int splits, int chunk_bytes, hipStream_t stream);
+int gemm32_splitk_launch(const GemmArgs& p, int splits, int chunk_bytes, hipStream_t stream);   // fp32 operands, K-major B
 int splitk_reduce_launch(const GemmStridedArgs& out, const float* workspace, int splits, hipStream_t stream);   // A, B, K, in_dtype of `out` unused
 bool gemm_wave128_192_ok(const GemmArgs& p, bool b_kmajor, int in_dtype, int tile_m = 192);   // the same for tiles of 192 x 256 / 128 x 256
 bool gemm_wave128_ok(const GemmArgs& p, bool b_kmajor, int in_dtype);

@@ -93,7 +93,7 @@ def _scale_ptr(s, device):
 _cu_count = {}   # device index -> compute units
 
 
-def _splitk_splits(device, M, N, k_bytes):
+def _splitk_splits(device, M, N, k_bytes, fp32=False):
     """Number of K splits for `matmul` (0 = none): products with less than half a round of 128x128 tiles and a long K
     give every tile to several workgroups (`mi355_gemm_splitk`) - one workgroup per CU, at least sixteen 64-byte K steps
     each, at most 32 slices and 64 MiB of fp32 partial sums.  Shapes with at most 64 rows on a side (and up to 128
@@ -109,6 +109,13 @@ def _splitk_splits(device, M, N, k_bytes):
         cus = _cu_count[idx] = max(1, _lib.load().mi355_query(_lib.Q_CU_COUNT))
     tiles = -(-M // 128) * -(-N // 128)
     ksteps = -(-k_bytes // 64)
+    if fp32:
+        # bound by the fp32 MFMA rate alone: whatever puts more CUs to work wins, down to eight K steps a slice (two
+        # workgroups per CU; flushed do_bench, 1024^3: 74 -> 24 us)
+        if tiles >= cus or ksteps < 16:
+            return 0
+        splits = min(-(-2 * cus // tiles), ksteps // 8, 32, (64 << 20) // (4 * M * N))
+        return splits if splits >= 2 else 0
     if tiles * 2 > cus or ksteps < 64:
         return 0
     # one workgroup per CU, at least 16 K steps each (flushed do_bench, bf16, us by number of splits - 1 / 2 / 4 / 8 / 16 /
@@ -187,8 +194,9 @@ def matmul(a, b, activation="", *, out_dtype=None, a_scale=None, b_scale=None, a
     act = _lib.ACT_LEAKY_RELU if activation == "leaky_relu" else _lib.ACT_NONE
     stream = _stream()
     md = hooks.enter("mi355_gemm", stream, hooks.matmul_launch_metadata, ("mi355_gemm", M, N, K_caller, _ELEM_BYTES[in_dt]))
-    if add is None and not softmax and in_dt != _lib.F32 and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor):
-        splits = _splitk_splits(device, M, N, K * _ELEM_BYTES[in_dt])
+    if (add is None and not softmax and isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor)
+            and (in_dt != _lib.F32 or (b.stride(0) == 1 and K % 4 == 0))):
+        splits = _splitk_splits(device, M, N, K * _ELEM_BYTES[in_dt], in_dt == _lib.F32)
         if splits:
             # few tiles, long K: every tile's K range is shared out (the fp32 partial sums live in a buffer from
             # torch's caching allocator, which orders its reuse on this stream)
