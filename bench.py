@@ -545,6 +545,41 @@ def main():
             r["gemm_of_this_ceiling"] = round(ref / r["tflops"], 3) if ref else None
             ceiling[key] = r
         extra["bare_mfma_ceiling_random_operands"] = ceiling
+        # A control for the same question from the other side: the same kernels on the same full-size inputs with a
+        # QUARTER of the CUs at work (64 persistent programs instead of 256, MI355_GEMM_PROGRAMS / MI355_ATTN_PROGRAMS).
+        # The board then stays below its power cap and at its full clock, and the rate per CU at work, as a fraction of
+        # the peak per CU, is what the kernel's cycles amount to at the clock the peak is quoted at.  (Fewer CUs also
+        # share the caches and the memory among fewer: a control, not a projection of the whole device.)
+        quarter = {}
+        table = secondary_workloads(lib, dev, n)
+        def headline():
+            qa = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+            qb = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+            qc = torch.empty(n, n, device=dev, dtype=torch.bfloat16)
+
+            def fn():
+                rc = lib.mi355_gemm(qa.data_ptr(), qb.data_ptr(), qc.data_ptr(), n, n, n, n, 1, n, 1, n, 1,
+                                    _lib.BF16, _lib.BF16, None, None, 0, stream)
+                assert rc == 0, rc
+
+            return fn, flops, "flops", {"peak": "bf16"}, 20
+        for key, build in (("bf16_gemm_8192", headline), ("fp8_e4m3_gemm_8192", table["fp8_e4m3_gemm_8192"]),
+                           ("mxfp4_gemm_8192", table["mxfp4_gemm_8192"]), ("attn_fwd_causal", table["attn_fwd_causal"])):
+            fn, work, _, info, _ = build()
+            os.environ["MI355_GEMM_PROGRAMS"] = os.environ["MI355_ATTN_PROGRAMS"] = "64"
+            lib.mi355_refresh_env()
+            try:
+                settle(fn, 0.1)
+                _, ms, _ = time_launches(fn, 10, 2)
+                rec = {"programs": 64, "ms": round(ms, 4), "tflops": round(work / ms / 1e9, 1),
+                       "frac_of_peak_per_cu_at_work": round(work / ms / 1e9 * 4 / PEAK[info["peak"]], 4)}
+                rec.update(observed_board_state(fn, 0.5))
+            finally:
+                del os.environ["MI355_GEMM_PROGRAMS"], os.environ["MI355_ATTN_PROGRAMS"]
+                lib.mi355_refresh_env()
+            quarter[key] = rec
+            del fn
+        extra["quarter_of_the_cus_at_full_clock"] = quarter
         out["extra"] = extra
 
     if not args.no_cpu:
